@@ -1,0 +1,146 @@
+"""ctypes binding of libmi355_aten.so (declared in include/mi355_aten.h).
+
+This is the only place that touches the C ABI.  There is no fallback: if the library has
+not been built, or its ABI version differs, loading raises and every operator wrapper
+fails with it.
+"""
+
+import ctypes
+from ctypes import POINTER, c_char_p, c_double, c_int, c_int32, c_int64, c_void_p
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi355_aten.so"
+ABI_VERSION = 1
+MAX_DIMS = 8
+
+# mi355_dtype
+F32, F16, BF16, F64, I32, I64, I16, I8, U8, BOOL = range(10)
+DTYPE = {
+    torch.float32: F32,
+    torch.float16: F16,
+    torch.bfloat16: BF16,
+    torch.float64: F64,
+    torch.int32: I32,
+    torch.int64: I64,
+    torch.int16: I16,
+    torch.int8: I8,
+    torch.uint8: U8,
+    torch.bool: BOOL,
+}
+# mi355_binary_op / mi355_unary_op / mi355_reduce_op
+ADD, MUL, MAXIMUM = 0, 1, 2
+RELU, CLAMP = 0, 1
+SUM, MEAN, AMAX, ARGMAX = 0, 1, 2, 3
+
+
+class TensorDesc(ctypes.Structure):
+    """struct mi355_tensor"""
+
+    _fields_ = [
+        ("data", c_void_p),
+        ("dtype", c_int32),
+        ("ndim", c_int32),
+        ("sizes", c_int64 * MAX_DIMS),
+        ("strides", c_int64 * MAX_DIMS),
+    ]
+
+
+_P = POINTER(TensorDesc)
+
+# name -> (restype, argtypes); mirrors include/mi355_aten.h one to one.
+SIGNATURES = {
+    "mi355_abi_version": (c_int, []),
+    "mi355_last_error": (c_char_p, []),
+    "mi355_binary": (c_int, [c_int, _P, _P, c_double, c_int64, _P, c_void_p]),
+    "mi355_unary": (c_int, [c_int, _P, c_int, c_double, c_double, c_int64, c_int64, _P, c_void_p]),
+    "mi355_where": (c_int, [_P, _P, _P, _P, c_void_p]),
+    "mi355_copy": (c_int, [_P, _P, c_void_p]),
+    "mi355_reduce_workspace_bytes": (c_int64, [c_int, c_int, c_int64, c_int64, c_int64]),
+    "mi355_reduce": (
+        c_int,
+        [c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_void_p],
+    ),
+    "mi355_softmax": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p]),
+    "mi355_layer_norm": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
+         c_double, c_void_p],
+    ),
+    "mi355_gemm": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
+         c_int64, c_int64, c_double, c_double, c_int, c_void_p],
+    ),
+    "mi355_index_select": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p],
+    ),
+    "mi355_gather": (c_int, [_P, c_int, _P, _P, c_void_p, c_void_p]),
+}
+
+_lib = None
+
+
+def load():
+    """dlopen the kernel library once; raise if it is missing or of another ABI."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build the HIP kernels first "
+            "(python -m backendbench_amd._build); there is no fallback path"
+        )
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if a declared symbol is not exported
+        fn.restype = restype
+        fn.argtypes = argtypes
+    got = lib.mi355_abi_version()
+    if got != ABI_VERSION:
+        raise RuntimeError(f"libmi355_aten.so has ABI {got}, the Python side expects {ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def check(rc):
+    if rc != 0:
+        msg = load().mi355_last_error()
+        raise RuntimeError(f"mi355 kernel library error {rc}: {msg.decode() if msg else '?'}")
+
+
+def dtype_code(dtype):
+    try:
+        return DTYPE[dtype]
+    except KeyError:
+        raise NotImplementedError(f"mi355 backend: dtype {dtype} is not supported") from None
+
+
+def desc(t, sizes=None, strides=None):
+    """mi355_tensor for `t`, optionally viewed with other sizes/strides (elements)."""
+    if sizes is None:
+        sizes = t.shape
+        strides = t.stride()
+    nd = len(sizes)
+    if nd > MAX_DIMS:
+        raise NotImplementedError(f"mi355 backend: {nd}-d tensors exceed the {MAX_DIMS}-d limit")
+    d = TensorDesc()
+    d.data = t.data_ptr()
+    d.dtype = dtype_code(t.dtype)
+    d.ndim = nd
+    for i in range(nd):
+        d.sizes[i] = sizes[i]
+        d.strides[i] = strides[i]
+    return d
+
+
+def current_stream_handle():
+    """hipStream_t of torch's current stream, so callers' events bracket our kernels."""
+    return torch.cuda.current_stream().cuda_stream
+
+
+def require_gpu():
+    if not torch.cuda.is_available():
+        raise RuntimeError("mi355 backend: no GPU visible; these operators only run on an MI355X (HIP) device")

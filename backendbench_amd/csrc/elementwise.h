@@ -1,0 +1,306 @@
+// Elementwise launch framework: one functor type F describes an op
+//   F::out_t, F::in0_t, F::in1_t, F::in2_t, F::NIN, out_t operator()(in0_t, in1_t, in2_t)
+// and three kernel shapes cover every layout:
+//   flat      all operands share one dense (possibly permuted) layout: 1-D pass, 128-bit
+//             accesses, grid-stride loop sized to the chip;
+//   strided   any strides/broadcast, index split with multiply-shift division; vectorised
+//             along the innermost dim when every operand is unit-stride or broadcast there;
+//   strided64 the same with 64-bit index math for > 2^31 work items.
+#pragma once
+#include "common.h"
+
+namespace mi355 {
+
+template <typename T, int N> struct alignas(sizeof(T) * N) VecN { T v[N]; };
+
+template <typename T, int N> __device__ __forceinline__ VecN<T, N> ld(const T* p) {
+  return *reinterpret_cast<const VecN<T, N>*>(p);
+}
+template <typename T, int N> __device__ __forceinline__ void st(T* p, const VecN<T, N>& v) {
+  *reinterpret_cast<VecN<T, N>*>(p) = v;
+}
+
+template <typename F> struct EwTraits {
+  static constexpr int NIN = F::NIN;
+  static constexpr int NT = NIN + 1;
+  static constexpr int max_size() {
+    int m = sizeof(typename F::out_t);
+    if (NIN > 0 && (int)sizeof(typename F::in0_t) > m) m = sizeof(typename F::in0_t);
+    if (NIN > 1 && (int)sizeof(typename F::in1_t) > m) m = sizeof(typename F::in1_t);
+    if (NIN > 2 && (int)sizeof(typename F::in2_t) > m) m = sizeof(typename F::in2_t);
+    return m;
+  }
+  static constexpr int V = 16 / max_size();  // elements per thread-vector
+};
+
+struct EwPtrs {
+  const void* in[3];
+  void* out;
+};
+
+template <typename F, int V, typename VA, typename VB, typename VC>
+__device__ __forceinline__ VecN<typename F::out_t, V> ew_apply(const F& f, const VA& a, const VB& b,
+                                                              const VC& c) {
+  VecN<typename F::out_t, V> r;
+#pragma unroll
+  for (int j = 0; j < V; ++j) r.v[j] = f(a.v[j], b.v[j], c.v[j]);
+  return r;
+}
+
+// ---------------------------------------------------------------- flat
+constexpr int kEwBlock = 256;
+constexpr int kEwUnroll = 4;
+
+template <typename F>
+__global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_t n) {
+  using TO = typename F::out_t;
+  using T0 = typename F::in0_t;
+  using T1 = typename F::in1_t;
+  using T2 = typename F::in2_t;
+  constexpr int V = EwTraits<F>::V;
+  constexpr int NIN = F::NIN;
+  const T0* a = static_cast<const T0*>(p.in[0]);
+  const T1* b = static_cast<const T1*>(p.in[1]);
+  const T2* c = static_cast<const T2*>(p.in[2]);
+  TO* o = static_cast<TO*>(p.out);
+
+  const int64_t nvec = n / V;
+  const int64_t stride = (int64_t)gridDim.x * kEwBlock;
+  int64_t i = (int64_t)blockIdx.x * kEwBlock + threadIdx.x;
+  for (; i + (kEwUnroll - 1) * stride < nvec; i += kEwUnroll * stride) {
+    VecN<T0, V> va[kEwUnroll];
+    VecN<T1, V> vb[kEwUnroll];
+    VecN<T2, V> vc[kEwUnroll];
+#pragma unroll
+    for (int u = 0; u < kEwUnroll; ++u) {
+      const int64_t e = (i + u * stride) * V;
+      va[u] = ld<T0, V>(a + e);
+      if constexpr (NIN > 1) vb[u] = ld<T1, V>(b + e);
+      if constexpr (NIN > 2) vc[u] = ld<T2, V>(c + e);
+    }
+#pragma unroll
+    for (int u = 0; u < kEwUnroll; ++u) {
+      const int64_t e = (i + u * stride) * V;
+      st<TO, V>(o + e, ew_apply<F, V>(f, va[u], vb[u], vc[u]));
+    }
+  }
+  for (; i < nvec; i += stride) {
+    const int64_t e = i * V;
+    VecN<T0, V> va = ld<T0, V>(a + e);
+    VecN<T1, V> vb;
+    VecN<T2, V> vc;
+    if constexpr (NIN > 1) vb = ld<T1, V>(b + e);
+    if constexpr (NIN > 2) vc = ld<T2, V>(c + e);
+    st<TO, V>(o + e, ew_apply<F, V>(f, va, vb, vc));
+  }
+  // ragged tail (< V elements), first threads of block 0
+  if (blockIdx.x == 0) {
+    const int64_t e = nvec * V + threadIdx.x;
+    if (e < n) {
+      T1 sb{};
+      T2 sc{};
+      if constexpr (NIN > 1) sb = b[e];
+      if constexpr (NIN > 2) sc = c[e];
+      o[e] = f(a[e], sb, sc);
+    }
+  }
+}
+
+// Same pass with scalar accesses, for operands whose base is not vector-aligned.
+template <typename F>
+__global__ __launch_bounds__(kEwBlock) void ew_flat_scalar_kernel(F f, EwPtrs p, int64_t n) {
+  using TO = typename F::out_t;
+  using T0 = typename F::in0_t;
+  using T1 = typename F::in1_t;
+  using T2 = typename F::in2_t;
+  constexpr int NIN = F::NIN;
+  const T0* a = static_cast<const T0*>(p.in[0]);
+  const T1* b = static_cast<const T1*>(p.in[1]);
+  const T2* c = static_cast<const T2*>(p.in[2]);
+  TO* o = static_cast<TO*>(p.out);
+  const int64_t stride = (int64_t)gridDim.x * kEwBlock;
+  for (int64_t e = (int64_t)blockIdx.x * kEwBlock + threadIdx.x; e < n; e += stride) {
+    T1 sb{};
+    T2 sc{};
+    if constexpr (NIN > 1) sb = b[e];
+    if constexpr (NIN > 2) sc = c[e];
+    o[e] = f(a[e], sb, sc);
+  }
+}
+
+// ---------------------------------------------------------------- strided
+// n / d for n < 2^31 as (umulhi(n, m) + n) >> s.
+struct FastDiv {
+  uint32_t d, m, s;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+  FastDiv f;
+  f.d = d;
+  f.s = 0;
+  while ((1ull << f.s) < d) ++f.s;
+  f.m = (uint32_t)(((1ull << 32) * ((1ull << f.s) - d)) / d + 1);
+  return f;
+}
+
+template <int NT> struct StridedArgs {
+  int32_t ndim;
+  uint32_t splat_mask;  // bit t: input t is broadcast along the vectorised inner dim
+  FastDiv div[MI355_MAX_DIMS];
+  int64_t sizes[MI355_MAX_DIMS];
+  int64_t strides[NT][MI355_MAX_DIMS];  // element strides; [NT-1] is the output
+};
+
+template <typename T, int V>
+__device__ __forceinline__ VecN<T, V> ld_or_splat(const T* p, bool splat) {
+  if (V == 1 || splat) {
+    VecN<T, V> r;
+    const T s = *p;
+#pragma unroll
+    for (int j = 0; j < V; ++j) r.v[j] = s;
+    return r;
+  }
+  return ld<T, V>(p);
+}
+
+// One work item = V consecutive elements of the innermost dim (V == 1: one element).
+template <typename F, int V, bool WIDE>
+__global__ __launch_bounds__(kEwBlock) void ew_strided_kernel(F f, EwPtrs p,
+                                                               StridedArgs<F::NIN + 1> a,
+                                                               int64_t total) {
+  using TO = typename F::out_t;
+  using T0 = typename F::in0_t;
+  using T1 = typename F::in1_t;
+  using T2 = typename F::in2_t;
+  constexpr int NIN = F::NIN;
+  constexpr int NT = NIN + 1;
+  const int64_t stride = (int64_t)gridDim.x * kEwBlock;
+  for (int64_t lin = (int64_t)blockIdx.x * kEwBlock + threadIdx.x; lin < total; lin += stride) {
+    int64_t off[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) off[t] = 0;
+    if constexpr (WIDE) {
+      int64_t rem = lin;
+      for (int k = a.ndim - 1; k >= 0; --k) {
+        const int64_t q = rem / a.sizes[k];
+        const int64_t idx = rem - q * a.sizes[k];
+        rem = q;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) off[t] += idx * a.strides[t][k];
+      }
+    } else {
+      uint32_t rem = (uint32_t)lin;
+      for (int k = a.ndim - 1; k >= 0; --k) {
+        const FastDiv d = a.div[k];
+        const uint32_t q = (uint32_t)(((uint64_t)__umulhi(rem, d.m) + rem) >> d.s);
+        const uint32_t idx = rem - q * d.d;
+        rem = q;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) off[t] += (int64_t)idx * a.strides[t][k];
+      }
+    }
+    VecN<T0, V> va = ld_or_splat<T0, V>(static_cast<const T0*>(p.in[0]) + off[0], a.splat_mask & 1u);
+    VecN<T1, V> vb;
+    VecN<T2, V> vc;
+    if constexpr (NIN > 1)
+      vb = ld_or_splat<T1, V>(static_cast<const T1*>(p.in[1]) + off[1], a.splat_mask & 2u);
+    if constexpr (NIN > 2)
+      vc = ld_or_splat<T2, V>(static_cast<const T2*>(p.in[2]) + off[2], a.splat_mask & 4u);
+    st<TO, V>(static_cast<TO*>(p.out) + off[NT - 1], ew_apply<F, V>(f, va, vb, vc));
+  }
+}
+
+// ---------------------------------------------------------------- host launcher
+template <typename F>
+int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_tensor* out,
+                       hipStream_t stream, const char* name) {
+  constexpr int NIN = F::NIN;
+  constexpr int NT = NIN + 1;
+  constexpr int V = EwTraits<F>::V;
+  const size_t esz[4] = {sizeof(typename F::in0_t), sizeof(typename F::in1_t),
+                         sizeof(typename F::in2_t), sizeof(typename F::out_t)};
+  for (int t = 0; t < NIN; ++t)
+    if (!same_shape(ins[t], out))
+      return set_error(MI355_ERR_INVALID, "%s: operand %d shape differs from output shape", name, t);
+  const int64_t n = numel(out);
+  if (n == 0) return MI355_OK;
+
+  const mi355_tensor* ts[NT];
+  for (int t = 0; t < NIN; ++t) ts[t] = ins[t];
+  ts[NIN] = out;
+  EwPtrs p{};
+  for (int t = 0; t < NIN; ++t) p.in[t] = ins[t]->data;
+  p.out = out->data;
+  const int max_blocks = kNumCU * 8;
+
+  if (same_dense_layout(ts, NT)) {
+    bool vec_ok = (reinterpret_cast<uintptr_t>(out->data) % (esz[3] * V)) == 0;
+    for (int t = 0; t < NIN; ++t)
+      vec_ok = vec_ok && (reinterpret_cast<uintptr_t>(ins[t]->data) % (esz[t] * V)) == 0;
+    if (vec_ok) {
+      const int grid = grid_for((n + V - 1) / V, kEwBlock * kEwUnroll, max_blocks);
+      hipLaunchKernelGGL(ew_flat_kernel<F>, dim3(grid), dim3(kEwBlock), 0, stream, f, p, n);
+    } else {
+      const int grid = grid_for(n, kEwBlock, max_blocks);
+      hipLaunchKernelGGL(ew_flat_scalar_kernel<F>, dim3(grid), dim3(kEwBlock), 0, stream, f, p, n);
+    }
+    return check_launch(name);
+  }
+
+  // Output stride for broadcast-free iteration must be real (no stride-0 output dims).
+  for (int i = 0; i < out->ndim; ++i)
+    if (out->sizes[i] > 1 && out->strides[i] == 0)
+      return set_error(MI355_ERR_INVALID, "%s: output has a broadcast (stride 0) dim", name);
+
+  const int64_t* strides[NT];
+  for (int t = 0; t < NT; ++t) strides[t] = ts[t]->strides;
+  Dims<NT> d = collapse_dims<NT>(out->ndim, out->sizes, strides);
+
+  // Vectorise along the innermost collapsed dim when every operand is unit-stride (or
+  // broadcast) there and every vector stays aligned.
+  const int last = d.ndim - 1;
+  bool vec_ok = V > 1 && d.sizes[last] % V == 0 && d.strides[NT - 1][last] == 1;
+  uint32_t splat = 0;
+  for (int t = 0; t < NT && vec_ok; ++t) {
+    const int64_t s = d.strides[t][last];
+    if (t < NIN && s == 0) {
+      splat |= 1u << t;
+      continue;
+    }
+    if (s != 1) vec_ok = false;
+    if (reinterpret_cast<uintptr_t>(ts[t]->data) % (esz[t == NIN ? 3 : t] * V)) vec_ok = false;
+    for (int k = 0; k < last; ++k)
+      if (d.strides[t][k] % V) vec_ok = false;
+  }
+
+  StridedArgs<NT> a{};
+  a.ndim = d.ndim;
+  a.splat_mask = vec_ok ? splat : 0u;
+  for (int k = 0; k < MI355_MAX_DIMS; ++k) {
+    a.sizes[k] = d.sizes[k];
+    for (int t = 0; t < NT; ++t) a.strides[t][k] = d.strides[t][k];
+  }
+  int64_t total = n;
+  if (vec_ok) {
+    a.sizes[last] /= V;
+    for (int t = 0; t < NT; ++t) a.strides[t][last] *= V;
+    total = n / V;
+  }
+  const bool wide = total >= (int64_t(1) << 31);
+  if (!wide)
+    for (int k = 0; k < d.ndim; ++k) a.div[k] = make_fastdiv((uint32_t)a.sizes[k]);
+  const int grid = grid_for(total, kEwBlock, kNumCU * 32);
+  if (vec_ok) {
+    if (wide)
+      hipLaunchKernelGGL((ew_strided_kernel<F, V, true>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+    else
+      hipLaunchKernelGGL((ew_strided_kernel<F, V, false>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+  } else {
+    if (wide)
+      hipLaunchKernelGGL((ew_strided_kernel<F, 1, true>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+    else
+      hipLaunchKernelGGL((ew_strided_kernel<F, 1, false>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+  }
+  return check_launch(name);
+}
+
+}  // namespace mi355

@@ -1,0 +1,230 @@
+// index_select / embedding (row gather) and gather (element gather).  Both move bits,
+// never values, so every dtype of a given width shares a kernel and results are exact.
+//
+//   rows_wave   rows of >= 64 copy units: one wave64 per output row, 128-bit units when
+//               alignment allows, four loads in flight per lane;
+//   rows_elem   short rows: one thread per copy unit;
+//   gather      one thread per output element (or per 4 consecutive 32-bit elements when
+//               the index tensor is dense), index stream coalesced.
+// An out-of-range index is never dereferenced: the output is zero-filled there and the
+// device error flag is raised.
+#include "elementwise.h"
+
+namespace mi355 {
+
+constexpr int kIxBlock = 256;
+
+template <typename I> __device__ __forceinline__ int64_t load_index(const void* p, int64_t j) {
+  return (int64_t) static_cast<const I*>(p)[j];
+}
+
+template <typename U, typename I>
+__global__ __launch_bounds__(kIxBlock) void index_rows_wave_kernel(const U* __restrict__ src, const void* __restrict__ index,
+                                                                  U* __restrict__ out, int64_t outer, int64_t n_src,
+                                                                  int64_t n_idx, int64_t row_units, int32_t* err) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t wave0 = (int64_t)blockIdx.x * (kIxBlock / kWave) + threadIdx.x / kWave;
+  const int64_t nwaves = (int64_t)gridDim.x * (kIxBlock / kWave);
+  const int64_t rows = outer * n_idx;
+  for (int64_t r = wave0; r < rows; r += nwaves) {
+    const int64_t o = r / n_idx, j = r - o * n_idx;
+    const int64_t idx = load_index<I>(index, j);
+    U* dst = out + r * row_units;
+    if (idx < 0 || idx >= n_src) {
+      if (err && lane == 0) *err = 1;
+      for (int64_t u = lane; u < row_units; u += kWave) dst[u] = U{};
+      continue;
+    }
+    const U* s = src + (o * n_src + idx) * row_units;
+    int64_t u = lane;
+    for (; u + 3 * kWave < row_units; u += 4 * kWave) {
+      const U a = s[u], b = s[u + kWave], c = s[u + 2 * kWave], d = s[u + 3 * kWave];
+      dst[u] = a;
+      dst[u + kWave] = b;
+      dst[u + 2 * kWave] = c;
+      dst[u + 3 * kWave] = d;
+    }
+    for (; u < row_units; u += kWave) dst[u] = s[u];
+  }
+}
+
+template <typename U, typename I>
+__global__ __launch_bounds__(kIxBlock) void index_rows_elem_kernel(const U* __restrict__ src, const void* __restrict__ index,
+                                                                  U* __restrict__ out, int64_t outer, int64_t n_src,
+                                                                  int64_t n_idx, int64_t row_units, int32_t* err) {
+  const int64_t total = outer * n_idx * row_units;
+  const int64_t stride = (int64_t)gridDim.x * kIxBlock;
+  for (int64_t e = (int64_t)blockIdx.x * kIxBlock + threadIdx.x; e < total; e += stride) {
+    const int64_t r = e / row_units, u = e - r * row_units;
+    const int64_t o = r / n_idx, j = r - o * n_idx;
+    const int64_t idx = load_index<I>(index, j);
+    if (idx < 0 || idx >= n_src) {
+      if (err) *err = 1;
+      out[e] = U{};
+    } else {
+      out[e] = src[(o * n_src + idx) * row_units + u];
+    }
+  }
+}
+
+struct U128 {
+  uint32_t w[4];
+} __attribute__((aligned(16)));
+
+template <typename U>
+static int run_index_select(const void* src, const void* index, int idx_dtype, void* out, int64_t outer, int64_t n_src,
+                            int64_t n_idx, int64_t row_units, int32_t* err, hipStream_t st) {
+  const int64_t rows = outer * n_idx;
+  const bool i64 = idx_dtype == MI355_I64;
+  if (row_units >= kWave) {
+    const int grid = grid_for(rows, kIxBlock / kWave, kNumCU * 32);
+    if (i64) hipLaunchKernelGGL((index_rows_wave_kernel<U, int64_t>), dim3(grid), dim3(kIxBlock), 0, st, (const U*)src, index, (U*)out, outer, n_src, n_idx, row_units, err);
+    else hipLaunchKernelGGL((index_rows_wave_kernel<U, int32_t>), dim3(grid), dim3(kIxBlock), 0, st, (const U*)src, index, (U*)out, outer, n_src, n_idx, row_units, err);
+  } else {
+    const int grid = grid_for(rows * row_units, kIxBlock, kNumCU * 32);
+    if (i64) hipLaunchKernelGGL((index_rows_elem_kernel<U, int64_t>), dim3(grid), dim3(kIxBlock), 0, st, (const U*)src, index, (U*)out, outer, n_src, n_idx, row_units, err);
+    else hipLaunchKernelGGL((index_rows_elem_kernel<U, int32_t>), dim3(grid), dim3(kIxBlock), 0, st, (const U*)src, index, (U*)out, outer, n_src, n_idx, row_units, err);
+  }
+  return check_launch("mi355_index_select");
+}
+
+// ---------------------------------------------------------------- gather
+struct GatherArgs {
+  int32_t ndim, dim;
+  int64_t sizes[MI355_MAX_DIMS];        // index (= out) sizes
+  int64_t idx_strides[MI355_MAX_DIMS];  // index strides
+  int64_t src_strides[MI355_MAX_DIMS];
+  int64_t src_dim_size;
+};
+
+// One thread per VEC consecutive output elements along the last dim (VEC == 4 needs a
+// dense index tensor and a last-dim size divisible by 4).
+template <typename U, int VEC>
+__global__ __launch_bounds__(kIxBlock) void gather_kernel(const U* __restrict__ src, const int64_t* __restrict__ index,
+                                                         U* __restrict__ out, GatherArgs a, int64_t total,
+                                                         int32_t* err) {
+  const int64_t stride = (int64_t)gridDim.x * kIxBlock;
+  const int last = a.ndim - 1;
+  for (int64_t w = (int64_t)blockIdx.x * kIxBlock + threadIdx.x; w < total; w += stride) {
+    const int64_t e = w * VEC;
+    int64_t rem = e, ioff = 0, soff = 0, last_coord = 0;
+    for (int k = last; k >= 0; --k) {
+      const int64_t q = rem / a.sizes[k];
+      const int64_t c = rem - q * a.sizes[k];
+      rem = q;
+      ioff += c * a.idx_strides[k];
+      if (k == last) last_coord = c;
+      if (k != a.dim) soff += c * a.src_strides[k];
+    }
+    if constexpr (VEC == 1) {
+      const int64_t idx = index[ioff];
+      if (idx < 0 || idx >= a.src_dim_size) {
+        if (err) *err = 1;
+        out[e] = U{};
+      } else {
+        out[e] = src[soff + idx * a.src_strides[a.dim]];
+      }
+    } else {
+      (void)last_coord;
+      // dense index: the VEC indices are adjacent in memory and 16-byte aligned pairs
+      const VecN<int64_t, 2> i01 = ld<int64_t, 2>(index + e);
+      const VecN<int64_t, 2> i23 = ld<int64_t, 2>(index + e + 2);
+      const int64_t ix[4] = {i01.v[0], i01.v[1], i23.v[0], i23.v[1]};
+      VecN<U, 4> r;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (ix[j] < 0 || ix[j] >= a.src_dim_size) {
+          if (err) *err = 1;
+          r.v[j] = U{};
+        } else {
+          const int64_t extra = a.dim == last ? 0 : (int64_t)j * a.src_strides[last];
+          r.v[j] = src[soff + extra + ix[j] * a.src_strides[a.dim]];
+        }
+      }
+      st<U, 4>(out + e, r);
+    }
+  }
+}
+
+template <typename U>
+static int run_gather(const mi355_tensor* src, int dim, const mi355_tensor* index, const mi355_tensor* out,
+                      int32_t* err, hipStream_t st) {
+  GatherArgs a{};
+  a.ndim = index->ndim;
+  a.dim = dim;
+  a.src_dim_size = src->sizes[dim];
+  bool idx_dense = true;
+  int64_t expect = 1;
+  for (int k = index->ndim - 1; k >= 0; --k) {
+    a.sizes[k] = index->sizes[k];
+    a.idx_strides[k] = index->strides[k];
+    a.src_strides[k] = src->strides[k];
+    if (index->sizes[k] != 1 && index->strides[k] != expect) idx_dense = false;
+    expect *= index->sizes[k];
+  }
+  const int64_t n = numel(out);
+  const int last = index->ndim - 1;
+  const bool vec = sizeof(U) == 4 && idx_dense && a.sizes[last] % 4 == 0 && aligned16(index->data) &&
+                   aligned16(out->data);
+  if (vec) {
+    const int grid = grid_for(n / 4, kIxBlock, kNumCU * 32);
+    hipLaunchKernelGGL((gather_kernel<U, 4>), dim3(grid), dim3(kIxBlock), 0, st, (const U*)src->data,
+                       (const int64_t*)index->data, (U*)out->data, a, n / 4, err);
+  } else {
+    const int grid = grid_for(n, kIxBlock, kNumCU * 32);
+    hipLaunchKernelGGL((gather_kernel<U, 1>), dim3(grid), dim3(kIxBlock), 0, st, (const U*)src->data,
+                       (const int64_t*)index->data, (U*)out->data, a, n, err);
+  }
+  return check_launch("mi355_gather");
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_index_select(const void* src, int elem_size, int64_t outer, int64_t n_src, int64_t inner,
+                                  const void* index, int idx_dtype, int64_t n_idx, void* out, int32_t* err_flag,
+                                  void* stream) {
+  MI355_REQUIRE(outer >= 0 && n_src >= 0 && inner >= 0 && n_idx >= 0, "mi355_index_select: negative extent");
+  MI355_REQUIRE(elem_size == 1 || elem_size == 2 || elem_size == 4 || elem_size == 8,
+                "mi355_index_select: elem_size %d", elem_size);
+  MI355_REQUIRE(idx_dtype == MI355_I32 || idx_dtype == MI355_I64, "mi355_index_select: index must be i32 or i64");
+  if (outer == 0 || inner == 0 || n_idx == 0) return MI355_OK;
+  MI355_REQUIRE(index != nullptr && out != nullptr, "mi355_index_select: NULL data pointer");
+  MI355_REQUIRE(src != nullptr || n_src == 0, "mi355_index_select: NULL src");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const int64_t row_bytes = inner * elem_size;
+  const uintptr_t align = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out) | (uintptr_t)row_bytes;
+  if (align % 16 == 0) return run_index_select<U128>(src, index, idx_dtype, out, outer, n_src, n_idx, row_bytes / 16, err_flag, st);
+  if (align % 8 == 0) return run_index_select<uint64_t>(src, index, idx_dtype, out, outer, n_src, n_idx, row_bytes / 8, err_flag, st);
+  if (align % 4 == 0) return run_index_select<uint32_t>(src, index, idx_dtype, out, outer, n_src, n_idx, row_bytes / 4, err_flag, st);
+  if (align % 2 == 0) return run_index_select<uint16_t>(src, index, idx_dtype, out, outer, n_src, n_idx, row_bytes / 2, err_flag, st);
+  return run_index_select<uint8_t>(src, index, idx_dtype, out, outer, n_src, n_idx, row_bytes, err_flag, st);
+}
+
+extern "C" int mi355_gather(const mi355_tensor* src, int dim, const mi355_tensor* index, const mi355_tensor* out,
+                            int32_t* err_flag, void* stream) {
+  int rc;
+  if ((rc = check_tensor(src, "mi355_gather", "src"))) return rc;
+  if ((rc = check_tensor(index, "mi355_gather", "index"))) return rc;
+  if ((rc = check_tensor(out, "mi355_gather", "out"))) return rc;
+  MI355_REQUIRE(index->dtype == MI355_I64, "mi355_gather: index must be i64");
+  MI355_REQUIRE(src->ndim == index->ndim && src->ndim >= 1, "mi355_gather: src and index must have equal ndim >= 1");
+  MI355_REQUIRE(dim >= 0 && dim < src->ndim, "mi355_gather: dim %d out of range", dim);
+  MI355_REQUIRE(same_shape(index, out) && out->dtype == src->dtype, "mi355_gather: out must have index's shape and src's dtype");
+  int64_t expect = 1;
+  for (int k = out->ndim - 1; k >= 0; --k) {
+    MI355_REQUIRE(out->sizes[k] == 1 || out->strides[k] == expect, "mi355_gather: out must be dense");
+    expect *= out->sizes[k];
+    if (k != dim) MI355_REQUIRE(index->sizes[k] <= src->sizes[k], "mi355_gather: index.size(%d) exceeds src.size(%d)", k, k);
+  }
+  if (numel(out) == 0) return MI355_OK;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (dtype_size(src->dtype)) {
+    case 1: return run_gather<uint8_t>(src, dim, index, out, err_flag, st);
+    case 2: return run_gather<uint16_t>(src, dim, index, out, err_flag, st);
+    case 4: return run_gather<uint32_t>(src, dim, index, out, err_flag, st);
+    case 8: return run_gather<uint64_t>(src, dim, index, out, err_flag, st);
+    default: return set_error(MI355_ERR_UNSUPPORTED, "mi355_gather: unsupported dtype");
+  }
+}

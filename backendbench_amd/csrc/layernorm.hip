@@ -1,0 +1,209 @@
+// native_layer_norm over the last N elements of M dense rows: returns y, mean, rstd.
+//
+//   wave   row fits a wave's registers: one HBM read; mean by wave all-reduce, then the
+//          centred second moment from the same registers (exact two-step statistics at
+//          single-pass traffic); y written once;
+//   block  longer rows: per-thread Welford accumulation, Chan's pairwise merge across
+//          lanes (shuffles) and waves (LDS), then the row is re-read (L2) to normalise.
+#include <type_traits>
+
+#include "rowtile.h"
+
+namespace mi355 {
+
+constexpr int kLnBlock = 256;
+
+template <typename T, typename W, typename S, int NV, bool VEC>
+__global__ __launch_bounds__(kLnBlock) void layernorm_wave_kernel(const T* __restrict__ x, const W* __restrict__ w,
+                                                                 const W* __restrict__ b, T* __restrict__ y,
+                                                                 S* __restrict__ mean_out, S* __restrict__ rstd_out,
+                                                                 int64_t rows, int64_t n, float eps) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t row = (int64_t)blockIdx.x * (kLnBlock / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;
+  using Tile = RowTile<T, NV, VEC>;
+  constexpr int V = Tile::V;
+  Tile t;
+  t.load(x + row * n, n, lane, 0.f);
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int j = 0; j < V; ++j) s += t.v[k][j];
+  const float inv_n = 1.f / (float)n;
+  const float mean = wave_allreduce(s, SumOp()) * inv_n;
+  float q = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float d = Tile::col(k, j, lane) < n ? t.v[k][j] - mean : 0.f;
+      q += d * d;
+    }
+  const float var = wave_allreduce(q, SumOp()) * inv_n;
+  const float rstd = rsqrtf(var + eps);
+  if (lane == 0) {
+    mean_out[row] = static_cast<S>(mean);
+    rstd_out[row] = static_cast<S>(rstd);
+  }
+  T* out = y + row * n;
+  if constexpr (VEC) {
+    // gamma/beta come through L2 as whole vectors, one per slab, shared by every row.
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int64_t c = Tile::col(k, 0, lane);
+      if (c < n) {
+        VecN<W, V> g, be;
+        if (w) g = ld<W, V>(w + c);
+        if (b) be = ld<W, V>(b + c);
+        Vec<T> r;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          float f = (t.v[k][j] - mean) * rstd;
+          if (w) f *= static_cast<float>(g.v[j]);
+          if (b) f += static_cast<float>(be.v[j]);
+          r.v[j] = static_cast<T>(f);
+        }
+        store_vec(out + c, r);
+      }
+    }
+  } else {
+    t.store(out, n, lane, [=](float v, int64_t c) {
+      float r = (v - mean) * rstd;
+      if (w) r *= static_cast<float>(w[c]);
+      if (b) r += static_cast<float>(b[c]);
+      return r;
+    });
+  }
+}
+
+// Welford state and Chan's merge.
+struct WF {
+  float n, mean, m2;
+};
+__device__ __forceinline__ void wf_update(WF& a, float x) {
+  a.n += 1.f;
+  const float d = x - a.mean;
+  a.mean += d / a.n;
+  a.m2 += d * (x - a.mean);
+}
+__device__ __forceinline__ WF wf_merge(WF a, WF b) {
+  const float n = a.n + b.n;
+  if (n == 0.f) return a;
+  const float d = b.mean - a.mean;
+  const float fb = b.n / n;
+  return {n, a.mean + d * fb, a.m2 + b.m2 + d * d * a.n * fb};
+}
+__device__ __forceinline__ WF wf_wave_reduce(WF a) {
+#pragma unroll
+  for (int k = 1; k < kWave; k <<= 1) {
+    WF o{__shfl_xor(a.n, k, kWave), __shfl_xor(a.mean, k, kWave), __shfl_xor(a.m2, k, kWave)};
+    a = wf_merge(a, o);
+  }
+  return a;
+}
+
+template <typename T, typename W, typename S, bool VEC>
+__global__ __launch_bounds__(kLnBlock) void layernorm_block_kernel(const T* __restrict__ x, const W* __restrict__ w,
+                                                                  const W* __restrict__ b, T* __restrict__ y,
+                                                                  S* __restrict__ mean_out, S* __restrict__ rstd_out,
+                                                                  int64_t n, float eps) {
+  constexpr int V = Vec<T>::N;
+  __shared__ WF smem[kLnBlock / kWave];
+  const T* row = x + (int64_t)blockIdx.x * n;
+  T* out = y + (int64_t)blockIdx.x * n;
+  WF a{0.f, 0.f, 0.f};
+  if constexpr (VEC) {
+    for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kLnBlock * V) {
+      const Vec<T> t = load_vec(row + c);
+#pragma unroll
+      for (int j = 0; j < V; ++j) wf_update(a, static_cast<float>(t.v[j]));
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < n; c += kLnBlock) wf_update(a, static_cast<float>(row[c]));
+  }
+  a = wf_wave_reduce(a);
+  if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = a;
+  __syncthreads();
+  a = smem[0];
+#pragma unroll
+  for (int k = 1; k < kLnBlock / kWave; ++k) a = wf_merge(a, smem[k]);
+  const float mean = a.mean;
+  const float rstd = rsqrtf(a.m2 / (float)n + eps);
+  if (threadIdx.x == 0) {
+    mean_out[blockIdx.x] = static_cast<S>(mean);
+    rstd_out[blockIdx.x] = static_cast<S>(rstd);
+  }
+  for (int64_t c = threadIdx.x; c < n; c += kLnBlock) {
+    float r = (static_cast<float>(row[c]) - mean) * rstd;
+    if (w) r *= static_cast<float>(w[c]);
+    if (b) r += static_cast<float>(b[c]);
+    out[c] = static_cast<T>(r);
+  }
+}
+
+template <typename T, typename W, typename S>
+static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void* mv, void* rv, int64_t M,
+                  int64_t N, double eps, hipStream_t st) {
+  const T* x = static_cast<const T*>(xv);
+  const W* w = static_cast<const W*>(wv);
+  const W* b = static_cast<const W*>(bv);
+  T* y = static_cast<T*>(yv);
+  S* mean = static_cast<S*>(mv);
+  S* rstd = static_cast<S*>(rv);
+  constexpr int V = Vec<T>::N;
+  const bool vec = N % V == 0 && aligned16(x) && aligned16(y) &&
+                   reinterpret_cast<uintptr_t>(w) % (sizeof(W) * V) == 0 &&
+                   reinterpret_cast<uintptr_t>(b) % (sizeof(W) * V) == 0;
+  const int64_t nblk = (M + kLnBlock / kWave - 1) / (kLnBlock / kWave);
+  MI355_REQUIRE(M < (int64_t(1) << 31), "mi355_layer_norm: too many rows (%lld)", (long long)M);
+  const bool done = dispatch_row_tile<T>(N, [&](auto nv) {
+    constexpr int NV = decltype(nv)::value;
+    if (vec) hipLaunchKernelGGL((layernorm_wave_kernel<T, W, S, NV, true>), dim3((unsigned)nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+    else hipLaunchKernelGGL((layernorm_wave_kernel<T, W, S, NV, false>), dim3((unsigned)nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+  });
+  if (!done) {
+    if (vec) hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, true>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, (float)eps);
+    else hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, false>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, (float)eps);
+  }
+  return check_launch("mi355_layer_norm");
+}
+
+template <typename T, typename W>
+static int run_ln_stat(int stat_dtype, int dtype, const void* x, const void* w, const void* b, void* y, void* m,
+                       void* r, int64_t M, int64_t N, double eps, hipStream_t st) {
+  if (stat_dtype == MI355_F32) return run_ln<T, W, float>(x, w, b, y, m, r, M, N, eps, st);
+  if (stat_dtype == dtype) return run_ln<T, W, T>(x, w, b, y, m, r, M, N, eps, st);
+  return set_error(MI355_ERR_UNSUPPORTED, "mi355_layer_norm: stat dtype must be f32 or the input dtype");
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_layer_norm(const void* x, int dtype, const void* weight, const void* bias, int w_dtype,
+                                void* y, void* mean, void* rstd, int stat_dtype, int64_t M, int64_t N, double eps,
+                                void* stream) {
+  MI355_REQUIRE(M >= 0 && N > 0, "mi355_layer_norm: bad extents M=%lld N=%lld", (long long)M, (long long)N);
+  if (M == 0) return MI355_OK;
+  MI355_REQUIRE(x && y && mean && rstd, "mi355_layer_norm: NULL data pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool has_w = weight != nullptr || bias != nullptr;
+  if (!has_w) w_dtype = dtype;
+  switch (dtype) {
+    case MI355_F32:
+      if (w_dtype == MI355_F32) return run_ln_stat<float, float>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);
+      break;
+    case MI355_F16:
+      if (w_dtype == MI355_F16) return run_ln_stat<f16_t, f16_t>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);
+      if (w_dtype == MI355_F32) return run_ln_stat<f16_t, float>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);
+      break;
+    case MI355_BF16:
+      if (w_dtype == MI355_BF16) return run_ln_stat<bf16_t, bf16_t>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);
+      if (w_dtype == MI355_F32) return run_ln_stat<bf16_t, float>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);
+      break;
+    default: break;
+  }
+  return set_error(MI355_ERR_UNSUPPORTED, "mi355_layer_norm: no kernel for x %s with weight %s", dtype_name(dtype),
+                   dtype_name(w_dtype));
+}

@@ -1,0 +1,423 @@
+// sum / mean / amax / argmax over the middle axis of a dense [outer, red, inner] view.
+//
+// Kernel shapes (picked by plan_reduce):
+//   rows_wave    inner == 1, many short rows: one wave64 per row, 128-bit loads, DPP +
+//                bpermute all-reduce, no LDS, no barrier;
+//   rows_block   inner == 1, long or few rows: one 256-thread block per (row, split),
+//                wave reduce then LDS combine across the four waves;
+//   rows_thread  inner == 1, red <= 32: one thread per row;
+//   cols         inner > 1: 64 lanes along inner (coalesced) x 4 along red, LDS combine;
+//   final        second pass over per-split partial states when a launch was split
+//                to fill the chip (few rows, long reduction).
+#include "common.h"
+
+#include <type_traits>
+
+namespace mi355 {
+
+// ---------------------------------------------------------------- reduction ops
+template <typename A> struct SumR {
+  using acc_t = A;
+  struct State { A s; };
+  static __device__ __forceinline__ State init() { return {A(0)}; }
+  static __device__ __forceinline__ void acc(State& st, A v, int64_t) { st.s += v; }
+  static __device__ __forceinline__ State combine(State a, State b) { return {a.s + b.s}; }
+  static __device__ __forceinline__ State shfl_xor(State a, int m) { return {__shfl_xor(a.s, m, kWave)}; }
+};
+template <typename A> struct AmaxR {
+  using acc_t = A;
+  struct State { A s; };
+  static __device__ __forceinline__ State init() {
+    if constexpr (IsFloat<A>::value) return {-INFINITY};
+    else if constexpr (sizeof(A) == 8) return {INT64_MIN};
+    else return {INT32_MIN};
+  }
+  static __device__ __forceinline__ void acc(State& st, A v, int64_t) { st.s = MaxNanOp()(st.s, v); }
+  static __device__ __forceinline__ State combine(State a, State b) { return {MaxNanOp()(a.s, b.s)}; }
+  static __device__ __forceinline__ State shfl_xor(State a, int m) { return {__shfl_xor(a.s, m, kWave)}; }
+};
+// (value, index) with ATen's order: NaN is the maximum, the lower index wins ties.
+template <typename A> struct ArgmaxR {
+  using acc_t = A;
+  struct State { A v; int64_t i; };
+  static __device__ __forceinline__ State init() { return {AmaxR<A>::init().s, INT64_MAX}; }
+  static __device__ __forceinline__ bool better(A v, int64_t i, A bv, int64_t bi) {
+    if constexpr (IsFloat<A>::value) {
+      const bool vn = v != v, bn = bv != bv;
+      if (vn || bn) return vn && (!bn || i < bi);
+    }
+    return v > bv || (v == bv && i < bi);
+  }
+  static __device__ __forceinline__ void acc(State& st, A v, int64_t i) {
+    if (better(v, i, st.v, st.i)) { st.v = v; st.i = i; }
+  }
+  static __device__ __forceinline__ State combine(State a, State b) {
+    return better(b.v, b.i, a.v, a.i) ? b : a;
+  }
+  static __device__ __forceinline__ State shfl_xor(State a, int m) {
+    return {__shfl_xor(a.v, m, kWave), (int64_t)__shfl_xor((long long)a.i, m, kWave)};
+  }
+};
+
+template <typename R> __device__ __forceinline__ typename R::State wave_reduce_state(typename R::State s) {
+#pragma unroll
+  for (int m = 1; m < kWave; m <<= 1) s = R::combine(s, R::shfl_xor(s, m));
+  return s;
+}
+// Scalar states take the DPP path.
+template <typename A> __device__ __forceinline__ typename SumR<A>::State wave_reduce(typename SumR<A>::State s, SumR<A>*) {
+  return {wave_allreduce(s.s, SumOp())};
+}
+template <typename A> __device__ __forceinline__ typename AmaxR<A>::State wave_reduce(typename AmaxR<A>::State s, AmaxR<A>*) {
+  return {wave_allreduce(s.s, MaxNanOp())};
+}
+template <typename A> __device__ __forceinline__ typename ArgmaxR<A>::State wave_reduce(typename ArgmaxR<A>::State s, ArgmaxR<A>*) {
+  return wave_reduce_state<ArgmaxR<A>>(s);
+}
+
+// Block reduce of a State (blockDim.x = 256): result valid in thread 0.
+template <typename R>
+__device__ __forceinline__ typename R::State block_reduce_state(typename R::State s, typename R::State* smem) {
+  s = wave_reduce(s, (R*)nullptr);
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int nwaves = blockDim.x / kWave;
+  if (lane == 0) smem[wave] = s;
+  __syncthreads();
+  if (threadIdx.x == 0)
+    for (int w = 1; w < nwaves; ++w) s = R::combine(s, smem[w]);
+  return s;
+}
+
+// How a final value leaves a kernel: SUM/AMAX write s, MEAN divides, ARGMAX writes i.
+enum { FIN_VALUE = 0, FIN_MEAN = 1, FIN_INDEX = 2 };
+template <typename R, typename O, int FIN>
+__device__ __forceinline__ void write_final(O* out, int64_t at, const typename R::State& st, double divisor) {
+  using A = typename R::acc_t;
+  if constexpr (FIN == FIN_INDEX) {
+    out[at] = (O)(((const typename ArgmaxR<A>::State&)st).i);
+  } else {
+    A v = *reinterpret_cast<const A*>(&st);
+    if constexpr (FIN == FIN_MEAN) v = v / (A)divisor;
+    out[at] = static_cast<O>(v);
+  }
+}
+
+// ---------------------------------------------------------------- kernels
+constexpr int kRedBlock = 256;
+
+// Accumulate x[base + lo .. base + hi) striding by `nthr` lanes starting at `tid`.
+template <typename T, typename R, bool VEC>
+__device__ __forceinline__ void accumulate_span(typename R::State& st, const T* row, int64_t lo, int64_t hi,
+                                                int tid, int nthr) {
+  using A = typename R::acc_t;
+  if constexpr (VEC) {
+    constexpr int V = Vec<T>::N;
+    // lo and hi are multiples of V (the planner guarantees it on the VEC path).
+    int64_t i = lo + (int64_t)tid * V;
+    const int64_t step = (int64_t)nthr * V;
+    for (; i + 3 * step < hi; i += 4 * step) {
+      Vec<T> v0 = load_vec(row + i), v1 = load_vec(row + i + step), v2 = load_vec(row + i + 2 * step),
+             v3 = load_vec(row + i + 3 * step);
+#pragma unroll
+      for (int j = 0; j < V; ++j) R::acc(st, (A)v0.v[j], i + j);
+#pragma unroll
+      for (int j = 0; j < V; ++j) R::acc(st, (A)v1.v[j], i + step + j);
+#pragma unroll
+      for (int j = 0; j < V; ++j) R::acc(st, (A)v2.v[j], i + 2 * step + j);
+#pragma unroll
+      for (int j = 0; j < V; ++j) R::acc(st, (A)v3.v[j], i + 3 * step + j);
+    }
+    for (; i < hi; i += step) {
+      Vec<T> v = load_vec(row + i);
+#pragma unroll
+      for (int j = 0; j < V; ++j) R::acc(st, (A)v.v[j], i + j);
+    }
+  } else {
+    for (int64_t i = lo + tid; i < hi; i += nthr) R::acc(st, (A)row[i], i);
+  }
+}
+
+template <typename T, typename O, typename R, int FIN, bool VEC>
+__global__ __launch_bounds__(kRedBlock) void rows_wave_kernel(const T* __restrict__ x, O* __restrict__ out,
+                                                             int64_t outer, int64_t red, double divisor) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t wave0 = (int64_t)blockIdx.x * (kRedBlock / kWave) + threadIdx.x / kWave;
+  const int64_t nwaves = (int64_t)gridDim.x * (kRedBlock / kWave);
+  for (int64_t row = wave0; row < outer; row += nwaves) {
+    typename R::State st = R::init();
+    accumulate_span<T, R, VEC>(st, x + row * red, 0, red, lane, kWave);
+    st = wave_reduce(st, (R*)nullptr);
+    if (lane == 0) write_final<R, O, FIN>(out, row, st, divisor);
+  }
+}
+
+// grid = (nsplit, outer).  PARTIAL: writes State to ws[row * nsplit + split].
+template <typename T, typename O, typename R, int FIN, bool VEC, bool PARTIAL>
+__global__ __launch_bounds__(kRedBlock) void rows_block_kernel(const T* __restrict__ x, O* __restrict__ out,
+                                                              typename R::State* __restrict__ ws, int64_t red,
+                                                              int64_t chunk, double divisor) {
+  __shared__ typename R::State smem[kRedBlock / kWave];
+  const int64_t row = blockIdx.y;
+  const int64_t lo = (int64_t)blockIdx.x * chunk;
+  const int64_t hi = lo + chunk < red ? lo + chunk : red;
+  typename R::State st = R::init();
+  accumulate_span<T, R, VEC>(st, x + row * red, lo, hi, threadIdx.x, kRedBlock);
+  st = block_reduce_state<R>(st, smem);
+  if (threadIdx.x == 0) {
+    if constexpr (PARTIAL) ws[row * gridDim.x + blockIdx.x] = st;
+    else write_final<R, O, FIN>(out, row, st, divisor);
+  }
+}
+
+template <typename T, typename O, typename R, int FIN>
+__global__ __launch_bounds__(kRedBlock) void rows_thread_kernel(const T* __restrict__ x, O* __restrict__ out,
+                                                               int64_t outer, int64_t red, double divisor) {
+  using A = typename R::acc_t;
+  const int64_t stride = (int64_t)gridDim.x * kRedBlock;
+  for (int64_t row = (int64_t)blockIdx.x * kRedBlock + threadIdx.x; row < outer; row += stride) {
+    typename R::State st = R::init();
+    const T* p = x + row * red;
+    for (int64_t i = 0; i < red; ++i) R::acc(st, (A)p[i], i);
+    write_final<R, O, FIN>(out, row, st, divisor);
+  }
+}
+
+// block = (64, 4); grid = (ceil(inner/64), nsplit, outer).
+template <typename T, typename O, typename R, int FIN, bool PARTIAL>
+__global__ __launch_bounds__(kRedBlock) void cols_kernel(const T* __restrict__ x, O* __restrict__ out,
+                                                        typename R::State* __restrict__ ws, int64_t red,
+                                                        int64_t inner, int64_t chunk, double divisor) {
+  using A = typename R::acc_t;
+  __shared__ typename R::State smem[4][kWave];
+  const int tx = threadIdx.x, ty = threadIdx.y;
+  const int64_t col = (int64_t)blockIdx.x * kWave + tx;
+  const int64_t o = blockIdx.z;
+  const int64_t lo = (int64_t)blockIdx.y * chunk;
+  const int64_t hi = lo + chunk < red ? lo + chunk : red;
+  typename R::State st = R::init();
+  if (col < inner) {
+    const T* p = x + o * red * inner + col;
+    for (int64_t r = lo + ty; r < hi; r += 4) R::acc(st, (A)p[r * inner], r);
+  }
+  smem[ty][tx] = st;
+  __syncthreads();
+  if (ty == 0 && col < inner) {
+    for (int k = 1; k < 4; ++k) st = R::combine(st, smem[k][tx]);
+    if constexpr (PARTIAL) ws[(o * gridDim.y + blockIdx.y) * inner + col] = st;
+    else write_final<R, O, FIN>(out, o * inner + col, st, divisor);
+  }
+}
+
+// partials [outer][nsplit][inner] -> out [outer][inner]
+template <typename O, typename R, int FIN>
+__global__ __launch_bounds__(kRedBlock) void final_kernel(const typename R::State* __restrict__ ws,
+                                                         O* __restrict__ out, int64_t outer, int64_t nsplit,
+                                                         int64_t inner, double divisor) {
+  const int64_t total = outer * inner;
+  const int64_t stride = (int64_t)gridDim.x * kRedBlock;
+  for (int64_t e = (int64_t)blockIdx.x * kRedBlock + threadIdx.x; e < total; e += stride) {
+    const int64_t o = e / inner, c = e - o * inner;
+    typename R::State st = ws[(o * nsplit) * inner + c];
+    for (int64_t s = 1; s < nsplit; ++s) st = R::combine(st, ws[(o * nsplit + s) * inner + c]);
+    write_final<R, O, FIN>(out, e, st, divisor);
+  }
+}
+
+// ---------------------------------------------------------------- planning
+enum Kind { ROWS_WAVE, ROWS_BLOCK, ROWS_THREAD, COLS };
+struct Plan {
+  Kind kind;
+  int64_t nsplit, chunk;
+};
+
+static Plan plan_reduce(int64_t outer, int64_t red, int64_t inner, int elem_size) {
+  Plan p{ROWS_BLOCK, 1, red};
+  const int V = 16 / elem_size;
+  const int64_t want_blocks = kNumCU * 4;
+  if (inner == 1) {
+    if (red <= 32 && outer >= 4096) { p.kind = ROWS_THREAD; return p; }
+    if (outer >= 2048 && red <= 16384) { p.kind = ROWS_WAVE; return p; }
+    p.kind = ROWS_BLOCK;
+    if (outer < 512) {
+      const int64_t unit = (int64_t)kRedBlock * V * 4;  // >= 4 vector loads per thread per split
+      int64_t ns = (want_blocks + outer - 1) / outer;
+      const int64_t max_ns = red / unit > 0 ? red / unit : 1;
+      if (ns > max_ns) ns = max_ns;
+      if (ns > 1) {
+        int64_t chunk = (red + ns - 1) / ns;
+        chunk = (chunk + kRedBlock * V - 1) / (kRedBlock * V) * (kRedBlock * V);
+        p.chunk = chunk;
+        p.nsplit = (red + chunk - 1) / chunk;
+      }
+    }
+    return p;
+  }
+  p.kind = COLS;
+  const int64_t base = outer * ((inner + kWave - 1) / kWave);
+  if (base < 512) {
+    int64_t ns = (want_blocks + base - 1) / base;
+    const int64_t max_ns = red / 32 > 0 ? red / 32 : 1;
+    if (ns > max_ns) ns = max_ns;
+    if (ns > 1) {
+      p.chunk = (red + ns - 1) / ns;
+      p.nsplit = (red + p.chunk - 1) / p.chunk;
+    }
+  }
+  return p;
+}
+
+template <typename T, typename O, typename R, int FIN>
+static int run_reduce(const void* xv, int64_t outer, int64_t red, int64_t inner, void* outv, void* wsv,
+                      int64_t ws_bytes, hipStream_t st) {
+  const T* x = static_cast<const T*>(xv);
+  O* out = static_cast<O*>(outv);
+  using State = typename R::State;
+  State* ws = static_cast<State*>(wsv);
+  const Plan p = plan_reduce(outer, red, inner, sizeof(T));
+  const double divisor = (double)red;
+  constexpr int V = Vec<T>::N;
+  if (p.nsplit > 1) {
+    const int64_t need = outer * p.nsplit * inner * (int64_t)sizeof(State);
+    MI355_REQUIRE(ws != nullptr && ws_bytes >= need,
+                  "mi355_reduce: workspace of %lld bytes needed, %lld given", (long long)need, (long long)ws_bytes);
+  }
+  switch (p.kind) {
+    case ROWS_THREAD: {
+      const int grid = grid_for(outer, kRedBlock, kNumCU * 16);
+      hipLaunchKernelGGL((rows_thread_kernel<T, O, R, FIN>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      break;
+    }
+    case ROWS_WAVE: {
+      const bool vec = aligned16(x) && red % V == 0;
+      const int grid = grid_for(outer, kRedBlock / kWave, kNumCU * 16);
+      if (vec) hipLaunchKernelGGL((rows_wave_kernel<T, O, R, FIN, true>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      else hipLaunchKernelGGL((rows_wave_kernel<T, O, R, FIN, false>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      break;
+    }
+    case ROWS_BLOCK: {
+      const bool vec = aligned16(x) && red % V == 0;
+      // grid.y carries rows: split oversize row counts over several launches.
+      for (int64_t r0 = 0; r0 < outer; r0 += 65535) {
+        const int64_t nr = outer - r0 < 65535 ? outer - r0 : 65535;
+        dim3 grid((unsigned)p.nsplit, (unsigned)nr);
+        const T* xr = x + r0 * red;
+        O* outr = out + r0;
+        State* wsr = ws ? ws + r0 * p.nsplit : nullptr;
+        if (p.nsplit > 1) {
+          if (vec) hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, true, true>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
+          else hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, false, true>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
+        } else {
+          if (vec) hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, true, false>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
+          else hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, false, false>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
+        }
+      }
+      break;
+    }
+    case COLS: {
+      const int64_t xb = (inner + kWave - 1) / kWave;
+      MI355_REQUIRE(xb < (int64_t(1) << 31) && p.nsplit < 65536, "mi355_reduce: inner extent too large");
+      for (int64_t o0 = 0; o0 < outer; o0 += 65535) {
+        const int64_t no = outer - o0 < 65535 ? outer - o0 : 65535;
+        dim3 grid((unsigned)xb, (unsigned)p.nsplit, (unsigned)no);
+        const T* xo = x + o0 * red * inner;
+        O* outo = out + o0 * inner;
+        State* wso = ws ? ws + o0 * p.nsplit * inner : nullptr;
+        if (p.nsplit > 1) hipLaunchKernelGGL((cols_kernel<T, O, R, FIN, true>), grid, dim3(kWave, 4), 0, st, xo, outo, wso, red, inner, p.chunk, divisor);
+        else hipLaunchKernelGGL((cols_kernel<T, O, R, FIN, false>), grid, dim3(kWave, 4), 0, st, xo, outo, wso, red, inner, p.chunk, divisor);
+      }
+      break;
+    }
+  }
+  int rc = check_launch("mi355_reduce");
+  if (rc) return rc;
+  if (p.nsplit > 1) {
+    const int grid = grid_for(outer * inner, kRedBlock, kNumCU * 8);
+    hipLaunchKernelGGL((final_kernel<O, R, FIN>), dim3(grid), dim3(kRedBlock), 0, st, ws, out, outer, p.nsplit, inner, divisor);
+    rc = check_launch("mi355_reduce(final)");
+  }
+  return rc;
+}
+
+template <typename T, typename O>
+static int run_op(int op, const void* x, int64_t outer, int64_t red, int64_t inner, void* out, void* ws,
+                  int64_t ws_bytes, hipStream_t st) {
+  using A = typename OpMath<T>::type;
+  using Acc = typename std::conditional<IsFloat<T>::value, A, int64_t>::type;  // ints sum in int64
+  switch (op) {
+    case MI355_SUM: return run_reduce<T, O, SumR<Acc>, FIN_VALUE>(x, outer, red, inner, out, ws, ws_bytes, st);
+    case MI355_MEAN:
+      if constexpr (IsFloat<T>::value) return run_reduce<T, O, SumR<Acc>, FIN_MEAN>(x, outer, red, inner, out, ws, ws_bytes, st);
+      else return set_error(MI355_ERR_UNSUPPORTED, "mi355_reduce: mean needs a floating dtype");
+    case MI355_AMAX: return run_reduce<T, O, AmaxR<A>, FIN_VALUE>(x, outer, red, inner, out, ws, ws_bytes, st);
+    default: return set_error(MI355_ERR_INVALID, "mi355_reduce: unknown op %d", op);
+  }
+}
+
+static size_t state_size(int op, int in_dtype) {
+  const bool is_f64 = in_dtype == MI355_F64, is_int = in_dtype == MI355_I32 || in_dtype == MI355_I64;
+  if (op == MI355_ARGMAX) return 16;
+  if (op == MI355_AMAX) return (is_f64 || in_dtype == MI355_I64) ? 8 : 4;
+  return (is_f64 || is_int) ? 8 : 4;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+// Bytes of scratch mi355_reduce needs for this problem (0 = single pass).
+extern "C" int64_t mi355_reduce_workspace_bytes(int op, int in_dtype, int64_t outer, int64_t red,
+                                                int64_t inner) {
+  const int es = dtype_size(in_dtype);
+  if (es == 0 || outer <= 0 || red <= 0 || inner <= 0) return 0;
+  const Plan p = plan_reduce(outer, red, inner, es);
+  if (p.nsplit <= 1) return 0;
+  return outer * p.nsplit * inner * (int64_t)state_size(op, in_dtype);
+}
+
+extern "C" int mi355_reduce(int op, const void* x, int in_dtype, int64_t outer, int64_t red, int64_t inner,
+                            void* out, int out_dtype, void* workspace, int64_t workspace_bytes, void* stream) {
+  MI355_REQUIRE(outer >= 0 && inner >= 0 && red > 0, "mi355_reduce: bad extents outer=%lld red=%lld inner=%lld",
+                (long long)outer, (long long)red, (long long)inner);
+  if (outer == 0 || inner == 0) return MI355_OK;
+  MI355_REQUIRE(x != nullptr && out != nullptr, "mi355_reduce: NULL data pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (op == MI355_ARGMAX) {
+    MI355_REQUIRE(out_dtype == MI355_I64, "mi355_reduce(argmax): out dtype must be i64");
+    switch (in_dtype) {
+      case MI355_F32: return run_reduce<float, int64_t, ArgmaxR<float>, FIN_INDEX>(x, outer, red, inner, out, workspace, workspace_bytes, st);
+      case MI355_F16: return run_reduce<f16_t, int64_t, ArgmaxR<float>, FIN_INDEX>(x, outer, red, inner, out, workspace, workspace_bytes, st);
+      case MI355_BF16: return run_reduce<bf16_t, int64_t, ArgmaxR<float>, FIN_INDEX>(x, outer, red, inner, out, workspace, workspace_bytes, st);
+      case MI355_F64: return run_reduce<double, int64_t, ArgmaxR<double>, FIN_INDEX>(x, outer, red, inner, out, workspace, workspace_bytes, st);
+      case MI355_I32: return run_reduce<int32_t, int64_t, ArgmaxR<int32_t>, FIN_INDEX>(x, outer, red, inner, out, workspace, workspace_bytes, st);
+      case MI355_I64: return run_reduce<int64_t, int64_t, ArgmaxR<int64_t>, FIN_INDEX>(x, outer, red, inner, out, workspace, workspace_bytes, st);
+      default: return set_error(MI355_ERR_UNSUPPORTED, "mi355_reduce(argmax): unsupported dtype %s", dtype_name(in_dtype));
+    }
+  }
+  const bool same = out_dtype == in_dtype;
+  switch (in_dtype) {
+    case MI355_F32:
+      if (same) return run_op<float, float>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      break;
+    case MI355_F16:
+      if (same) return run_op<f16_t, f16_t>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      if (out_dtype == MI355_F32) return run_op<f16_t, float>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      break;
+    case MI355_BF16:
+      if (same) return run_op<bf16_t, bf16_t>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      if (out_dtype == MI355_F32) return run_op<bf16_t, float>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      break;
+    case MI355_F64:
+      if (same) return run_op<double, double>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      break;
+    case MI355_I32:
+      if (op == MI355_AMAX && same) return run_op<int32_t, int32_t>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      if (op == MI355_SUM && out_dtype == MI355_I64) return run_op<int32_t, int64_t>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      break;
+    case MI355_I64:
+      if (same && op != MI355_MEAN) return run_op<int64_t, int64_t>(op, x, outer, red, inner, out, workspace, workspace_bytes, st);
+      break;
+    default: break;
+  }
+  return set_error(MI355_ERR_UNSUPPORTED, "mi355_reduce: no kernel for op %d, %s -> %s", op,
+                   dtype_name(in_dtype), dtype_name(out_dtype));
+}

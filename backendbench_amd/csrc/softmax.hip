@@ -1,0 +1,186 @@
+// _softmax over the middle axis of a dense [outer, dim, inner] view, fp32 math.
+//
+//   wave   inner == 1, row fits a wave's registers (<= 16 x 128-bit per lane): one HBM
+//          read, max and sum by wave all-reduce, one HBM write;
+//   block  inner == 1, longer rows: 256 threads keep an online (max, sum) pair in one
+//          pass, combine through LDS, then re-read the row (L2) to normalise;
+//   cols   inner > 1: one thread per (outer, inner) column, coalesced along inner,
+//          online pass then normalise pass.
+// exp(x - max) carries the special values: a +inf or NaN in the row, or a row of -inf,
+// turns the whole row into NaN, as ATen does.
+#include <type_traits>
+
+#include "rowtile.h"
+
+namespace mi355 {
+
+constexpr int kSmBlock = 256;
+
+template <typename T, typename O, int NV, bool VEC>
+__global__ __launch_bounds__(kSmBlock) void softmax_wave_kernel(const T* __restrict__ x, O* __restrict__ y,
+                                                               int64_t rows, int64_t n) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t row = (int64_t)blockIdx.x * (kSmBlock / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;
+  RowTile<T, NV, VEC> t;
+  constexpr int V = RowTile<T, NV, VEC>::V;
+  t.load(x + row * n, n, lane, -INFINITY);
+  float m = -INFINITY;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int j = 0; j < V; ++j) m = t.v[k][j] > m ? t.v[k][j] : m;
+  m = wave_allreduce(m, MaxOp());
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      t.v[k][j] = __expf(t.v[k][j] - m);
+      s += t.v[k][j];
+    }
+  // Padding lanes hold exp(-inf - m) = 0 unless m is -inf/NaN, where the row is NaN anyway.
+  s = wave_allreduce(s, SumOp());
+  const float inv = 1.f / s;
+  t.store(y + row * n, n, lane, [inv](float e, int64_t) { return e * inv; });
+}
+
+// Online (max, sum) pair; see the file header for the special-value rules.
+struct MS {
+  float m, s;
+};
+__device__ __forceinline__ void ms_update(MS& a, float x) {
+  if (x > a.m) {
+    a.s = a.s * __expf(a.m - x) + __expf(x - x);  // x - x is NaN for +inf
+    a.m = x;
+  } else if (x == -INFINITY) {
+    // contributes exactly zero
+  } else {
+    a.s += __expf(x - a.m);  // NaN x lands here and poisons the sum
+  }
+}
+__device__ __forceinline__ MS ms_combine(MS a, MS b) {
+  const float m = a.m > b.m ? a.m : b.m;
+  const float sa = a.m == -INFINITY ? a.s * 0.f : a.s * __expf(a.m - m);
+  const float sb = b.m == -INFINITY ? b.s * 0.f : b.s * __expf(b.m - m);
+  return {m, sa + sb};
+}
+__device__ __forceinline__ MS ms_wave_reduce(MS a) {
+#pragma unroll
+  for (int k = 1; k < kWave; k <<= 1) {
+    MS o{__shfl_xor(a.m, k, kWave), __shfl_xor(a.s, k, kWave)};
+    a = ms_combine(a, o);
+  }
+  return a;
+}
+
+template <typename T, typename O, bool VEC>
+__global__ __launch_bounds__(kSmBlock) void softmax_block_kernel(const T* __restrict__ x, O* __restrict__ y,
+                                                                int64_t n) {
+  constexpr int V = Vec<T>::N;
+  __shared__ MS smem[kSmBlock / kWave];
+  const T* row = x + (int64_t)blockIdx.x * n;
+  O* out = y + (int64_t)blockIdx.x * n;
+  MS a{-INFINITY, 0.f};
+  if constexpr (VEC) {
+    for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kSmBlock * V) {
+      const Vec<T> t = load_vec(row + c);
+#pragma unroll
+      for (int j = 0; j < V; ++j) ms_update(a, static_cast<float>(t.v[j]));
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < n; c += kSmBlock) ms_update(a, static_cast<float>(row[c]));
+  }
+  a = ms_wave_reduce(a);
+  if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = a;
+  __syncthreads();
+  a = smem[0];
+#pragma unroll
+  for (int w = 1; w < kSmBlock / kWave; ++w) a = ms_combine(a, smem[w]);
+  const float m = a.m, inv = 1.f / a.s;
+  if constexpr (VEC) {
+    for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kSmBlock * V) {
+      const Vec<T> t = load_vec(row + c);
+      VecN<O, V> r;
+#pragma unroll
+      for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(__expf(static_cast<float>(t.v[j]) - m) * inv);
+      st<O, V>(out + c, r);
+    }
+  } else {
+    for (int64_t c = threadIdx.x; c < n; c += kSmBlock)
+      out[c] = static_cast<O>(__expf(static_cast<float>(row[c]) - m) * inv);
+  }
+}
+
+template <typename T, typename O>
+__global__ __launch_bounds__(kSmBlock) void softmax_cols_kernel(const T* __restrict__ x, O* __restrict__ y,
+                                                               int64_t outer, int64_t n, int64_t inner) {
+  const int64_t total = outer * inner;
+  const int64_t stride = (int64_t)gridDim.x * kSmBlock;
+  for (int64_t e = (int64_t)blockIdx.x * kSmBlock + threadIdx.x; e < total; e += stride) {
+    const int64_t o = e / inner, c = e - o * inner;
+    const T* p = x + o * n * inner + c;
+    O* q = y + o * n * inner + c;
+    MS a{-INFINITY, 0.f};
+    for (int64_t r = 0; r < n; ++r) ms_update(a, static_cast<float>(p[r * inner]));
+    const float inv = 1.f / a.s;
+    for (int64_t r = 0; r < n; ++r)
+      q[r * inner] = static_cast<O>(__expf(static_cast<float>(p[r * inner]) - a.m) * inv);
+  }
+}
+
+template <typename T, typename O>
+static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64_t inner, hipStream_t st) {
+  const T* x = static_cast<const T*>(xv);
+  O* y = static_cast<O*>(yv);
+  constexpr int V = Vec<T>::N;
+  if (inner > 1) {
+    const int grid = grid_for(outer * inner, kSmBlock, kNumCU * 16);
+    hipLaunchKernelGGL((softmax_cols_kernel<T, O>), dim3(grid), dim3(kSmBlock), 0, st, x, y, outer, n, inner);
+    return check_launch("mi355_softmax(cols)");
+  }
+  const bool vec = n % V == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(y) % (sizeof(O) * V)) == 0;
+  const int64_t nblk = (outer + kSmBlock / kWave - 1) / (kSmBlock / kWave);
+  bool done = false;
+  if (nblk < (int64_t(1) << 31)) {
+    done = dispatch_row_tile<T>(n, [&](auto nv) {
+      constexpr int NV = decltype(nv)::value;
+      if (vec) hipLaunchKernelGGL((softmax_wave_kernel<T, O, NV, true>), dim3((unsigned)nblk), dim3(kSmBlock), 0, st, x, y, outer, n);
+      else hipLaunchKernelGGL((softmax_wave_kernel<T, O, NV, false>), dim3((unsigned)nblk), dim3(kSmBlock), 0, st, x, y, outer, n);
+    });
+  }
+  if (!done) {
+    MI355_REQUIRE(outer < (int64_t(1) << 31), "mi355_softmax: too many rows (%lld)", (long long)outer);
+    if (vec) hipLaunchKernelGGL((softmax_block_kernel<T, O, true>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
+    else hipLaunchKernelGGL((softmax_block_kernel<T, O, false>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
+  }
+  return check_launch("mi355_softmax");
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_softmax(const void* x, int in_dtype, void* y, int out_dtype, int64_t outer, int64_t dim,
+                             int64_t inner, void* stream) {
+  MI355_REQUIRE(outer >= 0 && dim >= 0 && inner >= 0, "mi355_softmax: negative extent");
+  if (outer == 0 || dim == 0 || inner == 0) return MI355_OK;
+  MI355_REQUIRE(x != nullptr && y != nullptr, "mi355_softmax: NULL data pointer");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (out_dtype == in_dtype) {
+    switch (in_dtype) {
+      case MI355_F32: return run_softmax<float, float>(x, y, outer, dim, inner, st);
+      case MI355_F16: return run_softmax<f16_t, f16_t>(x, y, outer, dim, inner, st);
+      case MI355_BF16: return run_softmax<bf16_t, bf16_t>(x, y, outer, dim, inner, st);
+      default: break;
+    }
+  } else if (out_dtype == MI355_F32) {  // half_to_float
+    switch (in_dtype) {
+      case MI355_F16: return run_softmax<f16_t, float>(x, y, outer, dim, inner, st);
+      case MI355_BF16: return run_softmax<bf16_t, float>(x, y, outer, dim, inner, st);
+      default: break;
+    }
+  }
+  return set_error(MI355_ERR_UNSUPPORTED, "mi355_softmax: no kernel for %s -> %s", dtype_name(in_dtype),
+                   dtype_name(out_dtype));
+}

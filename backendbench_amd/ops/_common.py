@@ -1,0 +1,148 @@
+"""Helpers shared by the operator wrappers: device management, dense/cast copies done
+with our own copy kernel, and the sticky out-of-range flag of the indexing kernels.
+
+The wrappers may run as the registered kernel of an ATen overload (torch.library
+override), so they never call an operator this backend overrides; allocation and view
+ops (empty, empty_like, empty_strided, expand, view, as_strided, to) are the only torch
+calls on tensors.
+"""
+
+import functools
+import os
+
+import torch
+
+from .. import _lib
+
+
+def _is_gpu(t):
+    return t.device.type == "cuda"
+
+
+def device_managed(fn):
+    """Run `fn` on the GPU whatever device the arguments live on.
+
+    Mirrors the contract the reference gives kernel authors
+    (BackendBench/prompts.py:18-24): CPU tensors are moved to the GPU, the result goes
+    back to the device of the first tensor argument, and a missing GPU is an error.
+    """
+
+    @functools.wraps(fn)
+    def wrapper(*args, **kwargs):
+        first = None
+        all_gpu = True
+        for a in args:
+            if isinstance(a, torch.Tensor):
+                if first is None:
+                    first = a
+                if a.device.type != "cuda":
+                    all_gpu = False
+        for a in kwargs.values():
+            if isinstance(a, torch.Tensor):
+                if first is None:
+                    first = a
+                if a.device.type != "cuda":
+                    all_gpu = False
+        if all_gpu:
+            return fn(*args, **kwargs)
+        _lib.require_gpu()
+        home = first.device
+        target = None
+        for a in list(args) + list(kwargs.values()):
+            if isinstance(a, torch.Tensor) and _is_gpu(a):
+                target = a.device
+                break
+        if target is None:
+            target = torch.device("cuda", torch.cuda.current_device())
+
+        def mv(a):
+            return a.to(target) if isinstance(a, torch.Tensor) and not _is_gpu(a) else a
+
+        out = fn(*[mv(a) for a in args], **{k: mv(v) for k, v in kwargs.items()})
+        if home.type == "cuda":
+            return out
+        if isinstance(out, torch.Tensor):
+            return out.to(home)
+        return tuple(o.to(home) for o in out)
+
+    return wrapper
+
+
+def launch(name, *args):
+    """Call one C entry point with the current stream appended; raise on failure."""
+    lib = _lib.load()
+    rc = getattr(lib, name)(*args, _lib.current_stream_handle())
+    if rc != 0:
+        _lib.check(rc)
+
+
+def copy_into(dst, src):
+    """dst[...] = src (cast + arbitrary strides) with the mi355_copy kernel."""
+    if dst.numel() == 0:
+        return dst
+    launch("mi355_copy", _lib.desc(src), _lib.desc(dst))
+    return dst
+
+
+def cast(t, dtype):
+    """`t` in `dtype`, layout preserved; no-op when the dtype already matches."""
+    if t.dtype == dtype:
+        return t
+    _lib.dtype_code(t.dtype)
+    _lib.dtype_code(dtype)
+    return copy_into(torch.empty_like(t, dtype=dtype), t)
+
+
+def dense(t):
+    """Row-major contiguous version of `t` (itself if it already is)."""
+    if t.is_contiguous():
+        return t
+    _lib.dtype_code(t.dtype)
+    return copy_into(torch.empty(t.shape, dtype=t.dtype, device=t.device), t)
+
+
+def prod(xs):
+    p = 1
+    for x in xs:
+        p *= x
+    return p
+
+
+def norm_dim(dim, ndim):
+    """ATen dim wrapping (a 0-d tensor accepts -1 and 0)."""
+    n = max(ndim, 1)
+    if not -n <= dim < n:
+        raise IndexError(f"Dimension out of range (expected to be in range of [{-n}, {n - 1}], but got {dim})")
+    return dim + n if dim < 0 else dim
+
+
+# ---- out-of-range indices ----------------------------------------------------------
+# The indexing kernels never dereference a bad index; they zero the output there and set a
+# device flag.  Reading the flag needs a device sync, so by default it is read only when
+# check_index_errors() is called (the evaluator does after every test); set
+# MI355_SYNC_INDEX_CHECK=1 to check after every indexing call, like the CPU kernels do.
+_flags = {}
+
+
+def index_error_flag(device):
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    f = _flags.get(key)
+    if f is None:
+        f = torch.zeros(1, dtype=torch.int32, device=device)
+        _flags[key] = f
+    return f
+
+
+def sync_index_check():
+    return os.environ.get("MI355_SYNC_INDEX_CHECK", "0") == "1"
+
+
+def check_index_errors():
+    """Raise IndexError if any indexing kernel saw an out-of-range index since the last call."""
+    bad = False
+    for f in _flags.values():
+        if int(f.item()) != 0:
+            bad = True
+            f.zero_()
+    if bad:
+        raise IndexError("index out of range in self")

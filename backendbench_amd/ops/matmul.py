@@ -1,0 +1,47 @@
+"""mm / addmm on the bf16/f16 MFMA kernel (fp32 accumulate) with a generic fallback."""
+
+import torch
+
+from .. import _lib
+from ._common import cast, device_managed, launch
+
+_GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+
+
+def _gemm(a, b, c, alpha, beta):
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError(f"mat1 and mat2 must be matrices, got {a.dim()}-D and {b.dim()}-D tensors")
+    if a.shape[1] != b.shape[0]:
+        raise RuntimeError(f"mat1 and mat2 shapes cannot be multiplied ({a.shape[0]}x{a.shape[1]} and "
+                           f"{b.shape[0]}x{b.shape[1]})")
+    if a.dtype != b.dtype:
+        raise RuntimeError(f"expected m1 and m2 to have the same dtype, but got: {a.dtype} != {b.dtype}")
+    if a.dtype not in _GEMM_DTYPES:
+        raise NotImplementedError(f"mi355 backend: matmul on {a.dtype} is not supported")
+    M, K = a.shape
+    N = b.shape[1]
+    out = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    if M == 0 or N == 0:
+        return out
+    if c is not None:
+        if c.dtype != a.dtype:
+            raise RuntimeError(f"self and mat2 must have the same dtype, but got {c.dtype} and {a.dtype}")
+        c = c.expand(M, N)  # raises like ATen when self cannot broadcast to [M, N]
+        c_ptr, c_rs, c_cs = c.data_ptr(), c.stride(0), c.stride(1)
+    else:
+        c_ptr, c_rs, c_cs = None, 0, 0
+    launch("mi355_gemm", a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), c_ptr,
+           c_rs, c_cs, out.data_ptr(), M, N, K, float(alpha), float(beta), _lib.dtype_code(a.dtype))
+    return out
+
+
+@device_managed
+def mm(self, mat2):
+    """aten.mm.default"""
+    return _gemm(self, mat2, None, 1.0, 0.0)
+
+
+@device_managed
+def addmm(self, mat1, mat2, *, beta=1, alpha=1):
+    """aten.addmm.default: beta * self + alpha * (mat1 @ mat2); beta == 0 never reads self."""
+    return _gemm(mat1, mat2, self, alpha, beta)

@@ -1,0 +1,231 @@
+"""sum / mean / amax / argmax, _softmax and native_layer_norm on the HIP row kernels.
+
+Every kernel sees a dense [outer, red, inner] view.  When the reduced dims are adjacent in
+a contiguous tensor that view is free; otherwise the operand is permuted/densified once
+with the copy kernel.
+"""
+
+import torch
+
+from .. import _lib
+from ._common import cast, copy_into, dense, device_managed, launch, norm_dim, prod
+
+_NATIVE_IN = (torch.float32, torch.float16, torch.bfloat16, torch.float64, torch.int32, torch.int64)
+_SMALL_INT = (torch.int16, torch.int8, torch.uint8, torch.bool)
+
+
+def _norm_dims(dim, ndim):
+    if dim is None:
+        return list(range(ndim))
+    if isinstance(dim, int):
+        dim = [dim]
+    dims = sorted({norm_dim(d, ndim) for d in dim}) if ndim > 0 else []
+    if len(dims) != len(list(dim)) and ndim > 0:
+        raise RuntimeError("dim appears multiple times in the list of dims")
+    if not dims:
+        return list(range(ndim))
+    return dims
+
+
+def _view3(x, dims):
+    """(dense tensor, outer, red, inner) with the dims in `dims` reduced."""
+    nd = x.dim()
+    if nd == 0:
+        return dense(x), 1, 1, 1
+    adjacent = dims == list(range(dims[0], dims[-1] + 1))
+    if adjacent:
+        xd = dense(x)
+        shape = x.shape
+        return xd, prod(shape[: dims[0]]), prod(shape[dims[0] : dims[-1] + 1]), prod(shape[dims[-1] + 1 :])
+    kept = [d for d in range(nd) if d not in dims]
+    xp = x.permute(kept + dims)
+    xd = copy_into(torch.empty(xp.shape, dtype=x.dtype, device=x.device), xp)
+    return xd, prod(x.shape[d] for d in kept), prod(x.shape[d] for d in dims), 1
+
+
+def _out_shape(x, dims, keepdim):
+    if x.dim() == 0:
+        return []
+    if keepdim:
+        return [1 if d in dims else s for d, s in enumerate(x.shape)]
+    return [s for d, s in enumerate(x.shape) if d not in dims]
+
+
+def _run_reduce(op, x, dims, keepdim, out_dtype):
+    """x: tensor of a natively reducible dtype with numel > 0 and red > 0."""
+    xd, outer, red, inner = _view3(x, dims)
+    out = torch.empty(_out_shape(x, dims, keepdim), dtype=out_dtype, device=x.device)
+    lib = _lib.load()
+    in_code, out_code = _lib.dtype_code(xd.dtype), _lib.dtype_code(out_dtype)
+    ws_bytes = lib.mi355_reduce_workspace_bytes(op, in_code, outer, red, inner)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    launch("mi355_reduce", op, xd.data_ptr(), in_code, outer, red, inner, out.data_ptr(), out_code,
+           ws.data_ptr() if ws is not None else None, ws_bytes)
+    return out
+
+
+def _sum_like(op, x, dim, keepdim, dtype, name):
+    dims = _norm_dims(dim, x.dim())
+    if dtype is None:
+        if x.dtype.is_floating_point:
+            dtype = x.dtype
+        elif op == _lib.MEAN:
+            raise RuntimeError(
+                f"{name}(): could not infer output dtype. Input dtype must be either a floating point or "
+                f"complex dtype. Got: {str(x.dtype).replace('torch.', '').capitalize()}")
+        else:
+            dtype = torch.int64
+    if dtype.is_complex or x.dtype.is_complex:
+        raise NotImplementedError("mi355 backend: complex reductions are not supported")
+    if op == _lib.MEAN and not dtype.is_floating_point:
+        raise RuntimeError(f"{name}(): could not infer output dtype. Optional dtype must be either a floating "
+                           f"point or complex dtype. Got: {str(dtype).replace('torch.', '').capitalize()}")
+    shape = _out_shape(x, dims, keepdim)
+    red = prod(x.shape[d] for d in dims) if x.dim() else 1
+    if x.numel() == 0:
+        fill = float("nan") if (op == _lib.MEAN and red == 0) else 0
+        return torch.full(shape, fill, dtype=dtype, device=x.device)
+    # Pick the dtype the kernel reads (`src`) and writes (`native_out`); cast around it.
+    if dtype.is_floating_point:
+        src = x if x.dtype.is_floating_point else cast(x, dtype)
+        if src.dtype != dtype and not (src.dtype in (torch.float16, torch.bfloat16) and dtype == torch.float32):
+            src = cast(src, dtype)
+        native_out = dtype
+    else:
+        src = cast(x, torch.int64) if x.dtype not in (torch.int32, torch.int64) else x
+        native_out = torch.int64
+    out = _run_reduce(op, src, dims, keepdim, native_out)
+    return cast(out, dtype)
+
+
+@device_managed
+def sum_dim(self, dim=None, keepdim=False, *, dtype=None):
+    """aten.sum.dim_IntList"""
+    return _sum_like(_lib.SUM, self, dim, keepdim, dtype, "sum")
+
+
+@device_managed
+def sum_default(self, *, dtype=None):
+    """aten.sum.default"""
+    return _sum_like(_lib.SUM, self, None, False, dtype, "sum")
+
+
+@device_managed
+def mean_dim(self, dim=None, keepdim=False, *, dtype=None):
+    """aten.mean.dim"""
+    return _sum_like(_lib.MEAN, self, dim, keepdim, dtype, "mean")
+
+
+@device_managed
+def mean_default(self, *, dtype=None):
+    """aten.mean.default"""
+    return _sum_like(_lib.MEAN, self, None, False, dtype, "mean")
+
+
+def _max_src(x):
+    if x.dtype in _NATIVE_IN:
+        return x
+    if x.dtype in _SMALL_INT:
+        return cast(x, torch.int32)  # value preserving
+    raise NotImplementedError(f"mi355 backend: dtype {x.dtype} is not supported")
+
+
+@device_managed
+def amax(self, dim=(), keepdim=False):
+    """aten.amax.default: NaN propagates; dim=[] reduces everything."""
+    dims = _norm_dims(list(dim), self.dim())
+    shape = _out_shape(self, dims, keepdim)
+    for d in dims:
+        if self.dim() and self.shape[d] == 0:
+            raise IndexError(f"amax(): Expected reduction dim {d} to have non-zero size.")
+    if self.numel() == 0:
+        return torch.empty(shape, dtype=self.dtype, device=self.device)
+    src = _max_src(self)
+    return cast(_run_reduce(_lib.AMAX, src, dims, keepdim, src.dtype), self.dtype)
+
+
+@device_managed
+def argmax(self, dim=None, keepdim=False):
+    """aten.argmax.default: first index of the maximum, NaN counts as maximum."""
+    if dim is None:
+        if self.numel() == 0:
+            raise IndexError("argmax(): Expected reduction dim to be specified for input.numel() == 0. Specify the reduction dim with the 'dim' argument.")
+        flat = dense(self).view(-1)
+        out = _run_reduce(_lib.ARGMAX, _max_src(flat), [0], False, torch.int64)
+        return out.view([1] * self.dim()) if keepdim else out
+    d = norm_dim(dim, self.dim())
+    if self.dim() and self.shape[d] == 0:
+        raise IndexError(f"argmax(): Expected reduction dim {d} to have non-zero size.")
+    dims = [d] if self.dim() else []
+    if self.numel() == 0:
+        return torch.empty(_out_shape(self, dims, keepdim), dtype=torch.int64, device=self.device)
+    return _run_reduce(_lib.ARGMAX, _max_src(self), dims, keepdim, torch.int64)
+
+
+@device_managed
+def softmax(self, dim, half_to_float):
+    """aten._softmax.default"""
+    if not self.dtype.is_floating_point:
+        raise RuntimeError("softmax expects a floating point input")
+    if half_to_float and self.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("conversion is supported for Half and BFloat16 type only")
+    out_dtype = torch.float32 if half_to_float else self.dtype
+    d = norm_dim(dim, self.dim())
+    out = torch.empty(self.shape, dtype=out_dtype, device=self.device)
+    if self.numel() == 0:
+        return out
+    if self.dtype == torch.float64:
+        raise NotImplementedError("mi355 backend: float64 softmax is not supported")
+    x = dense(self)
+    shape = x.shape if x.dim() else (1,)
+    launch("mi355_softmax", x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(out_dtype),
+           prod(shape[:d]), shape[d], prod(shape[d + 1 :]))
+    return out
+
+
+@device_managed
+def native_layer_norm(input, normalized_shape, weight, bias, eps):
+    """aten.native_layer_norm.default -> (y, mean, rstd).
+
+    mean/rstd are fp32 for f16/bf16 inputs (the accumulation type, as ATen's GPU kernels
+    return them) and shaped input.shape[:-k] + [1]*k.
+    """
+    k = len(normalized_shape)
+    if k == 0 or list(input.shape[input.dim() - k :]) != list(normalized_shape):
+        raise RuntimeError(
+            f"Given normalized_shape={list(normalized_shape)}, expected input with shape "
+            f"[*, {', '.join(str(s) for s in normalized_shape)}], but got input of size{list(input.shape)}")
+    for name, p in (("weight", weight), ("bias", bias)):
+        if p is not None and list(p.shape) != list(normalized_shape):
+            raise RuntimeError(f"Expected {name} to be of same shape as normalized_shape, but got {name} of shape "
+                               f"{list(p.shape)} and normalized_shape = {list(normalized_shape)}")
+    if input.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+        raise NotImplementedError(f"mi355 backend: layer norm on {input.dtype} is not supported")
+    lead = list(input.shape[: input.dim() - k])
+    M, N = prod(lead), prod(normalized_shape)
+    stat_dtype = torch.float32
+    y = torch.empty(input.shape, dtype=input.dtype, device=input.device)
+    mean = torch.empty(lead + [1] * k, dtype=stat_dtype, device=input.device)
+    rstd = torch.empty(lead + [1] * k, dtype=stat_dtype, device=input.device)
+    if M == 0:
+        return y, mean, rstd
+    if N == 0:
+        raise NotImplementedError("mi355 backend: layer norm over zero elements is not supported")
+    w_dtype = None
+    for p in (weight, bias):
+        if p is not None:
+            if w_dtype is not None and p.dtype != w_dtype:
+                raise RuntimeError("weight and bias must have the same dtype")
+            w_dtype = p.dtype
+    if w_dtype is not None and w_dtype != input.dtype:
+        if w_dtype != torch.float32:
+            weight = cast(weight, input.dtype) if weight is not None else None
+            bias = cast(bias, input.dtype) if bias is not None else None
+            w_dtype = input.dtype
+    x = dense(input)
+    w = dense(weight) if weight is not None else None
+    b = dense(bias) if bias is not None else None
+    launch("mi355_layer_norm", x.data_ptr(), _lib.dtype_code(x.dtype), w.data_ptr() if w is not None else None,
+           b.data_ptr() if b is not None else None, _lib.dtype_code(w_dtype or x.dtype), y.data_ptr(),
+           mean.data_ptr(), rstd.data_ptr(), _lib.dtype_code(stat_dtype), M, N, float(eps))
+    return y, mean, rstd

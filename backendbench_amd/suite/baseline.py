@@ -1,0 +1,409 @@
+"""The operator set's own test suite: headline shapes plus edge layouts.
+
+The reference's OpInfo / TorchBench / FACTO suites (BackendBench/suite/opinfo.py,
+torchbench.py, facto.py) need packages or downloads this environment does not have, so
+this module is the input source for the 19 operator slots: `perf_cases()` are the
+headline configurations (one per measured row: shapes, dtypes, distributions and the
+algorithmic bytes / flops used for roofline fractions) and `edge_cases()` are small
+inputs covering broadcasting, non-contiguous views, NaN / +-inf, ties, empty and 0-d
+tensors, integer dtypes and argument variants.  Every tensor is drawn on the CPU from a
+seeded generator and then moved, so any two devices see identical bits.
+"""
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List
+
+import torch
+
+from ..opregistry import get_operator
+from .base import OpTest, Test, TestSuite
+
+aten = torch.ops.aten
+
+
+@dataclass
+class Case:
+    key: str                 # e.g. "C2.softmax"
+    op: object               # OpOverload
+    make: Callable           # device -> (args, kwargs)
+    work: float = 0.0        # algorithmic bytes (bound == "hbm") or flops ("mfma") per call
+    bound: str = "hbm"
+    exact: bool = False      # outputs must be bit-identical to the reference
+    note: str = ""
+    extra: Dict = field(default_factory=dict)
+
+
+def _gen(seed):
+    return torch.Generator(device="cpu").manual_seed(seed)
+
+
+def normal(shape, dtype, mean=0.0, std=1.0, seed=0):
+    """N(mean, std) drawn in fp32 on the CPU, rounded once to `dtype`."""
+    t = torch.empty(shape, dtype=torch.float32)
+    t.normal_(mean, std, generator=_gen(seed))
+    return t.to(dtype)
+
+
+def randint(shape, high, seed=0, dtype=torch.int64, low=0):
+    return torch.randint(low, high, shape, generator=_gen(seed), dtype=dtype)
+
+
+def poison(t, frac=0.01, seed=0):
+    """Set `frac` of the elements to NaN, +inf, -inf (a third each) at seeded positions."""
+    flat = t.reshape(-1)
+    n = flat.numel()
+    k = max(3, int(n * frac)) if n >= 3 else 0
+    if k == 0:
+        return t
+    pos = torch.randperm(n, generator=_gen(seed))[:k]
+    third = k // 3
+    flat[pos[:third]] = float("nan")
+    flat[pos[third : 2 * third]] = float("inf")
+    flat[pos[2 * third :]] = float("-inf")
+    return t
+
+
+def _to(device, *tensors):
+    return [t.to(device) if isinstance(t, torch.Tensor) else t for t in tensors]
+
+
+# ---------------------------------------------------------------- headline configurations
+def perf_cases(scale: float = 1.0) -> List[Case]:
+    """One Case per measured row.  `scale` < 1 shrinks the leading extent of every shape
+    (same kernels, same layouts) for quick runs on small machines."""
+
+    def S(n, mult=1):
+        return max(mult, int(n * scale) // mult * mult)
+
+    bf16, f16, f32 = torch.bfloat16, torch.float16, torch.float32
+    cases = []
+
+    # C1: add.Tensor then relu, fp32 contiguous [4096, 4096]
+    m1 = S(4096)
+    cases.append(Case("C1.add", aten.add.Tensor,
+                      lambda d: (_to(d, normal((m1, 4096), f32, seed=1), normal((m1, 4096), f32, seed=2)), {}),
+                      work=3 * 4 * m1 * 4096))
+    cases.append(Case("C1.relu", aten.relu.default,
+                      lambda d: (_to(d, normal((m1, 4096), f32, seed=1) + normal((m1, 4096), f32, seed=2)), {}),
+                      work=2 * 4 * m1 * 4096, note="input is the C1 add result"))
+
+    # C2: row ops on bf16 [8192, 4096], N(0, 2)
+    m2, n2 = S(8192), 4096
+    x2 = lambda: normal((m2, n2), bf16, 0.0, 2.0, seed=3)
+    cases.append(Case("C2.softmax", aten._softmax.default, lambda d: (_to(d, x2(), -1, False), {}),
+                      work=2 * 2 * m2 * n2))
+    cases.append(Case("C2.layer_norm", aten.native_layer_norm.default,
+                      lambda d: (_to(d, x2(), [n2], normal((n2,), bf16, 1.0, 0.1, seed=4),
+                                     normal((n2,), bf16, 0.0, 0.1, seed=5), 1e-5), {}),
+                      work=2 * 2 * m2 * n2 + 2 * 2 * n2 + 2 * 4 * m2))
+    cases.append(Case("C2.sum", aten.sum.dim_IntList, lambda d: (_to(d, x2(), [-1]), {}),
+                      work=2 * m2 * n2 + 2 * m2))
+    cases.append(Case("C2.amax", aten.amax.default, lambda d: (_to(d, x2(), [-1]), {}),
+                      work=2 * m2 * n2 + 2 * m2))
+
+    # C3: mm / addmm, bf16, 7B MLP shapes
+    m3 = S(4096, 256)
+    for tag, (K, N) in (("up", (4096, 11008)), ("down", (11008, 4096))):
+        a = lambda K=K: normal((m3, K), bf16, seed=6)
+        b = lambda K=K, N=N: normal((K, N), bf16, 0.0, 0.02, seed=7)
+        flops = 2.0 * m3 * N * K
+        cases.append(Case(f"C3.mm_{tag}", aten.mm.default, lambda d, a=a, b=b: (_to(d, a(), b()), {}),
+                          work=flops, bound="mfma", extra={"bytes": 2 * (m3 * K + K * N + m3 * N)}))
+        cases.append(Case(f"C3.addmm_{tag}", aten.addmm.default,
+                          lambda d, a=a, b=b, N=N: (_to(d, normal((N,), bf16, 0.0, 0.02, seed=8), a(), b()), {}),
+                          work=flops, bound="mfma", extra={"bytes": 2 * (m3 * K + K * N + m3 * N + N)}))
+
+    # C4: indexing, bit-exact
+    v4, d4, n4 = S(128256), 4096, S(16384)
+    table = lambda: normal((v4, d4), bf16, 0.0, 0.02, seed=9)
+    idx = lambda: randint((n4,), v4, seed=10)
+    cases.append(Case("C4.embedding", aten.embedding.default, lambda d: (_to(d, table(), idx()), {}),
+                      work=2 * 2 * n4 * d4 + 8 * n4, exact=True))
+    cases.append(Case("C4.index_select", aten.index_select.default, lambda d: (_to(d, table(), 0, idx()), {}),
+                      work=2 * 2 * n4 * d4 + 8 * n4, exact=True))
+    g4 = S(2048)
+    cases.append(Case("C4.gather", aten.gather.default,
+                      lambda d: (_to(d, normal((g4, 4096), f32, seed=11), 1, randint((g4, 4096), 4096, seed=12)), {}),
+                      work=(4 + 8 + 4) * g4 * 4096, exact=True))
+    r4 = S(8192)
+    cases.append(Case("C4.argmax", aten.argmax.default,
+                      lambda d: (_to(d, normal((r4, 128256), f32, seed=13), -1), {}),
+                      work=4 * r4 * 128256 + 8 * r4, exact=True))
+
+    # C5: fp16 edge layouts with 1 % NaN / +-inf
+    b5 = S(64)
+    cases.append(Case("C5.mul_broadcast", aten.mul.Tensor,
+                      lambda d: (_to(d, normal((b5, 1, 2048), f16, seed=14), normal((1, 512, 2048), f16, seed=15)), {}),
+                      work=2 * (b5 * 512 * 2048 + b5 * 2048 + 512 * 2048)))
+    r5 = S(2048)
+    base = lambda seed: poison(normal((r5, 3072), f16, seed=seed), 0.01, seed=seed + 100)
+
+    def tview(device, seed):
+        return base(seed).to(device).t()  # [3072, r5] view with strides (1, 3072)
+
+    def cond_t(device):
+        return (normal((r5, 3072), f32, seed=19) > 0).to(device).t()
+
+    cases.append(Case("C5.where_t", aten.where.self, lambda d: ([cond_t(d), tview(d, 16), tview(d, 17)], {}),
+                      work=(1 + 2 + 2 + 2) * r5 * 3072, exact=True))
+    cases.append(Case("C5.maximum_t", aten.maximum.default, lambda d: ([tview(d, 16), tview(d, 17)], {}),
+                      work=3 * 2 * r5 * 3072))
+    cases.append(Case("C5.clamp_t", aten.clamp.default, lambda d: ([tview(d, 16), -1, 1], {}),
+                      work=2 * 2 * r5 * 3072))
+    return cases
+
+
+# ---------------------------------------------------------------- edge cases
+def edge_cases() -> List[Case]:
+    bf16, f16, f32, f64 = torch.bfloat16, torch.float16, torch.float32, torch.float64
+    i32, i64 = torch.int32, torch.int64
+    C: List[Case] = []
+    n = [0]
+
+    def add(op, make, exact=False, tag=""):
+        n[0] += 1
+        name = op.__name__.replace(".", "_")
+        C.append(Case(f"E{n[0]:03d}.{name}{('.' + tag) if tag else ''}", op, make, exact=exact))
+
+    special = lambda dt: torch.tensor([float("nan"), float("-inf"), -2.0, -0.0, 0.0, 3.0, float("inf"), 0.5], dtype=dt)
+
+    # ---- binary: add / mul / maximum
+    for op in (aten.add.Tensor, aten.mul.Tensor, aten.maximum.default):
+        for dt in (f32, f16, bf16):
+            add(op, lambda d, dt=dt: (_to(d, normal((33, 65), dt, seed=1), normal((33, 65), dt, seed=2)), {}), tag=f"{dt}".split(".")[-1])
+        add(op, lambda d: (_to(d, normal((4, 1, 16), f16, seed=3), normal((1, 5, 16), f16, seed=4)), {}), tag="bcast3")
+        add(op, lambda d: (_to(d, normal((7, 1), f32, seed=3), normal((1, 9), f32, seed=4)), {}), tag="outer")
+        add(op, lambda d: (_to(d, normal((6, 40), f32, seed=3), normal((40,), f32, seed=4)), {}), tag="rowvec")
+        add(op, lambda d: ([normal((48, 20), f16, seed=5).to(d).t(), normal((48, 20), f16, seed=6).to(d).t()], {}), tag="both_t")
+        add(op, lambda d: ([normal((48, 20), f32, seed=5).to(d).t(), normal((20, 48), f32, seed=6).to(d)], {}), tag="mixed_layout")
+        add(op, lambda d: ([normal((16, 64), f32, seed=5).to(d)[:, ::2], normal((16, 32), f32, seed=6).to(d)], {}), tag="strided")
+        add(op, lambda d: (_to(d, poison(normal((50, 30), f16, seed=7), 0.05, 8), poison(normal((50, 30), f16, seed=9), 0.05, 10)), {}), tag="naninf")
+        add(op, lambda d: (_to(d, special(f32), special(f32).flip(0)), {}), tag="special")
+        add(op, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), torch.empty(0, 128, dtype=f16)), {}), tag="empty")
+        add(op, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), normal((128,), f16, seed=1)), {}), tag="empty_bcast")
+        add(op, lambda d: (_to(d, torch.tensor(1.5, dtype=f16), torch.tensor(-2.25, dtype=f16)), {}), tag="0d")
+        add(op, lambda d: (_to(d, normal((5, 3), f32, seed=1), torch.tensor(2.0, dtype=f32)), {}), tag="0d_bcast")
+        add(op, lambda d: (_to(d, normal((9,), f16, seed=1), normal((9,), f32, seed=2)), {}), tag="promote_f16_f32")
+        add(op, lambda d: (_to(d, normal((9,), f16, seed=1), torch.tensor(0.5, dtype=f64)), {}), tag="promote_0d_f64")
+        add(op, lambda d: (_to(d, randint((9,), 100, 1, i32, -100), torch.tensor(0.5, dtype=f32)), {}), tag="promote_int_0d_f32")
+        add(op, lambda d: (_to(d, randint((17, 5), 100, 1, i64, -100), randint((17, 5), 100, 2, i64, -100)), {}), exact=True, tag="i64")
+        add(op, lambda d: (_to(d, randint((17, 5), 100, 1, i32, -100), randint((5,), 100, 2, i32, -100)), {}), exact=True, tag="i32")
+        add(op, lambda d: (_to(d, normal((4, 6), f64, seed=1), normal((4, 6), f64, seed=2)), {}), tag="f64")
+        add(op, lambda d: (_to(d, normal((3, 1000, 7), bf16, seed=1), normal((3, 1000, 7), bf16, seed=2)), {}), tag="odd_inner")
+    add(aten.add.Tensor, lambda d: (_to(d, normal((33, 65), f32, seed=1), normal((33, 65), f32, seed=2)), {"alpha": 2.5}), tag="alpha")
+    add(aten.add.Tensor, lambda d: (_to(d, normal((33, 65), bf16, seed=1), normal((65,), bf16, seed=2)), {"alpha": -1}), tag="alpha_bf16")
+    add(aten.add.Tensor, lambda d: (_to(d, randint((12,), 50, 1, i64), randint((12,), 50, 2, i64)), {"alpha": 3}), exact=True, tag="alpha_int")
+
+    # ---- unary: relu / clamp
+    for dt in (f32, f16, bf16):
+        t = f"{dt}".split(".")[-1]
+        add(aten.relu.default, lambda d, dt=dt: (_to(d, normal((33, 65), dt, seed=1)), {}), tag=t)
+        add(aten.clamp.default, lambda d, dt=dt: (_to(d, normal((33, 65), dt, seed=1), -0.5, 0.75), {}), tag=t)
+    for op, extra in ((aten.relu.default, ()), (aten.clamp.default, (-1, 1))):
+        add(op, lambda d, extra=extra: ([special(f32).to(d), *extra], {}), tag="special")
+        add(op, lambda d, extra=extra: ([poison(normal((40, 24), f16, seed=2), 0.05, 3).to(d).t(), *extra], {}), tag="naninf_t")
+        add(op, lambda d, extra=extra: ([normal((16, 64), f32, seed=5).to(d)[:, 1::3], *extra], {}), tag="strided")
+        add(op, lambda d, extra=extra: ([torch.empty(0, 128, dtype=f16).to(d), *extra], {}), tag="empty")
+        add(op, lambda d, extra=extra: ([torch.tensor(-1.5, dtype=f16).to(d), *extra], {}), tag="0d")
+        add(op, lambda d, extra=extra: ([randint((30,), 10, 1, i32, -10).to(d), *extra], {}), exact=True, tag="i32")
+        add(op, lambda d, extra=extra: ([normal((2, 3, 4, 5), f32, seed=1).to(d).permute(3, 1, 0, 2), *extra], {}), tag="perm4")
+    add(aten.clamp.default, lambda d: (_to(d, normal((50,), f32, seed=1), None, 0.25), {}), tag="max_only")
+    add(aten.clamp.default, lambda d: (_to(d, normal((50,), f32, seed=1), 0.25), {}), tag="min_only")
+    add(aten.clamp.default, lambda d: (_to(d, normal((50,), f32, seed=1), 2, 1), {}), tag="lo_gt_hi")
+    add(aten.clamp.default, lambda d: (_to(d, normal((50,), f32, seed=1), float("nan"), 1.0), {}), tag="nan_bound")
+    add(aten.clamp.default, lambda d: (_to(d, randint((50,), 10, 1, i32, -10), 0.5, 2), {}), tag="int_float_bounds")
+    add(aten.clamp.default, lambda d: (_to(d, normal((50,), bf16, seed=1), -0.3, 0.3), {}), tag="bf16_inexact_bounds")
+
+    # ---- where
+    cond = lambda shape, seed: normal(shape, f32, seed=seed) > 0
+    for dt in (f32, f16, bf16, i64):
+        mk = (lambda s, sd, dt=dt: randint(s, 100, sd, dt, -100)) if dt == i64 else (lambda s, sd, dt=dt: poison(normal(s, dt, seed=sd), 0.05, sd))
+        add(aten.where.self, lambda d, mk=mk: (_to(d, cond((33, 65), 1), mk((33, 65), 2), mk((33, 65), 3)), {}), exact=True, tag=f"{dt}".split(".")[-1])
+    add(aten.where.self, lambda d: (_to(d, cond((4, 1, 16), 1), normal((1, 5, 16), f16, seed=2), normal((4, 5, 1), f16, seed=3)), {}), exact=True, tag="bcast3")
+    add(aten.where.self, lambda d: ([cond((48, 20), 1).to(d).t(), normal((48, 20), f16, seed=2).to(d).t(), normal((48, 20), f16, seed=3).to(d).t()], {}), exact=True, tag="all_t")
+    add(aten.where.self, lambda d: ([cond((20, 48), 1).to(d), normal((48, 20), f16, seed=2).to(d).t(), normal((20, 48), f16, seed=3).to(d)], {}), exact=True, tag="mixed_layout")
+    add(aten.where.self, lambda d: (_to(d, cond((9,), 1), normal((9,), f16, seed=2), normal((9,), f32, seed=3)), {}), tag="promote")
+    add(aten.where.self, lambda d: (_to(d, cond((0, 128), 1), torch.empty(0, 128, dtype=f16), torch.empty(0, 128, dtype=f16)), {}), exact=True, tag="empty")
+    add(aten.where.self, lambda d: (_to(d, torch.tensor(True), torch.tensor(1.0), torch.tensor(2.0)), {}), exact=True, tag="0d")
+    add(aten.where.self, lambda d: (_to(d, cond((6, 7), 1), normal((6, 7), f32, seed=2), torch.tensor(0.0)), {}), exact=True, tag="0d_other")
+
+    # ---- reductions: sum / mean / amax / argmax
+    def red_variants(op, has_dtype, needs_list, allow_int=True, argmax=False):
+        def dims(v):
+            if argmax:
+                return v if not isinstance(v, list) else v[0]
+            return v if not needs_list or isinstance(v, list) else [v]
+        ex = argmax
+        for dt in (f32, f16, bf16):
+            t = f"{dt}".split(".")[-1]
+            add(op, lambda d, dt=dt: (_to(d, normal((37, 129), dt, seed=1), dims(-1)), {}), exact=ex, tag=f"last_{t}")
+            add(op, lambda d, dt=dt: (_to(d, normal((37, 129), dt, seed=1), dims(0)), {}), exact=ex, tag=f"first_{t}")
+        add(op, lambda d: (_to(d, normal((5, 300, 7), f32, seed=1), dims(1), True), {}), exact=ex, tag="mid_keepdim")
+        add(op, lambda d: (_to(d, normal((64, 4096), bf16, 0, 2, seed=1), dims(-1)), {}), exact=ex, tag="row4096")
+        add(op, lambda d: (_to(d, normal((3, 70001), f32, seed=1), dims(-1)), {}), exact=ex, tag="long_rows")
+        add(op, lambda d: (_to(d, normal((5000, 6), f32, seed=1), dims(-1)), {}), exact=ex, tag="short_rows")
+        add(op, lambda d: (_to(d, normal((2, 400000), f32, seed=1), dims(-1)), {}), exact=ex, tag="split_rows")
+        add(op, lambda d: (_to(d, normal((3000, 5), f32, seed=1), dims(0)), {}), exact=ex, tag="split_cols")
+        add(op, lambda d: ([normal((40, 24), f32, seed=2).to(d).t(), dims(-1)], {}), exact=ex, tag="transposed")
+        add(op, lambda d: (_to(d, torch.tensor(2.5, dtype=f32), *(() if argmax else (dims([]),))), {}), exact=ex, tag="0d")
+        if not argmax:
+            add(op, lambda d: (_to(d, normal((4, 5, 6), f32, seed=1), [0, 2]), {}), tag="dims_0_2")
+            add(op, lambda d: (_to(d, normal((4, 5, 6), f32, seed=1), [1, 2]), {}), tag="dims_1_2")
+            add(op, lambda d: (_to(d, normal((4, 5, 6), f32, seed=1), [-1, 0, 1], True), {}), tag="all_keepdim")
+            add(op, lambda d: (_to(d, normal((4, 5, 6), f32, seed=1), []), {}), tag="dim_empty_list")
+        add(op, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), dims(-1)), {}), exact=ex, tag="empty_outer")
+        if allow_int:
+            add(op, lambda d: (_to(d, randint((13, 50), 1000, 1, i32, -1000), dims(-1)), {}), exact=True, tag="i32")
+            add(op, lambda d: (_to(d, randint((13, 50), 1000, 1, i64, -1000), dims(0)), {}), exact=True, tag="i64")
+        if has_dtype:
+            add(op, lambda d: (_to(d, normal((37, 129), bf16, seed=1), dims(-1)), {"dtype": f32}), tag="dtype_f32")
+            add(op, lambda d: (_to(d, normal((37, 129), f32, seed=1), dims(-1)), {"dtype": bf16}), tag="dtype_bf16")
+
+    red_variants(aten.sum.dim_IntList, True, True)
+    red_variants(aten.mean.dim, True, True, allow_int=False)
+    red_variants(aten.amax.default, False, True)
+    red_variants(aten.argmax.default, False, False, argmax=True)
+    add(aten.sum.dim_IntList, lambda d: (_to(d, torch.empty(128, 0, dtype=f32), [-1]), {}), tag="empty_reduced")
+    add(aten.mean.dim, lambda d: (_to(d, torch.empty(4, 0, dtype=f32), [-1]), {}), tag="empty_reduced_nan")
+    add(aten.sum.dim_IntList, lambda d: (_to(d, normal((20, 30), f32, seed=1) > 0, [-1]), {}), exact=True, tag="bool")
+    add(aten.sum.dim_IntList, lambda d: (_to(d, normal((20, 30), f32, seed=1), None), {}), tag="dim_none")
+    add(aten.sum.default, lambda d: (_to(d, normal((300, 500), f32, seed=1)), {}), tag="all")
+    add(aten.sum.default, lambda d: (_to(d, normal((300, 500), bf16, seed=1)), {"dtype": f32}), tag="all_dtype")
+    add(aten.sum.default, lambda d: (_to(d, randint((300, 50), 10, 1, i32)), {}), exact=True, tag="all_int")
+    add(aten.mean.default, lambda d: (_to(d, normal((300, 500), f32, 3.0, 1.0, seed=1)), {}), tag="all")
+    add(aten.mean.default, lambda d: (_to(d, normal((30, 50), f16, seed=1)), {}), tag="all_f16")
+    nan_rows = lambda dt: torch.tensor([[1, float("nan"), 5, 5], [2, 7, 7, float("-inf")], [float("inf"), 1, float("inf"), 0],
+                                        [float("-inf")] * 4, [float("nan")] * 4], dtype=dt)
+    for dt in (f32, bf16):
+        t = f"{dt}".split(".")[-1]
+        add(aten.amax.default, lambda d, dt=dt: (_to(d, nan_rows(dt), [-1]), {}), tag=f"nan_ties_{t}")
+        add(aten.argmax.default, lambda d, dt=dt: (_to(d, nan_rows(dt), -1), {}), exact=True, tag=f"nan_ties_{t}")
+        add(aten.argmax.default, lambda d, dt=dt: (_to(d, nan_rows(dt), 0), {}), exact=True, tag=f"nan_ties_dim0_{t}")
+        add(aten.sum.dim_IntList, lambda d, dt=dt: (_to(d, nan_rows(dt), [-1]), {}), tag=f"nan_{t}")
+    add(aten.argmax.default, lambda d: (_to(d, normal((37, 129), f32, seed=1)), {}), exact=True, tag="flat")
+    add(aten.argmax.default, lambda d: (_to(d, normal((37, 129), f32, seed=1), None, True), {}), exact=True, tag="flat_keepdim")
+    add(aten.argmax.default, lambda d: (_to(d, normal((5, 300, 7), f32, seed=1), 1, True), {}), exact=True, tag="mid_keepdim2")
+    add(aten.argmax.default, lambda d: (_to(d, torch.zeros(6, 5000, dtype=f32), -1), {}), exact=True, tag="all_ties")
+    add(aten.argmax.default, lambda d: (_to(d, (normal((16, 70000), f32, seed=2) * 4).round(), -1), {}), exact=True, tag="many_ties")
+
+    # ---- _softmax
+    for dt in (f32, f16, bf16):
+        t = f"{dt}".split(".")[-1]
+        add(aten._softmax.default, lambda d, dt=dt: (_to(d, normal((37, 129), dt, 0, 2, seed=1), -1, False), {}), tag=f"last_{t}")
+        add(aten._softmax.default, lambda d, dt=dt: (_to(d, normal((37, 129), dt, 0, 2, seed=1), 0, False), {}), tag=f"first_{t}")
+    add(aten._softmax.default, lambda d: (_to(d, normal((16, 4096), bf16, 0, 2, seed=1), -1, False), {}), tag="row4096")
+    add(aten._softmax.default, lambda d: (_to(d, normal((4, 8192), f32, 0, 2, seed=1), 1, False), {}), tag="row8192_f32")
+    add(aten._softmax.default, lambda d: (_to(d, normal((3, 50000), f32, 0, 2, seed=1), -1, False), {}), tag="long_rows")
+    add(aten._softmax.default, lambda d: (_to(d, normal((3, 20000), bf16, 0, 2, seed=1), -1, False), {}), tag="long_rows_bf16")
+    add(aten._softmax.default, lambda d: (_to(d, normal((5, 300, 7), f32, seed=1), 1, False), {}), tag="mid")
+    add(aten._softmax.default, lambda d: ([normal((40, 24), f32, seed=2).to(d).t(), -1, False], {}), tag="transposed")
+    add(aten._softmax.default, lambda d: (_to(d, torch.tensor([[float("-inf"), float("-inf")], [float("inf"), 1.0], [float("nan"), 1.0],
+                                                                 [float("-inf"), 0.0], [1.0, 2.0]], dtype=f32), -1, False), {}), tag="special")
+    add(aten._softmax.default, lambda d: (_to(d, torch.cat([torch.full((2, 9000), float("-inf")), normal((2, 9000), f32, seed=1)], 0), -1, False), {}), tag="special_long")
+    add(aten._softmax.default, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), -1, False), {}), tag="empty")
+    add(aten._softmax.default, lambda d: (_to(d, torch.tensor(0.3, dtype=f32), 0, False), {}), tag="0d")
+    add(aten._softmax.default, lambda d: (_to(d, normal((37, 129), bf16, 0, 2, seed=1), -1, True), {}), tag="half_to_float")
+
+    # ---- native_layer_norm
+    for dt in (f32, f16, bf16):
+        t = f"{dt}".split(".")[-1]
+        add(aten.native_layer_norm.default,
+            lambda d, dt=dt: (_to(d, normal((37, 129), dt, 0, 2, seed=1), [129], normal((129,), dt, 1, 0.1, seed=2), normal((129,), dt, 0, 0.1, seed=3), 1e-5), {}), tag=t)
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((16, 4096), bf16, 0, 2, seed=1), [4096], normal((4096,), bf16, 1, 0.1, seed=2), normal((4096,), bf16, 0, 0.1, seed=3), 1e-5), {}), tag="row4096")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((16, 4096), bf16, 0, 2, seed=1), [4096], normal((4096,), f32, 1, 0.1, seed=2), normal((4096,), f32, 0, 0.1, seed=3), 1e-5), {}), tag="f32_params")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((3, 30000), f32, 5.0, 2, seed=1), [30000], normal((30000,), f32, 1, 0.1, seed=2), normal((30000,), f32, 0, 0.1, seed=3), 1e-5), {}), tag="long_rows")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((2, 3, 4, 5), f32, seed=1), [4, 5], normal((4, 5), f32, 1, 0.1, seed=2), normal((4, 5), f32, 0, 0.1, seed=3), 1e-5), {}), tag="multi_dim")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((37, 129), f32, seed=1), [129], None, None, 1e-5), {}), tag="no_affine")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((37, 129), f32, seed=1), [129], normal((129,), f32, 1, 0.1, seed=2), None, 1e-3), {}), tag="weight_only")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, torch.empty(0, 8, dtype=f32), [8], normal((8,), f32, seed=2), normal((8,), f32, seed=3), 1e-5), {}), tag="empty")
+    add(aten.native_layer_norm.default, lambda d: ([normal((24, 40), f32, seed=2).to(d).t(), [24], None, None, 1e-5], {}), tag="transposed")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((64, 1024), f32, 1000.0, 0.5, seed=1), [1024], None, None, 1e-5), {}), tag="large_mean")
+
+    # ---- mm / addmm
+    for dt in (bf16, f16, f32):
+        t = f"{dt}".split(".")[-1]
+        add(aten.mm.default, lambda d, dt=dt: (_to(d, normal((256, 128), dt, seed=1), normal((128, 512), dt, 0, 0.1, seed=2)), {}), tag=f"tile_{t}")
+        add(aten.mm.default, lambda d, dt=dt: (_to(d, normal((37, 53), dt, seed=1), normal((53, 29), dt, 0, 0.1, seed=2)), {}), tag=f"ragged_{t}")
+        add(aten.addmm.default, lambda d, dt=dt: (_to(d, normal((512,), dt, seed=3), normal((256, 128), dt, seed=1), normal((128, 512), dt, 0, 0.1, seed=2)), {}), tag=f"bias_{t}")
+    add(aten.mm.default, lambda d: (_to(d, normal((300, 264), bf16, seed=1), normal((264, 520), bf16, 0, 0.1, seed=2)), {}), tag="edge_tiles")
+    add(aten.mm.default, lambda d: (_to(d, normal((512, 1024), bf16, seed=1), normal((1024, 768), bf16, 0, 0.05, seed=2)), {}), tag="multi_tile")
+    add(aten.mm.default, lambda d: ([normal((512, 320), bf16, seed=1).to(d), normal((768, 320), bf16, 0, 0.05, seed=2).to(d).t()], {}), tag="b_transposed")
+    add(aten.mm.default, lambda d: ([normal((320, 512), bf16, seed=1).to(d).t(), normal((320, 768), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_transposed")
+    add(aten.mm.default, lambda d: (_to(d, torch.eye(256, dtype=bf16), normal((256, 256), bf16, seed=2)), {}), exact=True, tag="identity")
+    add(aten.mm.default, lambda d: (_to(d, torch.empty(2, 0, dtype=f32), torch.empty(0, 3, dtype=f32)), {}), tag="k0")
+    add(aten.mm.default, lambda d: (_to(d, torch.empty(0, 8, dtype=bf16), normal((8, 16), bf16, seed=1)), {}), tag="m0")
+    add(aten.addmm.default, lambda d: (_to(d, normal((256, 512), bf16, seed=3), normal((256, 128), bf16, seed=1), normal((128, 512), bf16, 0, 0.1, seed=2)), {"beta": 0.5, "alpha": 2.0}), tag="full_c_alpha_beta")
+    add(aten.addmm.default, lambda d: (_to(d, torch.full((512,), float("nan"), dtype=bf16), normal((256, 128), bf16, seed=1), normal((128, 512), bf16, 0, 0.1, seed=2)), {"beta": 0}), tag="beta0_nan")
+    add(aten.addmm.default, lambda d: (_to(d, normal((256, 1), f32, seed=3), normal((256, 64), f32, seed=1), normal((64, 40), f32, 0, 0.1, seed=2)), {}), tag="col_bias_f32")
+    add(aten.addmm.default, lambda d: (_to(d, normal((29,), f16, seed=3), normal((37, 53), f16, seed=1), normal((53, 29), f16, 0, 0.1, seed=2)), {"alpha": 0.5}), tag="ragged_f16")
+
+    # ---- index_select / embedding / gather
+    for dt in (bf16, f32, i64, torch.uint8):
+        t = f"{dt}".split(".")[-1]
+        src = (lambda s, dt=dt: randint(s, 200, 1, dt)) if not dt.is_floating_point else (lambda s, dt=dt: poison(normal(s, dt, seed=1), 0.02, 2))
+        add(aten.index_select.default, lambda d, src=src: (_to(d, src((50, 64)), 0, randint((33,), 50, 3)), {}), exact=True, tag=f"dim0_{t}")
+        add(aten.index_select.default, lambda d, src=src: (_to(d, src((7, 50, 9)), 1, randint((33,), 50, 3)), {}), exact=True, tag=f"dim1_{t}")
+        add(aten.index_select.default, lambda d, src=src: (_to(d, src((7, 50)), -1, randint((33,), 50, 3, i32)), {}), exact=True, tag=f"last_i32_{t}")
+        add(aten.embedding.default, lambda d, src=src: (_to(d, src((50, 64)), randint((4, 5), 50, 3)), {}), exact=True, tag=t)
+        add(aten.gather.default, lambda d, src=src: (_to(d, src((20, 64)), 1, randint((20, 64), 64, 3)), {}), exact=True, tag=f"dim1_{t}")
+        add(aten.gather.default, lambda d, src=src: (_to(d, src((20, 64)), 0, randint((11, 33), 20, 3)), {}), exact=True, tag=f"dim0_{t}")
+    add(aten.index_select.default, lambda d: (_to(d, normal((300, 4096), bf16, seed=1), 0, randint((100,), 300, 3)), {}), exact=True, tag="rows8k")
+    add(aten.index_select.default, lambda d: (_to(d, normal((300, 33), bf16, seed=1), 0, randint((100,), 300, 3)), {}), exact=True, tag="odd_row_bytes")
+    add(aten.index_select.default, lambda d: ([normal((64, 50), f32, seed=1).to(d).t(), 0, randint((33,), 50, 3).to(d)], {}), exact=True, tag="transposed_src")
+    add(aten.index_select.default, lambda d: (_to(d, normal((50, 64), f32, seed=1), 0, torch.tensor(7)), {}), exact=True, tag="0d_index")
+    add(aten.index_select.default, lambda d: (_to(d, normal((50, 64), f32, seed=1), 0, torch.empty(0, dtype=i64)), {}), exact=True, tag="empty_index")
+    add(aten.index_select.default, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), 1, randint((5,), 128, 3)), {}), exact=True, tag="empty_src")
+    add(aten.embedding.default, lambda d: (_to(d, normal((50, 64), bf16, seed=1), torch.tensor(3)), {}), exact=True, tag="0d_index")
+    add(aten.embedding.default, lambda d: (_to(d, normal((50, 64), bf16, seed=1), randint((2, 3, 4), 50, 3, i32)), {}), exact=True, tag="3d_i32")
+    add(aten.embedding.default, lambda d: (_to(d, normal((50, 64), bf16, seed=1), randint((9,), 50, 3), 0, False, False), {}), exact=True, tag="padding_idx_args")
+    add(aten.embedding.default, lambda d: (_to(d, normal((1000, 4096), bf16, 0, 0.02, seed=1), randint((257,), 1000, 3)), {}), exact=True, tag="rows8k")
+    add(aten.gather.default, lambda d: (_to(d, normal((5, 6, 7), f32, seed=1), 2, randint((5, 6, 3), 7, 3)), {}), exact=True, tag="3d_last")
+    add(aten.gather.default, lambda d: (_to(d, normal((5, 6, 7), f32, seed=1), 1, randint((4, 9, 7), 6, 3)), {}), exact=True, tag="3d_mid_smaller")
+    add(aten.gather.default, lambda d: ([normal((64, 20), f32, seed=1).to(d).t(), 1, randint((64, 20), 64, 3).to(d).t()], {}), exact=True, tag="transposed")
+    add(aten.gather.default, lambda d: (_to(d, normal((20, 64), f32, seed=1), 1, torch.empty(20, 0, dtype=i64)), {}), exact=True, tag="empty_index")
+    add(aten.gather.default, lambda d: (_to(d, torch.tensor(4.0), 0, torch.tensor(0)), {}), exact=True, tag="0d")
+    add(aten.gather.default, lambda d: (_to(d, normal((256, 512), f32, seed=1), 1, randint((256, 512), 512, 3)), {"sparse_grad": False}), exact=True, tag="vec_path")
+    return C
+
+
+class CaseTest(Test):
+    """Test over a Case: arguments are (re)drawn lazily from the seeded generator, so a
+    suite of multi-gigabyte cases holds no tensors until a test is read."""
+
+    def __init__(self, case, device):
+        super().__init__()
+        self.case = case
+        self.device = device
+        self._pending_kwargs = None
+
+    @property
+    def args(self):
+        args, self._pending_kwargs = self.case.make(self.device)
+        return list(args)
+
+    @property
+    def kwargs(self):
+        kw, self._pending_kwargs = self._pending_kwargs, None
+        return dict(kw) if kw is not None else dict(self.case.make(self.device)[1])
+
+
+def _as_test(case, device):
+    return CaseTest(case, device)
+
+
+def BaselineTestSuite(device="cuda", scale=1.0, filter=None):
+    """OpTests over the slots: edge cases as correctness tests, headline rows as
+    performance tests.  `filter`: list of op-name substrings (like the CLI's --ops)."""
+    per_op = {}
+    for case in edge_cases():
+        per_op.setdefault(case.op, ([], []))[0].append(case)
+    for case in perf_cases(scale):
+        per_op.setdefault(case.op, ([], []))[1].append(case)
+    optests = []
+    for op, (edges, perfs) in per_op.items():
+        name = op.__name__
+        if filter and not any(f in name for f in filter):
+            continue
+        optests.append(OpTest(get_operator(op), [_as_test(c, device) for c in edges],
+                              [_as_test(c, device) for c in perfs]))
+    return TestSuite(f"baseline_{device}", optests)

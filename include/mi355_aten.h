@@ -1,0 +1,174 @@
+/*
+ * mi355_aten.h — C ABI of libmi355_aten.so: hand-written HIP kernels (gfx950 / MI355X)
+ * for the core ATen operator set of a BackendBench directory backend.
+ *
+ * What each entry point replaces in the reference (meta-pytorch/BackendBench):
+ * the reference holds no kernels.  It holds one *slot* per operator overload — the
+ * module-level callable `<folder>_kernel_impl` that
+ * BackendBench/backends/directory.py:74-100 loads from
+ * `<ops_dir>/<folder>/<folder>_implementation*.py` and that
+ * BackendBench/eval.py:102,186,195 (or the torch dispatcher after
+ * BackendBench/__init__.py:70-101) calls with the ATen overload's arguments.
+ * The Python wrappers in backendbench_amd/ops fill those slots; the functions below
+ * are what those wrappers bind through ctypes.  Folder names are the ones
+ * BackendBench/scripts/op_map.py lists (line cited per entry point).
+ *
+ * Conventions (all entry points):
+ *   - every `void*` data pointer is a DEVICE pointer (tensor.data_ptr());
+ *   - sizes and strides are in ELEMENTS, int64;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); kernels are
+ *     only enqueued on it: no allocation, no synchronisation, no stream creation;
+ *   - return 0 on success, a negative mi355_status otherwise; mi355_last_error()
+ *     then returns a thread-local message.  Nothing is launched on error;
+ *   - zero-element outputs return 0 without launching.
+ */
+#ifndef MI355_ATEN_H
+#define MI355_ATEN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_ABI_VERSION 1
+#define MI355_MAX_DIMS 8
+
+typedef enum mi355_dtype {
+  MI355_F32 = 0,
+  MI355_F16 = 1,
+  MI355_BF16 = 2,
+  MI355_F64 = 3,
+  MI355_I32 = 4,
+  MI355_I64 = 5,
+  MI355_I16 = 6,
+  MI355_I8 = 7,
+  MI355_U8 = 8,
+  MI355_BOOL = 9,
+  MI355_DTYPE_COUNT = 10
+} mi355_dtype;
+
+typedef enum mi355_status {
+  MI355_OK = 0,
+  MI355_ERR_INVALID = -1,     /* bad argument (shape, stride, null pointer, alignment) */
+  MI355_ERR_UNSUPPORTED = -2, /* dtype / layout combination with no kernel            */
+  MI355_ERR_LAUNCH = -3       /* hipLaunchKernel reported an error                    */
+} mi355_status;
+
+/* Strided view of device memory.  ndim <= MI355_MAX_DIMS; stride 0 = broadcast. */
+typedef struct mi355_tensor {
+  void* data;
+  int32_t dtype; /* mi355_dtype */
+  int32_t ndim;
+  int64_t sizes[MI355_MAX_DIMS];
+  int64_t strides[MI355_MAX_DIMS];
+} mi355_tensor;
+
+int mi355_abi_version(void);
+const char* mi355_last_error(void);
+
+/* ---- elementwise -------------------------------------------------------------- */
+
+typedef enum mi355_binary_op { MI355_ADD = 0, MI355_MUL = 1, MI355_MAXIMUM = 2 } mi355_binary_op;
+
+/* out = a (op) b with a, b already broadcast to out's shape (stride 0 where expanded)
+ * and already of out's dtype.  MI355_ADD computes a + alpha*b (alpha_f for floating
+ * dtypes, alpha_i for integer dtypes).  MI355_MAXIMUM propagates NaN.
+ * Slots: add__Tensor (op_map.py:266), mul__Tensor (op_map.py:749),
+ * maximum__default (op_map.py:706). */
+int mi355_binary(int op, const mi355_tensor* a, const mi355_tensor* b, double alpha_f,
+                 int64_t alpha_i, const mi355_tensor* out, void* stream);
+
+typedef enum mi355_unary_op { MI355_RELU = 0, MI355_CLAMP = 1 } mi355_unary_op;
+
+/* out = relu(x) or clamp(x, lo, hi); x has out's shape and dtype.  `bounds` bit 0 = lo
+ * present, bit 1 = hi present.  NaN inputs stay NaN; lo > hi yields hi everywhere.
+ * Slots: relu__default (op_map.py:877), clamp__default (op_map.py:371). */
+int mi355_unary(int op, const mi355_tensor* x, int bounds, double lo_f, double hi_f,
+                int64_t lo_i, int64_t hi_i, const mi355_tensor* out, void* stream);
+
+/* out = cond ? a : b, bit-exact select.  cond is MI355_BOOL or MI355_U8; a, b have out's
+ * dtype; all three already broadcast to out's shape.
+ * Slot: where__self (op_map.py:1132). */
+int mi355_where(const mi355_tensor* cond, const mi355_tensor* a, const mi355_tensor* b,
+                const mi355_tensor* out, void* stream);
+
+/* dst = (dst dtype) src, any strides on either side, same shape (src may broadcast).
+ * Host-side helper for the slots above and below: type promotion and
+ * making an operand dense without calling another ATen kernel. */
+int mi355_copy(const mi355_tensor* src, const mi355_tensor* dst, void* stream);
+
+/* ---- reductions ----------------------------------------------------------------- */
+
+typedef enum mi355_reduce_op {
+  MI355_SUM = 0,
+  MI355_MEAN = 1,
+  MI355_AMAX = 2,
+  MI355_ARGMAX = 3
+} mi355_reduce_op;
+
+/* x is dense, viewed as [outer, red, inner]; reduces the middle axis; out is dense
+ * [outer, inner].  Accumulates in fp32 (f16/bf16/f32), fp64 (f64) or int64 (integers).
+ * out_dtype: x's dtype or the accumulation dtype for SUM/MEAN/AMAX; MI355_I64 for
+ * ARGMAX (first index among equal maxima, NaN counts as the maximum).  red == 0 is the
+ * caller's business (identity fill or error), not accepted here.  Few-row, long
+ * reductions are split over the chip and combined in a second pass: when
+ * mi355_reduce_workspace_bytes() is non-zero the caller passes that much device scratch
+ * (contents undefined before and after).
+ * Slots: sum__dim_IntList (op_map.py:1063), sum__default (:1061), mean__dim (:708),
+ * mean__default (:707), amax__default (:282), argmax__default (:300). */
+int64_t mi355_reduce_workspace_bytes(int op, int in_dtype, int64_t outer, int64_t red,
+                                     int64_t inner);
+int mi355_reduce(int op, const void* x, int in_dtype, int64_t outer, int64_t red,
+                 int64_t inner, void* out, int out_dtype, void* workspace,
+                 int64_t workspace_bytes, void* stream);
+
+/* y = softmax over the middle axis of dense x viewed as [outer, dim, inner]; fp32 math.
+ * out_dtype = in_dtype, or MI355_F32 for half_to_float.
+ * Slot: _softmax__default (op_map.py:193). */
+int mi355_softmax(const void* x, int in_dtype, void* y, int out_dtype, int64_t outer,
+                  int64_t dim, int64_t inner, void* stream);
+
+/* Layer norm over the last N elements of each of M dense rows.  weight/bias may be NULL
+ * and may differ in dtype from x (w_dtype).  mean/rstd are dense [M] in stat_dtype
+ * (MI355_F32 or x's dtype).  Biased variance, rstd = 1/sqrt(var + eps).
+ * Slot: native_layer_norm__default (op_map.py:776). */
+int mi355_layer_norm(const void* x, int dtype, const void* weight, const void* bias,
+                     int w_dtype, void* y, void* mean, void* rstd, int stat_dtype,
+                     int64_t M, int64_t N, double eps, void* stream);
+
+/* ---- matrix multiply -------------------------------------------------------------- */
+
+/* out[M,N] = beta * c + alpha * (a[M,K] @ b[K,N]), fp32 accumulate, out dense row-major
+ * in `dtype` (bf16 / f16 via MFMA; f32).  a, b, c carry explicit (row, col) element
+ * strides so transposed operands and a broadcast bias (c_rs = 0, c_cs = 1) need no copy.
+ * c may be NULL (then beta is ignored); beta == 0 never reads c.  K == 0 is accepted.
+ * Slots: mm__default (op_map.py:739), addmm__default (op_map.py:270). */
+int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs,
+               int64_t b_cs, const void* c, int64_t c_rs, int64_t c_cs, void* out,
+               int64_t M, int64_t N, int64_t K, double alpha, double beta, int dtype,
+               void* stream);
+
+/* ---- indexing --------------------------------------------------------------------- */
+
+/* src dense [outer, n_src, inner], out dense [outer, n_idx, inner]:
+ * out[o, j, :] = src[o, index[j], :].  elem_size in bytes (1, 2, 4, 8); idx_dtype
+ * MI355_I32 or MI355_I64; index dense.  An index outside [0, n_src) is never
+ * dereferenced: the row is zero-filled and *err_flag (device int32, may be NULL) is set
+ * to 1 — the host decides when to read it.
+ * Slots: index_select__default (op_map.py:571), embedding__default (op_map.py:447). */
+int mi355_index_select(const void* src, int elem_size, int64_t outer, int64_t n_src,
+                       int64_t inner, const void* index, int idx_dtype, int64_t n_idx,
+                       void* out, int32_t* err_flag, void* stream);
+
+/* out[...] = src[..., index[...], ...] along `dim`; out dense with index's shape, index
+ * MI355_I64 (any strides), src any strides, index.size(d) <= src.size(d) for d != dim.
+ * Same out-of-range convention as mi355_index_select.
+ * Slot: gather__default (op_map.py:510). */
+int mi355_gather(const mi355_tensor* src, int dim, const mi355_tensor* index,
+                 const mi355_tensor* out, int32_t* err_flag, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_ATEN_H */
