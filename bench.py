@@ -1,0 +1,234 @@
+#!/usr/bin/env python3
+"""Benchmark of the directory backend's HIP kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  A "step" is one pass of the headline row-op workload
+(BASELINE.json configs[1]): `_softmax`, `native_layer_norm`, `sum` and `amax` over the last
+dim of a bf16 [8192, 4096] tensor, each called once through the drop-in boundary
+(DirectoryBackend -> `<folder>_kernel_impl` -> ctypes -> libmi355_aten.so).  Inputs are
+resident in HBM before the clock starts; consecutive steps walk a pool of input copies larger
+than the last-level cache, so every step reads from HBM.  `value` is the algorithmic bytes of
+a step divided by the time of a step.
+
+Beside the step loop the script times every headline row of all five configurations the way
+the reference times GPU code (flush the cache, one event pair per repetition, mean), reports
+GB/s or TFLOP/s and the fraction of the MI355X peak per op under "per_op", times ATen on the
+host CPU for the same calls ("cpu_baseline", bounded samples) and reports the geometric mean
+speed-up over it.
+"""
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, TFLOP/s
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--launch", choices=["graph", "eager"], default="graph",
+                    help="replay the step loop from a HIP graph (default) or launch eagerly from Python")
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink factor for every shape (debug only)")
+    ap.add_argument("--ops", default="all", help="comma-separated substrings of per-op rows to time, or 'none'")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only-op", default=None, help="time just this per-op row in a loop (for profilers)")
+    ap.add_argument("--reps", type=int, default=50, help="repetitions for --only-op")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (every kernel works on one GPU's share); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels only run on an MI355X", file=sys.stderr)
+        sys.exit(1)
+
+    from backendbench_amd import eval as ev
+    from backendbench_amd.backends import DirectoryBackend
+    from backendbench_amd.suite import perf_cases
+
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda", 0)
+    backend = DirectoryBackend(os.path.join(ROOT, "generated_kernels"))
+    cases = perf_cases(args.scale)
+    by_key = {c.key: c for c in cases}
+
+    def impl_of(case):
+        return backend[case.op]
+
+    # ------------------------------------------------------------ profiler mode
+    if args.only_op:
+        case = by_key[args.only_op]
+        a, kw = case.make(dev)
+        f = impl_of(case)
+        for _ in range(3):
+            f(*a, **kw)
+        torch.cuda.synchronize()
+        for _ in range(args.reps):
+            ev._flush_cache(dev)
+            f(*a, **kw)
+        torch.cuda.synchronize()
+        print(json.dumps({"only_op": args.only_op, "reps": args.reps}))
+        return
+
+    # ------------------------------------------------------------ headline step loop (C2)
+    step_keys = ["C2.softmax", "C2.layer_norm", "C2.sum", "C2.amax"]
+    step_cases = [by_key[k] for k in step_keys]
+    step_bytes = sum(c.work for c in step_cases)
+    (x0, _, _), _ = by_key["C2.softmax"].make(dev)
+    (_, nshape, gamma, beta, eps), _ = by_key["C2.layer_norm"].make(dev)
+    pool_n = max(2, math.ceil(1.5 * 2**30 / (x0.numel() * x0.element_size())))  # >= 1.5 GiB of inputs
+    pool = [x0] + [x0.clone() for _ in range(pool_n - 1)]
+    softmax, layer_norm = impl_of(by_key["C2.softmax"]), impl_of(by_key["C2.layer_norm"])
+    rsum, ramax = impl_of(by_key["C2.sum"]), impl_of(by_key["C2.amax"])
+
+    def step(i):
+        x = pool[i % pool_n]
+        return softmax(x, -1, False), layer_norm(x, nshape, gamma, beta, eps), rsum(x, [-1]), ramax(x, [-1])
+
+    for i in range(3):  # first calls: library load, attribute set-up, allocator warm-up
+        keep = step(i)
+    torch.cuda.synchronize()
+
+    launch_mode = args.launch
+    graph = None
+    if launch_mode == "graph":
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                outs = [step(i) for i in range(pool_n)]  # one graph = one walk over the pool
+            torch.cuda.synchronize()
+        except Exception as exc:  # noqa: BLE001
+            print(f"bench.py: graph capture failed ({exc}); falling back to eager launches", file=sys.stderr)
+            graph, launch_mode = None, "eager"
+
+    def run_steps(n):
+        if graph is None:
+            for i in range(n):
+                step(i)
+        else:
+            done = 0
+            while done < n:
+                graph.replay()
+                done += pool_n
+
+    K = args.steps if graph is None else max(pool_n, args.steps // pool_n * pool_n)
+    W = args.warmup if graph is None else max(pool_n, math.ceil(args.warmup / pool_n) * pool_n)
+    run_steps(W)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_steps(K)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / K
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    del graph
+    outs = keep = None
+
+    # ------------------------------------------------------------ per-op timings
+    want = None if args.ops == "all" else ([] if args.ops == "none" else args.ops.split(","))
+    per_op = []
+    cpu_times = {}
+    for case in cases:
+        if want is not None and not any(w in case.key for w in want):
+            continue
+        a, kw = case.make(dev)
+        f = impl_of(case)
+        ms = ev.gpu_bench(lambda: f(*a, **kw))
+        row = {"op": case.key, "ms": round(ms, 5)}
+        if case.bound == "hbm":
+            gbs = case.work / (ms * 1e-3) / 1e9
+            row.update(bound="hbm", bytes=int(case.work), gbs=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4))
+        else:
+            tf = case.work / (ms * 1e-3) / 1e12
+            row.update(bound="mfma", flops=int(case.work), tflops=round(tf, 1), frac=round(tf / MFMA_BF16_PEAK_TFLOPS, 4))
+        if not args.no_cpu:
+            row["cpu_ms"], row["cpu_sample"] = cpu_time_ms(case, a, kw)
+            row["speedup_vs_cpu"] = round(row["cpu_ms"] / ms, 1)
+            cpu_times[case.key] = row["cpu_ms"]
+        per_op.append(row)
+        del a, kw
+        torch.cuda.empty_cache()
+
+    rows = {r["op"]: r for r in per_op}
+    # dominant kernel of the step = the op with the largest share of a step's GPU time
+    roofline = None
+    timed = [rows[k] for k in step_keys if k in rows]
+    if timed:
+        dom = max(timed, key=lambda r: r["ms"])
+        roofline = {"bound": "hbm", "kernel": dom["op"], "achieved": dom["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(dom["gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
+                    "bytes_per_launch": dom["bytes"], "avg_launch_ms": dom["ms"],
+                    "timing": "hip events on the launch stream, cache flushed before every launch, mean"}
+    cpu_baseline = None
+    if not args.no_cpu and all(k in cpu_times for k in step_keys):
+        cpu_ms = sum(cpu_times[k] for k in step_keys)
+        cpu_baseline = {"value": round(step_bytes / (cpu_ms * 1e-3) / 1e9, 2), "unit": "GB/s",
+                        "cores": torch.get_num_threads(), "kind": "port",
+                        "sample": "ATen CPU kernels (the oracle) on the same four calls at full size, "
+                                  "mean of a bounded number of runs each (see per_op[].cpu_sample)",
+                        "ms_per_step": round(cpu_ms, 3), "host_cpus": os.cpu_count()}
+    geomean = None
+    sp = [r["speedup_vs_cpu"] for r in per_op if "speedup_vs_cpu" in r]
+    if sp:
+        geomean = round(math.exp(sum(math.log(s) for s in sp) / len(sp)), 1)
+
+    line = {
+        "metric": "per-op GB/s or TFLOP/s + % of roofline on 1 MI355X; geomean speedup vs aten CPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 storage, fp32 accumulate", "data": "synthetic (seeded N(0,2) on CPU, copied to HBM)",
+        "config": {"workload": "C2 row ops on bf16 [8192,4096]: _softmax(dim=-1) + native_layer_norm([4096]) + "
+                               "sum(dim=-1) + amax(dim=-1), one call each per step",
+                   "bytes_per_step": int(step_bytes), "launch": launch_mode, "input_pool": pool_n,
+                   "scale": args.scale},
+        "roofline": roofline, "cpu_baseline": cpu_baseline,
+        "geomean_speedup_vs_cpu": geomean, "per_op": per_op,
+    }
+    print(json.dumps(line))
+
+
+def cpu_time_ms(case, args, kwargs):
+    """Mean ms per call of ATen on the host CPU for this row (the oracle, timed with the
+    reference's CPU recipe) on a bounded sample: GEMMs run 512 of their 4096 rows and are
+    scaled (cost is linear in M); everything else runs at full size with few repetitions."""
+    import torch
+
+    from oracle import aten_cpu
+
+    a = aten_cpu.to_cpu(list(args))
+    scale, note = 1.0, "full size"
+    if case.bound == "mfma":
+        pos = 1 if "addmm" in case.key else 0
+        M = a[pos].shape[0]
+        rows = min(M, 512)
+        a[pos] = a[pos][:rows].contiguous()
+        scale, note = M / rows, f"{rows} of {M} rows, time scaled x{M // rows}"
+    t0 = time.perf_counter()
+    case.op(*a, **kwargs)
+    first = time.perf_counter() - t0
+    runs = max(1, min(20, int(1.0 / max(first, 1e-4))))
+    warm = 1 if first > 0.2 else 2
+    sec = aten_cpu.time_call(case.op, a, kwargs, warmup=warm, runs=runs)
+    return round(sec * scale * 1e3, 4), f"{note}, {warm} warm-up + {runs} timed runs, {torch.get_num_threads()} threads"
+
+
+if __name__ == "__main__":
+    main()

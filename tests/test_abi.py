@@ -1,0 +1,81 @@
+"""The C-ABI library: it loads, exports every symbol include/mi355_aten.h declares, and the
+ctypes mirror of its struct and enums matches the header.  No compute calls (no GPU here)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from backendbench_amd import _lib
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "mi355_aten.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_[a-z_0-9]+)\s*\(", text)))
+
+
+def header_enum(name):
+    text = open(HEADER).read()
+    m = re.search(r"#define\s+%s\s+(\d+)" % name, text) or re.search(r"\b%s\s*=\s*(-?\d+)" % name, text)
+    assert m, name
+    return int(m.group(1))
+
+
+def test_header_declares_the_expected_entry_points():
+    fns = declared_functions()
+    assert "mi355_gemm" in fns and "mi355_softmax" in fns and "mi355_index_select" in fns
+    assert len(fns) == 13
+
+
+def test_every_declared_symbol_is_exported_and_bound():
+    lib = _lib.load()
+    for fn in declared_functions():
+        assert hasattr(lib, fn), f"{fn} is declared in the header but not exported"
+        assert fn in _lib.SIGNATURES, f"{fn} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == declared_functions()
+
+
+def test_abi_version_matches_header():
+    assert _lib.load().mi355_abi_version() == header_enum("MI355_ABI_VERSION") == _lib.ABI_VERSION
+
+
+def test_struct_layout_matches_header():
+    assert header_enum("MI355_MAX_DIMS") == _lib.MAX_DIMS == 8
+    assert ctypes.sizeof(_lib.TensorDesc) == 8 + 4 + 4 + 8 * 8 + 8 * 8
+    assert _lib.TensorDesc.sizes.offset == 16 and _lib.TensorDesc.strides.offset == 80
+
+
+@pytest.mark.parametrize("name,value", [("MI355_F32", _lib.F32), ("MI355_F16", _lib.F16), ("MI355_BF16", _lib.BF16),
+                                        ("MI355_F64", _lib.F64), ("MI355_I32", _lib.I32), ("MI355_I64", _lib.I64),
+                                        ("MI355_I16", _lib.I16), ("MI355_I8", _lib.I8), ("MI355_U8", _lib.U8),
+                                        ("MI355_BOOL", _lib.BOOL), ("MI355_ADD", _lib.ADD), ("MI355_MUL", _lib.MUL),
+                                        ("MI355_MAXIMUM", _lib.MAXIMUM), ("MI355_RELU", _lib.RELU),
+                                        ("MI355_CLAMP", _lib.CLAMP), ("MI355_SUM", _lib.SUM), ("MI355_MEAN", _lib.MEAN),
+                                        ("MI355_AMAX", _lib.AMAX), ("MI355_ARGMAX", _lib.ARGMAX)])
+def test_enum_values_match_header(name, value):
+    assert header_enum(name) == value
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    """Validation happens before any launch, so the error path is testable on the host."""
+    lib = _lib.load()
+    rc = lib.mi355_softmax(None, _lib.F32, None, _lib.F32, 4, 4, 1, None)
+    assert rc == -1 and b"NULL" in lib.mi355_last_error()
+    rc = lib.mi355_reduce(_lib.SUM, None, _lib.F32, 4, 0, 1, None, _lib.F32, None, 0, None)
+    assert rc == -1 and b"bad extents" in lib.mi355_last_error()
+    with pytest.raises(RuntimeError, match="bad extents"):
+        _lib.check(rc)
+    assert lib.mi355_gemm(None, 1, 1, None, 1, 1, None, 0, 0, None, 0, 8, 8, 1.0, 0.0, _lib.BF16, None) == 0
+
+
+def test_reduce_workspace_plan():
+    lib = _lib.load()
+    assert lib.mi355_reduce_workspace_bytes(_lib.SUM, _lib.BF16, 8192, 4096, 1) == 0      # wave per row
+    assert lib.mi355_reduce_workspace_bytes(_lib.ARGMAX, _lib.F32, 8192, 128256, 1) == 0  # block per row
+    ws = lib.mi355_reduce_workspace_bytes(_lib.SUM, _lib.F32, 1, 1 << 24, 1)              # one long row: split
+    assert ws > 0 and ws % 4 == 0
+    assert lib.mi355_reduce_workspace_bytes(_lib.ARGMAX, _lib.F32, 1, 1 << 24, 1) == ws * 4

@@ -1,0 +1,54 @@
+"""Result files: names, fields and summary rows (reference: BackendBench/output.py:116-288,
+expectations in test/test_output.py:116-172)."""
+
+import csv
+import json
+
+from backendbench_amd.eval import CorrectnessTestResult, PerformanceTestResult
+from backendbench_amd.output import overall_summary_text, prepare_results, save_results, summary_rows
+
+
+def results():
+    c = [CorrectnessTestResult("add.Tensor", "a1", True, max_abs_error=0.5, max_rel_error=0.25),
+         CorrectnessTestResult("add.Tensor", "a0", False, error_msg="bad", max_abs_error=2.0, max_rel_error=1.0),
+         CorrectnessTestResult("relu.default", "r0", True, max_abs_error=0.0, max_rel_error=0.0)]
+    p = [PerformanceTestResult("add.Tensor", "a1", 2.0, 1.0, 2.0, successfully_ran=True),
+         PerformanceTestResult("add.Tensor", "a0", 8.0, 1.0, 8.0, successfully_ran=True),
+         PerformanceTestResult("relu.default", "r0", None, None, 3.0, error_msg="x", successfully_ran=False)]
+    return c, p
+
+
+def test_prepare_results():
+    c, p = results()
+    everything, failed, summary = prepare_results(c, p)
+    assert [r["args"] for r in everything] == ["a0", "a0", "a1", "a1", "r0", "r0"]
+    assert [(r["op_name"], r["test_type"]) for r in failed] == [("add.Tensor", "correctness"), ("relu.default", "performance")]
+    s = summary["add.Tensor"]
+    assert s["correctness_tests"] == 2 and s["passed_correctness_tests"] == 1 and s["failed_correctness_tests"] == 1
+    assert s["correctness_rate"] == 0.5 and s["avg_speedup"] == 5.0 and abs(s["geomean_speedup"] - 4.0) < 1e-9
+    assert s["max_absolute_error"] == 2.0 and s["max_relative_error"] == 1.0
+    assert summary["relu.default"]["passed_performance_tests"] == 0 and summary["relu.default"]["geomean_speedup"] == 0.0
+    assert list(s) == ["operator", "total_tests", "correctness_tests", "performance_tests", "passed_correctness_tests",
+                       "passed_performance_tests", "failed_correctness_tests", "failed_performance_tests",
+                       "correctness_rate", "avg_speedup", "geomean_speedup", "max_absolute_error", "max_relative_error"]
+
+
+def test_summary_rows_and_text():
+    c, p = results()
+    rows = summary_rows(p, c)
+    assert rows == [("add.Tensor", "50.0000%", "4.0000x"), ("relu.default", "100.0000%", "1.0000x")]
+    text = overall_summary_text("cmd --x", 0.5, 2.0, 0.25, 1.0, p, c)
+    assert "# BackendBench Run Summary" in text and "| Correctness Score | 0.50 |" in text
+    assert "| Perf@1.0 Score | 0.25 |" in text and "| add.Tensor | 50.0000% | 4.0000x|" in text
+
+
+def test_save_results_writes_four_files(tmp_path):
+    c, p = results()
+    save_results(c, p, str(tmp_path / "out"), command="cmd", mean_correctness=0.5, geomean_perf=2.0, perf_at_p_score=0.25)
+    names = sorted(f.name for f in (tmp_path / "out").iterdir())
+    assert names == ["OVERALL_SUMMARY.md", "failed_tests.json", "full_results.json", "operator_summary.csv"]
+    assert len(json.loads((tmp_path / "out" / "full_results.json").read_text())) == 6
+    rows = list(csv.DictReader(open(tmp_path / "out" / "operator_summary.csv")))
+    assert {r["operator"] for r in rows} == {"add.Tensor", "relu.default"}
+    save_results(c, p, str(tmp_path / "bare"))
+    assert not (tmp_path / "bare" / "OVERALL_SUMMARY.md").exists()
