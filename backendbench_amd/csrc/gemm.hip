@@ -2,10 +2,12 @@
 //
 //   mfma     bf16 / f16, a K-contiguous, b either K-contiguous ("NT", e.g. weight.t()) or
 //            N-contiguous ("NN", row-major), 16-byte aligned rows.  256x256x64 block tile,
-//            four wave64 (2x2), each wave 128x128 = 8x8 v_mfma_f32_16x16x32 tiles with
-//            256 fp32 accumulators; A and B panels double-buffered in 128 KB of LDS in
-//            16-byte chunks XOR-swizzled by row so that both the 128-bit global->LDS
-//            writes and the MFMA fragment reads are bank-conflict free; block -> tile map
+//            eight wave64 (2x4, two per SIMD), each wave 128x64 = 8x4 v_mfma_f32_16x16x32
+//            tiles with 128 fp32 accumulators; A and B panels double-buffered in 128 KB of
+//            LDS, swizzled so that the 128-bit global->LDS writes and the fragment reads
+//            are bank-conflict free.  A row-major B stays N-contiguous in LDS and is
+//            transposed by the LDS read itself (ds_read_b64_tr_b16).  The next k-tile is
+//            in flight from HBM/L2 to registers during the MFMA phase; block -> tile map
 //            groups tiles per XCD so that one L2 serves neighbouring tiles.
 //   generic  any strides, bf16 / f16 / f32: 64x64 LDS tile, FMA inner loop.  Correctness
 //            path for shapes the MFMA kernel does not take.
@@ -36,14 +38,28 @@ template <> struct Mfma<f16_t> {
 };
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kGemmThreads = 256;
-constexpr int kRowBytes = BK * 2;                  // one tile row: 64 k-values = 128 B = 8 chunks
-constexpr int kPanelBytes = BM * kRowBytes;        // 32 KB per operand per stage
+constexpr int kGemmThreads = 512;                  // 8 waves: 2 (m) x 4 (n), each 128 x 64
+constexpr int kRowBytes = BK * 2;                  // K-contiguous panel row: 64 k = 128 B = 8 chunks
+constexpr int kPanelBytes = BM * kRowBytes;        // 32 KB per operand per stage (either layout)
 constexpr int kStageBytes = 2 * kPanelBytes;       // A + B
 constexpr int kGemmLds = 2 * kStageBytes;          // double buffered: 128 KB
 
-// Byte offset of 16-byte chunk `c` (0..7) of tile row `r` inside a panel.
-__device__ __forceinline__ int swz(int r, int c) { return r * kRowBytes + ((c ^ (r & 7)) << 4); }
+// K-contiguous panel ([row][k], A and the "NT" B): byte offset of 16-byte chunk c (0..7) of
+// row r.  The chunk index is XORed with (r + r/8) mod 8, which makes both any 8 consecutive
+// rows (32-bank LDS) and any 16 consecutive rows (64-bank LDS) hit distinct banks when the 16
+// lanes of an MFMA fragment read the same chunk of 16 rows; the 128-bit writes of a row's 8
+// chunks stay a full 128-byte line.
+__device__ __forceinline__ int swz_k(int r, int c) {
+  return r * kRowBytes + ((c ^ ((r + (r >> 3)) & 7)) << 4);
+}
+// N-contiguous panel ([k][n], the row-major "NN" B, 512 B per k): byte offset of 16-byte unit u
+// (0..31) of row k.  32-byte chunks are XORed with (k%4) | ((k/8)%2)*4 so that the transposing
+// 64-bit reads (4 k-rows x 32 B per 16 lanes, rows k..k+3 and k+8..k+11 per 32 lanes) spread
+// over all banks.
+__device__ __forceinline__ int swz_n(int k, int u) {
+  const int x = (k & 3) | (((k >> 3) & 1) << 2);
+  return k * (BN * 2) + ((((u >> 1) ^ x)) << 5) + ((u & 1) << 4);
+}
 
 struct GemmArgs {
   const void* a;
@@ -78,46 +94,56 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, int& tm, int& tn)
   tn = (pid % in_group) / rows;
 }
 
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+// ds_read_b64_tr_b16: within each block of 16 lanes, lane s supplies the address of 4
+// consecutive 16-bit elements ("row s/4, columns 4*(s%4)..+3" of a 4 x 16 block) and lane i
+// receives column i of the 4 rows.  With rows = k and columns = n this turns an N-contiguous
+// LDS panel into the K-contiguous MFMA operand.
+__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) s16x4*)(uintptr_t)(const_cast<unsigned char*>(p)));
+}
+
 template <typename T, bool B_NN>
 __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using frag_t = typename Mfma<T>::frag;
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave >> 2, wn = wave & 3;  // wave tile: rows wm*128.., cols wn*64..
   int tm, tn;
   tile_coords(g, tm, tn);
   const int bm = tm * BM, bn = tn * BN;
   const T* A = static_cast<const T*>(g.a);
   const T* B = static_cast<const T*>(g.b);
 
-  // ---- global -> register staging: 8 chunks of A and 8 of B per thread per k-tile
-  u32x4 ra[8], rb[8];
-  const int lc = tid & 7, lr = tid >> 3;  // A (and NT B): chunk lc of rows lr + 32*i
+  // ---- global -> register staging: 4 chunks of A and 4 of B per thread per k-tile
+  u32x4 ra[4], rb[4];
+  const int lc = tid & 7, lr = tid >> 3;    // K-contiguous panels: chunk lc of rows lr + 64*i
+  const int nu = tid & 31, kr = tid >> 5;   // NN B: 16-byte unit nu of k rows kr + 16*i
   auto load_tile = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int r = lr + 32 * i;
-      int gr = bm + r;
+    for (int i = 0; i < 4; ++i) {
+      int gr = bm + lr + 64 * i;
       gr = gr < g.M ? gr : g.M - 1;
       const int k = k0 + lc * 8;
       ra[i] = k < g.K ? *reinterpret_cast<const u32x4*>(A + (int64_t)gr * g.lda + k) : u32x4{0, 0, 0, 0};
     }
     if constexpr (!B_NN) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int r = lr + 32 * i;
-        int gn = bn + r;
+      for (int i = 0; i < 4; ++i) {
+        int gn = bn + lr + 64 * i;
         gn = gn < g.N ? gn : g.N - 1;
         const int k = k0 + lc * 8;
         rb[i] = k < g.K ? *reinterpret_cast<const u32x4*>(B + (int64_t)gn * g.ldb + k) : u32x4{0, 0, 0, 0};
       }
     } else {
-      const int nc = tid & 31, kr = tid >> 5;  // 8 n-values at n = nc*8, k rows kr + 8*i
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int k = k0 + kr + 8 * i;
-        int gn = bn + nc * 8;
-        gn = gn < g.N ? gn : 0;
+      for (int i = 0; i < 4; ++i) {
+        const int k = k0 + kr + 16 * i;
+        int gn = bn + nu * 8;
+        gn = gn < g.N ? gn : 0;  // N % 8 == 0: a unit is all-in or all-out; out-of-range columns are never stored
         rb[i] = k < g.K ? *reinterpret_cast<const u32x4*>(B + (int64_t)k * g.ldb + gn) : u32x4{0, 0, 0, 0};
       }
     }
@@ -126,61 +152,65 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
     unsigned char* pa = lds + stage * kStageBytes;
     unsigned char* pb = pa + kPanelBytes;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(pa + swz(lr + 32 * i, lc)) = ra[i];
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(pa + swz_k(lr + 64 * i, lc)) = ra[i];
     if constexpr (!B_NN) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(pb + swz(lr + 32 * i, lc)) = rb[i];
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(pb + swz_k(lr + 64 * i, lc)) = rb[i];
     } else {
-      // Transpose while writing: element e of the chunk is column n = nc*8 + e at row k.
-      const int nc = tid & 31, kr = tid >> 5;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int k = kr + 8 * i;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int n = nc * 8 + e;
-          const uint32_t w = rb[i][e >> 1];
-          const uint16_t h = (e & 1) ? (uint16_t)(w >> 16) : (uint16_t)(w & 0xFFFFu);
-          *reinterpret_cast<uint16_t*>(pb + swz(n, k >> 3) + ((k & 7) << 1)) = h;
-        }
-      }
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(pb + swz_n(kr + 16 * i, nu)) = rb[i];
     }
   };
 
-  f32x4 acc[8][8];
+  f32x4 acc[8][4];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int nk = (g.K + BK - 1) / BK;
   if (nk > 0) {
     load_tile(0);
     store_tile(0);
+    if (nk > 1) load_tile(BK);
   }
   __syncthreads();
-  const int fr = lane & 15, fc = lane >> 4;  // fragment row and 16-byte k-chunk of this lane
+  const int fr = lane & 15, fc = lane >> 4;  // fragment row (m or n) and k-group of this lane
   for (int kt = 0; kt < nk; ++kt) {
     const int stage = kt & 1;
-    if (kt + 1 < nk) load_tile((kt + 1) * BK);
     const unsigned char* pa = lds + stage * kStageBytes;
     const unsigned char* pb = pa + kPanelBytes;
 #pragma unroll
     for (int kk = 0; kk < BK / 32; ++kk) {
-      frag_t fa[8], fb[8];
+      frag_t fa[8], fb[4];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        fa[i] = *reinterpret_cast<const frag_t*>(pa + swz(wm * 128 + i * 16 + fr, kk * 4 + fc));
-        fb[i] = *reinterpret_cast<const frag_t*>(pb + swz(wn * 128 + i * 16 + fr, kk * 4 + fc));
+      for (int i = 0; i < 8; ++i)
+        fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k(wm * 128 + i * 16 + fr, kk * 4 + fc));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if constexpr (!B_NN) {
+          fb[j] = *reinterpret_cast<const frag_t*>(pb + swz_k(wn * 64 + j * 16 + fr, kk * 4 + fc));
+        } else {
+          // k = kk*32 + fc*8 + h*4 + (lane%16)/4, columns wn*64 + j*16 + 4*(lane%4) .. +3
+          const int kb = kk * 32 + fc * 8 + (fr >> 2);
+          const int n0 = wn * 64 + j * 16 + ((fr & 3) << 2);  // element column; 16-byte unit = n0/8
+          const s16x4 lo = lds_read_tr(pb + swz_n(kb, n0 >> 3) + ((n0 & 7) << 1));
+          const s16x4 hi = lds_read_tr(pb + swz_n(kb + 4, n0 >> 3) + ((n0 & 7) << 1));
+          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          fb[j] = __builtin_bit_cast(frag_t, both);
+        }
       }
 #pragma unroll
       for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < 4; ++j)
           // operands swapped: the lane ends up with 4 consecutive n of one row m
           acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
     }
-    if (kt + 1 < nk) store_tile(stage ^ 1);
+    if (kt + 1 < nk) {
+      store_tile(stage ^ 1);                       // tile kt+1, loaded during the previous compute phase
+      if (kt + 2 < nk) load_tile((kt + 2) * BK);  // in flight during the next compute phase
+    }
     __syncthreads();
   }
 
@@ -193,8 +223,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
     const int m = bm + wm * 128 + i * 16 + fr;
     if (m >= g.M) continue;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int n = bn + wn * 128 + j * 16 + fc * 4;
+    for (int j = 0; j < 4; ++j) {
+      const int n = bn + wn * 64 + j * 16 + fc * 4;
       if (n >= g.N) continue;  // N % 4 == 0 on this path: 4 columns are all in or all out
       VecN4<T> r;
 #pragma unroll

@@ -75,7 +75,9 @@ _INT_VIEW = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}
 
 
 def bit_equal(a, b):
-    """Same dtype, shape and bit pattern (NaN payloads included)."""
+    """Same dtype, shape and bit pattern (so -0.0 != 0.0), except that any NaN equals any NaN:
+    NaN payloads are not part of the contract (ATen's own CPU gather rewrites the payload of
+    bf16 NaNs it copies)."""
     if not (isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor)):
         return a == b
     if a.dtype != b.dtype or a.shape != b.shape:
@@ -86,7 +88,14 @@ def bit_equal(a, b):
     if a.dtype == torch.bool:
         return torch.equal(a, b)
     view = _INT_VIEW[a.element_size()]
-    return torch.equal(a.contiguous().view(view), b.contiguous().view(view))
+    a, b = a.contiguous(), b.contiguous()
+    ai, bi = a.view(view), b.view(view)
+    if a.dtype.is_floating_point:
+        nan_a, nan_b = a != a, b != b
+        if not torch.equal(nan_a, nan_b):
+            return False
+        return torch.equal(ai[~nan_a], bi[~nan_a])
+    return torch.equal(ai, bi)
 
 
 def _walk_pairs(a, b):

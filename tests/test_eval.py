@@ -37,6 +37,9 @@ def test_integer_outputs_are_compared_exactly():
     assert ev.allclose(x, x.clone(), exact=True)
     assert not ev.allclose(torch.tensor([1.0]), torch.tensor([1.0 + 1e-6]), exact=True)
     assert ev.bit_equal(torch.tensor([0.0]), torch.tensor([0.0])) and not ev.bit_equal(torch.tensor([0.0]), torch.tensor([-0.0]))
+    quiet = torch.tensor([0x7FC0, 0x3F80], dtype=torch.int16).view(torch.bfloat16)
+    other = torch.tensor([-1, 0x3F80], dtype=torch.int16).view(torch.bfloat16)      # another NaN payload
+    assert ev.bit_equal(quiet, other) and not ev.bit_equal(quiet, other.flip(0))
 
 
 def test_cpu_bench_call_count():
