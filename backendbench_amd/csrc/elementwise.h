@@ -19,6 +19,38 @@ template <typename T, int N> __device__ __forceinline__ VecN<T, N> ld(const T* p
 template <typename T, int N> __device__ __forceinline__ void st(T* p, const VecN<T, N>& v) {
   *reinterpret_cast<VecN<T, N>*>(p) = v;
 }
+// Streaming (non-temporal) forms for data touched exactly once: measured on MI355X, a
+// block-contiguous copy with non-temporal loads and stores runs at 5.8-6.4 TB/s against
+// 5.3-5.8 TB/s with plain accesses.  Vectors wider than 16 bytes are moved in 16-byte pieces.
+template <int BYTES> struct RawVec { typedef uint32_t type __attribute__((ext_vector_type(BYTES / 4))); };
+template <> struct RawVec<1> { typedef uint8_t type; };
+template <> struct RawVec<2> { typedef uint16_t type; };
+template <typename T, int N> __device__ __forceinline__ VecN<T, N> ld_nt(const T* p) {
+  constexpr int B = sizeof(T) * N;
+  if constexpr (B > 16) {
+    VecN<T, N> r;
+    using R = typename RawVec<16>::type;
+    R* dst = reinterpret_cast<R*>(&r);
+#pragma unroll
+    for (int i = 0; i < B / 16; ++i) dst[i] = __builtin_nontemporal_load(reinterpret_cast<const R*>(p) + i);
+    return r;
+  } else {
+    using R = typename RawVec<B>::type;
+    return __builtin_bit_cast(VecN<T, N>, __builtin_nontemporal_load(reinterpret_cast<const R*>(p)));
+  }
+}
+template <typename T, int N> __device__ __forceinline__ void st_nt(T* p, const VecN<T, N>& v) {
+  constexpr int B = sizeof(T) * N;
+  if constexpr (B > 16) {
+    using R = typename RawVec<16>::type;
+    const R* src = reinterpret_cast<const R*>(&v);
+#pragma unroll
+    for (int i = 0; i < B / 16; ++i) __builtin_nontemporal_store(src[i], reinterpret_cast<R*>(p) + i);
+  } else {
+    using R = typename RawVec<B>::type;
+    __builtin_nontemporal_store(__builtin_bit_cast(R, v), reinterpret_cast<R*>(p));
+  }
+}
 
 template <typename F> struct EwTraits {
   static constexpr int NIN = F::NIN;
@@ -51,6 +83,10 @@ __device__ __forceinline__ VecN<typename F::out_t, V> ew_apply(const F& f, const
 constexpr int kEwBlock = 256;
 constexpr int kEwUnroll = 4;
 
+// One block = one contiguous tile of kEwUnroll x 256 vectors per operand (16 KB each for
+// 128-bit vectors): all loads of the tile are issued before the first store, and the tile is a
+// single DRAM-friendly span — a grid-stride walk with the same number of loads in flight
+// measured 10-25 % slower on this chip.
 template <typename F>
 __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_t n) {
   using TO = typename F::out_t;
@@ -65,33 +101,36 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_
   TO* o = static_cast<TO*>(p.out);
 
   const int64_t nvec = n / V;
-  const int64_t stride = (int64_t)gridDim.x * kEwBlock;
-  int64_t i = (int64_t)blockIdx.x * kEwBlock + threadIdx.x;
-  for (; i + (kEwUnroll - 1) * stride < nvec; i += kEwUnroll * stride) {
-    VecN<T0, V> va[kEwUnroll];
-    VecN<T1, V> vb[kEwUnroll];
-    VecN<T2, V> vc[kEwUnroll];
+  constexpr int64_t TILE = (int64_t)kEwBlock * kEwUnroll;
+  for (int64_t base = (int64_t)blockIdx.x * TILE; base < nvec; base += (int64_t)gridDim.x * TILE) {
+    const int64_t i0 = base + threadIdx.x;
+    if (base + TILE <= nvec) {
+      VecN<T0, V> va[kEwUnroll];
+      VecN<T1, V> vb[kEwUnroll];
+      VecN<T2, V> vc[kEwUnroll];
 #pragma unroll
-    for (int u = 0; u < kEwUnroll; ++u) {
-      const int64_t e = (i + u * stride) * V;
-      va[u] = ld<T0, V>(a + e);
-      if constexpr (NIN > 1) vb[u] = ld<T1, V>(b + e);
-      if constexpr (NIN > 2) vc[u] = ld<T2, V>(c + e);
-    }
+      for (int u = 0; u < kEwUnroll; ++u) {
+        const int64_t e = (i0 + u * kEwBlock) * V;
+        va[u] = ld_nt<T0, V>(a + e);
+        if constexpr (NIN > 1) vb[u] = ld_nt<T1, V>(b + e);
+        if constexpr (NIN > 2) vc[u] = ld_nt<T2, V>(c + e);
+      }
 #pragma unroll
-    for (int u = 0; u < kEwUnroll; ++u) {
-      const int64_t e = (i + u * stride) * V;
-      st<TO, V>(o + e, ew_apply<F, V>(f, va[u], vb[u], vc[u]));
+      for (int u = 0; u < kEwUnroll; ++u) {
+        const int64_t e = (i0 + u * kEwBlock) * V;
+        st_nt<TO, V>(o + e, ew_apply<F, V>(f, va[u], vb[u], vc[u]));
+      }
+    } else {
+      for (int64_t i = i0; i < nvec; i += kEwBlock) {
+        const int64_t e = i * V;
+        VecN<T0, V> va = ld_nt<T0, V>(a + e);
+        VecN<T1, V> vb;
+        VecN<T2, V> vc;
+        if constexpr (NIN > 1) vb = ld_nt<T1, V>(b + e);
+        if constexpr (NIN > 2) vc = ld_nt<T2, V>(c + e);
+        st_nt<TO, V>(o + e, ew_apply<F, V>(f, va, vb, vc));
+      }
     }
-  }
-  for (; i < nvec; i += stride) {
-    const int64_t e = i * V;
-    VecN<T0, V> va = ld<T0, V>(a + e);
-    VecN<T1, V> vb;
-    VecN<T2, V> vc;
-    if constexpr (NIN > 1) vb = ld<T1, V>(b + e);
-    if constexpr (NIN > 2) vc = ld<T2, V>(c + e);
-    st<TO, V>(o + e, ew_apply<F, V>(f, va, vb, vc));
   }
   // ragged tail (< V elements), first threads of block 0
   if (blockIdx.x == 0) {
@@ -205,7 +244,7 @@ __global__ __launch_bounds__(kEwBlock) void ew_strided_kernel(F f, EwPtrs p,
       vb = ld_or_splat<T1, V>(static_cast<const T1*>(p.in[1]) + off[1], a.splat_mask & 2u);
     if constexpr (NIN > 2)
       vc = ld_or_splat<T2, V>(static_cast<const T2*>(p.in[2]) + off[2], a.splat_mask & 4u);
-    st<TO, V>(static_cast<TO*>(p.out) + off[NT - 1], ew_apply<F, V>(f, va, vb, vc));
+    st_nt<TO, V>(static_cast<TO*>(p.out) + off[NT - 1], ew_apply<F, V>(f, va, vb, vc));
   }
 }
 
@@ -237,7 +276,7 @@ int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_t
     for (int t = 0; t < NIN; ++t)
       vec_ok = vec_ok && (reinterpret_cast<uintptr_t>(ins[t]->data) % (esz[t] * V)) == 0;
     if (vec_ok) {
-      const int grid = grid_for((n + V - 1) / V, kEwBlock * kEwUnroll, max_blocks);
+      const int grid = grid_for((n + V - 1) / V, kEwBlock * kEwUnroll, 1 << 30);
       hipLaunchKernelGGL(ew_flat_kernel<F>, dim3(grid), dim3(kEwBlock), 0, stream, f, p, n);
     } else {
       const int grid = grid_for(n, kEwBlock, max_blocks);
@@ -288,7 +327,7 @@ int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_t
   const bool wide = total >= (int64_t(1) << 31);
   if (!wide)
     for (int k = 0; k < d.ndim; ++k) a.div[k] = make_fastdiv((uint32_t)a.sizes[k]);
-  const int grid = grid_for(total, kEwBlock, kNumCU * 32);
+  const int grid = grid_for(total, kEwBlock, 1 << 30);
   if (vec_ok) {
     if (wide)
       hipLaunchKernelGGL((ew_strided_kernel<F, V, true>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);

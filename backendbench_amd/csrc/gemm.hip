@@ -1,14 +1,14 @@
 // mm / addmm:  out[M,N] = beta * c + alpha * (a[M,K] @ b[K,N]),  fp32 accumulate.
 //
 //   mfma     bf16 / f16, a K-contiguous, b either K-contiguous ("NT", e.g. weight.t()) or
-//            N-contiguous ("NN", row-major), 16-byte aligned rows.  256x256x64 block tile,
-//            eight wave64 (2x4, two per SIMD), each wave 128x64 = 8x4 v_mfma_f32_16x16x32
-//            tiles with 128 fp32 accumulators; A and B panels double-buffered in 128 KB of
-//            LDS, swizzled so that the 128-bit global->LDS writes and the fragment reads
-//            are bank-conflict free.  A row-major B stays N-contiguous in LDS and is
-//            transposed by the LDS read itself (ds_read_b64_tr_b16).  The next k-tile is
-//            in flight from HBM/L2 to registers during the MFMA phase; block -> tile map
-//            groups tiles per XCD so that one L2 serves neighbouring tiles.
+//            N-contiguous ("NN", row-major), 16-byte aligned rows.  256x256x32 block tile,
+//            eight wave64 (2x4, two per SIMD), each wave 128x64 = 4x2 v_mfma_f32_32x32x16
+//            tiles with 128 fp32 accumulators; a four-stage 128 KB LDS ring, swizzled so
+//            that the 128-bit global->LDS writes and the fragment reads are bank-conflict
+//            free.  A row-major B stays N-contiguous in LDS and is transposed by the LDS
+//            read itself (ds_read_b64_tr_b16).  Tile it+3 is in flight from L2/HBM while
+//            tile `it` is multiplied; block -> tile map groups tiles per XCD so that one
+//            L2 serves neighbouring tiles.
 //   generic  any strides, bf16 / f16 / f32: 64x64 LDS tile, FMA inner loop.  Correctness
 //            path for shapes the MFMA kernel does not take.
 #include "common.h"
@@ -23,42 +23,33 @@ template <typename T> struct alignas(sizeof(T) * 4) VecN4 {
   T v[4];
 };
 
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// v_mfma_f32_32x32x16: measured at ~96 % of the 2.5 PFLOP/s bf16 peak on MI355X when issued
+// back to back; the 16x16x32 form tops out near 60 %, so the 32x32 form is the only one used.
+// Operand layout: lane l holds 8 consecutive k (k = (l/32)*8 + e) of row/column l%32; the
+// 32x32 result puts column l%32 and rows 8*(r/4) + (l/32)*4 + r%4 in register r of lane l.
 template <typename T> struct Mfma;
 template <> struct Mfma<bf16_t> {
   using frag = bf16x8;
-  static __device__ __forceinline__ f32x4 run(frag a, frag b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ f32x16 run(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct Mfma<f16_t> {
   using frag = f16x8;
-  static __device__ __forceinline__ f32x4 run(frag a, frag b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ f32x16 run(frag a, frag b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
 };
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kGemmThreads = 512;                  // 8 waves: 2 (m) x 4 (n), each 128 x 64
-constexpr int kRowBytes = BK * 2;                  // K-contiguous panel row: 64 k = 128 B = 8 chunks
-constexpr int kPanelBytes = BM * kRowBytes;        // 32 KB per operand per stage (either layout)
-constexpr int kStageBytes = 2 * kPanelBytes;       // A + B
-constexpr int kGemmLds = 2 * kStageBytes;          // double buffered: 128 KB
-
-// K-contiguous panel ([row][k], A and the "NT" B): byte offset of 16-byte chunk c (0..7) of
-// row r.  The chunk index is XORed with (r + r/8) mod 8, which makes both any 8 consecutive
-// rows (32-bank LDS) and any 16 consecutive rows (64-bank LDS) hit distinct banks when the 16
-// lanes of an MFMA fragment read the same chunk of 16 rows; the 128-bit writes of a row's 8
-// chunks stay a full 128-byte line.
-__device__ __forceinline__ int swz_k(int r, int c) {
-  return r * kRowBytes + ((c ^ ((r + (r >> 3)) & 7)) << 4);
-}
+constexpr int BM = 256, BN = 256;
 // N-contiguous panel ([k][n], the row-major "NN" B, 512 B per k): byte offset of 16-byte unit u
-// (0..31) of row k.  32-byte chunks are XORed with (k%4) | ((k/8)%2)*4 so that the transposing
-// 64-bit reads (4 k-rows x 32 B per 16 lanes, rows k..k+3 and k+8..k+11 per 32 lanes) spread
-// over all banks.
+// (0..31) of row k.  64-byte segments are rotated by k%4 (XOR on the segment index) so that a
+// transposing 64-bit read by 32 lanes — 4 consecutive k-rows x 64 B, see lds_read_tr — covers
+// four distinct 64-byte segments of the 256-byte bank window.
 __device__ __forceinline__ int swz_n(int k, int u) {
-  const int x = (k & 3) | (((k >> 3) & 1) << 2);
-  return k * (BN * 2) + ((((u >> 1) ^ x)) << 5) + ((u & 1) << 4);
+  return k * (BN * 2) + ((((u >> 2) ^ (k & 3))) << 6) + ((u & 3) << 4);
 }
 
 struct GemmArgs {
@@ -106,8 +97,27 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
       (__attribute__((address_space(3))) s16x4*)(uintptr_t)(const_cast<unsigned char*>(p)));
 }
 
-template <typename T, bool B_NN>
-__global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
+// ---------------------------------------------------------------- MFMA kernel
+// 256x256 block tile, BK = 32, a ring of four 32 KB LDS stages (A 256x32 + B 32x256 each).
+// In iteration `it` a wave (a) writes tile it+2 from registers into the ring, (b) starts the
+// global loads of tile it+3, (c) multiplies tile `it`, and already reads the first fragments
+// of tile it+1 — visible since the previous barrier — before it reaches the barrier, so the
+// MFMA pipe has work the moment the barrier opens.  The slot being overwritten held tile
+// it-2, which every wave finished before the previous barrier.
+constexpr int BK3 = 32;
+constexpr int kStages3 = 4;
+constexpr int kPanel3 = BM * BK3 * 2;        // 16 KB per operand per stage
+constexpr int kStage3 = 2 * kPanel3;         // 32 KB
+constexpr int kGemmLds = kStages3 * kStage3;  // 128 KB
+
+// K-contiguous panel with 64-byte rows (4 chunks): XOR with (r/4)%4 spreads 16 consecutive rows
+// reading the same chunk over the 16 16-byte positions of the 256-byte bank window.
+__device__ __forceinline__ int swz_k32(int r, int c) { return r * 64 + ((c ^ ((r >> 2) & 3)) << 4); }
+
+// KTAIL: K is not a multiple of BK3, so chunks past K are zero-filled (branch-free: the address
+// is clamped and the loaded value replaced); the common case compiles without the checks.
+template <typename T, bool B_NN, bool KTAIL>
+__global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using frag_t = typename Mfma<T>::frag;
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
@@ -118,122 +128,131 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_mfma_kernel(GemmArgs g) {
   const T* A = static_cast<const T*>(g.a);
   const T* B = static_cast<const T*>(g.b);
 
-  // ---- global -> register staging: 4 chunks of A and 4 of B per thread per k-tile
-  u32x4 ra[4], rb[4];
-  const int lc = tid & 7, lr = tid >> 3;    // K-contiguous panels: chunk lc of rows lr + 64*i
-  const int nu = tid & 31, kr = tid >> 5;   // NN B: 16-byte unit nu of k rows kr + 16*i
-  auto load_tile = [&](int k0) {
+  u32x4 ra[2], rb[2];
+  const int lc = tid & 3, lr = tid >> 2;   // K-contiguous panels: chunk lc of rows lr + 128*i
+  const int nu = tid & 31, kr = tid >> 5;  // NN B: 16-byte unit nu of k rows kr + 16*i
+  const u32x4 zero4 = {0, 0, 0, 0};
+  const T* a_ptr[2];
+  const T* b_ptr[2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      int gr = bm + lr + 64 * i;
-      gr = gr < g.M ? gr : g.M - 1;
-      const int k = k0 + lc * 8;
-      ra[i] = k < g.K ? *reinterpret_cast<const u32x4*>(A + (int64_t)gr * g.lda + k) : u32x4{0, 0, 0, 0};
-    }
+  for (int i = 0; i < 2; ++i) {
+    int gr = bm + lr + 128 * i;
+    gr = gr < g.M ? gr : g.M - 1;
+    a_ptr[i] = A + (int64_t)gr * g.lda + lc * 8;
     if constexpr (!B_NN) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int gn = bn + lr + 64 * i;
-        gn = gn < g.N ? gn : g.N - 1;
-        const int k = k0 + lc * 8;
-        rb[i] = k < g.K ? *reinterpret_cast<const u32x4*>(B + (int64_t)gn * g.ldb + k) : u32x4{0, 0, 0, 0};
-      }
+      int gn = bn + lr + 128 * i;
+      gn = gn < g.N ? gn : g.N - 1;
+      b_ptr[i] = B + (int64_t)gn * g.ldb + lc * 8;
     } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int k = k0 + kr + 16 * i;
-        int gn = bn + nu * 8;
-        gn = gn < g.N ? gn : 0;  // N % 8 == 0: a unit is all-in or all-out; out-of-range columns are never stored
-        rb[i] = k < g.K ? *reinterpret_cast<const u32x4*>(B + (int64_t)k * g.ldb + gn) : u32x4{0, 0, 0, 0};
-      }
+      int gn = bn + nu * 8;
+      gn = gn < g.N ? gn : 0;
+      b_ptr[i] = B + (int64_t)(kr + 16 * i) * g.ldb + gn;
     }
-  };
-  auto store_tile = [&](int stage) {
-    unsigned char* pa = lds + stage * kStageBytes;
-    unsigned char* pb = pa + kPanelBytes;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(pa + swz_k(lr + 64 * i, lc)) = ra[i];
-    if constexpr (!B_NN) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(pb + swz_k(lr + 64 * i, lc)) = rb[i];
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(pb + swz_n(kr + 16 * i, nu)) = rb[i];
-    }
-  };
-
-  f32x4 acc[8][4];
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  const int nk = (g.K + BK - 1) / BK;
-  if (nk > 0) {
-    load_tile(0);
-    store_tile(0);
-    if (nk > 1) load_tile(BK);
   }
-  __syncthreads();
-  const int fr = lane & 15, fc = lane >> 4;  // fragment row (m or n) and k-group of this lane
-  for (int kt = 0; kt < nk; ++kt) {
-    const int stage = kt & 1;
-    const unsigned char* pa = lds + stage * kStageBytes;
-    const unsigned char* pb = pa + kPanelBytes;
+  auto load_tile = [&](int t) {
+    const int k0 = t * BK3;
 #pragma unroll
-    for (int kk = 0; kk < BK / 32; ++kk) {
-      frag_t fa[8], fb[4];
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k(wm * 128 + i * 16 + fr, kk * 4 + fc));
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        if constexpr (!B_NN) {
-          fb[j] = *reinterpret_cast<const frag_t*>(pb + swz_k(wn * 64 + j * 16 + fr, kk * 4 + fc));
-        } else {
-          // k = kk*32 + fc*8 + h*4 + (lane%16)/4, columns wn*64 + j*16 + 4*(lane%4) .. +3
-          const int kb = kk * 32 + fc * 8 + (fr >> 2);
-          const int n0 = wn * 64 + j * 16 + ((fr & 3) << 2);  // element column; 16-byte unit = n0/8
-          const s16x4 lo = lds_read_tr(pb + swz_n(kb, n0 >> 3) + ((n0 & 7) << 1));
-          const s16x4 hi = lds_read_tr(pb + swz_n(kb + 4, n0 >> 3) + ((n0 & 7) << 1));
-          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          fb[j] = __builtin_bit_cast(frag_t, both);
-        }
+    for (int i = 0; i < 2; ++i) {
+      const bool in_a = !KTAIL || k0 + lc * 8 < g.K;
+      const u32x4 va = *reinterpret_cast<const u32x4*>(a_ptr[i] + (in_a ? k0 : 0));
+      ra[i] = in_a ? va : zero4;
+      if constexpr (!B_NN) {
+        const u32x4 vb = *reinterpret_cast<const u32x4*>(b_ptr[i] + (in_a ? k0 : 0));
+        rb[i] = in_a ? vb : zero4;
+      } else {
+        const bool in_b = !KTAIL || k0 + kr + 16 * i < g.K;
+        const u32x4 vb = *reinterpret_cast<const u32x4*>(b_ptr[i] + (int64_t)(in_b ? k0 : 0) * g.ldb);
+        rb[i] = in_b ? vb : zero4;
       }
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          // operands swapped: the lane ends up with 4 consecutive n of one row m
-          acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
     }
-    if (kt + 1 < nk) {
-      store_tile(stage ^ 1);                       // tile kt+1, loaded during the previous compute phase
-      if (kt + 2 < nk) load_tile((kt + 2) * BK);  // in flight during the next compute phase
+  };
+  auto store_tile = [&](int t) {
+    unsigned char* pa = lds + (t % kStages3) * kStage3;
+    unsigned char* pb = pa + kPanel3;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      *reinterpret_cast<u32x4*>(pa + swz_k32(lr + 128 * i, lc)) = ra[i];
+      if constexpr (!B_NN) *reinterpret_cast<u32x4*>(pb + swz_k32(lr + 128 * i, lc)) = rb[i];
+      else *reinterpret_cast<u32x4*>(pb + swz_n(kr + 16 * i, nu)) = rb[i];
     }
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  const int tr_k = fg * 8 + ((lane & 15) >> 2);
+  const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  auto read_frags = [&](int t, int ks, frag_t (&fa)[4], frag_t (&fb)[2]) {
+    const unsigned char* pa = lds + (t % kStages3) * kStage3;
+    const unsigned char* pb = pa + kPanel3;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k32(wm * 128 + i * 32 + fr, ks * 2 + fg));
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if constexpr (!B_NN) {
+        fb[j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * 64 + j * 32 + fr, ks * 2 + fg));
+      } else {
+        const int k = ks * 16 + tr_k;
+        const int n = wn * 64 + j * 32 + tr_n;
+        const s16x4 lo = lds_read_tr(pb + swz_n(k, n >> 3) + ((n & 7) << 1));
+        const s16x4 hi = lds_read_tr(pb + swz_n(k + 4, n >> 3) + ((n & 7) << 1));
+        fb[j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    }
+  };
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto mma = [&](frag_t (&fa)[4], frag_t (&fb)[2]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+  };
+
+  const int nk = (g.K + BK3 - 1) / BK3;
+  if (nk > 0) { load_tile(0); store_tile(0); }
+  if (nk > 1) { load_tile(1); store_tile(1); }
+  if (nk > 2) load_tile(2);
+  __syncthreads();
+  frag_t fa0[4], fb0[2], fa1[4], fb1[2];
+  if (nk > 0) read_frags(0, 0, fa0, fb0);
+  for (int it = 0; it < nk; ++it) {
+    if (it + 2 < nk) store_tile(it + 2);
+    if (it + 3 < nk) load_tile(it + 3);
+    read_frags(it, 1, fa1, fb1);
+    mma(fa0, fb0);
+    if (it + 1 < nk) read_frags(it + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
     __syncthreads();
   }
 
-  // ---- epilogue: lane holds C[m = fr][n = fc*4 .. +3] of each 16x16 tile
   T* D = static_cast<T*>(g.out);
   const T* C = static_cast<const T*>(g.c);
   const bool use_c = C != nullptr && g.beta != 0.f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int m = bm + wm * 128 + i * 16 + fr;
+  for (int i = 0; i < 4; ++i) {
+    const int m = bm + wm * 128 + i * 32 + fr;
     if (m >= g.M) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = bn + wn * 64 + j * 16 + fc * 4;
-      if (n >= g.N) continue;  // N % 4 == 0 on this path: 4 columns are all in or all out
-      VecN4<T> r;
+    for (int j = 0; j < 2; ++j) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float v = g.alpha * acc[i][j][e];
-        if (use_c) v += g.beta * static_cast<float>(C[(int64_t)m * g.c_rs + (int64_t)(n + e) * g.c_cs]);
-        r.v[e] = static_cast<T>(v);
+      for (int q = 0; q < 4; ++q) {
+        const int n = bn + wn * 64 + j * 32 + q * 8 + fg * 4;
+        if (n >= g.N) continue;
+        VecN4<T> r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = g.alpha * acc[i][j][q * 4 + e];
+          if (use_c) v += g.beta * static_cast<float>(C[(int64_t)m * g.c_rs + (int64_t)(n + e) * g.c_cs]);
+          r.v[e] = static_cast<T>(v);
+        }
+        *reinterpret_cast<VecN4<T>*>(D + (int64_t)m * g.N + n) = r;
       }
-      *reinterpret_cast<VecN4<T>*>(D + (int64_t)m * g.N + n) = r;
     }
   }
 }
@@ -313,22 +332,25 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       g.tiles_n = (int32_t)((N + BN - 1) / BN);
       const int64_t nblocks = (int64_t)g.tiles_m * g.tiles_n;
       MI355_REQUIRE(nblocks < (int64_t(1) << 31), "mi355_gemm: too many tiles");
-      static thread_local bool attr_set[2] = {false, false};
-      if (b_nt) {
-        auto kern = gemm_mfma_kernel<T, false>;
-        if (!attr_set[0]) {
-          hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
-          attr_set[0] = true;
-        }
-        hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(kGemmThreads), kGemmLds, st, g);
-      } else {
-        auto kern = gemm_mfma_kernel<T, true>;
-        if (!attr_set[1]) {
-          hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
-          attr_set[1] = true;
-        }
-        hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(kGemmThreads), kGemmLds, st, g);
+      const bool ktail = K % BK3 != 0;
+      const void* kern =
+          b_nt ? (ktail ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, false, false>)
+               : (ktail ? (const void*)gemm_mfma_kernel<T, true, true> : (const void*)gemm_mfma_kernel<T, true, false>);
+      const int nthreads = 512;
+      // 128 KB of dynamic LDS needs the attribute once per kernel and process.
+      static thread_local const void* attr_done[8] = {};
+      bool seen = false;
+      for (const void* k : attr_done) seen = seen || k == kern;
+      if (!seen) {
+        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
+        if (e != hipSuccess)
+          return set_error(MI355_ERR_LAUNCH, "mi355_gemm: cannot reserve %d bytes of LDS: %s", kGemmLds, hipGetErrorString(e));
+        for (const void*& k : attr_done)
+          if (k == nullptr) { k = kern; break; }
       }
+      void* params[] = {&g};
+      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks), dim3(nthreads), params, kGemmLds, st);
+      if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma): launch failed: %s", hipGetErrorString(e));
       return check_launch("mi355_gemm(mfma)");
     }
   }

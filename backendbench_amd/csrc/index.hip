@@ -4,8 +4,10 @@
 //   rows_wave   rows of >= 64 copy units: one wave64 per output row, 128-bit units when
 //               alignment allows, four loads in flight per lane;
 //   rows_elem   short rows: one thread per copy unit;
-//   gather      one thread per output element (or per 4 consecutive 32-bit elements when
-//               the index tensor is dense), index stream coalesced.
+//   gather_rows gather along the last dim of dense operands: the source row is staged in LDS
+//               with coalesced loads and the indices are resolved there;
+//   gather      any other layout: one thread per output element (or per 4 consecutive 32-bit
+//               elements when the index tensor is dense), index stream coalesced.
 // An out-of-range index is never dereferenced: the output is zero-filled there and the
 // device error flag is raised.
 #include "elementwise.h"
@@ -13,6 +15,7 @@
 namespace mi355 {
 
 constexpr int kIxBlock = 256;
+typedef u32x4 U128;  // 16-byte copy unit
 
 template <typename I> __device__ __forceinline__ int64_t load_index(const void* p, int64_t j) {
   return (int64_t) static_cast<const I*>(p)[j];
@@ -32,19 +35,21 @@ __global__ __launch_bounds__(kIxBlock) void index_rows_wave_kernel(const U* __re
     U* dst = out + r * row_units;
     if (idx < 0 || idx >= n_src) {
       if (err && lane == 0) *err = 1;
-      for (int64_t u = lane; u < row_units; u += kWave) dst[u] = U{};
+      for (int64_t u = lane; u < row_units; u += kWave) dst[u] = U(0);
       continue;
     }
     const U* s = src + (o * n_src + idx) * row_units;
+    // rows are read and written once: streaming (non-temporal) accesses, four loads in flight
     int64_t u = lane;
     for (; u + 3 * kWave < row_units; u += 4 * kWave) {
-      const U a = s[u], b = s[u + kWave], c = s[u + 2 * kWave], d = s[u + 3 * kWave];
-      dst[u] = a;
-      dst[u + kWave] = b;
-      dst[u + 2 * kWave] = c;
-      dst[u + 3 * kWave] = d;
+      const U a = __builtin_nontemporal_load(s + u), b = __builtin_nontemporal_load(s + u + kWave),
+              c = __builtin_nontemporal_load(s + u + 2 * kWave), d = __builtin_nontemporal_load(s + u + 3 * kWave);
+      __builtin_nontemporal_store(a, dst + u);
+      __builtin_nontemporal_store(b, dst + u + kWave);
+      __builtin_nontemporal_store(c, dst + u + 2 * kWave);
+      __builtin_nontemporal_store(d, dst + u + 3 * kWave);
     }
-    for (; u < row_units; u += kWave) dst[u] = s[u];
+    for (; u < row_units; u += kWave) __builtin_nontemporal_store(__builtin_nontemporal_load(s + u), dst + u);
   }
 }
 
@@ -60,16 +65,13 @@ __global__ __launch_bounds__(kIxBlock) void index_rows_elem_kernel(const U* __re
     const int64_t idx = load_index<I>(index, j);
     if (idx < 0 || idx >= n_src) {
       if (err) *err = 1;
-      out[e] = U{};
+      out[e] = U(0);
     } else {
       out[e] = src[(o * n_src + idx) * row_units + u];
     }
   }
 }
 
-struct U128 {
-  uint32_t w[4];
-} __attribute__((aligned(16)));
 
 template <typename U>
 static int run_index_select(const void* src, const void* index, int idx_dtype, void* out, int64_t outer, int64_t n_src,
@@ -146,6 +148,55 @@ __global__ __launch_bounds__(kIxBlock) void gather_kernel(const U* __restrict__ 
   }
 }
 
+// Gather along the last dim of a dense [rows, len] source with a dense [rows, n_idx] index:
+// one block stages (its share of) the source row in LDS with coalesced 128-bit loads, then
+// resolves four indices per thread per step from LDS — the index stream and the output stay
+// fully coalesced and no random access leaves the CU.  grid = (splits, rows).
+template <typename U>
+__global__ __launch_bounds__(kIxBlock) void gather_rows_lds_kernel(const U* __restrict__ src, const int64_t* __restrict__ index,
+                                                                  U* __restrict__ out, int64_t len, int64_t n_idx,
+                                                                  int64_t per_split, int32_t* err) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  U* row = reinterpret_cast<U*>(smem_raw);
+  const int64_t r = blockIdx.y;
+  const U* s = src + r * len;
+  constexpr int UV = 16 / sizeof(U);
+  if (len % UV == 0 && (reinterpret_cast<uintptr_t>(s) & 15) == 0) {
+    for (int64_t i = (int64_t)threadIdx.x * UV; i < len; i += (int64_t)kIxBlock * UV)
+      st<U, UV>(row + i, ld_nt<U, UV>(s + i));
+  } else {
+    for (int64_t i = threadIdx.x; i < len; i += kIxBlock) row[i] = s[i];
+  }
+  __syncthreads();
+  const int64_t j0 = (int64_t)blockIdx.x * per_split;
+  const int64_t j1 = j0 + per_split < n_idx ? j0 + per_split : n_idx;
+  const int64_t* ix = index + r * n_idx;
+  U* o = out + r * n_idx;
+  const bool vec = n_idx % 4 == 0 && per_split % 4 == 0 && (reinterpret_cast<uintptr_t>(ix) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(o) % (4 * sizeof(U))) == 0;
+  if (vec) {
+    for (int64_t j = j0 + (int64_t)threadIdx.x * 4; j < j1; j += (int64_t)kIxBlock * 4) {
+      const VecN<int64_t, 2> a = ld_nt<int64_t, 2>(ix + j), b = ld_nt<int64_t, 2>(ix + j + 2);
+      const int64_t id[4] = {a.v[0], a.v[1], b.v[0], b.v[1]};
+      VecN<U, 4> v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool ok = id[e] >= 0 && id[e] < len;
+        if (!ok && err) *err = 1;
+        v.v[e] = ok ? row[id[e]] : U(0);
+      }
+      st_nt<U, 4>(o + j, v);
+    }
+  } else {
+    for (int64_t j = j0 + threadIdx.x; j < j1; j += kIxBlock) {
+      const int64_t id = ix[j];
+      const bool ok = id >= 0 && id < len;
+      if (!ok && err) *err = 1;
+      o[j] = ok ? row[id] : U(0);
+    }
+  }
+}
+
 template <typename U>
 static int run_gather(const mi355_tensor* src, int dim, const mi355_tensor* index, const mi355_tensor* out,
                       int32_t* err, hipStream_t st) {
@@ -164,6 +215,35 @@ static int run_gather(const mi355_tensor* src, int dim, const mi355_tensor* inde
   }
   const int64_t n = numel(out);
   const int last = index->ndim - 1;
+  // LDS-staged path: last-dim gather, dense source and index, matching outer extents.
+  {
+    bool ok = dim == last && idx_dense;
+    int64_t expect_s = 1, rows = 1;
+    for (int k = last; k >= 0 && ok; --k) {
+      if (src->sizes[k] != 1 && src->strides[k] != expect_s) ok = false;
+      expect_s *= src->sizes[k];
+      if (k != last) {
+        if (index->sizes[k] != src->sizes[k]) ok = false;
+        rows *= index->sizes[k];
+      }
+    }
+    const int64_t len = src->sizes[last], n_idx = index->sizes[last];
+    if (ok && len > 0 && len * (int64_t)sizeof(U) <= 64 * 1024 && rows < 65536 && n_idx >= len / 8) {
+      int64_t splits = 1;
+      if (rows < 512) {
+        splits = n_idx / 4096;
+        if (splits < 1) splits = 1;
+        if (splits > 64) splits = 64;
+      }
+      int64_t per_split = (n_idx + splits - 1) / splits;
+      per_split = (per_split + 3) / 4 * 4;
+      splits = (n_idx + per_split - 1) / per_split;
+      hipLaunchKernelGGL((gather_rows_lds_kernel<U>), dim3((unsigned)splits, (unsigned)rows), dim3(kIxBlock),
+                         (size_t)(len * sizeof(U)), st, (const U*)src->data, (const int64_t*)index->data,
+                         (U*)out->data, len, n_idx, per_split, err);
+      return check_launch("mi355_gather(lds)");
+    }
+  }
   const bool vec = sizeof(U) == 4 && idx_dense && a.sizes[last] % 4 == 0 && aligned16(index->data) &&
                    aligned16(out->data);
   if (vec) {

@@ -1,8 +1,8 @@
 // native_layer_norm over the last N elements of M dense rows: returns y, mean, rstd.
 //
-//   wave   row fits a wave's registers: one HBM read; mean by wave all-reduce, then the
-//          centred second moment from the same registers (exact two-step statistics at
-//          single-pass traffic); y written once;
+//   tile   row fits the registers of 1, 2 or 4 cooperating waves: one HBM read; mean by
+//          all-reduce, then the centred second moment from the same registers (exact
+//          two-step statistics at single-pass traffic); y written once;
 //   block  longer rows: per-thread Welford accumulation, Chan's pairwise merge across
 //          lanes (shuffles) and waves (LDS), then the row is re-read (L2) to normalise.
 #include <type_traits>
@@ -11,38 +11,41 @@
 
 namespace mi355 {
 
-constexpr int kLnBlock = 256;
+constexpr int kLnBlock = kRowBlock;
 
-template <typename T, typename W, typename S, int NV, bool VEC>
-__global__ __launch_bounds__(kLnBlock) void layernorm_wave_kernel(const T* __restrict__ x, const W* __restrict__ w,
-                                                                 const W* __restrict__ b, T* __restrict__ y,
+template <typename T, typename Wt, typename S, int NV, bool VEC, int W>
+__global__ __launch_bounds__(kLnBlock) void layernorm_tile_kernel(const T* __restrict__ x, const Wt* __restrict__ w,
+                                                                 const Wt* __restrict__ b, T* __restrict__ y,
                                                                  S* __restrict__ mean_out, S* __restrict__ rstd_out,
                                                                  int64_t rows, int64_t n, float eps) {
-  const int lane = threadIdx.x % kWave;
-  const int64_t row = (int64_t)blockIdx.x * (kLnBlock / kWave) + threadIdx.x / kWave;
-  if (row >= rows) return;
-  using Tile = RowTile<T, NV, VEC>;
+  using Tile = RowTile<T, NV, VEC, W>;
   constexpr int V = Tile::V;
-  Tile t;
-  t.load(x + row * n, n, lane, 0.f);
+  __shared__ float red_a[kLnBlock / kWave], red_b[kLnBlock / kWave];
+  const int t = threadIdx.x % Tile::GROUP;
+  int64_t row = (int64_t)blockIdx.x * Tile::ROWS_PER_BLOCK + threadIdx.x / Tile::GROUP;
+  const bool active = row < rows;  // inactive groups still walk through the barriers
+  if (!active) row = rows - 1;
+  Tile tile;
+  tile.load(x + row * n, n, t, 0.f);
   float s = 0.f;
 #pragma unroll
   for (int k = 0; k < NV; ++k)
 #pragma unroll
-    for (int j = 0; j < V; ++j) s += t.v[k][j];
+    for (int j = 0; j < V; ++j) s += tile.v[k][j];
   const float inv_n = 1.f / (float)n;
-  const float mean = wave_allreduce(s, SumOp()) * inv_n;
+  const float mean = group_allreduce<W>(s, SumOp(), red_a) * inv_n;
   float q = 0.f;
 #pragma unroll
   for (int k = 0; k < NV; ++k)
 #pragma unroll
     for (int j = 0; j < V; ++j) {
-      const float d = Tile::col(k, j, lane) < n ? t.v[k][j] - mean : 0.f;
+      const float d = Tile::col(k, j, t) < n ? tile.v[k][j] - mean : 0.f;
       q += d * d;
     }
-  const float var = wave_allreduce(q, SumOp()) * inv_n;
+  const float var = group_allreduce<W>(q, SumOp(), red_b) * inv_n;
   const float rstd = rsqrtf(var + eps);
-  if (lane == 0) {
+  if (!active) return;
+  if (t == 0) {
     mean_out[row] = static_cast<S>(mean);
     rstd_out[row] = static_cast<S>(rstd);
   }
@@ -51,24 +54,24 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_wave_kernel(const T* __res
     // gamma/beta come through L2 as whole vectors, one per slab, shared by every row.
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-      const int64_t c = Tile::col(k, 0, lane);
+      const int64_t c = Tile::col(k, 0, t);
       if (c < n) {
-        VecN<W, V> g, be;
-        if (w) g = ld<W, V>(w + c);
-        if (b) be = ld<W, V>(b + c);
-        Vec<T> r;
+        VecN<Wt, V> g, be;
+        if (w) g = ld<Wt, V>(w + c);
+        if (b) be = ld<Wt, V>(b + c);
+        VecN<T, V> r;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-          float f = (t.v[k][j] - mean) * rstd;
+          float f = (tile.v[k][j] - mean) * rstd;
           if (w) f *= static_cast<float>(g.v[j]);
           if (b) f += static_cast<float>(be.v[j]);
           r.v[j] = static_cast<T>(f);
         }
-        store_vec(out + c, r);
+        st_nt<T, V>(out + c, r);
       }
     }
   } else {
-    t.store(out, n, lane, [=](float v, int64_t c) {
+    tile.store(out, n, t, [=](float v, int64_t c) {
       float r = (v - mean) * rstd;
       if (w) r *= static_cast<float>(w[c]);
       if (b) r += static_cast<float>(b[c]);
@@ -155,12 +158,13 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
   const bool vec = N % V == 0 && aligned16(x) && aligned16(y) &&
                    reinterpret_cast<uintptr_t>(w) % (sizeof(W) * V) == 0 &&
                    reinterpret_cast<uintptr_t>(b) % (sizeof(W) * V) == 0;
-  const int64_t nblk = (M + kLnBlock / kWave - 1) / (kLnBlock / kWave);
   MI355_REQUIRE(M < (int64_t(1) << 31), "mi355_layer_norm: too many rows (%lld)", (long long)M);
-  const bool done = dispatch_row_tile<T>(N, [&](auto nv) {
-    constexpr int NV = decltype(nv)::value;
-    if (vec) hipLaunchKernelGGL((layernorm_wave_kernel<T, W, S, NV, true>), dim3((unsigned)nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
-    else hipLaunchKernelGGL((layernorm_wave_kernel<T, W, S, NV, false>), dim3((unsigned)nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+  const bool done = dispatch_row_tile<T>(N, vec, [&](auto nv, auto wv, auto v) {
+    constexpr int NV = decltype(nv)::value, WG = decltype(wv)::value;
+    constexpr bool VEC = decltype(v)::value;
+    constexpr int rpb = kLnBlock / (kWave * WG);
+    const unsigned nblk = (unsigned)((M + rpb - 1) / rpb);
+    hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, VEC, WG>), dim3(nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
   });
   if (!done) {
     if (vec) hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, true>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, (float)eps);

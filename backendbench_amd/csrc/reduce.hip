@@ -116,8 +116,8 @@ __device__ __forceinline__ void accumulate_span(typename R::State& st, const T* 
     int64_t i = lo + (int64_t)tid * V;
     const int64_t step = (int64_t)nthr * V;
     for (; i + 3 * step < hi; i += 4 * step) {
-      Vec<T> v0 = load_vec(row + i), v1 = load_vec(row + i + step), v2 = load_vec(row + i + 2 * step),
-             v3 = load_vec(row + i + 3 * step);
+      Vec<T> v0 = load_vec_nt(row + i), v1 = load_vec_nt(row + i + step), v2 = load_vec_nt(row + i + 2 * step),
+             v3 = load_vec_nt(row + i + 3 * step);
 #pragma unroll
       for (int j = 0; j < V; ++j) R::acc(st, (A)v0.v[j], i + j);
 #pragma unroll
@@ -128,7 +128,7 @@ __device__ __forceinline__ void accumulate_span(typename R::State& st, const T* 
       for (int j = 0; j < V; ++j) R::acc(st, (A)v3.v[j], i + 3 * step + j);
     }
     for (; i < hi; i += step) {
-      Vec<T> v = load_vec(row + i);
+      Vec<T> v = load_vec_nt(row + i);
 #pragma unroll
       for (int j = 0; j < V; ++j) R::acc(st, (A)v.v[j], i + j);
     }

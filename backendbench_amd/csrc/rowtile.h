@@ -1,8 +1,11 @@
-// A row held in the registers of one wave64: NV slabs of 64 lanes x V elements (V = one
-// 128-bit load), converted to fp32 on load.  Used by the single-pass softmax and layer
-// norm kernels: the row is read from HBM once, reduced with wave all-reduces, and written
-// once.  VEC=false keeps the same register shape with scalar, lane-interleaved accesses
-// for rows whose base is not 16-byte aligned.
+// A row held in the registers of W cooperating wave64s (W = 1, 2 or 4 waves of one 256-thread
+// block): NV slabs of 64*W lanes x V elements (V = one 128-bit load), converted to fp32 on
+// load.  Used by the single-pass softmax and layer norm kernels: the row is read from HBM
+// once (non-temporal 128-bit loads), reduced with wave all-reduces plus one LDS exchange when
+// W > 1, and written once.  Spreading a row over more waves keeps the per-lane tile at <= 32
+// values, so eight waves fit on a SIMD and all rows of a launch are resident at once.
+// VEC = false keeps the same register shape with scalar, lane-interleaved accesses for rows
+// whose base is not 16-byte aligned (W = 1 only).
 #pragma once
 #include <type_traits>
 
@@ -11,26 +14,29 @@
 
 namespace mi355 {
 
-template <typename T, int NV, bool VEC> struct RowTile {
+constexpr int kRowBlock = 256;  // threads per block of every row-tile kernel
+
+template <typename T, int NV, bool VEC, int W> struct RowTile {
   static constexpr int V = 16 / sizeof(T);
-  static constexpr int CAP = NV * V * kWave;  // elements one wave can hold
+  static constexpr int GROUP = kWave * W;        // lanes cooperating on one row
+  static constexpr int ROWS_PER_BLOCK = kRowBlock / GROUP;
   float v[NV][V];
 
-  // Column of element (k, j) for this lane.
-  static __device__ __forceinline__ int64_t col(int k, int j, int lane) {
-    if constexpr (VEC) return ((int64_t)k * kWave + lane) * V + j;
-    else return ((int64_t)k * V + j) * kWave + lane;
+  // Column of element (k, j) for lane `t` (0 .. GROUP-1) of the row group.
+  static __device__ __forceinline__ int64_t col(int k, int j, int t) {
+    if constexpr (VEC) return ((int64_t)k * GROUP + t) * V + j;
+    else return ((int64_t)k * V + j) * GROUP + t;
   }
 
-  __device__ __forceinline__ void load(const T* row, int64_t n, int lane, float pad) {
+  __device__ __forceinline__ void load(const T* row, int64_t n, int t, float pad) {
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       if constexpr (VEC) {
-        const int64_t c = col(k, 0, lane);
+        const int64_t c = col(k, 0, t);
         if (c < n) {  // n % V == 0 on this path: a vector is all-in or all-out
-          const Vec<T> t = load_vec(row + c);
+          const VecN<T, V> x = ld_nt<T, V>(row + c);
 #pragma unroll
-          for (int j = 0; j < V; ++j) v[k][j] = static_cast<float>(t.v[j]);
+          for (int j = 0; j < V; ++j) v[k][j] = static_cast<float>(x.v[j]);
         } else {
 #pragma unroll
           for (int j = 0; j < V; ++j) v[k][j] = pad;
@@ -38,7 +44,7 @@ template <typename T, int NV, bool VEC> struct RowTile {
       } else {
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-          const int64_t c = col(k, j, lane);
+          const int64_t c = col(k, j, t);
           v[k][j] = c < n ? static_cast<float>(row[c]) : pad;
         }
       }
@@ -47,21 +53,21 @@ template <typename T, int NV, bool VEC> struct RowTile {
 
   // out[c] = f(v, c) for every in-range element, written in the slab layout.
   template <typename O, typename Fn>
-  __device__ __forceinline__ void store(O* row, int64_t n, int lane, Fn f) const {
+  __device__ __forceinline__ void store(O* row, int64_t n, int t, Fn f) const {
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       if constexpr (VEC) {
-        const int64_t c = col(k, 0, lane);
+        const int64_t c = col(k, 0, t);
         if (c < n) {
-          VecN<O, V> t;
+          VecN<O, V> x;
 #pragma unroll
-          for (int j = 0; j < V; ++j) t.v[j] = static_cast<O>(f(v[k][j], c + j));
-          st<O, V>(row + c, t);
+          for (int j = 0; j < V; ++j) x.v[j] = static_cast<O>(f(v[k][j], c + j));
+          st_nt<O, V>(row + c, x);
         }
       } else {
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-          const int64_t c = col(k, j, lane);
+          const int64_t c = col(k, j, t);
           if (c < n) row[c] = static_cast<O>(f(v[k][j], c));
         }
       }
@@ -69,15 +75,60 @@ template <typename T, int NV, bool VEC> struct RowTile {
   }
 };
 
-// Calls body(std::integral_constant<int, NV>) for the smallest NV in {1,2,4,8,16} whose
-// tile holds n elements of T; returns false when the row is too long for registers.
-template <typename T, typename Body> inline bool dispatch_row_tile(int64_t n, Body body) {
-  constexpr int64_t unit = (16 / sizeof(T)) * kWave;
-  if (n <= unit) { body(std::integral_constant<int, 1>()); return true; }
-  if (n <= 2 * unit) { body(std::integral_constant<int, 2>()); return true; }
-  if (n <= 4 * unit) { body(std::integral_constant<int, 4>()); return true; }
-  if (n <= 8 * unit) { body(std::integral_constant<int, 8>()); return true; }
-  if (n <= 16 * unit) { body(std::integral_constant<int, 16>()); return true; }
+// All-reduce over the W waves of a row group.  `smem` has one slot per wave of the block and
+// must not be reused by the caller before the next __syncthreads().  Every thread of the
+// block has to call this (it contains a barrier when W > 1).
+template <int W, typename T, typename Op>
+__device__ __forceinline__ T group_allreduce(T v, Op op, T* smem) {
+  v = wave_allreduce(v, op);
+  if constexpr (W == 1) {
+    return v;
+  } else {
+    const int wave = threadIdx.x / kWave;
+    if (threadIdx.x % kWave == 0) smem[wave] = v;
+    __syncthreads();
+    const int first = wave / W * W;
+    T r = smem[first];
+#pragma unroll
+    for (int i = 1; i < W; ++i) r = op(r, smem[first + i]);
+    return r;
+  }
+}
+
+// Picks (NV, W) for rows of n elements of T and calls body(NV, W, VEC) with integral
+// constants; false when the row does not fit 16 slabs over 4 waves.  Aligned rows get at most
+// 32 values per lane (W grows instead); unaligned rows use one wave and the scalar layout.
+template <typename T, typename Body> inline bool dispatch_row_tile(int64_t n, bool vec, Body body) {
+  constexpr int V = 16 / sizeof(T);
+  using std::integral_constant;
+#define MI355_ROW(NV_, W_, VEC_)                                                              \
+  {                                                                                           \
+    body(integral_constant<int, NV_>(), integral_constant<int, W_>(), integral_constant<bool, VEC_>()); \
+    return true;                                                                              \
+  }
+  if (!vec) {
+    const int64_t unit = V * kWave;
+    if (n <= unit) MI355_ROW(1, 1, false)
+    if (n <= 2 * unit) MI355_ROW(2, 1, false)
+    if (n <= 4 * unit) MI355_ROW(4, 1, false)
+    if (n <= 8 * unit) MI355_ROW(8, 1, false)
+    if (n <= 16 * unit) MI355_ROW(16, 1, false)
+    return false;
+  }
+  constexpr int NV32 = 32 / V;  // slabs that make 32 values per lane
+  if (n <= 32 * kWave) {
+    const int64_t unit = V * kWave;
+    if (n <= unit) MI355_ROW(1, 1, true)
+    if (n <= 2 * unit) MI355_ROW(2, 1, true)
+    if (NV32 >= 4 && n <= 4 * unit) MI355_ROW(4, 1, true)
+    MI355_ROW(NV32, 1, true)
+  }
+  if (n <= 32 * kWave * 2) MI355_ROW(NV32, 2, true)
+  const int64_t unit4 = V * kWave * 4;
+  if (n <= NV32 * unit4) MI355_ROW(NV32, 4, true)
+  if (NV32 < 8 && n <= 8 * unit4) MI355_ROW(8, 4, true)
+  if (n <= 16 * unit4) MI355_ROW(16, 4, true)
+#undef MI355_ROW
   return false;
 }
 

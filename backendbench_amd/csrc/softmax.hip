@@ -1,7 +1,7 @@
 // _softmax over the middle axis of a dense [outer, dim, inner] view, fp32 math.
 //
-//   wave   inner == 1, row fits a wave's registers (<= 16 x 128-bit per lane): one HBM
-//          read, max and sum by wave all-reduce, one HBM write;
+//   tile   inner == 1, row fits the registers of 1, 2 or 4 cooperating waves: one HBM read,
+//          max and sum by wave all-reduce (+ one LDS exchange between waves), one HBM write;
 //   block  inner == 1, longer rows: 256 threads keep an online (max, sum) pair in one
 //          pass, combine through LDS, then re-read the row (L2) to normalise;
 //   cols   inner > 1: one thread per (outer, inner) column, coalesced along inner,
@@ -14,35 +14,38 @@
 
 namespace mi355 {
 
-constexpr int kSmBlock = 256;
+constexpr int kSmBlock = kRowBlock;
 
-template <typename T, typename O, int NV, bool VEC>
-__global__ __launch_bounds__(kSmBlock) void softmax_wave_kernel(const T* __restrict__ x, O* __restrict__ y,
+template <typename T, typename O, int NV, bool VEC, int W>
+__global__ __launch_bounds__(kSmBlock) void softmax_tile_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                int64_t rows, int64_t n) {
-  const int lane = threadIdx.x % kWave;
-  const int64_t row = (int64_t)blockIdx.x * (kSmBlock / kWave) + threadIdx.x / kWave;
-  if (row >= rows) return;
-  RowTile<T, NV, VEC> t;
-  constexpr int V = RowTile<T, NV, VEC>::V;
-  t.load(x + row * n, n, lane, -INFINITY);
+  using Tile = RowTile<T, NV, VEC, W>;
+  constexpr int V = Tile::V;
+  __shared__ float red_max[kSmBlock / kWave], red_sum[kSmBlock / kWave];
+  const int t = threadIdx.x % Tile::GROUP;
+  int64_t row = (int64_t)blockIdx.x * Tile::ROWS_PER_BLOCK + threadIdx.x / Tile::GROUP;
+  const bool active = row < rows;  // inactive groups still walk through the barriers
+  if (!active) row = rows - 1;
+  Tile tile;
+  tile.load(x + row * n, n, t, -INFINITY);
   float m = -INFINITY;
 #pragma unroll
   for (int k = 0; k < NV; ++k)
 #pragma unroll
-    for (int j = 0; j < V; ++j) m = t.v[k][j] > m ? t.v[k][j] : m;
-  m = wave_allreduce(m, MaxOp());
+    for (int j = 0; j < V; ++j) m = tile.v[k][j] > m ? tile.v[k][j] : m;
+  m = group_allreduce<W>(m, MaxOp(), red_max);
   float s = 0.f;
 #pragma unroll
   for (int k = 0; k < NV; ++k)
 #pragma unroll
     for (int j = 0; j < V; ++j) {
-      t.v[k][j] = __expf(t.v[k][j] - m);
-      s += t.v[k][j];
+      tile.v[k][j] = __expf(tile.v[k][j] - m);
+      s += tile.v[k][j];
     }
   // Padding lanes hold exp(-inf - m) = 0 unless m is -inf/NaN, where the row is NaN anyway.
-  s = wave_allreduce(s, SumOp());
+  s = group_allreduce<W>(s, SumOp(), red_sum);
   const float inv = 1.f / s;
-  t.store(y + row * n, n, lane, [inv](float e, int64_t) { return e * inv; });
+  if (active) tile.store(y + row * n, n, t, [inv](float e, int64_t) { return e * inv; });
 }
 
 // Online (max, sum) pair; see the file header for the special-value rules.
@@ -140,13 +143,14 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
     return check_launch("mi355_softmax(cols)");
   }
   const bool vec = n % V == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(y) % (sizeof(O) * V)) == 0;
-  const int64_t nblk = (outer + kSmBlock / kWave - 1) / (kSmBlock / kWave);
   bool done = false;
-  if (nblk < (int64_t(1) << 31)) {
-    done = dispatch_row_tile<T>(n, [&](auto nv) {
-      constexpr int NV = decltype(nv)::value;
-      if (vec) hipLaunchKernelGGL((softmax_wave_kernel<T, O, NV, true>), dim3((unsigned)nblk), dim3(kSmBlock), 0, st, x, y, outer, n);
-      else hipLaunchKernelGGL((softmax_wave_kernel<T, O, NV, false>), dim3((unsigned)nblk), dim3(kSmBlock), 0, st, x, y, outer, n);
+  if (outer < (int64_t(1) << 31)) {
+    done = dispatch_row_tile<T>(n, vec, [&](auto nv, auto w, auto v) {
+      constexpr int NV = decltype(nv)::value, W = decltype(w)::value;
+      constexpr bool VEC = decltype(v)::value;
+      constexpr int rpb = kSmBlock / (kWave * W);
+      const unsigned nblk = (unsigned)((outer + rpb - 1) / rpb);
+      hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, VEC, W>), dim3(nblk), dim3(kSmBlock), 0, st, x, y, outer, n);
     });
   }
   if (!done) {
