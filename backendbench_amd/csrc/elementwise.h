@@ -1,8 +1,8 @@
 // Elementwise launch framework: one functor type F describes an op
 //   F::out_t, F::in0_t, F::in1_t, F::in2_t, F::NIN, out_t operator()(in0_t, in1_t, in2_t)
 // and three kernel shapes cover every layout:
-//   flat      all operands share one dense (possibly permuted) layout: 1-D pass, 128-bit
-//             accesses, grid-stride loop sized to the chip;
+//   flat      all operands share one dense (possibly permuted) layout: 1-D pass, one
+//             contiguous 16 KB tile per operand per block, non-temporal 128-bit accesses;
 //   strided   any strides/broadcast, index split with multiply-shift division; vectorised
 //             along the innermost dim when every operand is unit-stride or broadcast there;
 //   strided64 the same with 64-bit index math for > 2^31 work items.

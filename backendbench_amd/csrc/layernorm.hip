@@ -13,20 +13,41 @@ namespace mi355 {
 
 constexpr int kLnBlock = kRowBlock;
 
-template <typename T, typename Wt, typename S, int NV, bool VEC, int W>
-__global__ __launch_bounds__(kLnBlock) void layernorm_tile_kernel(const T* __restrict__ x, const Wt* __restrict__ w,
-                                                                 const Wt* __restrict__ b, T* __restrict__ y,
-                                                                 S* __restrict__ mean_out, S* __restrict__ rstd_out,
-                                                                 int64_t rows, int64_t n, float eps) {
-  using Tile = RowTile<T, NV, VEC, W>;
+// BLOCK = 1024 (many rows): gamma and beta are staged once per block in LDS (dynamic,
+// 2 * n * sizeof(Wt) bytes) and serve the 1024 / (64 W) rows of the block.  Fetching them from
+// L2 for every row makes every wave of the launch hammer the same 16 KB — the few L2 channels
+// that hold them — and cost ~15 % of the kernel's time.  BLOCK = 256 (few rows) reads them
+// straight from L2 and keeps more blocks in flight.
+template <typename T, typename Wt, typename S, int NV, bool VEC, int W, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restrict__ x, const Wt* __restrict__ w,
+                                                              const Wt* __restrict__ b, T* __restrict__ y,
+                                                              S* __restrict__ mean_out, S* __restrict__ rstd_out,
+                                                              int64_t rows, int64_t n, float eps) {
+  using Tile = RowTile<T, NV, VEC, W, BLOCK>;
   constexpr int V = Tile::V;
-  __shared__ float red_a[kLnBlock / kWave], red_b[kLnBlock / kWave];
+  constexpr bool STAGE = VEC && BLOCK > kLnBlock;
+  extern __shared__ __attribute__((aligned(32))) unsigned char ln_smem[];
+  __shared__ float red_a[BLOCK / kWave], red_b[BLOCK / kWave];
+  const Wt* gs = w;
+  const Wt* bs = b;
   const int t = threadIdx.x % Tile::GROUP;
   int64_t row = (int64_t)blockIdx.x * Tile::ROWS_PER_BLOCK + threadIdx.x / Tile::GROUP;
   const bool active = row < rows;  // inactive groups still walk through the barriers
   if (!active) row = rows - 1;
   Tile tile;
   tile.load(x + row * n, n, t, 0.f);
+  if constexpr (STAGE) {
+    Wt* gl = reinterpret_cast<Wt*>(ln_smem);
+    Wt* bl = gl + n;
+    constexpr int WV = 16 / sizeof(Wt);
+    for (int64_t c = (int64_t)threadIdx.x * WV; c < n; c += (int64_t)BLOCK * WV) {
+      if (w) st<Wt, WV>(gl + c, ld<Wt, WV>(w + c));
+      if (b) st<Wt, WV>(bl + c, ld<Wt, WV>(b + c));
+    }
+    gs = gl;
+    bs = bl;  // visible after the barrier inside the first group_allreduce (W > 1) or the one below
+    if constexpr (W == 1) __syncthreads();
+  }
   float s = 0.f;
 #pragma unroll
   for (int k = 0; k < NV; ++k)
@@ -51,14 +72,13 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_tile_kernel(const T* __res
   }
   T* out = y + row * n;
   if constexpr (VEC) {
-    // gamma/beta come through L2 as whole vectors, one per slab, shared by every row.
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int64_t c = Tile::col(k, 0, t);
       if (c < n) {
         VecN<Wt, V> g, be;
-        if (w) g = ld<Wt, V>(w + c);
-        if (b) be = ld<Wt, V>(b + c);
+        if (w) g = ld<Wt, V>(gs + c);
+        if (b) be = ld<Wt, V>(bs + c);
         VecN<T, V> r;
 #pragma unroll
         for (int j = 0; j < V; ++j) {
@@ -155,16 +175,25 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
   S* mean = static_cast<S*>(mv);
   S* rstd = static_cast<S*>(rv);
   constexpr int V = Vec<T>::N;
+  const bool has_params = w != nullptr || b != nullptr;
   const bool vec = N % V == 0 && aligned16(x) && aligned16(y) &&
                    reinterpret_cast<uintptr_t>(w) % (sizeof(W) * V) == 0 &&
-                   reinterpret_cast<uintptr_t>(b) % (sizeof(W) * V) == 0;
+                   reinterpret_cast<uintptr_t>(b) % (sizeof(W) * V) == 0 && N % (16 / sizeof(W)) == 0;
   MI355_REQUIRE(M < (int64_t(1) << 31), "mi355_layer_norm: too many rows (%lld)", (long long)M);
+  const size_t param_bytes = 2 * (size_t)N * sizeof(W);
   const bool done = dispatch_row_tile<T>(N, vec, [&](auto nv, auto wv, auto v) {
     constexpr int NV = decltype(nv)::value, WG = decltype(wv)::value;
     constexpr bool VEC = decltype(v)::value;
-    constexpr int rpb = kLnBlock / (kWave * WG);
-    const unsigned nblk = (unsigned)((M + rpb - 1) / rpb);
-    hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, VEC, WG>), dim3(nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+    constexpr int BIG = 1024;
+    constexpr int rpb_big = BIG / (kWave * WG), rpb = kLnBlock / (kWave * WG);
+    // Enough rows to fill the chip with 1024-thread blocks: share gamma/beta through LDS.
+    if (VEC && has_params && param_bytes <= 48 * 1024 && M >= (int64_t)rpb_big * 2 * kNumCU) {
+      const unsigned nblk = (unsigned)((M + rpb_big - 1) / rpb_big);
+      hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, VEC, WG, BIG>), dim3(nblk), dim3(BIG), param_bytes, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+    } else {
+      const unsigned nblk = (unsigned)((M + rpb - 1) / rpb);
+      hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, VEC, WG, kLnBlock>), dim3(nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+    }
   });
   if (!done) {
     if (vec) hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, true>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, (float)eps);

@@ -16,10 +16,10 @@ namespace mi355 {
 
 constexpr int kRowBlock = 256;  // threads per block of every row-tile kernel
 
-template <typename T, int NV, bool VEC, int W> struct RowTile {
+template <typename T, int NV, bool VEC, int W, int BLOCK = kRowBlock> struct RowTile {
   static constexpr int V = 16 / sizeof(T);
   static constexpr int GROUP = kWave * W;        // lanes cooperating on one row
-  static constexpr int ROWS_PER_BLOCK = kRowBlock / GROUP;
+  static constexpr int ROWS_PER_BLOCK = BLOCK / GROUP;
   float v[NV][V];
 
   // Column of element (k, j) for lane `t` (0 .. GROUP-1) of the row group.

@@ -11,11 +11,13 @@ resident in HBM before the clock starts; consecutive steps walk a pool of input 
 than the last-level cache, so every step reads from HBM.  `value` is the algorithmic bytes of
 a step divided by the time of a step.
 
-Beside the step loop the script times every headline row of all five configurations the way
-the reference times GPU code (flush the cache, one event pair per repetition, mean), reports
-GB/s or TFLOP/s and the fraction of the MI355X peak per op under "per_op", times ATen on the
-host CPU for the same calls ("cpu_baseline", bounded samples) and reports the geometric mean
-speed-up over it.
+Beside the step loop the script times every headline row of all five configurations: `ms` is
+the mean time per launch of a HIP graph that holds one launch per member of a pool of input
+copies (cold inputs, one event pair around the replays; agrees with rocprofv3's per-kernel
+average), `ms_flush_events` is the reference's own GPU recipe (flush the cache, one event pair
+per repetition, mean).  It reports GB/s or TFLOP/s and the fraction of the MI355X peak per op
+under "per_op", times ATen on the host CPU for the same calls ("cpu_baseline", bounded samples)
+and reports the geometric mean speed-up over it.
 """
 
 import argparse
@@ -30,6 +32,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, TFLOP/s
+# HBM bytes per launch from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
+# same counter reads for a plain 128 MiB copy); measured once per kernel with rocprofv3 --pmc,
+# summary in profiles/layernorm_tile_kernel__C2_layer_norm.md.  Not re-measured by this script.
+MEASURED_TRAFFIC_BYTES = {"C2.layer_norm": 134_490_000}
 
 
 def parse():
@@ -42,8 +48,7 @@ def parse():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink factor for every shape (debug only)")
     ap.add_argument("--ops", default="all", help="comma-separated substrings of per-op rows to time, or 'none'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only-op", default=None, help="time just this per-op row in a loop (for profilers)")
-    ap.add_argument("--reps", type=int, default=50, help="repetitions for --only-op")
+    ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy")
     return ap.parse_args()
 
 
@@ -74,18 +79,21 @@ def main():
         return backend[case.op]
 
     # ------------------------------------------------------------ profiler mode
+    # One op only, timed exactly like its per_op row, so that a profiler's per-kernel average
+    # covers the same launches.  "calib.copy" is a plain 128 MiB -> 128 MiB copy with the
+    # library's copy kernel (known traffic, for scaling hardware byte counters).
     if args.only_op:
-        case = by_key[args.only_op]
-        a, kw = case.make(dev)
-        f = impl_of(case)
-        for _ in range(3):
-            f(*a, **kw)
-        torch.cuda.synchronize()
-        for _ in range(args.reps):
-            ev._flush_cache(dev)
-            f(*a, **kw)
-        torch.cuda.synchronize()
-        print(json.dumps({"only_op": args.only_op, "reps": args.reps}))
+        if args.only_op == "calib.copy":
+            from backendbench_amd.ops._common import copy_into
+
+            src = torch.empty(32 * 2**20, dtype=torch.float32, device=dev).normal_()
+            f, a, kw, work = (lambda s: copy_into(torch.empty_like(s), s)), [src], {}, 2 * src.numel() * 4
+        else:
+            case = by_key[args.only_op]
+            a, kw = case.make(dev)
+            f, work = impl_of(case), case.work
+        ms, how = graph_bench(f, a, kw)
+        print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "work": work, "timing": how}))
         return
 
     # ------------------------------------------------------------ headline step loop (C2)
@@ -175,7 +183,8 @@ def main():
     if timed:
         dom = max(timed, key=lambda r: r["ms"])
         roofline = {"bound": "hbm", "kernel": dom["op"], "achieved": dom["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(dom["gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
+                    "frac": round(dom["gbs"] / HBM_PEAK_GBS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(dom["op"]) if args.scale == 1.0 else None,
                     "bytes_per_launch": dom["bytes"], "avg_launch_ms": dom["ms"],
                     "timing": dom["timing"]}
     cpu_baseline = None
