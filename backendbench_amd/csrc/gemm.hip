@@ -4,11 +4,14 @@
 //            N-contiguous ("NN", row-major), 16-byte aligned rows.  256x256x32 block tile,
 //            eight wave64 (2x4, two per SIMD), each wave 128x64 = 4x2 v_mfma_f32_32x32x16
 //            tiles with 128 fp32 accumulators; a four-stage 128 KB LDS ring, swizzled so
-//            that the 128-bit global->LDS writes and the fragment reads are bank-conflict
-//            free.  A row-major B stays N-contiguous in LDS and is transposed by the LDS
-//            read itself (ds_read_b64_tr_b16).  Tile it+3 is in flight from L2/HBM while
-//            tile `it` is multiplied; block -> tile map groups tiles per XCD so that one
-//            L2 serves neighbouring tiles.
+//            that the fills and the fragment reads are bank-conflict free.  A row-major B
+//            stays N-contiguous in LDS and is transposed by the LDS read itself
+//            (ds_read_b64_tr_b16).  Block -> tile map groups tiles per XCD so that one L2
+//            serves neighbouring tiles.  Two fill paths:
+//              gemm_mfma_dma_kernel  K % 32 == 0: panels go global -> LDS directly
+//                                    (global_load_lds_dwordx4), three tiles ahead; MFMAs and
+//                                    LDS reads of a wave are interleaved one to one;
+//              gemm_mfma_kernel      K tail: global -> registers -> LDS with zero fill.
 //   generic  any strides, bf16 / f16 / f32: 64x64 LDS tile, FMA inner loop.  Correctness
 //            path for shapes the MFMA kernel does not take.
 #include "common.h"
@@ -63,6 +66,7 @@ struct GemmArgs {
   int32_t M, N, K;
   float alpha, beta;
   int32_t tiles_m, tiles_n;
+  int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
 };
 
 // Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous
@@ -95,6 +99,69 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
       (__attribute__((address_space(3))) s16x4*)(uintptr_t)(const_cast<unsigned char*>(p)));
+}
+
+// ---------------------------------------------------------------- epilogue
+// A wave's 128x64 result: register r of acc[i][j] in lane l is C[m0 + 32 i + l%32][n0 + 32 j +
+// 8 (r/4) + 4 (l/32) + r%4] (operands were swapped, so a lane owns runs of 4 consecutive n).
+// Writing those 8-byte runs straight to global memory leaves every 128-byte line to be
+// assembled from 16 stores in L2, and the epilogue then costs more than a tenth of the whole
+// GEMM.  Instead the wave applies alpha / beta * c in fp32, parks the rounded tile in its own
+// 16 KB slice of the (now idle) LDS ring, and reads it back row-major: every global store
+// instruction then writes 8 complete 128-byte rows.  Must be called by all waves after the
+// last barrier of the main loop (the ring is no longer read).
+template <typename T>
+__device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x16 (&acc)[4][2], unsigned char* lds,
+                                                  int wave, int lane, int m0, int n0) {
+  const int fr = lane & 31, fg = lane >> 5;
+  const T* C = static_cast<const T*>(g.c);
+  const bool use_c = C != nullptr && g.beta != 0.f;
+  unsigned char* slab = lds + wave * (128 * 128);  // 128 rows x 128 bytes
+  // 16-byte slot s of row r lives at slot s ^ ((r/2) % 8): two-way conflicts at most on both sides
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = i * 32 + fr;
+    const int m = m0 + row;
+    const int mc = m < g.M ? m : g.M - 1;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int nl = j * 32 + q * 8 + fg * 4;
+        int n = n0 + nl;
+        n = n + 4 <= g.N ? n : 0;  // out-of-range columns are computed on valid addresses and never stored
+        float cv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (use_c) {
+          if (g.c_vec) {
+            const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (int64_t)mc * g.c_rs + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(t.v[e]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(C[(int64_t)mc * g.c_rs + (int64_t)(n + e) * g.c_cs]);
+          }
+        }
+        VecN4<T> r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float v = g.alpha * acc[i][j][q * 4 + e];
+          r.v[e] = static_cast<T>(use_c ? v + g.beta * cv[e] : v);
+        }
+        const int slot = (j * 4 + q) ^ ((row >> 1) & 7);
+        *reinterpret_cast<VecN4<T>*>(slab + row * 128 + slot * 16 + fg * 8) = r;
+      }
+    }
+  }
+  // same wave wrote and reads: LDS operations of a wave complete in order
+  T* D = static_cast<T*>(g.out);
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    const int chunk = t * kWave + lane;  // 1024 chunks of 16 bytes, 8 per row
+    const int row = chunk >> 3, s = chunk & 7;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(slab + row * 128 + ((s ^ ((row >> 1) & 7)) << 4));
+    const int m = m0 + row, n = n0 + s * 8;
+    if (m < g.M && n < g.N) *reinterpret_cast<u32x4*>(D + (int64_t)m * g.N + n) = v;  // N % 8 == 0 on this path
+  }
 }
 
 // ---------------------------------------------------------------- MFMA kernel
@@ -231,30 +298,166 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
     __syncthreads();
   }
 
-  T* D = static_cast<T*>(g.out);
-  const T* C = static_cast<const T*>(g.c);
-  const bool use_c = C != nullptr && g.beta != 0.f;
+  store_tile_result<T>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
+}
+
+// ---------------------------------------------------------------- MFMA kernel, direct-to-LDS fills
+// Same tiling, ring and fragment reads as gemm_mfma_kernel, but the panels are filled with
+// global_load_lds_dwordx4: each wave-level load moves 64 x 16 bytes from global memory straight
+// into 1 KB of LDS (lane l lands at M0 + 16 l), without passing through VGPRs and without
+// ds_write instructions.  Because the LDS position of a lane is fixed, the swizzle is applied
+// on the global side: a lane fetches the chunk that belongs at its LDS position.
+// Tile it+3 is requested at the start of iteration `it` into the slot tile it-1 just left, and
+// must have landed by the end of iteration it+1 (s_waitcnt vmcnt(4): only the four loads of
+// the newest tile may still be in flight), so every tile has two iterations to arrive.  The
+// loads are issued from inline asm, so the compiler's own wait-count bookkeeping does not see
+// them and adds no waits of its own.  Needs K % 32 == 0 (no zero fill on this path).
+__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_offset, const void* gptr) {
+  asm volatile("s_mov_b32 m0, %0\n\t"
+               "s_nop 0\n\t"
+               "global_load_lds_dwordx4 %1, off" ::"s"(lds_byte_offset), "v"(gptr)
+               : "memory");
+}
+
+template <typename T, bool B_NN>
+__global__ __launch_bounds__(512) void gemm_mfma_dma_kernel(GemmArgs g) {
+  constexpr int S = kStages3;   // ring depth
+  constexpr bool PF = true;     // fragments of the next tile are read before the barrier
+  constexpr bool SCHED = true;  // pin the MFMA / DS-read interleave
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  using frag_t = typename Mfma<T>::frag;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 2, wn = wave & 3;
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  const int bm = tm * BM, bn = tn * BN;
+  const T* A = static_cast<const T*>(g.a);
+  const T* B = static_cast<const T*>(g.b);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;  // LDS-relative address of the ring
+
+  // Per-lane source pointers of this wave's four 1 KB regions per tile (two per panel): region
+  // q = wave + 8 i of a panel is LDS bytes [q*1024, q*1024 + 1024).
+  const T* a_src[2];
+  const T* b_src[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = bm + wm * 128 + i * 32 + fr;
-    if (m >= g.M) continue;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = bn + wn * 64 + j * 32 + q * 8 + fg * 4;
-        if (n >= g.N) continue;
-        VecN4<T> r;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          float v = g.alpha * acc[i][j][q * 4 + e];
-          if (use_c) v += g.beta * static_cast<float>(C[(int64_t)m * g.c_rs + (int64_t)(n + e) * g.c_cs]);
-          r.v[e] = static_cast<T>(v);
-        }
-        *reinterpret_cast<VecN4<T>*>(D + (int64_t)m * g.N + n) = r;
-      }
+  for (int i = 0; i < 2; ++i) {
+    const int q = wave + 8 * i;
+    {  // K-contiguous A panel: region q = rows 16q .. 16q+15, 4 chunks per row
+      const int r = 16 * q + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gr = bm + r;
+      gr = gr < g.M ? gr : g.M - 1;
+      a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+    }
+    if constexpr (!B_NN) {
+      const int r = 16 * q + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gn = bn + r;
+      gn = gn < g.N ? gn : g.N - 1;
+      b_src[i] = B + (int64_t)gn * g.ldb + c * 8;
+    } else {  // N-contiguous B panel: region q = k rows 2q, 2q+1, 32 units per row
+      const int k = 2 * q + (lane >> 5), pos = lane & 31;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gn = bn + u * 8;
+      gn = gn < g.N ? gn : 0;
+      b_src[i] = B + (int64_t)k * g.ldb + gn;
     }
   }
+  auto request_tile = [&](int t) {
+    const uint32_t stage = lds_base + (uint32_t)(t % S) * kStage3;
+    const int64_t k0 = (int64_t)t * BK3;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t region = (uint32_t)(wave + 8 * i) * 1024u;
+      lds_dma16(stage + region, a_src[i] + k0);
+      if constexpr (!B_NN) lds_dma16(stage + kPanel3 + region, b_src[i] + k0);
+      else lds_dma16(stage + kPanel3 + region, b_src[i] + k0 * g.ldb);
+    }
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  const int tr_k = fg * 8 + ((lane & 15) >> 2);
+  const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  auto read_frags = [&](int t, int ks, frag_t (&fa)[4], frag_t (&fb)[2]) {
+    const unsigned char* pa = lds + (t % S) * kStage3;
+    const unsigned char* pb = pa + kPanel3;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k32(wm * 128 + i * 32 + fr, ks * 2 + fg));
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if constexpr (!B_NN) {
+        fb[j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * 64 + j * 32 + fr, ks * 2 + fg));
+      } else {
+        const int k = ks * 16 + tr_k;
+        const int n = wn * 64 + j * 32 + tr_n;
+        const s16x4 lo = lds_read_tr(pb + swz_n(k, n >> 3) + ((n & 7) << 1));
+        const s16x4 hi = lds_read_tr(pb + swz_n(k + 4, n >> 3) + ((n & 7) << 1));
+        fb[j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    }
+  };
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto mma = [&](frag_t (&fa)[4], frag_t (&fb)[2]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+  };
+
+  // Ring of S stages; PF = fragments of the next tile are read before the barrier.  At the wait
+  // point of iteration `it`, tile it+1+PF must have landed; the S-2-PF newer tiles may fly on.
+  constexpr int FLY = S - 2 - (PF ? 1 : 0);
+  const int nk = g.K / BK3;
+  for (int t = 0; t < S - 1 && t < nk; ++t) request_tile(t);
+  if (nk >= S - 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * FLY) : "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  frag_t fa0[4], fb0[2], fa1[4], fb1[2];
+  read_frags(0, 0, fa0, fb0);
+  int it = 0;
+  // Steady state: no conditions inside, so the body is one scheduling region.  The MFMAs of a
+  // 16-k step are interleaved with the LDS reads of the following step (SCHED: one MFMA, then
+  // one or two DS reads), so the matrix pipe and the LDS pipe of a wave work at the same time.
+  for (; it + S - 1 < nk; ++it) {
+    request_tile(it + S - 1);
+    read_frags(it, 1, fa1, fb1);
+    mma(fa0, fb0);
+    if constexpr (PF) read_frags(it + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    if constexpr (SCHED) {
+#define MI355_MFMA_THEN_READS                              \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       \
+  __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);       \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       \
+  __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS
+      MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS
+#undef MI355_MFMA_THEN_READS
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * FLY) : "memory");
+    __syncthreads();
+    if constexpr (!PF) read_frags(it + 1, 0, fa0, fb0);
+  }
+  for (; it < nk; ++it) {  // drain: nothing left to request
+    read_frags(it, 1, fa1, fb1);
+    mma(fa0, fb0);
+    if (PF && it + 1 < nk) read_frags(it + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (!PF && it + 1 < nk) read_frags(it + 1, 0, fa0, fb0);
+  }
+
+  store_tile_result<T>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
 }
 
 // ---------------------------------------------------------------- generic fallback
@@ -320,12 +523,13 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     // Tiny problems are cheaper on the generic kernel than on a mostly empty 256x256 tile.
     const bool worth = M * N >= 128 * 128 && K >= 32;
     if (a_ok && (b_nt || b_nn) && K % 8 == 0 && N % 8 == 0 && fits && worth && K > 0 &&
-        reinterpret_cast<uintptr_t>(out) % 8 == 0) {
+        aligned16(out)) {
       GemmArgs g{};
       g.a = a; g.b = b; g.c = c; g.out = out;
       g.lda = a_rs;
       g.ldb = b_nt ? b_cs : b_rs;
       g.c_rs = c_rs; g.c_cs = c_cs;
+      g.c_vec = c != nullptr && c_cs == 1 && c_rs % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 8 == 0;
       g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
       g.alpha = (float)alpha; g.beta = (float)beta;
       g.tiles_m = (int32_t)((M + BM - 1) / BM);
@@ -333,10 +537,9 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const int64_t nblocks = (int64_t)g.tiles_m * g.tiles_n;
       MI355_REQUIRE(nblocks < (int64_t(1) << 31), "mi355_gemm: too many tiles");
       const bool ktail = K % BK3 != 0;
-      const void* kern =
-          b_nt ? (ktail ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, false, false>)
-               : (ktail ? (const void*)gemm_mfma_kernel<T, true, true> : (const void*)gemm_mfma_kernel<T, true, false>);
-      const int nthreads = 512;
+      const void* kern;
+      if (ktail) kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
+      else kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
       // 128 KB of dynamic LDS needs the attribute once per kernel and process.
       static thread_local const void* attr_done[8] = {};
       bool seen = false;
@@ -349,7 +552,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
           if (k == nullptr) { k = kern; break; }
       }
       void* params[] = {&g};
-      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks), dim3(nthreads), params, kGemmLds, st);
+      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks), dim3(512), params, kGemmLds, st);
       if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma): launch failed: %s", hipGetErrorString(e));
       return check_launch("mi355_gemm(mfma)");
     }
