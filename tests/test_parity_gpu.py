@@ -235,3 +235,38 @@ def test_live_dispatcher_override_runs_our_kernels(backend):
         assert ev.allclose(a.cpu(), b.cpu())
     again = block()  # override gone
     assert ev.allclose(plain[0].cpu(), again[0].cpu())
+
+
+def test_hip_graph_replays_match_eager(backend):
+    """The kernels are launched on torch's current stream, so a HIP graph captures them.  Every
+    replay (with eager work and synchronisations in between) must reproduce the eager result."""
+    announce("hip graph capture/replay")
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(512, 4096, generator=g) * 2).bfloat16().cuda()
+    w = (torch.randn(4096, 512, generator=g) * 0.02).bfloat16().cuda()
+    gamma, beta = torch.ones(4096).bfloat16().cuda(), torch.zeros(4096).bfloat16().cuda()
+    idx = torch.randint(0, 512, (300,), generator=g).cuda()
+
+    def work(inp):
+        y, mean, rstd = backend[aten.native_layer_norm.default](inp, [4096], gamma, beta, 1e-5)
+        p = backend[aten._softmax.default](y, -1, False)
+        h = backend[aten.mm.default](p, w)
+        s = backend[aten.sum.dim_IntList](h, [-1])
+        e = backend[aten.embedding.default](inp, idx)
+        a = backend[aten.argmax.default](h.float(), -1)
+        return y, p, h, s, e, a, mean
+
+    eager = [t.clone() for t in work(x)]   # also the warm-up: library load, LDS attribute, error flag
+    torch.cuda.synchronize()
+    static_in = x.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = work(static_in)
+    for rep in range(4):
+        static_in.copy_(x if rep % 2 == 0 else x.flip(0))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = eager if rep % 2 == 0 else [t.clone() for t in work(x.flip(0))]
+        torch.cuda.synchronize()
+        for o, e_ in zip(outs, want):
+            assert ev.allclose(e_.cpu(), o.cpu(), exact=not o.dtype.is_floating_point), f"replay {rep} differs"
