@@ -30,7 +30,7 @@ DTYPE = {
     torch.bool: BOOL,
 }
 # mi355_binary_op / mi355_unary_op / mi355_reduce_op
-ADD, MUL, MAXIMUM = 0, 1, 2
+ADD, MUL, MAXIMUM, MINIMUM = 0, 1, 2, 3
 RELU, CLAMP = 0, 1
 SUM, MEAN, AMAX, ARGMAX = 0, 1, 2, 3
 
@@ -62,7 +62,7 @@ SIGNATURES = {
         c_int,
         [c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_void_p],
     ),
-    "mi355_softmax": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p]),
+    "mi355_softmax": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "mi355_layer_norm": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,

@@ -37,6 +37,20 @@ template <typename T> struct MaximumF {
   }
 };
 
+template <typename T> struct MinimumF {
+  using out_t = T; using in0_t = T; using in1_t = T; using in2_t = Unused;
+  static constexpr int NIN = 2;
+  using M = typename OpMath<T>::type;
+  __device__ __forceinline__ T operator()(T a, T b, Unused) const {
+    const M x = static_cast<M>(a), y = static_cast<M>(b);
+    if constexpr (IsFloat<T>::value) {
+      if (x != x) return a;
+      if (y != y) return b;
+    }
+    return x < y ? a : b;
+  }
+};
+
 // ---- unary -----------------------------------------------------------------------
 template <typename T> struct ReluF {
   using out_t = T; using in0_t = T; using in1_t = Unused; using in2_t = Unused;
@@ -140,6 +154,7 @@ extern "C" int mi355_binary(int op, const mi355_tensor* a, const mi355_tensor* b
       }
       case MI355_MUL: return launch_elementwise(MulF<T>{}, ins, out, st, "mi355_binary(mul)");
       case MI355_MAXIMUM: return launch_elementwise(MaximumF<T>{}, ins, out, st, "mi355_binary(maximum)");
+      case MI355_MINIMUM: return launch_elementwise(MinimumF<T>{}, ins, out, st, "mi355_binary(minimum)");
       default: return set_error(MI355_ERR_INVALID, "mi355_binary: unknown op %d", op);
     }
   });

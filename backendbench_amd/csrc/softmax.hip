@@ -1,4 +1,4 @@
-// _softmax over the middle axis of a dense [outer, dim, inner] view, fp32 math.
+// _softmax / _log_softmax over the middle axis of a dense [outer, dim, inner] view, fp32 math.
 //
 //   tile   inner == 1, row fits the registers of 1, 2 or 4 cooperating waves: one HBM read,
 //          max and sum by wave all-reduce (+ one LDS exchange between waves), one HBM write;
@@ -16,7 +16,7 @@ namespace mi355 {
 
 constexpr int kSmBlock = kRowBlock;
 
-template <typename T, typename O, int NV, bool VEC, int W>
+template <typename T, typename O, int NV, bool VEC, int W, bool LOG>
 __global__ __launch_bounds__(kSmBlock) void softmax_tile_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                int64_t rows, int64_t n) {
   using Tile = RowTile<T, NV, VEC, W>;
@@ -39,13 +39,20 @@ __global__ __launch_bounds__(kSmBlock) void softmax_tile_kernel(const T* __restr
   for (int k = 0; k < NV; ++k)
 #pragma unroll
     for (int j = 0; j < V; ++j) {
-      tile.v[k][j] = __expf(tile.v[k][j] - m);
-      s += tile.v[k][j];
+      const float d = tile.v[k][j] - m;
+      const float e = __expf(d);
+      tile.v[k][j] = LOG ? d : e;  // log-softmax keeps x - max and subtracts log(sum) at the end
+      s += e;
     }
   // Padding lanes hold exp(-inf - m) = 0 unless m is -inf/NaN, where the row is NaN anyway.
   s = group_allreduce<W>(s, SumOp(), red_sum);
-  const float inv = 1.f / s;
-  if (active) tile.store(y + row * n, n, t, [inv](float e, int64_t) { return e * inv; });
+  if constexpr (LOG) {
+    const float ls = __logf(s);
+    if (active) tile.store(y + row * n, n, t, [ls](float d, int64_t) { return d - ls; });
+  } else {
+    const float inv = 1.f / s;
+    if (active) tile.store(y + row * n, n, t, [inv](float e, int64_t) { return e * inv; });
+  }
 }
 
 // Online (max, sum) pair; see the file header for the special-value rules.
@@ -77,7 +84,7 @@ __device__ __forceinline__ MS ms_wave_reduce(MS a) {
   return a;
 }
 
-template <typename T, typename O, bool VEC>
+template <typename T, typename O, bool VEC, bool LOG>
 __global__ __launch_bounds__(kSmBlock) void softmax_block_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                 int64_t n) {
   constexpr int V = Vec<T>::N;
@@ -100,22 +107,23 @@ __global__ __launch_bounds__(kSmBlock) void softmax_block_kernel(const T* __rest
   a = smem[0];
 #pragma unroll
   for (int w = 1; w < kSmBlock / kWave; ++w) a = ms_combine(a, smem[w]);
-  const float m = a.m, inv = 1.f / a.s;
+  const float m = a.m, inv = 1.f / a.s, ls = __logf(a.s);
+  auto fin = [=](float v) { return LOG ? (v - m) - ls : __expf(v - m) * inv; };
   if constexpr (VEC) {
     for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kSmBlock * V) {
       const Vec<T> t = load_vec(row + c);
       VecN<O, V> r;
 #pragma unroll
-      for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(__expf(static_cast<float>(t.v[j]) - m) * inv);
+      for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(fin(static_cast<float>(t.v[j])));
       st<O, V>(out + c, r);
     }
   } else {
     for (int64_t c = threadIdx.x; c < n; c += kSmBlock)
-      out[c] = static_cast<O>(__expf(static_cast<float>(row[c]) - m) * inv);
+      out[c] = static_cast<O>(fin(static_cast<float>(row[c])));
   }
 }
 
-template <typename T, typename O>
+template <typename T, typename O, bool LOG>
 __global__ __launch_bounds__(kSmBlock) void softmax_cols_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                int64_t outer, int64_t n, int64_t inner) {
   const int64_t total = outer * inner;
@@ -126,20 +134,22 @@ __global__ __launch_bounds__(kSmBlock) void softmax_cols_kernel(const T* __restr
     O* q = y + o * n * inner + c;
     MS a{-INFINITY, 0.f};
     for (int64_t r = 0; r < n; ++r) ms_update(a, static_cast<float>(p[r * inner]));
-    const float inv = 1.f / a.s;
-    for (int64_t r = 0; r < n; ++r)
-      q[r * inner] = static_cast<O>(__expf(static_cast<float>(p[r * inner]) - a.m) * inv);
+    const float inv = 1.f / a.s, ls = __logf(a.s);
+    for (int64_t r = 0; r < n; ++r) {
+      const float v = static_cast<float>(p[r * inner]);
+      q[r * inner] = static_cast<O>(LOG ? (v - a.m) - ls : __expf(v - a.m) * inv);
+    }
   }
 }
 
-template <typename T, typename O>
+template <typename T, typename O, bool LOG>
 static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64_t inner, hipStream_t st) {
   const T* x = static_cast<const T*>(xv);
   O* y = static_cast<O*>(yv);
   constexpr int V = Vec<T>::N;
   if (inner > 1) {
     const int grid = grid_for(outer * inner, kSmBlock, kNumCU * 16);
-    hipLaunchKernelGGL((softmax_cols_kernel<T, O>), dim3(grid), dim3(kSmBlock), 0, st, x, y, outer, n, inner);
+    hipLaunchKernelGGL((softmax_cols_kernel<T, O, LOG>), dim3(grid), dim3(kSmBlock), 0, st, x, y, outer, n, inner);
     return check_launch("mi355_softmax(cols)");
   }
   const bool vec = n % V == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(y) % (sizeof(O) * V)) == 0;
@@ -150,13 +160,13 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
       constexpr bool VEC = decltype(v)::value;
       constexpr int rpb = kSmBlock / (kWave * W);
       const unsigned nblk = (unsigned)((outer + rpb - 1) / rpb);
-      hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, VEC, W>), dim3(nblk), dim3(kSmBlock), 0, st, x, y, outer, n);
+      hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, VEC, W, LOG>), dim3(nblk), dim3(kSmBlock), 0, st, x, y, outer, n);
     });
   }
   if (!done) {
     MI355_REQUIRE(outer < (int64_t(1) << 31), "mi355_softmax: too many rows (%lld)", (long long)outer);
-    if (vec) hipLaunchKernelGGL((softmax_block_kernel<T, O, true>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
-    else hipLaunchKernelGGL((softmax_block_kernel<T, O, false>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
+    if (vec) hipLaunchKernelGGL((softmax_block_kernel<T, O, true, LOG>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
+    else hipLaunchKernelGGL((softmax_block_kernel<T, O, false, LOG>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
   }
   return check_launch("mi355_softmax");
 }
@@ -165,23 +175,28 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
 
 using namespace mi355;
 
+template <typename T, typename O>
+static int run_softmax_any(int log_softmax, const void* x, void* y, int64_t outer, int64_t dim, int64_t inner, hipStream_t st) {
+  return log_softmax ? run_softmax<T, O, true>(x, y, outer, dim, inner, st) : run_softmax<T, O, false>(x, y, outer, dim, inner, st);
+}
+
 extern "C" int mi355_softmax(const void* x, int in_dtype, void* y, int out_dtype, int64_t outer, int64_t dim,
-                             int64_t inner, void* stream) {
+                             int64_t inner, int log_softmax, void* stream) {
   MI355_REQUIRE(outer >= 0 && dim >= 0 && inner >= 0, "mi355_softmax: negative extent");
   if (outer == 0 || dim == 0 || inner == 0) return MI355_OK;
   MI355_REQUIRE(x != nullptr && y != nullptr, "mi355_softmax: NULL data pointer");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (out_dtype == in_dtype) {
     switch (in_dtype) {
-      case MI355_F32: return run_softmax<float, float>(x, y, outer, dim, inner, st);
-      case MI355_F16: return run_softmax<f16_t, f16_t>(x, y, outer, dim, inner, st);
-      case MI355_BF16: return run_softmax<bf16_t, bf16_t>(x, y, outer, dim, inner, st);
+      case MI355_F32: return run_softmax_any<float, float>(log_softmax, x, y, outer, dim, inner, st);
+      case MI355_F16: return run_softmax_any<f16_t, f16_t>(log_softmax, x, y, outer, dim, inner, st);
+      case MI355_BF16: return run_softmax_any<bf16_t, bf16_t>(log_softmax, x, y, outer, dim, inner, st);
       default: break;
     }
   } else if (out_dtype == MI355_F32) {  // half_to_float
     switch (in_dtype) {
-      case MI355_F16: return run_softmax<f16_t, float>(x, y, outer, dim, inner, st);
-      case MI355_BF16: return run_softmax<bf16_t, float>(x, y, outer, dim, inner, st);
+      case MI355_F16: return run_softmax_any<f16_t, float>(log_softmax, x, y, outer, dim, inner, st);
+      case MI355_BF16: return run_softmax_any<bf16_t, float>(log_softmax, x, y, outer, dim, inner, st);
       default: break;
     }
   }

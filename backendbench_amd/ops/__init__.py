@@ -1,16 +1,21 @@
 """ATen-semantics wrappers over libmi355_aten.so, one callable per operator slot.
 
 SLOTS maps the directory-backend folder name (BackendBench/utils.py:289-308 naming) to the
-callable that fills `<folder>_kernel_impl`.
+callable that fills `<folder>_kernel_impl`.  CORE_SLOTS are the 19 overloads of the core
+operator set; VARIANT_SLOTS are their in-place / out= / sibling overloads
+(BackendBench/scripts/op_map.py lists them on the same `canonical:` lines), served by the
+same kernels.
 """
 
 from ._common import check_index_errors
-from .elementwise import add, clamp, maximum, mul, relu, where
+from .elementwise import (add, add_, clamp, clamp_, clamp_max, clamp_min, clamp_tensor, maximum, minimum, mul, mul_,
+                          out_variant, relu, relu_, where)
 from .index import embedding, gather, index_select
 from .matmul import addmm, mm
-from .reduce import (amax, argmax, mean_default, mean_dim, native_layer_norm, softmax, sum_default, sum_dim)
+from .reduce import (amax, argmax, log_softmax, mean_default, mean_dim, native_layer_norm, softmax, sum_default,
+                     sum_dim)
 
-SLOTS = {
+CORE_SLOTS = {
     "add__Tensor": add,
     "mul__Tensor": mul,
     "maximum__default": maximum,
@@ -32,4 +37,36 @@ SLOTS = {
     "gather__default": gather,
 }
 
-__all__ = ["SLOTS", "check_index_errors", *sorted(f.__name__ for f in SLOTS.values())]
+VARIANT_SLOTS = {
+    # in-place overloads (folder names keep the trailing underscore: add_.Tensor -> add___Tensor)
+    "add___Tensor": add_,
+    "mul___Tensor": mul_,
+    "relu___default": relu_,
+    "clamp___default": clamp_,
+    # sibling overloads on the same kernels
+    "minimum__default": minimum,
+    "clamp_min__default": clamp_min,
+    "clamp_max__default": clamp_max,
+    "clamp__Tensor": clamp_tensor,
+    "_log_softmax__default": log_softmax,
+    # out= overloads
+    "add__out": out_variant(add),
+    "mul__out": out_variant(mul),
+    "maximum__out": out_variant(maximum),
+    "relu__out": out_variant(relu),
+    "clamp__out": out_variant(clamp),
+    "where__self_out": out_variant(where),
+    "sum__IntList_out": out_variant(sum_dim),
+    "mean__out": out_variant(mean_dim),
+    "amax__out": out_variant(amax),
+    "argmax__out": out_variant(argmax),
+    "_softmax__out": out_variant(softmax),
+    "mm__out": out_variant(mm),
+    "addmm__out": out_variant(addmm),
+    "index_select__out": out_variant(index_select),
+    "gather__out": out_variant(gather),
+}
+
+SLOTS = {**CORE_SLOTS, **VARIANT_SLOTS}
+
+__all__ = ["SLOTS", "CORE_SLOTS", "VARIANT_SLOTS", "check_index_errors"]

@@ -10,7 +10,7 @@ import math
 import torch
 
 from .. import _lib
-from ._common import cast, device_managed, launch
+from ._common import cast, copy_into, device_managed, launch
 
 
 def _out_like_inputs(shape, dtype, inputs):
@@ -31,7 +31,24 @@ def _out_like_inputs(shape, dtype, inputs):
     return torch.empty(shape, dtype=dtype, device=inputs[0].device)
 
 
+def _alpha_args(dtype, alpha):
+    if dtype.is_floating_point:
+        return float(alpha), 0
+    if isinstance(alpha, float) and not float(alpha).is_integer():
+        raise RuntimeError("For integral input tensors, argument alpha must not be a floating point number.")
+    return 0.0, int(alpha)
+
+
+def _as_operand(self, other):
+    """A Python number as second operand (the dispatcher unwraps the 0-d tensor that
+    add.Scalar / `x *= 2` build) becomes a 0-d tensor of the promoted dtype on self's device."""
+    if isinstance(other, torch.Tensor):
+        return other
+    return torch.full((), other, dtype=torch.result_type(self, other), device=self.device)
+
+
 def _binary(op, a, b, alpha=1):
+    b = _as_operand(a, b)
     dtype = torch.result_type(a, b)
     if dtype.is_complex:
         raise NotImplementedError(f"mi355 backend: binary ops on {dtype} are not supported")
@@ -43,15 +60,45 @@ def _binary(op, a, b, alpha=1):
     out = _out_like_inputs(shape, dtype, (a, b))
     if out.numel() == 0:
         return out
-    if dtype.is_floating_point:
-        alpha_f, alpha_i = float(alpha), 0
-    else:
-        if isinstance(alpha, float) and not float(alpha).is_integer():
-            raise RuntimeError("For integral input tensors, argument alpha must not be a floating point number.")
-        alpha_f, alpha_i = 0.0, int(alpha)
+    alpha_f, alpha_i = _alpha_args(dtype, alpha)
     launch("mi355_binary", op, _lib.desc(a.expand(shape)), _lib.desc(b.expand(shape)), alpha_f, alpha_i,
            _lib.desc(out))
     return out
+
+
+def _binary_inplace(op, functional, self, other, **kw):
+    """self (op)= other: the result type must be castable to self's dtype and broadcasting must
+    not change self's shape, as for every ATen in-place overload.  `functional` is the
+    out-of-place wrapper, used when the arithmetic dtype differs from self's or self is on the CPU."""
+    other = _as_operand(self, other)
+    dtype = torch.result_type(self, other)
+    full = torch.broadcast_shapes(self.shape, other.shape)
+    if tuple(full) != tuple(self.shape):
+        raise RuntimeError(f"output with shape {list(self.shape)} doesn't match the broadcast shape {list(full)}")
+    if not torch.can_cast(dtype, self.dtype):
+        raise RuntimeError(f"result type {str(dtype).replace('torch.', '').capitalize()} can't be cast to the "
+                           f"desired output type {str(self.dtype).replace('torch.', '').capitalize()}")
+    if dtype != self.dtype or dtype == torch.bool or not _is_gpu_tensor(self):
+        return copy_into_any(self, functional(self, other, **kw))
+    if self.numel() == 0:
+        return self
+    alpha_f, alpha_i = _alpha_args(dtype, kw.get("alpha", 1))
+    b = cast(other if _is_gpu_tensor(other) else other.to(self.device), dtype)
+    launch("mi355_binary", op, _lib.desc(self), _lib.desc(b.expand(self.shape)), alpha_f, alpha_i, _lib.desc(self))
+    return self
+
+
+def _is_gpu_tensor(t):
+    return t.device.type == "cuda"
+
+
+def copy_into_any(dst, src):
+    """dst[...] = src across devices: our copy kernel on the GPU, torch's transfer otherwise."""
+    if _is_gpu_tensor(dst) and _is_gpu_tensor(src):
+        copy_into(dst, src.expand(dst.shape) if tuple(src.shape) != tuple(dst.shape) else src)
+    else:
+        dst.copy_(src)  # host <-> device transfer (only reached with CPU tensors)
+    return dst
 
 
 @device_managed
@@ -60,10 +107,20 @@ def add(self, other, *, alpha=1):
     return _binary(_lib.ADD, self, other, alpha)
 
 
+def add_(self, other, *, alpha=1):
+    """aten.add_.Tensor"""
+    return _binary_inplace(_lib.ADD, add, self, other, alpha=alpha)
+
+
 @device_managed
 def mul(self, other):
     """aten.mul.Tensor"""
     return _binary(_lib.MUL, self, other)
+
+
+def mul_(self, other):
+    """aten.mul_.Tensor"""
+    return _binary_inplace(_lib.MUL, mul, self, other)
 
 
 @device_managed
@@ -72,9 +129,15 @@ def maximum(self, other):
     return _binary(_lib.MAXIMUM, self, other)
 
 
-def _unary(op, x, out_dtype, bounds=0, lo=None, hi=None):
+@device_managed
+def minimum(self, other):
+    """aten.minimum.default: NaN in either operand wins."""
+    return _binary(_lib.MINIMUM, self, other)
+
+
+def _unary(op, x, out_dtype, bounds=0, lo=None, hi=None, inplace=False):
     x = cast(x, out_dtype)
-    out = _out_like_inputs(x.shape, out_dtype, (x,))
+    out = x if inplace else _out_like_inputs(x.shape, out_dtype, (x,))
     if out.numel() == 0:
         return out
     if out_dtype.is_floating_point:
@@ -89,12 +152,35 @@ def _unary(op, x, out_dtype, bounds=0, lo=None, hi=None):
     return out
 
 
+def _check_relu_dtype(t):
+    if t.dtype == torch.bool or t.dtype.is_complex:
+        raise RuntimeError(f"relu is not implemented for {t.dtype}")
+
+
 @device_managed
 def relu(self):
     """aten.relu.default"""
-    if self.dtype == torch.bool or self.dtype.is_complex:
-        raise RuntimeError(f"relu is not implemented for {self.dtype}")
+    _check_relu_dtype(self)
     return _unary(_lib.RELU, self, self.dtype)
+
+
+def relu_(self):
+    """aten.relu_.default"""
+    _check_relu_dtype(self)
+    if not _is_gpu_tensor(self):
+        return copy_into_any(self, relu(self))
+    _unary(_lib.RELU, self, self.dtype, inplace=True)
+    return self
+
+
+def _clamp_dtype(self, bounds):
+    dtype = self.dtype
+    for bound in bounds:
+        if bound is not None:
+            dtype = torch.result_type(torch.empty((), dtype=dtype, device="meta").expand(1), bound)
+    if dtype == torch.bool or dtype.is_complex:
+        raise NotImplementedError(f"mi355 backend: clamp on {dtype} is not supported")
+    return dtype
 
 
 @device_managed
@@ -102,14 +188,48 @@ def clamp(self, min=None, max=None):
     """aten.clamp.default: Scalar bounds; at least one must be given."""
     if min is None and max is None:
         raise RuntimeError("torch.clamp: At least one of 'min' or 'max' must not be None")
-    dtype = self.dtype
-    for bound in (min, max):
-        if bound is not None:
-            dtype = torch.result_type(torch.empty((), dtype=dtype, device="meta").expand(1), bound)
-    if dtype == torch.bool or dtype.is_complex:
-        raise NotImplementedError(f"mi355 backend: clamp on {dtype} is not supported")
     bounds = (1 if min is not None else 0) | (2 if max is not None else 0)
-    return _unary(_lib.CLAMP, self, dtype, bounds, min, max)
+    return _unary(_lib.CLAMP, self, _clamp_dtype(self, (min, max)), bounds, min, max)
+
+
+def clamp_(self, min=None, max=None):
+    """aten.clamp_.default"""
+    if min is None and max is None:
+        raise RuntimeError("torch.clamp: At least one of 'min' or 'max' must not be None")
+    dtype = _clamp_dtype(self, (min, max))
+    if not torch.can_cast(dtype, self.dtype):
+        raise RuntimeError(f"result type {str(dtype).replace('torch.', '').capitalize()} can't be cast to the "
+                           f"desired output type {str(self.dtype).replace('torch.', '').capitalize()}")
+    if dtype != self.dtype or not _is_gpu_tensor(self):
+        return copy_into_any(self, clamp(self, min, max))
+    bounds = (1 if min is not None else 0) | (2 if max is not None else 0)
+    _unary(_lib.CLAMP, self, dtype, bounds, min, max, inplace=True)
+    return self
+
+
+@device_managed
+def clamp_min(self, min):
+    """aten.clamp_min.default"""
+    return _unary(_lib.CLAMP, self, _clamp_dtype(self, (min,)), 1, min, None)
+
+
+@device_managed
+def clamp_max(self, max):
+    """aten.clamp_max.default"""
+    return _unary(_lib.CLAMP, self, _clamp_dtype(self, (max,)), 2, None, max)
+
+
+@device_managed
+def clamp_tensor(self, min=None, max=None):
+    """aten.clamp.Tensor: tensor bounds, min(max(self, lo), hi) with NaN propagation."""
+    if min is None and max is None:
+        raise RuntimeError("torch.clamp: At least one of 'min' or 'max' must not be None")
+    out = self
+    if min is not None:
+        out = _binary(_lib.MAXIMUM, out, min)
+    if max is not None:
+        out = _binary(_lib.MINIMUM, out, max)
+    return out
 
 
 @device_managed
@@ -127,3 +247,23 @@ def where(condition, self, other):
     launch("mi355_where", _lib.desc(condition.expand(shape)), _lib.desc(a.expand(shape)),
            _lib.desc(b.expand(shape)), _lib.desc(out))
     return out
+
+
+def out_variant(functional):
+    """`<op>.out(..., out=Tensor)` from the functional wrapper: compute, resize `out` if its
+    shape differs (as ATen does), then store with a cast into `out`'s dtype and return `out`."""
+
+    def impl(*args, out, **kwargs):
+        res = functional(*args, **kwargs)
+        if not torch.can_cast(res.dtype, out.dtype):
+            raise RuntimeError(f"result type {str(res.dtype).replace('torch.', '').capitalize()} can't be cast to "
+                               f"the desired output type {str(out.dtype).replace('torch.', '').capitalize()}")
+        if tuple(out.shape) != tuple(res.shape):
+            out.resize_(res.shape)
+        if res.device != out.device:
+            res = res.to(out.device)
+        return copy_into_any(out, res)
+
+    impl.__name__ = functional.__name__ + "_out"
+    impl.__doc__ = f"out= variant of {functional.__name__}"
+    return impl

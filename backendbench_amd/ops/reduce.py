@@ -162,9 +162,7 @@ def argmax(self, dim=None, keepdim=False):
     return _run_reduce(_lib.ARGMAX, _max_src(self), dims, keepdim, torch.int64)
 
 
-@device_managed
-def softmax(self, dim, half_to_float):
-    """aten._softmax.default"""
+def _softmax_impl(self, dim, half_to_float, log):
     if not self.dtype.is_floating_point:
         raise RuntimeError("softmax expects a floating point input")
     if half_to_float and self.dtype not in (torch.float16, torch.bfloat16):
@@ -179,8 +177,20 @@ def softmax(self, dim, half_to_float):
     x = dense(self)
     shape = x.shape if x.dim() else (1,)
     launch("mi355_softmax", x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(out_dtype),
-           prod(shape[:d]), shape[d], prod(shape[d + 1 :]))
+           prod(shape[:d]), shape[d], prod(shape[d + 1 :]), 1 if log else 0)
     return out
+
+
+@device_managed
+def softmax(self, dim, half_to_float):
+    """aten._softmax.default"""
+    return _softmax_impl(self, dim, half_to_float, False)
+
+
+@device_managed
+def log_softmax(self, dim, half_to_float):
+    """aten._log_softmax.default"""
+    return _softmax_impl(self, dim, half_to_float, True)
 
 
 @device_managed

@@ -2,7 +2,7 @@
 
 The reference's OpInfo / TorchBench / FACTO suites (BackendBench/suite/opinfo.py,
 torchbench.py, facto.py) need packages or downloads this environment does not have, so
-this module is the input source for the 19 operator slots: `perf_cases()` are the
+this module is the input source for the operator slots: `perf_cases()` are the
 headline configurations (one per measured row: shapes, dtypes, distributions and the
 algorithmic bytes / flops used for roofline fractions) and `edge_cases()` are small
 inputs covering broadcasting, non-contiguous views, NaN / +-inf, ties, empty and 0-d
@@ -168,7 +168,7 @@ def edge_cases() -> List[Case]:
     special = lambda dt: torch.tensor([float("nan"), float("-inf"), -2.0, -0.0, 0.0, 3.0, float("inf"), 0.5], dtype=dt)
 
     # ---- binary: add / mul / maximum
-    for op in (aten.add.Tensor, aten.mul.Tensor, aten.maximum.default):
+    for op in (aten.add.Tensor, aten.mul.Tensor, aten.maximum.default, aten.minimum.default):
         for dt in (f32, f16, bf16):
             add(op, lambda d, dt=dt: (_to(d, normal((33, 65), dt, seed=1), normal((33, 65), dt, seed=2)), {}), tag=f"{dt}".split(".")[-1])
         add(op, lambda d: (_to(d, normal((4, 1, 16), f16, seed=3), normal((1, 5, 16), f16, seed=4)), {}), tag="bcast3")
@@ -213,6 +213,16 @@ def edge_cases() -> List[Case]:
     add(aten.clamp.default, lambda d: (_to(d, normal((50,), f32, seed=1), float("nan"), 1.0), {}), tag="nan_bound")
     add(aten.clamp.default, lambda d: (_to(d, randint((50,), 10, 1, i32, -10), 0.5, 2), {}), tag="int_float_bounds")
     add(aten.clamp.default, lambda d: (_to(d, normal((50,), bf16, seed=1), -0.3, 0.3), {}), tag="bf16_inexact_bounds")
+
+    for op, b in ((aten.clamp_min.default, -0.25), (aten.clamp_max.default, 0.5)):
+        add(op, lambda d, b=b: (_to(d, poison(normal((33, 65), f32, seed=1), 0.05, 2), b), {}), tag="f32_naninf")
+        add(op, lambda d, b=b: ([normal((40, 24), bf16, seed=2).to(d).t(), b], {}), tag="bf16_t")
+        add(op, lambda d, b=b: (_to(d, randint((30,), 10, 1, i32, -10), 2), {}), exact=True, tag="i32")
+        add(op, lambda d, b=b: (_to(d, torch.empty(0, 128, dtype=f16), b), {}), tag="empty")
+    add(aten.clamp.Tensor, lambda d: (_to(d, poison(normal((33, 65), f32, seed=1), 0.05, 2), normal((33, 65), f32, -1, 0.2, seed=3), normal((33, 65), f32, 1, 0.2, seed=4)), {}), tag="both")
+    add(aten.clamp.Tensor, lambda d: (_to(d, normal((6, 40), f16, seed=1), normal((40,), f16, -0.5, 0.1, seed=3), None), {}), tag="min_bcast")
+    add(aten.clamp.Tensor, lambda d: (_to(d, normal((6, 40), bf16, seed=1), None, torch.tensor(0.25, dtype=bf16)), {}), tag="max_0d")
+    add(aten.clamp.Tensor, lambda d: (_to(d, normal((50,), f32, seed=1), torch.full((50,), float("nan")), normal((50,), f32, 1, 0.1, seed=2)), {}), tag="nan_bound")
 
     # ---- where
     cond = lambda shape, seed: normal(shape, f32, seed=seed) > 0
@@ -304,6 +314,17 @@ def edge_cases() -> List[Case]:
     add(aten._softmax.default, lambda d: (_to(d, torch.tensor(0.3, dtype=f32), 0, False), {}), tag="0d")
     add(aten._softmax.default, lambda d: (_to(d, normal((37, 129), bf16, 0, 2, seed=1), -1, True), {}), tag="half_to_float")
 
+    for dt in (f32, f16, bf16):
+        t = f"{dt}".split(".")[-1]
+        add(aten._log_softmax.default, lambda d, dt=dt: (_to(d, normal((37, 129), dt, 0, 2, seed=1), -1, False), {}), tag=f"last_{t}")
+    add(aten._log_softmax.default, lambda d: (_to(d, normal((16, 4096), bf16, 0, 2, seed=1), -1, False), {}), tag="row4096")
+    add(aten._log_softmax.default, lambda d: (_to(d, normal((3, 50000), f32, 0, 2, seed=1), -1, False), {}), tag="long_rows")
+    add(aten._log_softmax.default, lambda d: (_to(d, normal((5, 300, 7), f32, seed=1), 1, False), {}), tag="mid")
+    add(aten._log_softmax.default, lambda d: (_to(d, torch.tensor([[float("-inf"), float("-inf")], [float("inf"), 1.0], [float("nan"), 1.0],
+                                                                     [float("-inf"), 0.0], [1.0, 2.0]], dtype=f32), -1, False), {}), tag="special")
+    add(aten._log_softmax.default, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), -1, False), {}), tag="empty")
+    add(aten._log_softmax.default, lambda d: (_to(d, normal((37, 129), bf16, 0, 2, seed=1), -1, True), {}), tag="half_to_float")
+
     # ---- native_layer_norm
     for dt in (f32, f16, bf16):
         t = f"{dt}".split(".")[-1]
@@ -393,7 +414,9 @@ def _as_test(case, device):
 
 def BaselineTestSuite(device="cuda", scale=1.0, filter=None):
     """OpTests over the slots: edge cases as correctness tests, headline rows as
-    performance tests.  `filter`: list of op-name substrings (like the CLI's --ops)."""
+    performance tests.  `filter`: list of operator names matched exactly, with or without
+    the overload ("_softmax", "add.Tensor"), as the reference's OpInfo suite matches --ops
+    (BackendBench/suite/opinfo.py:91)."""
     per_op = {}
     for case in edge_cases():
         per_op.setdefault(case.op, ([], []))[0].append(case)
@@ -402,7 +425,7 @@ def BaselineTestSuite(device="cuda", scale=1.0, filter=None):
     optests = []
     for op, (edges, perfs) in per_op.items():
         name = op.__name__
-        if filter and not any(f in name for f in filter):
+        if filter and name not in filter and name.split(".")[0] not in filter:
             continue
         optests.append(OpTest(get_operator(op), [_as_test(c, device) for c in edges],
                               [_as_test(c, device) for c in perfs]))

@@ -69,13 +69,20 @@ const char* mi355_last_error(void);
 
 /* ---- elementwise -------------------------------------------------------------- */
 
-typedef enum mi355_binary_op { MI355_ADD = 0, MI355_MUL = 1, MI355_MAXIMUM = 2 } mi355_binary_op;
+typedef enum mi355_binary_op {
+  MI355_ADD = 0,
+  MI355_MUL = 1,
+  MI355_MAXIMUM = 2,
+  MI355_MINIMUM = 3
+} mi355_binary_op;
 
 /* out = a (op) b with a, b already broadcast to out's shape (stride 0 where expanded)
  * and already of out's dtype.  MI355_ADD computes a + alpha*b (alpha_f for floating
- * dtypes, alpha_i for integer dtypes).  MI355_MAXIMUM propagates NaN.
+ * dtypes, alpha_i for integer dtypes).  MI355_MAXIMUM / MI355_MINIMUM propagate NaN.
+ * `out` may be `a` itself (in-place overloads).
  * Slots: add__Tensor (op_map.py:266), mul__Tensor (op_map.py:749),
- * maximum__default (op_map.py:706). */
+ * maximum__default (op_map.py:706), minimum__default (op_map.py:717); with both,
+ * clamp__Tensor (op_map.py:372). */
 int mi355_binary(int op, const mi355_tensor* a, const mi355_tensor* b, double alpha_f,
                  int64_t alpha_i, const mi355_tensor* out, void* stream);
 
@@ -83,7 +90,9 @@ typedef enum mi355_unary_op { MI355_RELU = 0, MI355_CLAMP = 1 } mi355_unary_op;
 
 /* out = relu(x) or clamp(x, lo, hi); x has out's shape and dtype.  `bounds` bit 0 = lo
  * present, bit 1 = hi present.  NaN inputs stay NaN; lo > hi yields hi everywhere.
- * Slots: relu__default (op_map.py:877), clamp__default (op_map.py:371). */
+ * `out` may be `x` itself (in-place overloads).
+ * Slots: relu__default (op_map.py:877), clamp__default (op_map.py:371),
+ * clamp_min__default (op_map.py:369), clamp_max__default (op_map.py:367). */
 int mi355_unary(int op, const mi355_tensor* x, int bounds, double lo_f, double hi_f,
                 int64_t lo_i, int64_t hi_i, const mi355_tensor* out, void* stream);
 
@@ -123,11 +132,11 @@ int mi355_reduce(int op, const void* x, int in_dtype, int64_t outer, int64_t red
                  int64_t inner, void* out, int out_dtype, void* workspace,
                  int64_t workspace_bytes, void* stream);
 
-/* y = softmax over the middle axis of dense x viewed as [outer, dim, inner]; fp32 math.
- * out_dtype = in_dtype, or MI355_F32 for half_to_float.
- * Slot: _softmax__default (op_map.py:193). */
+/* y = softmax (log_softmax != 0: log-softmax) over the middle axis of dense x viewed as
+ * [outer, dim, inner]; fp32 math.  out_dtype = in_dtype, or MI355_F32 for half_to_float.
+ * Slots: _softmax__default (op_map.py:193), _log_softmax__default (op_map.py:151). */
 int mi355_softmax(const void* x, int in_dtype, void* y, int out_dtype, int64_t outer,
-                  int64_t dim, int64_t inner, void* stream);
+                  int64_t dim, int64_t inner, int log_softmax, void* stream);
 
 /* Layer norm over the last N elements of each of M dense rows.  weight/bias may be NULL
  * and may differ in dtype from x (w_dtype).  mean/rstd are dense [M] in stat_dtype

@@ -4,7 +4,7 @@ Follows BackendBench/eval.py:99-100 (`ref = op(*args, **kwargs)`) with the argum
 to the CPU, plus the two places where ATen's CPU and GPU kernels differ in *signature*
 rather than in mathematics and the device convention is the one the backend follows:
 
-* `_softmax(x, dim, half_to_float=True)`: the CPU kernel refuses it; the reference value is
+* `_softmax` / `_log_softmax(x, dim, half_to_float=True)`: the CPU kernel refuses it; the reference value is
   `_softmax(x.float(), dim, False)` (the same mathematics: fp32 softmax of the upcast input).
 * `native_layer_norm` on f16/bf16 input: the CPU kernel returns mean/rstd rounded to the
   input dtype, GPU kernels return them in fp32.  y comes from the plain call; mean/rstd come
@@ -31,7 +31,7 @@ def reference(op, args, kwargs=None):
     args = to_cpu(list(args))
     kwargs = to_cpu(dict(kwargs or {}))
     name = op.__name__
-    if name == "_softmax.default" and len(args) >= 3 and args[2]:
+    if name in ("_softmax.default", "_log_softmax.default") and len(args) >= 3 and args[2]:
         return op(args[0].float(), args[1], False)
     if name == "native_layer_norm.default" and args[0].dtype in (torch.float16, torch.bfloat16):
         x, shape, w, b, eps = args

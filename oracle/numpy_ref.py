@@ -23,6 +23,30 @@ def maximum(a, b):
         return np.where(np.isnan(a) | np.isnan(b), np.nan, np.where(a > b, a, b)) if a.dtype.kind == "f" else np.maximum(a, b)
 
 
+def minimum(a, b):
+    """minimum(Tensor self, Tensor other): elementwise min, NaN if either is NaN."""
+    with np.errstate(invalid="ignore"):
+        return np.where(np.isnan(a) | np.isnan(b), np.nan, np.where(a < b, a, b)) if a.dtype.kind == "f" else np.minimum(a, b)
+
+
+def clamp_tensor(x, lo=None, hi=None):
+    """clamp.Tensor(Tensor self, Tensor? min, Tensor? max): minimum(maximum(x, min), max)."""
+    y = x
+    if lo is not None:
+        y = maximum(*np.broadcast_arrays(np.asarray(y, dtype=np.result_type(y, lo)), np.asarray(lo, dtype=np.result_type(y, lo))))
+    if hi is not None:
+        y = minimum(*np.broadcast_arrays(np.asarray(y, dtype=np.result_type(y, hi)), np.asarray(hi, dtype=np.result_type(y, hi))))
+    return y
+
+
+def log_softmax(x, dim):
+    """_log_softmax: (x - max) - log(sum(exp(x - max))) along dim."""
+    with np.errstate(invalid="ignore", over="ignore", divide="ignore"):
+        m = np.max(x, axis=dim, keepdims=True)
+        d = x - m
+        return d - np.log(np.exp(d).sum(axis=dim, keepdims=True))
+
+
 def relu(x):
     """relu(Tensor self): max(x, 0) with NaN kept."""
     with np.errstate(invalid="ignore"):

@@ -53,7 +53,7 @@ def test_struct_layout_matches_header():
                                         ("MI355_F64", _lib.F64), ("MI355_I32", _lib.I32), ("MI355_I64", _lib.I64),
                                         ("MI355_I16", _lib.I16), ("MI355_I8", _lib.I8), ("MI355_U8", _lib.U8),
                                         ("MI355_BOOL", _lib.BOOL), ("MI355_ADD", _lib.ADD), ("MI355_MUL", _lib.MUL),
-                                        ("MI355_MAXIMUM", _lib.MAXIMUM), ("MI355_RELU", _lib.RELU),
+                                        ("MI355_MAXIMUM", _lib.MAXIMUM), ("MI355_MINIMUM", _lib.MINIMUM), ("MI355_RELU", _lib.RELU),
                                         ("MI355_CLAMP", _lib.CLAMP), ("MI355_SUM", _lib.SUM), ("MI355_MEAN", _lib.MEAN),
                                         ("MI355_AMAX", _lib.AMAX), ("MI355_ARGMAX", _lib.ARGMAX)])
 def test_enum_values_match_header(name, value):
@@ -63,7 +63,7 @@ def test_enum_values_match_header(name, value):
 def test_argument_errors_are_reported_without_a_gpu():
     """Validation happens before any launch, so the error path is testable on the host."""
     lib = _lib.load()
-    rc = lib.mi355_softmax(None, _lib.F32, None, _lib.F32, 4, 4, 1, None)
+    rc = lib.mi355_softmax(None, _lib.F32, None, _lib.F32, 4, 4, 1, 0, None)
     assert rc == -1 and b"NULL" in lib.mi355_last_error()
     rc = lib.mi355_reduce(_lib.SUM, None, _lib.F32, 4, 0, 1, None, _lib.F32, None, 0, None)
     assert rc == -1 and b"bad extents" in lib.mi355_last_error()

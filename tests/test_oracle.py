@@ -71,6 +71,16 @@ def numpy_result(case, args, kwargs):
         return numpy_ref.mul(a[0], a[1])
     if n == "maximum.default":
         return numpy_ref.maximum(*np.broadcast_arrays(a[0], a[1]))
+    if n == "minimum.default":
+        return numpy_ref.minimum(*np.broadcast_arrays(a[0], a[1]))
+    if n == "clamp_min.default":
+        return numpy_ref.clamp(a[0], a[1], None)
+    if n == "clamp_max.default":
+        return numpy_ref.clamp(a[0], None, a[1])
+    if n == "clamp.Tensor":
+        return numpy_ref.clamp_tensor(a[0], a[1], a[2] if len(a) > 2 else None)
+    if n == "_log_softmax.default":
+        return numpy_ref.log_softmax(a[0], a[1])
     if n == "relu.default":
         return numpy_ref.relu(a[0])
     if n == "clamp.default":

@@ -30,7 +30,7 @@ PERF = perf_cases()
 def backend():
     assert torch.cuda.is_available(), "these tests need the MI355X"
     b = DirectoryBackend(os.path.join(ROOT, "generated_kernels"))
-    assert len(b.compiled_kernels) == 19
+    assert len(b.compiled_kernels) == 43
     return b
 
 
@@ -270,3 +270,174 @@ def test_hip_graph_replays_match_eager(backend):
         torch.cuda.synchronize()
         for o, e_ in zip(outs, want):
             assert ev.allclose(e_.cpu(), o.cpu(), exact=not o.dtype.is_floating_point), f"replay {rep} differs"
+
+
+def _t(shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def _inplace_cases():
+    f32, bf16, f16, i32 = torch.float32, torch.bfloat16, torch.float16, torch.int32
+    return [
+        ("add_.same", aten.add_.Tensor, lambda: ([_t((33, 65)), _t((33, 65), seed=1)], {})),
+        ("add_.alpha_bcast", aten.add_.Tensor, lambda: ([_t((33, 65), bf16), _t((65,), bf16, seed=1)], {"alpha": -0.5})),
+        ("add_.mixed_dtype", aten.add_.Tensor, lambda: ([_t((17, 40), bf16), _t((17, 40), f32, seed=1)], {})),
+        ("add_.transposed_self", aten.add_.Tensor, lambda: ([_t((40, 24), f16).t(), _t((24, 40), f16, seed=1)], {})),
+        ("add_.int", aten.add_.Tensor, lambda: ([torch.arange(60, dtype=i32).reshape(6, 10), torch.arange(10, dtype=i32)], {"alpha": 3})),
+        ("add_.zero_d_other", aten.add_.Tensor, lambda: ([_t((9, 9)), torch.tensor(2.5)], {})),
+        ("add_.empty", aten.add_.Tensor, lambda: ([torch.empty(0, 8), torch.empty(0, 8)], {})),
+        ("mul_.same", aten.mul_.Tensor, lambda: ([_t((128, 130), bf16), _t((128, 130), bf16, seed=1)], {})),
+        ("mul_.bcast_col", aten.mul_.Tensor, lambda: ([_t((31, 70)), _t((31, 1), seed=1)], {})),
+        ("mul_.sliced_self", aten.mul_.Tensor, lambda: ([_t((20, 64))[:, 3:35], _t((20, 32), seed=1)], {})),
+        ("relu_.f16", aten.relu_.default, lambda: ([_t((1000,), f16)], {})),
+        ("relu_.transposed", aten.relu_.default, lambda: ([_t((12, 50)).t()], {})),
+        ("relu_.int", aten.relu_.default, lambda: ([torch.arange(-20, 20, dtype=i32)], {})),
+        ("clamp_.both", aten.clamp_.default, lambda: ([_t((33, 65)), -0.25, 0.5], {})),
+        ("clamp_.min_only", aten.clamp_.default, lambda: ([_t((33, 65), bf16), 0.0], {})),
+        ("clamp_.max_kw", aten.clamp_.default, lambda: ([_t((7, 5, 3), f16)], {"max": 0.1})),
+    ]
+
+
+@pytest.mark.parametrize("case", _inplace_cases(), ids=[c[0] for c in _inplace_cases()])
+def test_inplace_overloads_write_through_self(backend, case):
+    """add_/mul_/relu_/clamp_ return `self` itself, leave its layout alone, and hold the values
+    ATen's in-place overload leaves in a CPU clone of the same inputs."""
+    key, op, make = case
+    announce(key)
+    args, kwargs = make()
+    args = [a.cuda() if isinstance(a, torch.Tensor) else a for a in args]
+    base = args[0]
+    cpu_args = [a.cpu().clone() if isinstance(a, torch.Tensor) else a for a in args]
+    if not base.is_contiguous():   # clone() would densify: rebuild the same view on the CPU
+        cpu_args[0] = torch.empty_strided(base.shape, base.stride(), dtype=base.dtype).copy_(base.cpu())
+    ptr, stride = base.data_ptr(), base.stride()
+    res = backend[op](*args, **kwargs)
+    torch.cuda.synchronize()
+    ref = op(*cpu_args, **kwargs)
+    assert res is base and res.data_ptr() == ptr and res.stride() == stride
+    assert ev.allclose(ref, res.cpu(), exact=not ref.dtype.is_floating_point), key
+
+
+def test_inplace_overloads_reject_what_aten_rejects(backend):
+    announce("in-place error behaviour")
+    ints = torch.arange(6, device="cuda")
+    for op, args in ((aten.add_.Tensor, [ints, torch.ones(6, device="cuda")]),          # float result into int self
+                     (aten.mul_.Tensor, [torch.ones(6, device="cuda"), torch.ones(2, 6, device="cuda")]),  # self would grow
+                     (aten.clamp_.default, [torch.ones(3, device="cuda")])):
+        cpu_args = [a.cpu().clone() if isinstance(a, torch.Tensor) else a for a in args]
+        expected = aten_cpu.raises(op, cpu_args)
+        assert expected is not None, op
+        with pytest.raises(expected):
+            backend[op](*args)
+    assert torch.equal(ints.cpu(), torch.arange(6))   # nothing was written
+
+
+def _out_cases():
+    f32, bf16, i64 = torch.float32, torch.bfloat16, torch.int64
+    idx = torch.tensor([4, 0, 4, 2])
+    gidx = torch.randint(0, 9, (9, 5), generator=torch.Generator().manual_seed(5))
+    cond = _t((6, 30), seed=9) > 0
+    return [
+        ("add.out", aten.add.out, [_t((6, 30)), _t((30,), seed=1)], {"alpha": 2}, ((6, 30), f32)),
+        ("add.out_cast", aten.add.out, [_t((6, 30)), _t((6, 30), seed=1)], {}, ((6, 30), bf16)),
+        ("add.out_resized", aten.add.out, [_t((6, 30)), _t((6, 30), seed=1)], {}, ((0,), f32)),
+        ("mul.out", aten.mul.out, [_t((6, 30), bf16), _t((6, 30), bf16, seed=1)], {}, ((6, 30), bf16)),
+        ("maximum.out", aten.maximum.out, [_t((6, 30)), _t((6, 30), seed=1)], {}, ((6, 30), f32)),
+        ("relu.out", aten.relu.out, [_t((6, 30))], {}, ((6, 30), f32)),
+        ("clamp.out", aten.clamp.out, [_t((6, 30)), -0.1, 0.3], {}, ((6, 30), f32)),
+        ("where.self_out", aten.where.self_out, [cond, _t((6, 30)), _t((6, 30), seed=1)], {}, ((6, 30), f32)),
+        ("sum.IntList_out", aten.sum.IntList_out, [_t((6, 30, 4)), [1]], {"keepdim": True}, ((6, 1, 4), f32)),
+        ("sum.IntList_out_dtype", aten.sum.IntList_out, [_t((6, 30), bf16), [-1]], {"dtype": f32}, ((6,), f32)),
+        ("mean.out", aten.mean.out, [_t((6, 30)), [0]], {}, ((30,), f32)),
+        ("amax.out", aten.amax.out, [_t((6, 30)), [-1]], {}, ((6,), f32)),
+        ("argmax.out", aten.argmax.out, [_t((6, 30)), 1], {}, ((6,), i64)),
+        ("_softmax.out", aten._softmax.out, [_t((6, 30)), -1, False], {}, ((6, 30), f32)),
+        ("mm.out", aten.mm.out, [_t((64, 96), bf16), _t((96, 32), bf16, seed=1)], {}, ((64, 32), bf16)),
+        ("addmm.out", aten.addmm.out, [_t((32,)), _t((64, 96)), _t((96, 32), seed=1)], {"beta": 0.5, "alpha": 2.0}, ((64, 32), f32)),
+        ("index_select.out", aten.index_select.out, [_t((9, 5)), 0, idx], {}, ((4, 5), f32)),
+        ("gather.out", aten.gather.out, [_t((9, 5)), 0, gidx], {}, ((9, 5), f32)),
+    ]
+
+
+@pytest.mark.parametrize("case", _out_cases(), ids=[c[0] for c in _out_cases()])
+def test_out_overloads_fill_the_given_tensor(backend, case):
+    """`<op>.out(..., out=t)` returns `t` itself holding what ATen's out= overload writes on the
+    CPU, including the cast into `t`'s dtype and the resize of a wrongly shaped `t`."""
+    import warnings
+
+    key, op, args, kwargs, (oshape, odtype) = case
+    announce(key)
+    out = torch.full(oshape, 7, dtype=odtype).cuda()
+    gpu_args = [a.cuda() if isinstance(a, torch.Tensor) else a for a in args]
+    res = backend[op](*gpu_args, out=out, **kwargs)
+    torch.cuda.synchronize()
+    from backendbench_amd.ops import check_index_errors
+
+    check_index_errors()
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        ref = op(*args, out=torch.full(oshape, 7, dtype=odtype), **kwargs)
+    assert res is out
+    assert ev.allclose(ref, res.cpu(), exact=not ref.dtype.is_floating_point or key in ("where.self_out", "index_select.out", "gather.out")), key
+
+
+def test_out_overload_rejects_a_narrowing_cast(backend):
+    announce("out= error behaviour")
+    a = torch.ones(4, device="cuda")
+    out = torch.zeros(4, dtype=torch.int32, device="cuda")
+    assert aten_cpu.raises(aten.add.out, [a.cpu(), a.cpu()], {"out": out.cpu()}) is RuntimeError
+    with pytest.raises(RuntimeError):
+        backend[aten.add.out](a, a, out=out)
+
+
+def test_variant_overloads_through_the_live_dispatcher(backend):
+    """Python's in-place operators, out= keywords and the sibling overloads reach the variant
+    slots under enable(), with results equal to the stock run."""
+    import backendbench_amd
+    import backendbench_amd.ops.elementwise as e
+    import backendbench_amd.ops.reduce as r
+    from backendbench_amd.ops import _common
+
+    announce("enable(): in-place / out= / sibling overloads")
+    x0 = _t((48, 200), torch.bfloat16, seed=1).cuda()
+    y0 = _t((48, 200), torch.bfloat16, seed=2).cuda()
+    lo = _t((200,), torch.bfloat16, seed=3, scale=0.1).cuda() - 0.5
+
+    def work():
+        x = x0.clone()
+        x += y0
+        x *= 0.5
+        x.mul_(y0)
+        z = torch.empty_like(x)
+        torch.add(x, y0, alpha=2, out=z)
+        z.relu_()
+        z.clamp_(max=1.5)
+        c = torch.clamp(x, min=lo)
+        m = torch.minimum(c, y0)
+        lp = torch.log_softmax(m.float(), dim=-1)
+        cm = torch.clamp_min(x, -0.25).clamp_max(0.75)
+        return x, z, c, m, lp, cm
+
+    plain = work()
+    calls = []
+    orig = _common.launch
+
+    def spy(name, *a):
+        calls.append((name, a[0] if name in ("mi355_binary", "mi355_unary") else None))
+        return orig(name, *a)
+
+    with backendbench_amd.BackendBench.enable(kernel_dir=os.path.join(ROOT, "generated_kernels"), dispatch_key="CUDA"):
+        e.launch = r.launch = spy
+        try:
+            ours = work()
+            torch.cuda.synchronize()
+        finally:
+            e.launch = r.launch = orig
+    from backendbench_amd import _lib
+
+    names = [n for n, _ in calls]
+    assert names.count("mi355_binary") >= 6 and names.count("mi355_unary") >= 4 and "mi355_softmax" in names
+    assert ("mi355_binary", _lib.MINIMUM) in calls and ("mi355_binary", _lib.MAXIMUM) in calls
+    for a, b in zip(plain, ours):
+        assert a.dtype == b.dtype and ev.allclose(a.cpu(), b.cpu())
