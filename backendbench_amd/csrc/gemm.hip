@@ -177,8 +177,11 @@ constexpr int kPanel3 = BM * BK3 * 2;        // 16 KB per operand per stage
 constexpr int kStage3 = 2 * kPanel3;         // 32 KB
 constexpr int kGemmLds = kStages3 * kStage3;  // 128 KB
 
-// K-contiguous panel with 64-byte rows (4 chunks): XOR with (r/4)%4 spreads 16 consecutive rows
-// reading the same chunk over the 16 16-byte positions of the 256-byte bank window.
+// K-contiguous panel with 64-byte rows (4 chunks): four consecutive rows fill the four 64-byte
+// segments of the 256-byte bank window and the XOR with (r/4)%4 moves each group of four rows
+// to another 16-byte position.  The 16 lanes of one ds_read_b128 pass hold rows {0-3, 12-15,
+// 20-27} or {4-11, 16-19, 28-31} of a fragment (see swz_k64): in both sets (r/4)%4 takes every
+// value once, so a pass touches 16 distinct positions (SQ_LDS_BANK_CONFLICT reads 0).
 __device__ __forceinline__ int swz_k32(int r, int c) { return r * 64 + ((c ^ ((r >> 2) & 3)) << 4); }
 
 // KTAIL: K is not a multiple of BK3, so chunks past K are zero-filled (branch-free: the address
@@ -460,6 +463,180 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma_kernel(GemmArgs g) {
   store_tile_result<T>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
 }
 
+// ---------------------------------------------------------------- MFMA kernel, full-line A fills
+// Row-major ("NN") B and K % 64 == 0.  As gemm_mfma_dma_kernel, except that the A panel is
+// fetched 64 k (one whole 128-byte line per row) at a time: with 32-k steps every line of A is
+// requested twice, 64 bytes each, which halves the useful width of each L2 request and was
+// measured to hold the A stream to ~13.5 TB/s chip-wide against ~21.5 TB/s for whole lines.
+// LDS: three A slots of 256 x 64 (32 KB, rows of 128 B, swz_k64) and four B slots of 32 x 256
+// (16 KB, swz_n) = 160 KB.  A step is still 32 k.  At the start of an even step t the A slot
+// that steps t-2, t-1 used is refilled with k-range of steps t+4, t+5 (four loads per lane);
+// every step t refills the B slot of step t-1 with step t+3 (two loads per lane).  The first
+// fragments of step t+1 are read before the barrier that ends step t, so at that barrier the
+// panels of step t+2 must have landed: only the loads issued in step t itself may still fly
+// (s_waitcnt vmcnt(6) after an even step, vmcnt(2) after an odd one).
+constexpr int kASlot64 = BM * 64 * 2;                 // 32 KB
+constexpr int kBRing64 = 3 * kASlot64;                // B slots start here
+constexpr int kGemmLds64 = kBRing64 + 4 * kPanel3;    // 160 KB
+// K-contiguous panel with 128-byte rows (8 chunks).  A ds_read_b128 is served in four passes of
+// 16 lanes, and the passes are not runs of consecutive lanes: measured on gfx950 they are lanes
+// {0-3, 12-15, 20-27}, {4-11, 16-19, 28-31} and the same sets + 32.  A fragment read puts rows
+// r0 + lane%32 in the lanes, so the rows of one pass are {0-3, 12-15, 20-27} or the rest; the
+// XOR term (bits 1, 3, 4 of the row) takes all eight values over the even rows of either set
+// and over the odd rows, which with the row parity selecting the 128-byte half gives the 16
+// lanes of a pass 16 distinct 16-byte positions of the 256-byte bank window.
+__device__ __forceinline__ int swz_k64(int r, int c) {
+  return r * 128 + ((c ^ (((r >> 1) & 1) | ((r >> 2) & 6))) << 4);
+}
+
+template <typename T>
+__global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  using frag_t = typename Mfma<T>::frag;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 2, wn = wave & 3;
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  const int bm = tm * BM, bn = tn * BN;
+  const T* A = static_cast<const T*>(g.a);
+  const T* B = static_cast<const T*>(g.b);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  // A: region q = wave + 8 i (i < 4) of a slot is rows 8q .. 8q+7, eight 16-byte chunks per row.
+  // B: region q = wave + 8 i (i < 2) of a slot is k rows 2q, 2q+1, 32 units per row.
+  const T* a_src[4];
+  const T* b_src[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 8 * (wave + 8 * i) + (lane >> 3), slot = lane & 7;
+    const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
+    int gr = bm + r;
+    gr = gr < g.M ? gr : g.M - 1;
+    a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int k = 2 * (wave + 8 * i) + (lane >> 5), pos = lane & 31;
+    const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+    int gn = bn + u * 8;
+    gn = gn < g.N ? gn : 0;
+    b_src[i] = B + (int64_t)k * g.ldb + gn;
+  }
+  // a_slot: byte offset of the A slot to fill; t: first of the two steps it will hold.
+  auto request_a = [&](int t, uint32_t a_slot) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      lds_dma16(lds_base + a_slot + (uint32_t)(wave + 8 * i) * 1024u, a_src[i] + (int64_t)t * BK3);
+  };
+  auto request_b = [&](int t) {
+    const uint32_t stage = lds_base + kBRing64 + (uint32_t)(t & 3) * kPanel3;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      lds_dma16(stage + (uint32_t)(wave + 8 * i) * 1024u, b_src[i] + (int64_t)t * BK3 * g.ldb);
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  const int tr_k = fg * 8 + ((lane & 15) >> 2);
+  const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  // Fragments of 16-k sub-step ks (0, 1) of step t, whose A data is half `half` of `a_slot`.
+  auto read_frags = [&](int t, uint32_t a_slot, int half, int ks, frag_t (&fa)[4], frag_t (&fb)[2]) {
+    const unsigned char* pa = lds + a_slot;
+    const unsigned char* pb = lds + kBRing64 + (t & 3) * kPanel3;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 128 + i * 32 + fr, half * 4 + ks * 2 + fg));
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int k = ks * 16 + tr_k;
+      const int n = wn * 64 + j * 32 + tr_n;
+      const s16x4 lo = lds_read_tr(pb + swz_n(k, n >> 3) + ((n & 7) << 1));
+      const s16x4 hi = lds_read_tr(pb + swz_n(k + 4, n >> 3) + ((n & 7) << 1));
+      fb[j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
+  };
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto mma = [&](frag_t (&fa)[4], frag_t (&fb)[2]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+  };
+  auto next_slot = [](uint32_t s) { return s + kASlot64 == (uint32_t)kBRing64 ? 0u : s + kASlot64; };
+
+#define MI355_MFMA_THEN_READS                              \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       \
+  __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);       \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       \
+  __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+#define MI355_STEP_SCHEDULE                                                                   \
+  MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS     \
+  MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS MI355_MFMA_THEN_READS
+
+  const int nk = g.K / BK3;  // even: K % 64 == 0
+  request_a(0, 0);
+  if (nk > 2) request_a(2, kASlot64);
+  request_b(0);
+  if (nk > 1) request_b(1);
+  if (nk > 2) request_b(2);
+  if (nk > 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  frag_t fa0[4], fb0[2], fa1[4], fb1[2];
+  uint32_t cur = 0;  // A slot of steps t, t+1
+  read_frags(0, cur, 0, 0, fa0, fb0);
+  int t = 0;
+  // Steady state, two steps per trip and no conditions inside: each half is one scheduling
+  // region in which the MFMAs of a 16-k sub-step are interleaved with the LDS reads of the
+  // following one.
+  for (; t + 5 < nk; t += 2) {
+    const uint32_t nxt = next_slot(cur);
+    // even step t
+    request_a(t + 4, next_slot(nxt));
+    request_b(t + 3);
+    read_frags(t, cur, 0, 1, fa1, fb1);
+    mma(fa0, fb0);
+    read_frags(t + 1, cur, 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    MI355_STEP_SCHEDULE
+    asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    __syncthreads();
+    // odd step t+1
+    request_b(t + 4);
+    read_frags(t + 1, cur, 1, 1, fa1, fb1);
+    mma(fa0, fb0);
+    read_frags(t + 2, nxt, 0, 0, fa0, fb0);
+    mma(fa1, fb1);
+    MI355_STEP_SCHEDULE
+    asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    __syncthreads();
+    cur = nxt;
+  }
+#undef MI355_STEP_SCHEDULE
+#undef MI355_MFMA_THEN_READS
+  for (; t < nk; ++t) {  // drain: every A slot is already requested, B may lack up to two steps
+    const int half = t & 1;
+    if (t + 3 < nk) request_b(t + 3);
+    read_frags(t, cur, half, 1, fa1, fb1);
+    mma(fa0, fb0);
+    const uint32_t nxt = half ? next_slot(cur) : cur;
+    if (t + 1 < nk) read_frags(t + 1, nxt, half ^ 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    cur = nxt;
+  }
+
+  store_tile_result<T>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
+}
+
 // ---------------------------------------------------------------- generic fallback
 constexpr int GT = 64, GK = 16;
 template <typename T>
@@ -538,21 +715,28 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       MI355_REQUIRE(nblocks < (int64_t(1) << 31), "mi355_gemm: too many tiles");
       const bool ktail = K % BK3 != 0;
       const void* kern;
-      if (ktail) kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
-      else kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
-      // 128 KB of dynamic LDS needs the attribute once per kernel and process.
+      int lds_bytes = kGemmLds;
+      if (ktail) {
+        kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
+      } else if (!b_nt && K % 64 == 0) {
+        kern = (const void*)gemm_mfma_dma64_kernel<T>;
+        lds_bytes = kGemmLds64;
+      } else {
+        kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
+      }
+      // More than 64 KB of dynamic LDS needs the attribute once per kernel and process.
       static thread_local const void* attr_done[8] = {};
       bool seen = false;
       for (const void* k : attr_done) seen = seen || k == kern;
       if (!seen) {
-        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds);
+        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess)
-          return set_error(MI355_ERR_LAUNCH, "mi355_gemm: cannot reserve %d bytes of LDS: %s", kGemmLds, hipGetErrorString(e));
+          return set_error(MI355_ERR_LAUNCH, "mi355_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
         for (const void*& k : attr_done)
           if (k == nullptr) { k = kern; break; }
       }
       void* params[] = {&g};
-      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks), dim3(512), params, kGemmLds, st);
+      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks), dim3(512), params, lds_bytes, st);
       if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma): launch failed: %s", hipGetErrorString(e));
       return check_launch("mi355_gemm(mfma)");
     }

@@ -348,6 +348,8 @@ def edge_cases() -> List[Case]:
         add(aten.addmm.default, lambda d, dt=dt: (_to(d, normal((512,), dt, seed=3), normal((256, 128), dt, seed=1), normal((128, 512), dt, 0, 0.1, seed=2)), {}), tag=f"bias_{t}")
     add(aten.mm.default, lambda d: (_to(d, normal((300, 264), bf16, seed=1), normal((264, 520), bf16, 0, 0.1, seed=2)), {}), tag="edge_tiles")
     add(aten.mm.default, lambda d: (_to(d, normal((512, 1024), bf16, seed=1), normal((1024, 768), bf16, 0, 0.05, seed=2)), {}), tag="multi_tile")
+    for k in (32, 64, 96, 128, 192, 320, 448):   # every prologue / steady-state / drain length of the K loops
+        add(aten.mm.default, lambda d, k=k: (_to(d, normal((260, k), bf16, seed=1), normal((k, 264), bf16, 0, 0.1, seed=2)), {}), tag=f"ksteps_{k}")
     add(aten.mm.default, lambda d: ([normal((512, 320), bf16, seed=1).to(d), normal((768, 320), bf16, 0, 0.05, seed=2).to(d).t()], {}), tag="b_transposed")
     add(aten.mm.default, lambda d: ([normal((320, 512), bf16, seed=1).to(d).t(), normal((320, 768), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_transposed")
     add(aten.mm.default, lambda d: (_to(d, torch.eye(256, dtype=bf16), normal((256, 256), bf16, seed=2)), {}), exact=True, tag="identity")
