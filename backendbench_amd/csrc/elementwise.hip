@@ -32,6 +32,7 @@ template <typename T> struct MaximumF {
     if constexpr (IsFloat<T>::value) {
       if (x != x) return a;
       if (y != y) return b;
+      if (x == y) return __builtin_signbit(x) ? b : a;  // IEEE 754-2019 maximum: +0 above -0
     }
     return x > y ? a : b;
   }
@@ -46,6 +47,7 @@ template <typename T> struct MinimumF {
     if constexpr (IsFloat<T>::value) {
       if (x != x) return a;
       if (y != y) return b;
+      if (x == y) return __builtin_signbit(x) ? a : b;  // IEEE 754-2019 minimum: -0 below +0
     }
     return x < y ? a : b;
   }
@@ -58,7 +60,8 @@ template <typename T> struct ReluF {
   using M = typename OpMath<T>::type;
   __device__ __forceinline__ T operator()(T a, Unused, Unused) const {
     const M x = static_cast<M>(a);
-    return x <= M(0) ? static_cast<T>(M(0)) : a;  // NaN <= 0 is false: NaN passes through
+    // NaN < 0 and -0.0 < 0 are false: both pass through unchanged, as on ATen's CPU kernel
+    return x < M(0) ? static_cast<T>(M(0)) : a;
   }
 };
 template <typename T> struct ClampF {

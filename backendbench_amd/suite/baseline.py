@@ -199,6 +199,9 @@ def edge_cases() -> List[Case]:
         t = f"{dt}".split(".")[-1]
         add(aten.relu.default, lambda d, dt=dt: (_to(d, normal((33, 65), dt, seed=1)), {}), tag=t)
         add(aten.clamp.default, lambda d, dt=dt: (_to(d, normal((33, 65), dt, seed=1), -0.5, 0.75), {}), tag=t)
+    for dt in (f32, bf16, torch.float64):   # sign of zero and NaN survive bit for bit
+        add(aten.relu.default, lambda d, dt=dt: (_to(d, torch.tensor([-0.0, 0.0, -1.0, float("nan"), float("-inf"), float("inf"), 2.5], dtype=dt)), {}),
+            exact=True, tag=f"signed_zero_{str(dt)[6:]}")
     for op, extra in ((aten.relu.default, ()), (aten.clamp.default, (-1, 1))):
         add(op, lambda d, extra=extra: ([special(f32).to(d), *extra], {}), tag="special")
         add(op, lambda d, extra=extra: ([poison(normal((40, 24), f16, seed=2), 0.05, 3).to(d).t(), *extra], {}), tag="naninf_t")
