@@ -201,8 +201,36 @@ __device__ __forceinline__ VecN<T, V> ld_or_splat(const T* p, bool splat) {
   return ld<T, V>(p);
 }
 
-// One work item = V consecutive elements of the innermost dim (V == 1: one element).
-template <typename F, int V, bool WIDE>
+// One work item = V consecutive elements of the innermost dim (V == 1: one element).  A block
+// takes U * kEwBlock consecutive work items, U per thread: the U index splits and loads are all
+// issued before the first store, as in the flat kernel.
+template <typename F, int NT, bool WIDE>
+__device__ __forceinline__ void ew_split_index(const StridedArgs<NT>& a, int64_t lin, int64_t (&off)[NT]) {
+#pragma unroll
+  for (int t = 0; t < NT; ++t) off[t] = 0;
+  if constexpr (WIDE) {
+    int64_t rem = lin;
+    for (int k = a.ndim - 1; k >= 0; --k) {
+      const int64_t q = rem / a.sizes[k];
+      const int64_t idx = rem - q * a.sizes[k];
+      rem = q;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) off[t] += idx * a.strides[t][k];
+    }
+  } else {
+    uint32_t rem = (uint32_t)lin;
+    for (int k = a.ndim - 1; k >= 0; --k) {
+      const FastDiv d = a.div[k];
+      const uint32_t q = (uint32_t)(((uint64_t)__umulhi(rem, d.m) + rem) >> d.s);
+      const uint32_t idx = rem - q * d.d;
+      rem = q;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) off[t] += (int64_t)idx * a.strides[t][k];
+    }
+  }
+}
+
+template <typename F, int V, bool WIDE, int U>
 __global__ __launch_bounds__(kEwBlock) void ew_strided_kernel(F f, EwPtrs p,
                                                                StridedArgs<F::NIN + 1> a,
                                                                int64_t total) {
@@ -212,39 +240,30 @@ __global__ __launch_bounds__(kEwBlock) void ew_strided_kernel(F f, EwPtrs p,
   using T2 = typename F::in2_t;
   constexpr int NIN = F::NIN;
   constexpr int NT = NIN + 1;
-  const int64_t stride = (int64_t)gridDim.x * kEwBlock;
-  for (int64_t lin = (int64_t)blockIdx.x * kEwBlock + threadIdx.x; lin < total; lin += stride) {
-    int64_t off[NT];
+  const int64_t stride = (int64_t)gridDim.x * kEwBlock * U;
+  for (int64_t base = (int64_t)blockIdx.x * kEwBlock * U + threadIdx.x; base < total; base += stride) {
+    VecN<T0, V> va[U];
+    VecN<T1, V> vb[U];
+    VecN<T2, V> vc[U];
+    int64_t out_off[U];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) off[t] = 0;
-    if constexpr (WIDE) {
-      int64_t rem = lin;
-      for (int k = a.ndim - 1; k >= 0; --k) {
-        const int64_t q = rem / a.sizes[k];
-        const int64_t idx = rem - q * a.sizes[k];
-        rem = q;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) off[t] += idx * a.strides[t][k];
-      }
-    } else {
-      uint32_t rem = (uint32_t)lin;
-      for (int k = a.ndim - 1; k >= 0; --k) {
-        const FastDiv d = a.div[k];
-        const uint32_t q = (uint32_t)(((uint64_t)__umulhi(rem, d.m) + rem) >> d.s);
-        const uint32_t idx = rem - q * d.d;
-        rem = q;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) off[t] += (int64_t)idx * a.strides[t][k];
+    for (int j = 0; j < U; ++j) {
+      const int64_t lin = base + (int64_t)j * kEwBlock;
+      if (lin < total) {
+        int64_t off[NT];
+        ew_split_index<F, NT, WIDE>(a, lin, off);
+        out_off[j] = off[NT - 1];
+        va[j] = ld_or_splat<T0, V>(static_cast<const T0*>(p.in[0]) + off[0], a.splat_mask & 1u);
+        if constexpr (NIN > 1)
+          vb[j] = ld_or_splat<T1, V>(static_cast<const T1*>(p.in[1]) + off[1], a.splat_mask & 2u);
+        if constexpr (NIN > 2)
+          vc[j] = ld_or_splat<T2, V>(static_cast<const T2*>(p.in[2]) + off[2], a.splat_mask & 4u);
       }
     }
-    VecN<T0, V> va = ld_or_splat<T0, V>(static_cast<const T0*>(p.in[0]) + off[0], a.splat_mask & 1u);
-    VecN<T1, V> vb;
-    VecN<T2, V> vc;
-    if constexpr (NIN > 1)
-      vb = ld_or_splat<T1, V>(static_cast<const T1*>(p.in[1]) + off[1], a.splat_mask & 2u);
-    if constexpr (NIN > 2)
-      vc = ld_or_splat<T2, V>(static_cast<const T2*>(p.in[2]) + off[2], a.splat_mask & 4u);
-    st_nt<TO, V>(static_cast<TO*>(p.out) + off[NT - 1], ew_apply<F, V>(f, va, vb, vc));
+#pragma unroll
+    for (int j = 0; j < U; ++j)
+      if (base + (int64_t)j * kEwBlock < total)
+        st_nt<TO, V>(static_cast<TO*>(p.out) + out_off[j], ew_apply<F, V>(f, va[j], vb[j], vc[j]));
   }
 }
 
@@ -327,17 +346,24 @@ int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_t
   const bool wide = total >= (int64_t(1) << 31);
   if (!wide)
     for (int k = 0; k < d.ndim; ++k) a.div[k] = make_fastdiv((uint32_t)a.sizes[k]);
+  // Large vectorised problems: four work items per thread, so that a block owns 4 * 256 vectors.
+  constexpr int kStridedUnroll = 4;
+  if (vec_ok && !wide && total >= (int64_t)kEwBlock * kStridedUnroll * kNumCU * 4) {
+    const int grid = grid_for(total, kEwBlock * kStridedUnroll, 1 << 30);
+    hipLaunchKernelGGL((ew_strided_kernel<F, V, false, kStridedUnroll>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+    return check_launch(name);
+  }
   const int grid = grid_for(total, kEwBlock, 1 << 30);
   if (vec_ok) {
     if (wide)
-      hipLaunchKernelGGL((ew_strided_kernel<F, V, true>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+      hipLaunchKernelGGL((ew_strided_kernel<F, V, true, 1>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
     else
-      hipLaunchKernelGGL((ew_strided_kernel<F, V, false>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+      hipLaunchKernelGGL((ew_strided_kernel<F, V, false, 1>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
   } else {
     if (wide)
-      hipLaunchKernelGGL((ew_strided_kernel<F, 1, true>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+      hipLaunchKernelGGL((ew_strided_kernel<F, 1, true, 1>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
     else
-      hipLaunchKernelGGL((ew_strided_kernel<F, 1, false>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+      hipLaunchKernelGGL((ew_strided_kernel<F, 1, false, 1>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
   }
   return check_launch(name);
 }
