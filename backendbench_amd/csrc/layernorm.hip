@@ -100,27 +100,29 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
   }
 }
 
-// Welford state and Chan's merge.
-struct WF {
-  float n, mean, m2;
+// Welford state and Chan's merge, in the accumulation type A (float; double for f64 input).
+template <typename T> struct LnAcc { using type = float; };
+template <> struct LnAcc<double> { using type = double; };
+template <typename A> struct WF {
+  A n, mean, m2;
 };
-__device__ __forceinline__ void wf_update(WF& a, float x) {
-  a.n += 1.f;
-  const float d = x - a.mean;
+template <typename A> __device__ __forceinline__ void wf_update(WF<A>& a, A x) {
+  a.n += A(1);
+  const A d = x - a.mean;
   a.mean += d / a.n;
   a.m2 += d * (x - a.mean);
 }
-__device__ __forceinline__ WF wf_merge(WF a, WF b) {
-  const float n = a.n + b.n;
-  if (n == 0.f) return a;
-  const float d = b.mean - a.mean;
-  const float fb = b.n / n;
+template <typename A> __device__ __forceinline__ WF<A> wf_merge(WF<A> a, WF<A> b) {
+  const A n = a.n + b.n;
+  if (n == A(0)) return a;
+  const A d = b.mean - a.mean;
+  const A fb = b.n / n;
   return {n, a.mean + d * fb, a.m2 + b.m2 + d * d * a.n * fb};
 }
-__device__ __forceinline__ WF wf_wave_reduce(WF a) {
+template <typename A> __device__ __forceinline__ WF<A> wf_wave_reduce(WF<A> a) {
 #pragma unroll
   for (int k = 1; k < kWave; k <<= 1) {
-    WF o{__shfl_xor(a.n, k, kWave), __shfl_xor(a.mean, k, kWave), __shfl_xor(a.m2, k, kWave)};
+    WF<A> o{__shfl_xor(a.n, k, kWave), __shfl_xor(a.mean, k, kWave), __shfl_xor(a.m2, k, kWave)};
     a = wf_merge(a, o);
   }
   return a;
@@ -131,19 +133,20 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_block_kernel(const T* __re
                                                                   const W* __restrict__ b, T* __restrict__ y,
                                                                   S* __restrict__ mean_out, S* __restrict__ rstd_out,
                                                                   int64_t n, float eps) {
+  using A = typename LnAcc<T>::type;
   constexpr int V = Vec<T>::N;
-  __shared__ WF smem[kLnBlock / kWave];
+  __shared__ WF<A> smem[kLnBlock / kWave];
   const T* row = x + (int64_t)blockIdx.x * n;
   T* out = y + (int64_t)blockIdx.x * n;
-  WF a{0.f, 0.f, 0.f};
+  WF<A> a{A(0), A(0), A(0)};
   if constexpr (VEC) {
     for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kLnBlock * V) {
       const Vec<T> t = load_vec(row + c);
 #pragma unroll
-      for (int j = 0; j < V; ++j) wf_update(a, static_cast<float>(t.v[j]));
+      for (int j = 0; j < V; ++j) wf_update(a, static_cast<A>(t.v[j]));
     }
   } else {
-    for (int64_t c = threadIdx.x; c < n; c += kLnBlock) wf_update(a, static_cast<float>(row[c]));
+    for (int64_t c = threadIdx.x; c < n; c += kLnBlock) wf_update(a, static_cast<A>(row[c]));
   }
   a = wf_wave_reduce(a);
   if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = a;
@@ -151,16 +154,18 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_block_kernel(const T* __re
   a = smem[0];
 #pragma unroll
   for (int k = 1; k < kLnBlock / kWave; ++k) a = wf_merge(a, smem[k]);
-  const float mean = a.mean;
-  const float rstd = rsqrtf(a.m2 / (float)n + eps);
+  const A mean = a.mean;
+  A rstd;
+  if constexpr (std::is_same<A, double>::value) rstd = 1.0 / sqrt(a.m2 / (double)n + (double)eps);
+  else rstd = rsqrtf(a.m2 / (float)n + eps);
   if (threadIdx.x == 0) {
     mean_out[blockIdx.x] = static_cast<S>(mean);
     rstd_out[blockIdx.x] = static_cast<S>(rstd);
   }
   for (int64_t c = threadIdx.x; c < n; c += kLnBlock) {
-    float r = (static_cast<float>(row[c]) - mean) * rstd;
-    if (w) r *= static_cast<float>(w[c]);
-    if (b) r += static_cast<float>(b[c]);
+    A r = (static_cast<A>(row[c]) - mean) * rstd;
+    if (w) r *= static_cast<A>(w[c]);
+    if (b) r += static_cast<A>(b[c]);
     out[c] = static_cast<T>(r);
   }
 }
@@ -181,7 +186,9 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
                    reinterpret_cast<uintptr_t>(b) % (sizeof(W) * V) == 0 && N % (16 / sizeof(W)) == 0;
   MI355_REQUIRE(M < (int64_t(1) << 31), "mi355_layer_norm: too many rows (%lld)", (long long)M);
   const size_t param_bytes = 2 * (size_t)N * sizeof(W);
-  const bool done = dispatch_row_tile<T>(N, vec, [&](auto nv, auto wv, auto v) {
+  bool done = false;
+  if constexpr (!std::is_same<T, double>::value)  // f64 rows take the block kernel (double accumulation)
+  done = dispatch_row_tile<T>(N, vec, [&](auto nv, auto wv, auto v) {
     constexpr int NV = decltype(nv)::value, WG = decltype(wv)::value;
     constexpr bool VEC = decltype(v)::value;
     constexpr int BIG = 1024;
@@ -230,6 +237,9 @@ extern "C" int mi355_layer_norm(const void* x, int dtype, const void* weight, co
     case MI355_F16:
       if (w_dtype == MI355_F16) return run_ln_stat<f16_t, f16_t>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);
       if (w_dtype == MI355_F32) return run_ln_stat<f16_t, float>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);
+      break;
+    case MI355_F64:
+      if (w_dtype == MI355_F64) return run_ln_stat<double, double>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);
       break;
     case MI355_BF16:
       if (w_dtype == MI355_BF16) return run_ln_stat<bf16_t, bf16_t>(stat_dtype, dtype, x, weight, bias, y, mean, rstd, M, N, eps, st);

@@ -1,4 +1,5 @@
-// _softmax / _log_softmax over the middle axis of a dense [outer, dim, inner] view, fp32 math.
+// _softmax / _log_softmax over the middle axis of a dense [outer, dim, inner] view, fp32 math
+// (fp64 for f64 input, on the block and cols kernels only).
 //
 //   tile   inner == 1, row fits the registers of 1, 2 or 4 cooperating waves: one HBM read,
 //          max and sum by wave all-reduce (+ one LDS exchange between waves), one HBM write;
@@ -55,30 +56,42 @@ __global__ __launch_bounds__(kSmBlock) void softmax_tile_kernel(const T* __restr
   }
 }
 
-// Online (max, sum) pair; see the file header for the special-value rules.
-struct MS {
-  float m, s;
+// Online (max, sum) pair in the accumulation type A (float; double for f64 input); see the
+// file header for the special-value rules.
+template <typename A> __device__ __forceinline__ A sm_exp(A x) {
+  if constexpr (std::is_same<A, double>::value) return exp(x);
+  else return __expf(x);
+}
+template <typename A> __device__ __forceinline__ A sm_log(A x) {
+  if constexpr (std::is_same<A, double>::value) return log(x);
+  else return __logf(x);
+}
+template <typename T> struct SmAcc { using type = float; };
+template <> struct SmAcc<double> { using type = double; };
+
+template <typename A> struct MS {
+  A m, s;
 };
-__device__ __forceinline__ void ms_update(MS& a, float x) {
+template <typename A> __device__ __forceinline__ void ms_update(MS<A>& a, A x) {
   if (x > a.m) {
-    a.s = a.s * __expf(a.m - x) + __expf(x - x);  // x - x is NaN for +inf
+    a.s = a.s * sm_exp(a.m - x) + sm_exp(x - x);  // x - x is NaN for +inf
     a.m = x;
   } else if (x == -INFINITY) {
     // contributes exactly zero
   } else {
-    a.s += __expf(x - a.m);  // NaN x lands here and poisons the sum
+    a.s += sm_exp(x - a.m);  // NaN x lands here and poisons the sum
   }
 }
-__device__ __forceinline__ MS ms_combine(MS a, MS b) {
-  const float m = a.m > b.m ? a.m : b.m;
-  const float sa = a.m == -INFINITY ? a.s * 0.f : a.s * __expf(a.m - m);
-  const float sb = b.m == -INFINITY ? b.s * 0.f : b.s * __expf(b.m - m);
+template <typename A> __device__ __forceinline__ MS<A> ms_combine(MS<A> a, MS<A> b) {
+  const A m = a.m > b.m ? a.m : b.m;
+  const A sa = a.m == -INFINITY ? a.s * A(0) : a.s * sm_exp(a.m - m);
+  const A sb = b.m == -INFINITY ? b.s * A(0) : b.s * sm_exp(b.m - m);
   return {m, sa + sb};
 }
-__device__ __forceinline__ MS ms_wave_reduce(MS a) {
+template <typename A> __device__ __forceinline__ MS<A> ms_wave_reduce(MS<A> a) {
 #pragma unroll
   for (int k = 1; k < kWave; k <<= 1) {
-    MS o{__shfl_xor(a.m, k, kWave), __shfl_xor(a.s, k, kWave)};
+    MS<A> o{__shfl_xor(a.m, k, kWave), __shfl_xor(a.s, k, kWave)};
     a = ms_combine(a, o);
   }
   return a;
@@ -87,19 +100,20 @@ __device__ __forceinline__ MS ms_wave_reduce(MS a) {
 template <typename T, typename O, bool VEC, bool LOG>
 __global__ __launch_bounds__(kSmBlock) void softmax_block_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                 int64_t n) {
+  using A = typename SmAcc<T>::type;
   constexpr int V = Vec<T>::N;
-  __shared__ MS smem[kSmBlock / kWave];
+  __shared__ MS<A> smem[kSmBlock / kWave];
   const T* row = x + (int64_t)blockIdx.x * n;
   O* out = y + (int64_t)blockIdx.x * n;
-  MS a{-INFINITY, 0.f};
+  MS<A> a{-INFINITY, A(0)};
   if constexpr (VEC) {
     for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kSmBlock * V) {
       const Vec<T> t = load_vec(row + c);
 #pragma unroll
-      for (int j = 0; j < V; ++j) ms_update(a, static_cast<float>(t.v[j]));
+      for (int j = 0; j < V; ++j) ms_update(a, static_cast<A>(t.v[j]));
     }
   } else {
-    for (int64_t c = threadIdx.x; c < n; c += kSmBlock) ms_update(a, static_cast<float>(row[c]));
+    for (int64_t c = threadIdx.x; c < n; c += kSmBlock) ms_update(a, static_cast<A>(row[c]));
   }
   a = ms_wave_reduce(a);
   if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = a;
@@ -107,37 +121,38 @@ __global__ __launch_bounds__(kSmBlock) void softmax_block_kernel(const T* __rest
   a = smem[0];
 #pragma unroll
   for (int w = 1; w < kSmBlock / kWave; ++w) a = ms_combine(a, smem[w]);
-  const float m = a.m, inv = 1.f / a.s, ls = __logf(a.s);
-  auto fin = [=](float v) { return LOG ? (v - m) - ls : __expf(v - m) * inv; };
+  const A m = a.m, inv = A(1) / a.s, ls = sm_log(a.s);
+  auto fin = [=](A v) { return LOG ? (v - m) - ls : sm_exp(v - m) * inv; };
   if constexpr (VEC) {
     for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kSmBlock * V) {
       const Vec<T> t = load_vec(row + c);
       VecN<O, V> r;
 #pragma unroll
-      for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(fin(static_cast<float>(t.v[j])));
+      for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(fin(static_cast<A>(t.v[j])));
       st<O, V>(out + c, r);
     }
   } else {
     for (int64_t c = threadIdx.x; c < n; c += kSmBlock)
-      out[c] = static_cast<O>(fin(static_cast<float>(row[c])));
+      out[c] = static_cast<O>(fin(static_cast<A>(row[c])));
   }
 }
 
 template <typename T, typename O, bool LOG>
 __global__ __launch_bounds__(kSmBlock) void softmax_cols_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                int64_t outer, int64_t n, int64_t inner) {
+  using A = typename SmAcc<T>::type;
   const int64_t total = outer * inner;
   const int64_t stride = (int64_t)gridDim.x * kSmBlock;
   for (int64_t e = (int64_t)blockIdx.x * kSmBlock + threadIdx.x; e < total; e += stride) {
     const int64_t o = e / inner, c = e - o * inner;
     const T* p = x + o * n * inner + c;
     O* q = y + o * n * inner + c;
-    MS a{-INFINITY, 0.f};
-    for (int64_t r = 0; r < n; ++r) ms_update(a, static_cast<float>(p[r * inner]));
-    const float inv = 1.f / a.s, ls = __logf(a.s);
+    MS<A> a{-INFINITY, A(0)};
+    for (int64_t r = 0; r < n; ++r) ms_update(a, static_cast<A>(p[r * inner]));
+    const A inv = A(1) / a.s, ls = sm_log(a.s);
     for (int64_t r = 0; r < n; ++r) {
-      const float v = static_cast<float>(p[r * inner]);
-      q[r * inner] = static_cast<O>(LOG ? (v - a.m) - ls : __expf(v - a.m) * inv);
+      const A v = static_cast<A>(p[r * inner]);
+      q[r * inner] = static_cast<O>(LOG ? (v - a.m) - ls : sm_exp(v - a.m) * inv);
     }
   }
 }
@@ -154,6 +169,7 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
   }
   const bool vec = n % V == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(y) % (sizeof(O) * V)) == 0;
   bool done = false;
+  if constexpr (!std::is_same<T, double>::value)  // f64 rows take the block kernel (double accumulation)
   if (outer < (int64_t(1) << 31)) {
     done = dispatch_row_tile<T>(n, vec, [&](auto nv, auto w, auto v) {
       constexpr int NV = decltype(nv)::value, W = decltype(w)::value;
@@ -191,6 +207,7 @@ extern "C" int mi355_softmax(const void* x, int in_dtype, void* y, int out_dtype
       case MI355_F32: return run_softmax_any<float, float>(log_softmax, x, y, outer, dim, inner, st);
       case MI355_F16: return run_softmax_any<f16_t, f16_t>(log_softmax, x, y, outer, dim, inner, st);
       case MI355_BF16: return run_softmax_any<bf16_t, bf16_t>(log_softmax, x, y, outer, dim, inner, st);
+      case MI355_F64: return run_softmax_any<double, double>(log_softmax, x, y, outer, dim, inner, st);
       default: break;
     }
   } else if (out_dtype == MI355_F32) {  // half_to_float

@@ -172,8 +172,6 @@ def _softmax_impl(self, dim, half_to_float, log):
     out = torch.empty(self.shape, dtype=out_dtype, device=self.device)
     if self.numel() == 0:
         return out
-    if self.dtype == torch.float64:
-        raise NotImplementedError("mi355 backend: float64 softmax is not supported")
     x = dense(self)
     shape = x.shape if x.dim() else (1,)
     launch("mi355_softmax", x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(out_dtype),
@@ -197,7 +195,7 @@ def log_softmax(self, dim, half_to_float):
 def native_layer_norm(input, normalized_shape, weight, bias, eps):
     """aten.native_layer_norm.default -> (y, mean, rstd).
 
-    mean/rstd are fp32 for f16/bf16 inputs (the accumulation type, as ATen's GPU kernels
+    mean/rstd are fp32 for f16/bf16 inputs, fp64 for f64 (the accumulation type, as ATen's GPU kernels
     return them) and shaped input.shape[:-k] + [1]*k.
     """
     k = len(normalized_shape)
@@ -209,11 +207,11 @@ def native_layer_norm(input, normalized_shape, weight, bias, eps):
         if p is not None and list(p.shape) != list(normalized_shape):
             raise RuntimeError(f"Expected {name} to be of same shape as normalized_shape, but got {name} of shape "
                                f"{list(p.shape)} and normalized_shape = {list(normalized_shape)}")
-    if input.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+    if input.dtype not in (torch.float32, torch.float16, torch.bfloat16, torch.float64):
         raise NotImplementedError(f"mi355 backend: layer norm on {input.dtype} is not supported")
     lead = list(input.shape[: input.dim() - k])
     M, N = prod(lead), prod(normalized_shape)
-    stat_dtype = torch.float32
+    stat_dtype = torch.float64 if input.dtype == torch.float64 else torch.float32
     y = torch.empty(input.shape, dtype=input.dtype, device=input.device)
     mean = torch.empty(lead + [1] * k, dtype=stat_dtype, device=input.device)
     rstd = torch.empty(lead + [1] * k, dtype=stat_dtype, device=input.device)
@@ -228,7 +226,7 @@ def native_layer_norm(input, normalized_shape, weight, bias, eps):
                 raise RuntimeError("weight and bias must have the same dtype")
             w_dtype = p.dtype
     if w_dtype is not None and w_dtype != input.dtype:
-        if w_dtype != torch.float32:
+        if w_dtype != torch.float32 or input.dtype == torch.float64:
             weight = cast(weight, input.dtype) if weight is not None else None
             bias = cast(bias, input.dtype) if bias is not None else None
             w_dtype = input.dtype

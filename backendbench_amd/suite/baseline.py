@@ -328,6 +328,13 @@ def edge_cases() -> List[Case]:
     add(aten._log_softmax.default, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), -1, False), {}), tag="empty")
     add(aten._log_softmax.default, lambda d: (_to(d, normal((37, 129), bf16, 0, 2, seed=1), -1, True), {}), tag="half_to_float")
 
+    f64 = torch.float64
+    add(aten._softmax.default, lambda d: (_to(d, normal((37, 129), f64, 0, 2, seed=1), -1, False), {}), tag="last_f64")
+    add(aten._softmax.default, lambda d: (_to(d, normal((5, 30, 7), f64, seed=1), 1, False), {}), tag="mid_f64")
+    add(aten._log_softmax.default, lambda d: (_to(d, normal((3, 5000), f64, 0, 2, seed=1), -1, False), {}), tag="long_rows_f64")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((33, 300), f64, 3, 2, seed=1), [300], normal((300,), f64, 1, 0.1, seed=2), normal((300,), f64, 0, 0.1, seed=3), 1e-5), {}), tag="f64")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((4, 6, 10), f64, seed=1), [6, 10], None, None, 1e-5), {}), tag="f64_no_affine_2d")
+
     # ---- native_layer_norm
     for dt in (f32, f16, bf16):
         t = f"{dt}".split(".")[-1]

@@ -197,14 +197,14 @@ def _argmax(d):
 
 
 def _softmax(d):
-    dt = d.dtype(ints=False, f64=False)
+    dt = d.dtype(ints=False)
     x = d.tensor(d.shape(), dt, 2.0, special=d.r.random() < 0.3)
     dim = d.r.randrange(-x.dim(), x.dim()) if x.dim() else d.r.choice([0, -1])
-    return [x, dim, dt != torch.float32 and d.r.random() < 0.3], {}
+    return [x, dim, dt in (torch.float16, torch.bfloat16) and d.r.random() < 0.3], {}
 
 
 def _layer_norm(d):
-    dt = d.dtype(ints=False, f64=False)
+    dt = d.dtype(ints=False)
     shape = d.shape(min_rank=1)
     if shape[-1] == 0:
         shape[-1] = 7
