@@ -6,7 +6,8 @@ fails with it.
 """
 
 import ctypes
-from ctypes import POINTER, c_char_p, c_double, c_int, c_int32, c_int64, c_void_p
+import struct
+from ctypes import c_char_p, c_double, c_int, c_int32, c_int64, c_void_p
 from pathlib import Path
 
 import torch
@@ -47,7 +48,12 @@ class TensorDesc(ctypes.Structure):
     ]
 
 
-_P = POINTER(TensorDesc)
+# `const mi355_tensor*` arguments are passed as the 144 packed bytes of the struct (built by
+# desc() with one struct.pack): several times cheaper per call than filling a ctypes Structure.
+_P = c_char_p
+_DESC = struct.Struct("=Qii8q8q")
+assert _DESC.size == ctypes.sizeof(TensorDesc)
+_PAD = (0,) * MAX_DIMS
 
 # name -> (restype, argtypes); mirrors include/mi355_aten.h one to one.
 SIGNATURES = {
@@ -119,25 +125,32 @@ def dtype_code(dtype):
 
 
 def desc(t, sizes=None, strides=None):
-    """mi355_tensor for `t`, optionally viewed with other sizes/strides (elements)."""
+    """Packed `struct mi355_tensor` for `t`, optionally viewed with other sizes/strides (elements)."""
     if sizes is None:
         sizes = t.shape
         strides = t.stride()
     nd = len(sizes)
     if nd > MAX_DIMS:
         raise NotImplementedError(f"mi355 backend: {nd}-d tensors exceed the {MAX_DIMS}-d limit")
-    d = TensorDesc()
-    d.data = t.data_ptr()
-    d.dtype = dtype_code(t.dtype)
-    d.ndim = nd
-    for i in range(nd):
-        d.sizes[i] = sizes[i]
-        d.strides[i] = strides[i]
-    return d
+    try:
+        code = DTYPE[t.dtype]
+    except KeyError:
+        raise NotImplementedError(f"mi355 backend: dtype {t.dtype} is not supported") from None
+    pad = _PAD[nd:]
+    return _DESC.pack(t.data_ptr(), code, nd, *sizes, *pad, *strides, *pad)
+
+
+try:  # raw hipStream_t of the current stream without building a torch.cuda.Stream object
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+    _cur_device = torch._C._cuda_getDevice
+except AttributeError:  # pragma: no cover - older/newer torch without these bindings
+    _raw_stream = _cur_device = None
 
 
 def current_stream_handle():
     """hipStream_t of torch's current stream, so callers' events bracket our kernels."""
+    if _raw_stream is not None:
+        return _raw_stream(_cur_device())
     return torch.cuda.current_stream().cuda_stream
 
 

@@ -6,7 +6,8 @@
 //   rows_block   inner == 1, long or few rows: one 256-thread block per (row, split),
 //                wave reduce then LDS combine across the four waves;
 //   rows_thread  inner == 1, red <= 32: one thread per row;
-//   cols         inner > 1: 64 lanes along inner (coalesced) x 4 along red, LDS combine;
+//   cols         inner > 1: 64 lanes along inner (coalesced, one 128-bit load each when inner
+//                allows) x 4 along red, LDS combine;
 //   final        second pass over per-split partial states when a launch was split
 //                to fill the chip (few rows, long reduction).
 #include "common.h"
@@ -217,10 +218,89 @@ __global__ __launch_bounds__(kRedBlock) void final_kernel(const typename R::Stat
   const int64_t stride = (int64_t)gridDim.x * kRedBlock;
   for (int64_t e = (int64_t)blockIdx.x * kRedBlock + threadIdx.x; e < total; e += stride) {
     const int64_t o = e / inner, c = e - o * inner;
-    typename R::State st = ws[(o * nsplit) * inner + c];
-    for (int64_t s = 1; s < nsplit; ++s) st = R::combine(st, ws[(o * nsplit + s) * inner + c]);
+    const typename R::State* p = ws + (o * nsplit) * inner + c;
+    typename R::State st = R::init();
+    int64_t s = 0;
+    for (; s + 8 <= nsplit; s += 8) {  // eight independent loads in flight, then combine in order
+      typename R::State part[8];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) part[k] = p[(s + k) * inner];
+#pragma unroll
+      for (int k = 0; k < 8; ++k) st = R::combine(st, part[k]);
+    }
+    for (; s < nsplit; ++s) st = R::combine(st, p[s * inner]);
     write_final<R, O, FIN>(out, e, st, divisor);
   }
+}
+
+// As cols_kernel with one 128-bit load per lane: lane tx owns V consecutive columns, so a wave
+// reads 1 KB of every row it visits, and four row loads are in flight per thread.
+// block = (64, 4); grid = (ceil(inner / (64 V)), nsplit, outer).  inner % V == 0, x 16-byte aligned.
+template <typename T, typename O, typename R, int FIN, bool PARTIAL>
+__global__ __launch_bounds__(kRedBlock) void cols_vec_kernel(const T* __restrict__ x, O* __restrict__ out,
+                                                            typename R::State* __restrict__ ws, int64_t red,
+                                                            int64_t inner, int64_t chunk, double divisor) {
+  using A = typename R::acc_t;
+  using State = typename R::State;
+  constexpr int V = Vec<T>::N;
+  __shared__ State smem[3][kWave][V];
+  const int tx = threadIdx.x, ty = threadIdx.y;
+  const int64_t col = ((int64_t)blockIdx.x * kWave + tx) * V;
+  const int64_t o = blockIdx.z;
+  const int64_t lo = (int64_t)blockIdx.y * chunk;
+  const int64_t hi = lo + chunk < red ? lo + chunk : red;
+  State st[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) st[j] = R::init();
+  if (col < inner) {
+    const T* p = x + o * red * inner + col;
+    int64_t r = lo + ty;
+    for (; r + 12 < hi; r += 16) {
+      const Vec<T> v0 = load_vec_nt(p + r * inner), v1 = load_vec_nt(p + (r + 4) * inner),
+                   v2 = load_vec_nt(p + (r + 8) * inner), v3 = load_vec_nt(p + (r + 12) * inner);
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        R::acc(st[j], (A)v0.v[j], r);
+        R::acc(st[j], (A)v1.v[j], r + 4);
+        R::acc(st[j], (A)v2.v[j], r + 8);
+        R::acc(st[j], (A)v3.v[j], r + 12);
+      }
+    }
+    for (; r < hi; r += 4) {
+      const Vec<T> v = load_vec_nt(p + r * inner);
+#pragma unroll
+      for (int j = 0; j < V; ++j) R::acc(st[j], (A)v.v[j], r);
+    }
+  }
+  if (ty > 0) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) smem[ty - 1][tx][j] = st[j];
+  }
+  __syncthreads();
+  if (ty == 0 && col < inner) {
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      for (int k = 0; k < 3; ++k) st[j] = R::combine(st[j], smem[k][tx][j]);
+      if constexpr (PARTIAL) ws[(o * gridDim.y + blockIdx.y) * inner + col + j] = st[j];
+      else write_final<R, O, FIN>(out, o * inner + col + j, st[j], divisor);
+    }
+  }
+}
+
+// Second pass for split rows (inner == 1): one wave per output, lanes stride over the row's
+// nsplit partial states, then a wave reduce.  (A single thread walking a thousand partials
+// one after the other costs several times the first pass.)
+template <typename O, typename R, int FIN>
+__global__ __launch_bounds__(kRedBlock) void final_rows_kernel(const typename R::State* __restrict__ ws,
+                                                              O* __restrict__ out, int64_t outer, int64_t nsplit,
+                                                              double divisor) {
+  const int lane = threadIdx.x % kWave;
+  const int64_t row = (int64_t)blockIdx.x * (kRedBlock / kWave) + threadIdx.x / kWave;
+  if (row >= outer) return;  // whole waves leave together
+  typename R::State st = R::init();
+  for (int64_t s = lane; s < nsplit; s += kWave) st = R::combine(st, ws[row * nsplit + s]);
+  st = wave_reduce(st, (R*)nullptr);
+  if (lane == 0) write_final<R, O, FIN>(out, row, st, divisor);
 }
 
 // ---------------------------------------------------------------- planning
@@ -253,10 +333,12 @@ static Plan plan_reduce(int64_t outer, int64_t red, int64_t inner, int elem_size
     return p;
   }
   p.kind = COLS;
-  const int64_t base = outer * ((inner + kWave - 1) / kWave);
-  if (base < 512) {
+  const int64_t per_block = inner % V == 0 ? (int64_t)kWave * V : kWave;  // columns per block (vector / scalar form)
+  const int64_t base = outer * ((inner + per_block - 1) / per_block);
+  if (base < want_blocks) {
     int64_t ns = (want_blocks + base - 1) / base;
-    const int64_t max_ns = red / 32 > 0 ? red / 32 : 1;
+    int64_t max_ns = red / 16 > 0 ? red / 16 : 1;  // >= 4 rows per thread per split
+    if (max_ns > 64) max_ns = 64;                    // keeps the second pass short
     if (ns > max_ns) ns = max_ns;
     if (ns > 1) {
       p.chunk = (red + ns - 1) / ns;
@@ -314,7 +396,8 @@ static int run_reduce(const void* xv, int64_t outer, int64_t red, int64_t inner,
       break;
     }
     case COLS: {
-      const int64_t xb = (inner + kWave - 1) / kWave;
+      const bool vec = V > 1 && inner % V == 0 && aligned16(x);
+      const int64_t xb = vec ? (inner + kWave * V - 1) / (kWave * V) : (inner + kWave - 1) / kWave;
       MI355_REQUIRE(xb < (int64_t(1) << 31) && p.nsplit < 65536, "mi355_reduce: inner extent too large");
       for (int64_t o0 = 0; o0 < outer; o0 += 65535) {
         const int64_t no = outer - o0 < 65535 ? outer - o0 : 65535;
@@ -322,8 +405,13 @@ static int run_reduce(const void* xv, int64_t outer, int64_t red, int64_t inner,
         const T* xo = x + o0 * red * inner;
         O* outo = out + o0 * inner;
         State* wso = ws ? ws + o0 * p.nsplit * inner : nullptr;
-        if (p.nsplit > 1) hipLaunchKernelGGL((cols_kernel<T, O, R, FIN, true>), grid, dim3(kWave, 4), 0, st, xo, outo, wso, red, inner, p.chunk, divisor);
-        else hipLaunchKernelGGL((cols_kernel<T, O, R, FIN, false>), grid, dim3(kWave, 4), 0, st, xo, outo, wso, red, inner, p.chunk, divisor);
+        if (vec) {
+          if (p.nsplit > 1) hipLaunchKernelGGL((cols_vec_kernel<T, O, R, FIN, true>), grid, dim3(kWave, 4), 0, st, xo, outo, wso, red, inner, p.chunk, divisor);
+          else hipLaunchKernelGGL((cols_vec_kernel<T, O, R, FIN, false>), grid, dim3(kWave, 4), 0, st, xo, outo, wso, red, inner, p.chunk, divisor);
+        } else {
+          if (p.nsplit > 1) hipLaunchKernelGGL((cols_kernel<T, O, R, FIN, true>), grid, dim3(kWave, 4), 0, st, xo, outo, wso, red, inner, p.chunk, divisor);
+          else hipLaunchKernelGGL((cols_kernel<T, O, R, FIN, false>), grid, dim3(kWave, 4), 0, st, xo, outo, wso, red, inner, p.chunk, divisor);
+        }
       }
       break;
     }
@@ -331,8 +419,13 @@ static int run_reduce(const void* xv, int64_t outer, int64_t red, int64_t inner,
   int rc = check_launch("mi355_reduce");
   if (rc) return rc;
   if (p.nsplit > 1) {
-    const int grid = grid_for(outer * inner, kRedBlock, kNumCU * 8);
-    hipLaunchKernelGGL((final_kernel<O, R, FIN>), dim3(grid), dim3(kRedBlock), 0, st, ws, out, outer, p.nsplit, inner, divisor);
+    if (inner == 1) {
+      const int grid = (int)((outer + kRedBlock / kWave - 1) / (kRedBlock / kWave));  // outer < 512 on this path
+      hipLaunchKernelGGL((final_rows_kernel<O, R, FIN>), dim3(grid), dim3(kRedBlock), 0, st, ws, out, outer, p.nsplit, divisor);
+    } else {
+      const int grid = grid_for(outer * inner, kRedBlock, kNumCU * 8);
+      hipLaunchKernelGGL((final_kernel<O, R, FIN>), dim3(grid), dim3(kRedBlock), 0, st, ws, out, outer, p.nsplit, inner, divisor);
+    }
     rc = check_launch("mi355_reduce(final)");
   }
   return rc;

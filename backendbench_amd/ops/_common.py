@@ -35,14 +35,15 @@ def device_managed(fn):
             if isinstance(a, torch.Tensor):
                 if first is None:
                     first = a
-                if a.device.type != "cuda":
+                if not a.is_cuda:
                     all_gpu = False
-        for a in kwargs.values():
-            if isinstance(a, torch.Tensor):
-                if first is None:
-                    first = a
-                if a.device.type != "cuda":
-                    all_gpu = False
+        if kwargs:
+            for a in kwargs.values():
+                if isinstance(a, torch.Tensor):
+                    if first is None:
+                        first = a
+                    if not a.is_cuda:
+                        all_gpu = False
         if all_gpu:
             return fn(*args, **kwargs)
         _lib.require_gpu()
@@ -68,12 +69,29 @@ def device_managed(fn):
     return wrapper
 
 
+_entry = {}
+
+
 def launch(name, *args):
     """Call one C entry point with the current stream appended; raise on failure."""
-    lib = _lib.load()
-    rc = getattr(lib, name)(*args, _lib.current_stream_handle())
+    fn = _entry.get(name)
+    if fn is None:
+        fn = _entry[name] = getattr(_lib.load(), name)
+    rc = fn(*args, _lib.current_stream_handle())
     if rc != 0:
         _lib.check(rc)
+
+
+def row_major_strides(shape):
+    strides = [1] * len(shape)
+    for i in range(len(shape) - 2, -1, -1):
+        strides[i] = strides[i + 1] * max(shape[i + 1], 1)
+    return strides
+
+
+def new_dense(shape, dtype, device):
+    """Uninitialised row-major tensor (empty_strided parses its arguments faster than empty)."""
+    return torch.empty_strided(shape, row_major_strides(shape), dtype=dtype, device=device)
 
 
 def copy_into(dst, src):
@@ -98,7 +116,7 @@ def dense(t):
     if t.is_contiguous():
         return t
     _lib.dtype_code(t.dtype)
-    return copy_into(torch.empty(t.shape, dtype=t.dtype, device=t.device), t)
+    return copy_into(new_dense(t.shape, t.dtype, t.device), t)
 
 
 def prod(xs):

@@ -10,7 +10,7 @@ import math
 import torch
 
 from .. import _lib
-from ._common import cast, copy_into, device_managed, launch
+from ._common import cast, copy_into, device_managed, launch, new_dense
 
 
 def _out_like_inputs(shape, dtype, inputs):
@@ -18,17 +18,48 @@ def _out_like_inputs(shape, dtype, inputs):
     ATen's TensorIterator does), row-major otherwise."""
     lead = None
     for t in inputs:
-        if tuple(t.shape) == tuple(shape):
+        if t.shape == shape:
             if lead is None:
                 lead = t
             elif t.stride() != lead.stride():
                 lead = None
                 break
-    if lead is not None and not lead.is_contiguous():
-        out = torch.empty_like(lead, dtype=dtype)  # preserve_format: dense permutations survive
-        if out.stride() == lead.stride():
+    if lead is not None:
+        out = torch.empty_like(lead) if lead.dtype == dtype else torch.empty_like(lead, dtype=dtype)
+        if lead.is_contiguous() or out.stride() == lead.stride():  # preserve_format: dense permutations survive
             return out
-    return torch.empty(shape, dtype=dtype, device=inputs[0].device)
+    return new_dense(shape, dtype, inputs[0].device)
+
+
+def _broadcast_shape(*shapes):
+    """torch.broadcast_shapes without its Python-side overhead (it costs more than a kernel launch)."""
+    n = 0
+    for s in shapes:
+        if len(s) > n:
+            n = len(s)
+    out = [1] * n
+    for s in shapes:
+        off = n - len(s)
+        for i, v in enumerate(s):
+            cur = out[off + i]
+            if cur == v or v == 1:
+                continue
+            if cur == 1:
+                out[off + i] = v
+            else:
+                raise RuntimeError(f"The size of tensor a ({cur}) must match the size of tensor b ({v}) at "
+                                   f"non-singleton dimension {off + i}")
+    return torch.Size(out)
+
+
+def _desc_as(t, shape):
+    """Descriptor of `t` broadcast to `shape` (stride 0 on the broadcast dims), without expand()."""
+    if t.shape == shape:
+        return _lib.desc(t)
+    off = len(shape) - t.dim()
+    strides = [0] * off + [0 if n == 1 and shape[off + i] != 1 else st
+                           for i, (n, st) in enumerate(zip(t.shape, t.stride()))]
+    return _lib.desc(t, shape, strides)
 
 
 def _alpha_args(dtype, alpha):
@@ -49,20 +80,19 @@ def _as_operand(self, other):
 
 def _binary(op, a, b, alpha=1):
     b = _as_operand(a, b)
-    dtype = torch.result_type(a, b)
+    dtype = a.dtype if a.dtype == b.dtype else torch.result_type(a, b)
     if dtype.is_complex:
         raise NotImplementedError(f"mi355 backend: binary ops on {dtype} are not supported")
     if dtype == torch.bool:  # or / and / or: compute in u8, any non-zero is True
         return cast(_binary(op, cast(a, torch.uint8), cast(b, torch.uint8), 1 if alpha else 0), torch.bool)
-    shape = torch.broadcast_shapes(a.shape, b.shape)
+    shape = a.shape if a.shape == b.shape else _broadcast_shape(a.shape, b.shape)
     a = cast(a, dtype)
     b = cast(b, dtype)
     out = _out_like_inputs(shape, dtype, (a, b))
     if out.numel() == 0:
         return out
     alpha_f, alpha_i = _alpha_args(dtype, alpha)
-    launch("mi355_binary", op, _lib.desc(a.expand(shape)), _lib.desc(b.expand(shape)), alpha_f, alpha_i,
-           _lib.desc(out))
+    launch("mi355_binary", op, _desc_as(a, shape), _desc_as(b, shape), alpha_f, alpha_i, _lib.desc(out))
     return out
 
 
@@ -71,20 +101,21 @@ def _binary_inplace(op, functional, self, other, **kw):
     not change self's shape, as for every ATen in-place overload.  `functional` is the
     out-of-place wrapper, used when the arithmetic dtype differs from self's or self is on the CPU."""
     other = _as_operand(self, other)
-    dtype = torch.result_type(self, other)
-    full = torch.broadcast_shapes(self.shape, other.shape)
-    if tuple(full) != tuple(self.shape):
+    dtype = self.dtype if self.dtype == other.dtype else torch.result_type(self, other)
+    full = self.shape if self.shape == other.shape else _broadcast_shape(self.shape, other.shape)
+    if full != self.shape:
         raise RuntimeError(f"output with shape {list(self.shape)} doesn't match the broadcast shape {list(full)}")
-    if not torch.can_cast(dtype, self.dtype):
+    if dtype != self.dtype and not torch.can_cast(dtype, self.dtype):
         raise RuntimeError(f"result type {str(dtype).replace('torch.', '').capitalize()} can't be cast to the "
                            f"desired output type {str(self.dtype).replace('torch.', '').capitalize()}")
-    if dtype != self.dtype or dtype == torch.bool or not _is_gpu_tensor(self):
+    if dtype != self.dtype or dtype == torch.bool or not self.is_cuda:
         return copy_into_any(self, functional(self, other, **kw))
     if self.numel() == 0:
         return self
     alpha_f, alpha_i = _alpha_args(dtype, kw.get("alpha", 1))
-    b = cast(other if _is_gpu_tensor(other) else other.to(self.device), dtype)
-    launch("mi355_binary", op, _lib.desc(self), _lib.desc(b.expand(self.shape)), alpha_f, alpha_i, _lib.desc(self))
+    b = cast(other if other.is_cuda else other.to(self.device), dtype)
+    mine = _lib.desc(self)
+    launch("mi355_binary", op, mine, _desc_as(b, self.shape), alpha_f, alpha_i, mine)
     return self
 
 
@@ -94,8 +125,9 @@ def _is_gpu_tensor(t):
 
 def copy_into_any(dst, src):
     """dst[...] = src across devices: our copy kernel on the GPU, torch's transfer otherwise."""
-    if _is_gpu_tensor(dst) and _is_gpu_tensor(src):
-        copy_into(dst, src.expand(dst.shape) if tuple(src.shape) != tuple(dst.shape) else src)
+    if dst.is_cuda and src.is_cuda:
+        if dst.numel():
+            launch("mi355_copy", _desc_as(src, dst.shape), _lib.desc(dst))
     else:
         dst.copy_(src)  # host <-> device transfer (only reached with CPU tensors)
     return dst
@@ -137,7 +169,7 @@ def minimum(self, other):
 
 def _unary(op, x, out_dtype, bounds=0, lo=None, hi=None, inplace=False):
     x = cast(x, out_dtype)
-    out = x if inplace else _out_like_inputs(x.shape, out_dtype, (x,))
+    out = x if inplace else torch.empty_like(x)  # preserve_format: dense permutations keep their layout
     if out.numel() == 0:
         return out
     if out_dtype.is_floating_point:
@@ -174,10 +206,16 @@ def relu_(self):
 
 
 def _clamp_dtype(self, bounds):
+    """Result dtype of clamp with Python-number bounds: a float bound lifts an integer tensor to
+    the default float dtype, anything else keeps self's dtype (result_type of a dimensioned
+    tensor with scalars)."""
     dtype = self.dtype
-    for bound in bounds:
-        if bound is not None:
-            dtype = torch.result_type(torch.empty((), dtype=dtype, device="meta").expand(1), bound)
+    if not dtype.is_floating_point:
+        for bound in bounds:
+            if isinstance(bound, float):
+                dtype = torch.get_default_dtype()
+            elif bound is not None and not isinstance(bound, (int, bool)):
+                dtype = torch.result_type(torch.empty((), dtype=dtype, device="meta").expand(1), bound)
     if dtype == torch.bool or dtype.is_complex:
         raise NotImplementedError(f"mi355 backend: clamp on {dtype} is not supported")
     return dtype
@@ -237,15 +275,17 @@ def where(condition, self, other):
     """aten.where.self: bit-exact select with broadcasting."""
     if condition.dtype not in (torch.bool, torch.uint8):
         raise RuntimeError(f"where expected condition to be a boolean tensor, but got a tensor with dtype {condition.dtype}")
-    dtype = torch.result_type(self, other)
-    shape = torch.broadcast_shapes(condition.shape, self.shape, other.shape)
+    dtype = self.dtype if self.dtype == other.dtype else torch.result_type(self, other)
+    if condition.shape == self.shape == other.shape:
+        shape = self.shape
+    else:
+        shape = _broadcast_shape(condition.shape, self.shape, other.shape)
     a = cast(self, dtype)
     b = cast(other, dtype)
     out = _out_like_inputs(shape, dtype, (condition, a, b))
     if out.numel() == 0:
         return out
-    launch("mi355_where", _lib.desc(condition.expand(shape)), _lib.desc(a.expand(shape)),
-           _lib.desc(b.expand(shape)), _lib.desc(out))
+    launch("mi355_where", _desc_as(condition, shape), _desc_as(a, shape), _desc_as(b, shape), _lib.desc(out))
     return out
 
 

@@ -3,7 +3,7 @@
 import torch
 
 from .. import _lib
-from ._common import cast, device_managed, launch
+from ._common import cast, device_managed, launch, new_dense
 
 _GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
 
@@ -20,7 +20,7 @@ def _gemm(a, b, c, alpha, beta):
         raise NotImplementedError(f"mi355 backend: matmul on {a.dtype} is not supported")
     M, K = a.shape
     N = b.shape[1]
-    out = torch.empty((M, N), dtype=a.dtype, device=a.device)
+    out = new_dense((M, N), a.dtype, a.device)
     if M == 0 or N == 0:
         return out
     if c is not None:

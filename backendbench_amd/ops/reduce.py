@@ -8,7 +8,7 @@ with the copy kernel.
 import torch
 
 from .. import _lib
-from ._common import cast, copy_into, dense, device_managed, launch, norm_dim, prod
+from ._common import cast, copy_into, dense, device_managed, launch, new_dense, norm_dim, prod
 
 _NATIVE_IN = (torch.float32, torch.float16, torch.bfloat16, torch.float64, torch.int32, torch.int64)
 _SMALL_INT = (torch.int16, torch.int8, torch.uint8, torch.bool)
@@ -39,7 +39,7 @@ def _view3(x, dims):
         return xd, prod(shape[: dims[0]]), prod(shape[dims[0] : dims[-1] + 1]), prod(shape[dims[-1] + 1 :])
     kept = [d for d in range(nd) if d not in dims]
     xp = x.permute(kept + dims)
-    xd = copy_into(torch.empty(xp.shape, dtype=x.dtype, device=x.device), xp)
+    xd = copy_into(new_dense(xp.shape, x.dtype, x.device), xp)
     return xd, prod(x.shape[d] for d in kept), prod(x.shape[d] for d in dims), 1
 
 
@@ -54,11 +54,11 @@ def _out_shape(x, dims, keepdim):
 def _run_reduce(op, x, dims, keepdim, out_dtype):
     """x: tensor of a natively reducible dtype with numel > 0 and red > 0."""
     xd, outer, red, inner = _view3(x, dims)
-    out = torch.empty(_out_shape(x, dims, keepdim), dtype=out_dtype, device=x.device)
+    out = new_dense(_out_shape(x, dims, keepdim), out_dtype, x.device)
     lib = _lib.load()
     in_code, out_code = _lib.dtype_code(xd.dtype), _lib.dtype_code(out_dtype)
     ws_bytes = lib.mi355_reduce_workspace_bytes(op, in_code, outer, red, inner)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    ws = new_dense((ws_bytes,), torch.uint8, x.device) if ws_bytes else None
     launch("mi355_reduce", op, xd.data_ptr(), in_code, outer, red, inner, out.data_ptr(), out_code,
            ws.data_ptr() if ws is not None else None, ws_bytes)
     return out
@@ -139,7 +139,7 @@ def amax(self, dim=(), keepdim=False):
         if self.dim() and self.shape[d] == 0:
             raise IndexError(f"amax(): Expected reduction dim {d} to have non-zero size.")
     if self.numel() == 0:
-        return torch.empty(shape, dtype=self.dtype, device=self.device)
+        return new_dense(shape, self.dtype, self.device)
     src = _max_src(self)
     return cast(_run_reduce(_lib.AMAX, src, dims, keepdim, src.dtype), self.dtype)
 
@@ -158,7 +158,7 @@ def argmax(self, dim=None, keepdim=False):
         raise IndexError(f"argmax(): Expected reduction dim {d} to have non-zero size.")
     dims = [d] if self.dim() else []
     if self.numel() == 0:
-        return torch.empty(_out_shape(self, dims, keepdim), dtype=torch.int64, device=self.device)
+        return new_dense(_out_shape(self, dims, keepdim), torch.int64, self.device)
     return _run_reduce(_lib.ARGMAX, _max_src(self), dims, keepdim, torch.int64)
 
 
@@ -169,7 +169,7 @@ def _softmax_impl(self, dim, half_to_float, log):
         raise RuntimeError("conversion is supported for Half and BFloat16 type only")
     out_dtype = torch.float32 if half_to_float else self.dtype
     d = norm_dim(dim, self.dim())
-    out = torch.empty(self.shape, dtype=out_dtype, device=self.device)
+    out = new_dense(self.shape, out_dtype, self.device)
     if self.numel() == 0:
         return out
     x = dense(self)
@@ -212,9 +212,9 @@ def native_layer_norm(input, normalized_shape, weight, bias, eps):
     lead = list(input.shape[: input.dim() - k])
     M, N = prod(lead), prod(normalized_shape)
     stat_dtype = torch.float64 if input.dtype == torch.float64 else torch.float32
-    y = torch.empty(input.shape, dtype=input.dtype, device=input.device)
-    mean = torch.empty(lead + [1] * k, dtype=stat_dtype, device=input.device)
-    rstd = torch.empty(lead + [1] * k, dtype=stat_dtype, device=input.device)
+    y = new_dense(input.shape, input.dtype, input.device)
+    mean = new_dense(lead + [1] * k, stat_dtype, input.device)
+    rstd = new_dense(lead + [1] * k, stat_dtype, input.device)
     if M == 0:
         return y, mean, rstd
     if N == 0:

@@ -441,3 +441,26 @@ def test_variant_overloads_through_the_live_dispatcher(backend):
     assert ("mi355_binary", _lib.MINIMUM) in calls and ("mi355_binary", _lib.MAXIMUM) in calls
     for a, b in zip(plain, ours):
         assert a.dtype == b.dtype and ev.allclose(a.cpu(), b.cpu())
+
+
+def test_trace_replay_scores_every_op_correct(backend):
+    """A text trace in the reference's TorchBench format (BackendBench/data_loaders.py:43-91,
+    suite/torchbench.py:39-105) with transformer-shaped inputs, replayed through
+    eval_one_op as the reference's `--suite torchbench` does: tensors are drawn on the GPU,
+    the reference value is the stock ATen kernel on the same tensors (eval.py:100), every
+    operator must score 1.0."""
+    from backendbench_amd.suite.trace import TraceTestSuite
+
+    suite = TraceTestSuite("trace", os.path.join(ROOT, "tests", "golden", "transformer_block_trace.txt"), topn=None)
+    seen = 0
+    for t in suite:
+        announce(f"trace {t.op.__name__}")
+        torch.manual_seed(seen)
+        c, p, cr, pr = ev.eval_one_op(t.op, backend[t.op], t.correctness_tests, t.performance_tests)
+        bad = [r for r in cr if not r.is_correct]
+        assert c == 1.0, f"{t.op.__name__}: {[(r.args, r.error_msg, r.max_abs_error) for r in bad]}"
+        assert all(r.successfully_ran for r in pr), [r.error_msg for r in pr if not r.successfully_ran]
+        print(f"[trace] {t.op.__name__:32s} speedup over the stock GPU kernel {p:6.2f}x  "
+              + " ".join(f"{r.speedup:.2f}" for r in pr), flush=True)
+        seen += 1
+    assert seen == 20

@@ -1,5 +1,7 @@
 """Suite containers and this operator set's own cases."""
 
+import re
+
 import torch
 
 from backendbench_amd.suite import BaselineTestSuite, SmokeTestSuite, edge_cases, perf_cases
@@ -94,3 +96,26 @@ def test_trace_suite(tmp_path):
     tests = list(ops[0].correctness_tests)
     assert len(tests) == 1 and tests[0].args[0].shape == (64, 8)      # largest input first, duplicates merged
     assert len(list(TraceTestSuite("t", str(p), filter=["sum"]))) == 1
+
+
+def test_committed_trace_fixture_parses():
+    """tests/golden/transformer_block_trace.txt: 20 operators, every line a valid argument string
+    whose operator resolves to one of the directory backend's slots."""
+    import os
+
+    from backendbench_amd.ops import SLOTS
+    from backendbench_amd.utils import deserialize_args, op_name_to_folder_name
+
+    path = os.path.join(os.path.dirname(__file__), "golden", "transformer_block_trace.txt")
+    suite = TraceTestSuite("trace", path)
+    ops = list(suite)
+    assert len(ops) == 20
+    n_inputs = 0
+    for t in ops:
+        assert op_name_to_folder_name(t.op.__name__) in SLOTS, t.op
+        for text in t.inputs:
+            small = re.sub(r"\d{3,}", "4", text)   # same structure, tiny extents: parse without the memory
+            args, kwargs = deserialize_args(small)
+            assert any(isinstance(a, torch.Tensor) for a in args)
+            n_inputs += 1
+    assert n_inputs == 44
