@@ -13,7 +13,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi355_aten.so"
-ABI_VERSION = 1
+ABI_VERSION = 2
 MAX_DIMS = 8
 
 # mi355_dtype
@@ -74,10 +74,11 @@ SIGNATURES = {
         [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
          c_double, c_void_p],
     ),
+    "mi355_gemm_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int]),
     "mi355_gemm": (
         c_int,
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
-         c_int64, c_int64, c_double, c_double, c_int, c_void_p],
+         c_int64, c_int64, c_double, c_double, c_int, c_void_p, c_int64, c_void_p],
     ),
     "mi355_index_select": (
         c_int,

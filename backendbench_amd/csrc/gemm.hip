@@ -14,6 +14,8 @@
 //              gemm_mfma_kernel      K tail: global -> registers -> LDS with zero fill.
 //   generic  any strides, bf16 / f16 / f32: 64x64 LDS tile, FMA inner loop.  Correctness
 //            path for shapes the MFMA kernel does not take.
+#include <type_traits>
+
 #include "common.h"
 
 namespace mi355 {
@@ -67,7 +69,60 @@ struct GemmArgs {
   float alpha, beta;
   int32_t tiles_m, tiles_n;
   int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
+  // Split-K (128x128 kernels only): blockIdx.y = split, which covers k in [split * ksplit,
+  // min(K, (split + 1) * ksplit)) and writes its raw fp32 tile to ws[split][M][N].
+  float* ws;
+  int32_t ksplit;
 };
+
+// fp32 partial tile of one split: register r of acc[i][j] in lane l is
+// C[m0 + 32 i + l%32][n0 + 32 j + 8 (r/4) + 4 (l/32) + r%4]; N % 4 == 0 on the MFMA paths.
+template <int MI>
+__device__ __forceinline__ void store_partial_tile(const GemmArgs& g, const f32x16 (&acc)[MI][2], int lane, int m0,
+                                                   int n0) {
+  const int fr = lane & 31, fg = lane >> 5;
+  float* W = g.ws + (int64_t)blockIdx.y * g.M * g.N;
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+    const int m = m0 + i * 32 + fr;
+    if (m >= g.M) continue;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + j * 32 + q * 8 + fg * 4;
+        if (n >= g.N) continue;
+        f32x4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = acc[i][j][q * 4 + e];
+        *reinterpret_cast<f32x4*>(W + (int64_t)m * g.N + n) = r;
+      }
+  }
+}
+
+// out = alpha * sum over splits of ws + beta * c, four consecutive n per thread.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_splitk_finish_kernel(GemmArgs g, int nsplit) {
+  const int64_t quads = (int64_t)g.M * g.N / 4;
+  const T* C = static_cast<const T*>(g.c);
+  const bool use_c = C != nullptr && g.beta != 0.f;
+  T* D = static_cast<T*>(g.out);
+  const int64_t plane = (int64_t)g.M * g.N;
+  for (int64_t qd = (int64_t)blockIdx.x * 256 + threadIdx.x; qd < quads; qd += (int64_t)gridDim.x * 256) {
+    const int64_t e0 = qd * 4;
+    f32x4 sum = *reinterpret_cast<const f32x4*>(g.ws + e0);
+    for (int sp = 1; sp < nsplit; ++sp) sum += *reinterpret_cast<const f32x4*>(g.ws + sp * plane + e0);
+    const int64_t m = e0 / g.N, n = e0 - m * g.N;
+    VecN4<T> r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = g.alpha * sum[e];
+      if (use_c) v += g.beta * static_cast<float>(C[m * g.c_rs + (n + e) * g.c_cs]);
+      r.v[e] = static_cast<T>(v);
+    }
+    *reinterpret_cast<VecN4<T>*>(D + e0) = r;
+  }
+}
 
 // Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous
 // band of tile ids, then walk the band in groups of 8 tile-rows so A and B panels repeat
@@ -102,7 +157,7 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
 }
 
 // ---------------------------------------------------------------- epilogue
-// A wave's 128x64 result: register r of acc[i][j] in lane l is C[m0 + 32 i + l%32][n0 + 32 j +
+// A wave's (32 MI)x64 result: register r of acc[i][j] in lane l is C[m0 + 32 i + l%32][n0 + 32 j +
 // 8 (r/4) + 4 (l/32) + r%4] (operands were swapped, so a lane owns runs of 4 consecutive n).
 // Writing those 8-byte runs straight to global memory leaves every 128-byte line to be
 // assembled from 16 stores in L2, and the epilogue then costs more than a tenth of the whole
@@ -110,16 +165,16 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
 // 16 KB slice of the (now idle) LDS ring, and reads it back row-major: every global store
 // instruction then writes 8 complete 128-byte rows.  Must be called by all waves after the
 // last barrier of the main loop (the ring is no longer read).
-template <typename T>
-__device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x16 (&acc)[4][2], unsigned char* lds,
+template <typename T, int MI>
+__device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x16 (&acc)[MI][2], unsigned char* lds,
                                                   int wave, int lane, int m0, int n0) {
   const int fr = lane & 31, fg = lane >> 5;
   const T* C = static_cast<const T*>(g.c);
   const bool use_c = C != nullptr && g.beta != 0.f;
-  unsigned char* slab = lds + wave * (128 * 128);  // 128 rows x 128 bytes
+  unsigned char* slab = lds + wave * (MI * 32 * 128);  // MI * 32 rows x 128 bytes
   // 16-byte slot s of row r lives at slot s ^ ((r/2) % 8): two-way conflicts at most on both sides
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < MI; ++i) {
     const int row = i * 32 + fr;
     const int m = m0 + row;
     const int mc = m < g.M ? m : g.M - 1;
@@ -155,8 +210,8 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
   // same wave wrote and reads: LDS operations of a wave complete in order
   T* D = static_cast<T*>(g.out);
 #pragma unroll
-  for (int t = 0; t < 16; ++t) {
-    const int chunk = t * kWave + lane;  // 1024 chunks of 16 bytes, 8 per row
+  for (int t = 0; t < MI * 4; ++t) {
+    const int chunk = t * kWave + lane;  // MI * 256 chunks of 16 bytes, 8 per row
     const int row = chunk >> 3, s = chunk & 7;
     const u32x4 v = *reinterpret_cast<const u32x4*>(slab + row * 128 + ((s ^ ((row >> 1) & 7)) << 4));
     const int m = m0 + row, n = n0 + s * 8;
@@ -301,7 +356,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
     __syncthreads();
   }
 
-  store_tile_result<T>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
+  store_tile_result<T, 4>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
 }
 
 // ---------------------------------------------------------------- MFMA kernel, direct-to-LDS fills
@@ -460,7 +515,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma_kernel(GemmArgs g) {
     if (!PF && it + 1 < nk) read_frags(it + 1, 0, fa0, fb0);
   }
 
-  store_tile_result<T>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
+  store_tile_result<T, 4>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
 }
 
 // ---------------------------------------------------------------- MFMA kernel, full-line A fills
@@ -634,7 +689,311 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
     cur = nxt;
   }
 
-  store_tile_result<T>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
+  store_tile_result<T, 4>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
+}
+
+// ---------------------------------------------------------------- MFMA kernel, 128x128 tiles
+// For problems that do not fill the chip with 256x256 tiles.  Four waves (2x2), each a 64x64
+// corner (2x2 MFMA blocks, 64 accumulators), 32-k steps, a ring of four 16 KB stages
+// (A 128x32 + B 32x128) filled by global_load_lds_dwordx4 three steps ahead exactly as in
+// gemm_mfma_dma_kernel; 64 KB of LDS, so two workgroups share a CU.  K % 32 == 0.
+constexpr int SBM = 128, SBN = 128;
+constexpr int kSPanel = SBM * BK3 * 2;            // 8 KB per operand per stage
+constexpr int kSStage = 2 * kSPanel;              // 16 KB
+constexpr int kSmallLds = kStages3 * kSStage;     // 64 KB
+// N-contiguous B panel of the 128-wide tile: 256 B per k row, 64-byte segments rotated by k % 4.
+__device__ __forceinline__ int swz_n128(int k, int u) {
+  return k * (SBN * 2) + ((((u >> 2) ^ (k & 3))) << 6) + ((u & 3) << 4);
+}
+
+template <typename T, bool B_NN, bool SPLIT>
+__global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
+  constexpr int S = kStages3;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  using frag_t = typename Mfma<T>::frag;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  const int bm = tm * SBM, bn = tn * SBN;
+  const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
+  const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
+  const T* A = static_cast<const T*>(g.a) + kbeg;
+  const T* B = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  // Region q = wave + 4 i (i < 2) of a panel is LDS bytes [q * 1024, q * 1024 + 1024).
+  const T* a_src[2];
+  const T* b_src[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = wave + 4 * i;
+    {  // K-contiguous A panel: region q = rows 16q .. 16q+15, 4 chunks per row
+      const int r = 16 * q + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gr = bm + r;
+      gr = gr < g.M ? gr : g.M - 1;
+      a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+    }
+    if constexpr (!B_NN) {
+      const int r = 16 * q + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gn = bn + r;
+      gn = gn < g.N ? gn : g.N - 1;
+      b_src[i] = B + (int64_t)gn * g.ldb + c * 8;
+    } else {  // N-contiguous B panel: region q = k rows 4q .. 4q+3, 16 units per row
+      const int k = 4 * q + (lane >> 4), pos = lane & 15;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gn = bn + u * 8;
+      gn = gn < g.N ? gn : 0;
+      b_src[i] = B + (int64_t)k * g.ldb + gn;
+    }
+  }
+  auto request_tile = [&](int t) {
+    const uint32_t stage = lds_base + (uint32_t)(t % S) * kSStage;
+    const int64_t k0 = (int64_t)t * BK3;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
+      lds_dma16(stage + region, a_src[i] + k0);
+      if constexpr (!B_NN) lds_dma16(stage + kSPanel + region, b_src[i] + k0);
+      else lds_dma16(stage + kSPanel + region, b_src[i] + k0 * g.ldb);
+    }
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  const int tr_k = fg * 8 + ((lane & 15) >> 2);
+  const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  auto read_frags = [&](int t, int ks, frag_t (&fa)[2], frag_t (&fb)[2]) {
+    const unsigned char* pa = lds + (t % S) * kSStage;
+    const unsigned char* pb = pa + kSPanel;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k32(wm * 64 + i * 32 + fr, ks * 2 + fg));
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if constexpr (!B_NN) {
+        fb[j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * 64 + j * 32 + fr, ks * 2 + fg));
+      } else {
+        const int k = ks * 16 + tr_k;
+        const int n = wn * 64 + j * 32 + tr_n;
+        const s16x4 lo = lds_read_tr(pb + swz_n128(k, n >> 3) + ((n & 7) << 1));
+        const s16x4 hi = lds_read_tr(pb + swz_n128(k + 4, n >> 3) + ((n & 7) << 1));
+        fb[j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto mma = [&](frag_t (&fa)[2], frag_t (&fb)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+  };
+
+  // At the wait point of step `it`, tile it+2 must have landed (its first fragments are read
+  // before the next barrier); only the newest tile's four loads may still be in flight.
+  const int nk = (kend - kbeg) / BK3;
+  for (int t = 0; t < S - 1 && t < nk; ++t) request_tile(t);
+  if (nk >= S - 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  frag_t fa0[2], fb0[2], fa1[2], fb1[2];
+  read_frags(0, 0, fa0, fb0);
+  int it = 0;
+  for (; it + S - 1 < nk; ++it) {
+    request_tile(it + S - 1);
+    read_frags(it, 1, fa1, fb1);
+    mma(fa0, fb0);
+    read_frags(it + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    __syncthreads();
+  }
+  for (; it < nk; ++it) {  // drain: nothing left to request
+    read_frags(it, 1, fa1, fb1);
+    mma(fa0, fb0);
+    if (it + 1 < nk) read_frags(it + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  if constexpr (SPLIT) store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
+  else store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
+}
+
+// ---------------------------------------------------------------- MFMA kernel, fp32
+// v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate; 157 TFLOP/s dense peak).  Same shape as the
+// 128x128 half-precision kernel in bytes: four waves (2x2) of 64x64, 16-k steps (64-byte rows),
+// a ring of four 16 KB stages (A 128x16 + B 16x128 fp32) filled by global_load_lds_dwordx4
+// three steps ahead.  A lane reads one 16-byte chunk (4 consecutive k) per operand block and
+// feeds MFMA e (e = 0..3) with its element e: the two k slots of that MFMA are then k = e of
+// the lower chunk (lanes 0-31) and of the upper chunk (lanes 32-63) — any pairing works as long
+// as both operands use the same one.  Row-major B has no transposing LDS read at 32 bits: a
+// lane gathers its four k with four ds_read_b32, rows of the panel offset by 128 bytes every
+// four k so that the two lane halves use different banks.  K % 16 == 0, N % 4 == 0.
+constexpr int FBK = 16;
+// [k][n] fp32 panel, 512 B per k row; 16-byte unit u of row k sits at u ^ (8 * ((k / 4) % 2)).
+__device__ __forceinline__ int swz_nf(int k, int n) {
+  return k * (SBN * 4) + (((n >> 2) ^ (((k >> 2) & 1) << 3)) << 4) + ((n & 3) << 2);
+}
+
+template <bool B_NN, bool SPLIT>
+__global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
+  constexpr int S = kStages3;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  const int bm = tm * SBM, bn = tn * SBN;
+  const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
+  const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
+  const float* A = static_cast<const float*>(g.a) + kbeg;
+  const float* B = static_cast<const float*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  const float* a_src[2];
+  const float* b_src[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = wave + 4 * i;
+    {  // K-contiguous panel: region q = rows 16q .. 16q+15, 4 chunks of 4 floats per row
+      const int r = 16 * q + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gr = bm + r;
+      gr = gr < g.M ? gr : g.M - 1;
+      a_src[i] = A + (int64_t)gr * g.lda + c * 4;
+    }
+    if constexpr (!B_NN) {
+      const int r = 16 * q + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gn = bn + r;
+      gn = gn < g.N ? gn : g.N - 1;
+      b_src[i] = B + (int64_t)gn * g.ldb + c * 4;
+    } else {  // N-contiguous panel: region q = k rows 2q, 2q+1, 32 units of 4 floats per row
+      const int k = 2 * q + (lane >> 5), pos = lane & 31;
+      const int u = pos ^ (((k >> 2) & 1) << 3);
+      int gn = bn + u * 4;
+      gn = gn < g.N ? gn : 0;
+      b_src[i] = B + (int64_t)k * g.ldb + gn;
+    }
+  }
+  auto request_tile = [&](int t) {
+    const uint32_t stage = lds_base + (uint32_t)(t % S) * kSStage;
+    const int64_t k0 = (int64_t)t * FBK;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
+      lds_dma16(stage + region, a_src[i] + k0);
+      if constexpr (!B_NN) lds_dma16(stage + kSPanel + region, b_src[i] + k0);
+      else lds_dma16(stage + kSPanel + region, b_src[i] + k0 * g.ldb);
+    }
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  // Operand blocks of 8-k sub-step ks (0, 1) of step t: 4 floats per lane and block.
+  auto read_frags = [&](int t, int ks, f32x4 (&fa)[2], f32x4 (&fb)[2]) {
+    const unsigned char* pa = lds + (t % S) * kSStage;
+    const unsigned char* pb = pa + kSPanel;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      fa[i] = *reinterpret_cast<const f32x4*>(pa + swz_k32(wm * 64 + i * 32 + fr, ks * 2 + fg));
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if constexpr (!B_NN) {
+        fb[j] = *reinterpret_cast<const f32x4*>(pb + swz_k32(wn * 64 + j * 32 + fr, ks * 2 + fg));
+      } else {
+        const int n = wn * 64 + j * 32 + fr;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          fb[j][e] = *reinterpret_cast<const float*>(pb + swz_nf(ks * 8 + fg * 4 + e, n));
+      }
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto mma = [&](f32x4 (&fa)[2], f32x4 (&fb)[2]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][e], fa[i][e], acc[i][j], 0, 0, 0);
+  };
+
+  const int nk = (kend - kbeg) / FBK;
+  for (int t = 0; t < S - 1 && t < nk; ++t) request_tile(t);
+  if (nk >= S - 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  f32x4 fa0[2], fb0[2], fa1[2], fb1[2];
+  read_frags(0, 0, fa0, fb0);
+  int it = 0;
+  for (; it + S - 1 < nk; ++it) {
+    request_tile(it + S - 1);
+    read_frags(it, 1, fa1, fb1);
+    mma(fa0, fb0);
+    read_frags(it + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    __syncthreads();
+  }
+  for (; it < nk; ++it) {
+    read_frags(it, 1, fa1, fb1);
+    mma(fa0, fb0);
+    if (it + 1 < nk) read_frags(it + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  if constexpr (SPLIT) {
+    store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
+    return;
+  }
+  // Register r of acc[i][j] in lane l is C[m0 + 32 i + l%32][n0 + 32 j + 8 (r/4) + 4 (l/32) + r%4]:
+  // four consecutive n per lane and r/4, stored as one 16-byte vector.
+  const float* C = static_cast<const float*>(g.c);
+  const bool use_c = C != nullptr && g.beta != 0.f;
+  float* D = static_cast<float*>(g.out);
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = bm + wm * 64 + i * 32 + fr;
+    if (m >= g.M) continue;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = bn + wn * 64 + j * 32 + q * 8 + fg * 4;
+        if (n >= g.N) continue;  // N % 4 == 0: a vector is all-in or all-out
+        f32x4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float v = g.alpha * acc[i][j][q * 4 + e];
+          if (use_c) v += g.beta * C[(int64_t)m * g.c_rs + (int64_t)(n + e) * g.c_cs];
+          r[e] = v;
+        }
+        *reinterpret_cast<f32x4*>(D + (int64_t)m * g.N + n) = r;
+      }
+  }
 }
 
 // ---------------------------------------------------------------- generic fallback
@@ -687,10 +1046,46 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
   }
 }
 
+// Split-K plan for problems with few 128x128 tiles and a long K: how many splits, and the k
+// extent of each (a multiple of the kernel's k step).  Splits are added until the launch has
+// about two workgroups per CU, each split keeps at least eight k steps, and the fp32 partials
+// (written and read once) stay below a small multiple of the bytes of A and B.
+struct SplitPlan {
+  int nsplit, ksplit;
+};
+static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
+  const int bk = elem_size == 4 ? FBK : BK3;
+  const int64_t tiles = ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN);
+  SplitPlan p{1, (int)K};
+  if (tiles >= kNumCU / 2 || K % bk != 0) return p;
+  int64_t ns = (2 * kNumCU + tiles - 1) / tiles;
+  const int64_t by_k = K / (8 * bk);
+  if (ns > by_k) ns = by_k;
+  if (ns > 64) ns = 64;
+  // fp32 MFMAs run at a sixteenth of the half-precision rate, so fp32 problems can afford more
+  // partial traffic per operand byte before the split stops paying.
+  const int64_t budget = (M * K + K * N) * elem_size * (elem_size == 4 ? 4 : 2);
+  while (ns > 1 && ns * M * N * 8 > budget) --ns;
+  if (ns <= 1) return p;
+  int64_t ks = (K + ns - 1) / ns;
+  ks = (ks + bk - 1) / bk * bk;
+  p.ksplit = (int)ks;
+  p.nsplit = (int)((K + ks - 1) / ks);
+  return p;
+}
+
+template <typename T>
+static int finish_splitk(const GemmArgs& g, int nsplit, hipStream_t st) {
+  const int64_t quads = (int64_t)g.M * g.N / 4;
+  const int grid = grid_for(quads, 256, kNumCU * 8);
+  hipLaunchKernelGGL((gemm_splitk_finish_kernel<T>), dim3(grid), dim3(256), 0, st, g, nsplit);
+  return check_launch("mi355_gemm(split-k finish)");
+}
+
 template <typename T>
 static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs,
                     const void* c, int64_t c_rs, int64_t c_cs, void* out, int64_t M, int64_t N, int64_t K,
-                    double alpha, double beta, hipStream_t st) {
+                    double alpha, double beta, void* workspace, int64_t workspace_bytes, hipStream_t st) {
   constexpr bool can_mfma = sizeof(T) == 2;
   if constexpr (can_mfma) {
     const bool a_ok = a_cs == 1 && a_rs % 8 == 0 && aligned16(a);
@@ -711,12 +1106,31 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       g.alpha = (float)alpha; g.beta = (float)beta;
       g.tiles_m = (int32_t)((M + BM - 1) / BM);
       g.tiles_n = (int32_t)((N + BN - 1) / BN);
-      const int64_t nblocks = (int64_t)g.tiles_m * g.tiles_n;
+      int64_t nblocks = (int64_t)g.tiles_m * g.tiles_n;
       MI355_REQUIRE(nblocks < (int64_t(1) << 31), "mi355_gemm: too many tiles");
       const bool ktail = K % BK3 != 0;
       const void* kern;
       int lds_bytes = kGemmLds;
-      if (ktail) {
+      int threads = 512;
+      int nsplit = 1;
+      // Fewer 256x256 tiles than three quarters of the CUs: 128x128 tiles, two workgroups per CU.
+      if (!ktail && nblocks < kNumCU * 3 / 4) {
+        g.tiles_m = (int32_t)((M + SBM - 1) / SBM);
+        g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
+        nblocks = (int64_t)g.tiles_m * g.tiles_n;
+        const SplitPlan sp = plan_splitk(M, N, K, sizeof(T));
+        if (sp.nsplit > 1 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 &&
+            reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+          nsplit = sp.nsplit;
+          g.ws = static_cast<float*>(workspace);
+          g.ksplit = sp.ksplit;
+          kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, true> : (const void*)gemm_mfma_small_kernel<T, true, true>;
+        } else {
+          kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, false> : (const void*)gemm_mfma_small_kernel<T, true, false>;
+        }
+        lds_bytes = kSmallLds;
+        threads = 256;
+      } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
       } else if (!b_nt && K % 64 == 0) {
         kern = (const void*)gemm_mfma_dma64_kernel<T>;
@@ -725,7 +1139,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
       }
       // More than 64 KB of dynamic LDS needs the attribute once per kernel and process.
-      static thread_local const void* attr_done[8] = {};
+      static thread_local const void* attr_done[12] = {};
       bool seen = false;
       for (const void* k : attr_done) seen = seen || k == kern;
       if (!seen) {
@@ -736,9 +1150,57 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
           if (k == nullptr) { k = kern; break; }
       }
       void* params[] = {&g};
-      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks), dim3(512), params, lds_bytes, st);
+      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks, (unsigned)nsplit), dim3(threads), params, lds_bytes, st);
       if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma): launch failed: %s", hipGetErrorString(e));
-      return check_launch("mi355_gemm(mfma)");
+      const int rc = check_launch("mi355_gemm(mfma)");
+      if (rc || nsplit == 1) return rc;
+      return finish_splitk<T>(g, nsplit, st);
+    }
+  }
+  if constexpr (std::is_same<T, float>::value) {
+    const bool a_ok = a_cs == 1 && a_rs % 4 == 0 && aligned16(a);
+    const bool b_nt = b_rs == 1 && b_cs % 4 == 0 && aligned16(b);
+    const bool b_nn = b_cs == 1 && b_rs % 4 == 0 && aligned16(b);
+    const bool fits = M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
+    if (a_ok && (b_nt || b_nn) && K % FBK == 0 && K > 0 && N % 4 == 0 && fits && M * N >= 64 * 64 && aligned16(out)) {
+      GemmArgs g{};
+      g.a = a; g.b = b; g.c = c; g.out = out;
+      g.lda = a_rs;
+      g.ldb = b_nt ? b_cs : b_rs;
+      g.c_rs = c_rs; g.c_cs = c_cs;
+      g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
+      g.alpha = (float)alpha; g.beta = (float)beta;
+      g.tiles_m = (int32_t)((M + SBM - 1) / SBM);
+      g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
+      const int64_t nblocks = (int64_t)g.tiles_m * g.tiles_n;
+      MI355_REQUIRE(nblocks < (int64_t(1) << 31), "mi355_gemm: too many tiles");
+      int nsplit = 1;
+      const SplitPlan sp = plan_splitk(M, N, K, 4);
+      if (sp.nsplit > 1 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 &&
+          reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+        nsplit = sp.nsplit;
+        g.ws = static_cast<float*>(workspace);
+        g.ksplit = sp.ksplit;
+      }
+      const void* kern;
+      if (nsplit > 1) kern = b_nt ? (const void*)gemm_mfma_f32_kernel<false, true> : (const void*)gemm_mfma_f32_kernel<true, true>;
+      else kern = b_nt ? (const void*)gemm_mfma_f32_kernel<false, false> : (const void*)gemm_mfma_f32_kernel<true, false>;
+      static thread_local const void* attr_done[4] = {};
+      bool seen = false;
+      for (const void* k : attr_done) seen = seen || k == kern;
+      if (!seen) {
+        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kSmallLds);
+        if (e != hipSuccess)
+          return set_error(MI355_ERR_LAUNCH, "mi355_gemm: cannot reserve %d bytes of LDS: %s", kSmallLds, hipGetErrorString(e));
+        for (const void*& k : attr_done)
+          if (k == nullptr) { k = kern; break; }
+      }
+      void* params[] = {&g};
+      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks, (unsigned)nsplit), dim3(256), params, kSmallLds, st);
+      if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma f32): launch failed: %s", hipGetErrorString(e));
+      const int rc = check_launch("mi355_gemm(mfma f32)");
+      if (rc || nsplit == 1) return rc;
+      return finish_splitk<float>(g, nsplit, st);
     }
   }
   const int64_t gx = (N + GT - 1) / GT, gy = (M + GT - 1) / GT;
@@ -753,18 +1215,27 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
 
 using namespace mi355;
 
+extern "C" int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype) {
+  const int es = dtype_size(dtype);
+  if (M <= 0 || N <= 0 || K <= 0 || (es != 2 && es != 4)) return 0;
+  if (dtype != MI355_BF16 && dtype != MI355_F16 && dtype != MI355_F32) return 0;
+  const SplitPlan p = plan_splitk(M, N, K, es);
+  return p.nsplit > 1 ? (int64_t)p.nsplit * M * N * 4 : 0;
+}
+
 extern "C" int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs,
                           const void* c, int64_t c_rs, int64_t c_cs, void* out, int64_t M, int64_t N, int64_t K,
-                          double alpha, double beta, int dtype, void* stream) {
+                          double alpha, double beta, int dtype, void* workspace, int64_t workspace_bytes,
+                          void* stream) {
   MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, "mi355_gemm: negative extent");
   if (M == 0 || N == 0) return MI355_OK;
   MI355_REQUIRE(out != nullptr, "mi355_gemm: NULL out");
   MI355_REQUIRE(K == 0 || (a != nullptr && b != nullptr), "mi355_gemm: NULL operand");
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (dtype) {
-    case MI355_BF16: return run_gemm<bf16_t>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, st);
-    case MI355_F16: return run_gemm<f16_t>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, st);
-    case MI355_F32: return run_gemm<float>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, st);
+    case MI355_BF16: return run_gemm<bf16_t>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
+    case MI355_F16: return run_gemm<f16_t>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
+    case MI355_F32: return run_gemm<float>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
     default: return set_error(MI355_ERR_UNSUPPORTED, "mi355_gemm: unsupported dtype %s", dtype_name(dtype));
   }
 }

@@ -1,4 +1,4 @@
-"""mm / addmm on the bf16/f16 MFMA kernel (fp32 accumulate) with a generic fallback."""
+"""mm / addmm on the bf16/f16/f32 MFMA kernels (fp32 accumulate) with a generic fallback."""
 
 import torch
 
@@ -6,6 +6,15 @@ from .. import _lib
 from ._common import cast, device_managed, launch, new_dense
 
 _GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+_SPLITK_MAX_OUT = 128 * 128 * 128  # the planner never splits problems with 128 or more 128x128 tiles
+_ws_fn = None
+
+
+def _workspace_bytes():
+    global _ws_fn
+    if _ws_fn is None:
+        _ws_fn = _lib.load().mi355_gemm_workspace_bytes
+    return _ws_fn
 
 
 def _gemm(a, b, c, alpha, beta):
@@ -30,8 +39,15 @@ def _gemm(a, b, c, alpha, beta):
         c_ptr, c_rs, c_cs = c.data_ptr(), c.stride(0), c.stride(1)
     else:
         c_ptr, c_rs, c_cs = None, 0, 0
+    code = _lib.dtype_code(a.dtype)
+    ws, ws_bytes = None, 0
+    if M * N < _SPLITK_MAX_OUT:  # only skinny / small outputs are ever split along K
+        ws_bytes = _workspace_bytes()(M, N, K, code)
+        if ws_bytes:
+            ws = new_dense((ws_bytes,), torch.uint8, a.device)
     launch("mi355_gemm", a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), c_ptr,
-           c_rs, c_cs, out.data_ptr(), M, N, K, float(alpha), float(beta), _lib.dtype_code(a.dtype))
+           c_rs, c_cs, out.data_ptr(), M, N, K, float(alpha), float(beta), code,
+           ws.data_ptr() if ws is not None else None, ws_bytes)
     return out
 
 

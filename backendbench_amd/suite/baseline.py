@@ -361,6 +361,17 @@ def edge_cases() -> List[Case]:
     for k in (32, 64, 96, 128, 192, 320, 448):   # every prologue / steady-state / drain length of the K loops
         add(aten.mm.default, lambda d, k=k: (_to(d, normal((260, k), bf16, seed=1), normal((k, 264), bf16, 0, 0.1, seed=2)), {}), tag=f"ksteps_{k}")
     add(aten.mm.default, lambda d: ([normal((512, 320), bf16, seed=1).to(d), normal((768, 320), bf16, 0, 0.05, seed=2).to(d).t()], {}), tag="b_transposed")
+    for k in (16, 32, 48, 64, 80, 272):   # fp32 MFMA path: every prologue / steady-state / drain length
+        add(aten.mm.default, lambda d, k=k: (_to(d, normal((132, k), f32, seed=1), normal((k, 140), f32, 0, 0.1, seed=2)), {}), tag=f"f32_ksteps_{k}")
+    add(aten.mm.default, lambda d: ([normal((300, 96), f32, seed=1).to(d), normal((260, 96), f32, 0, 0.1, seed=2).to(d).t()], {}), tag="f32_b_transposed")
+    add(aten.addmm.default, lambda d: ([normal((260,), f32, seed=3).to(d), normal((300, 96), f32, seed=1).to(d), normal((260, 96), f32, 0, 0.1, seed=2).to(d).t()], {"beta": 0.5, "alpha": 2.0}), tag="f32_linear")
+    add(aten.mm.default, lambda d: (_to(d, torch.eye(128, dtype=f32), normal((128, 128), f32, seed=2)), {}), exact=True, tag="f32_identity")
+    # skinny problems with a long K: split along K over the chip, fp32 partials, finishing pass
+    add(aten.mm.default, lambda d: (_to(d, normal((16, 2048), bf16, seed=1), normal((2048, 1024), bf16, 0, 0.05, seed=2)), {}), tag="splitk_bf16")
+    add(aten.mm.default, lambda d: (_to(d, normal((40, 2144), f16, seed=1), normal((2144, 520), f16, 0, 0.05, seed=2)), {}), tag="splitk_ragged_f16")
+    add(aten.addmm.default, lambda d: ([normal((1024,), bf16, seed=3).to(d), normal((24, 4096), bf16, seed=1).to(d), normal((1024, 4096), bf16, 0, 0.02, seed=2).to(d).t()], {"beta": 0.5, "alpha": 2.0}), tag="splitk_linear_bf16")
+    add(aten.addmm.default, lambda d: ([normal((200,), f32, seed=3).to(d), normal((64, 1024), f32, seed=1).to(d), normal((200, 1024), f32, 0, 0.05, seed=2).to(d).t()], {}), tag="splitk_linear_f32")
+    add(aten.mm.default, lambda d: (_to(d, normal((64, 1040), f32, seed=1), normal((1040, 256), f32, 0, 0.05, seed=2)), {}), tag="splitk_f32")
     add(aten.mm.default, lambda d: ([normal((320, 512), bf16, seed=1).to(d).t(), normal((320, 768), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_transposed")
     add(aten.mm.default, lambda d: (_to(d, torch.eye(256, dtype=bf16), normal((256, 256), bf16, seed=2)), {}), exact=True, tag="identity")
     add(aten.mm.default, lambda d: (_to(d, torch.empty(2, 0, dtype=f32), torch.empty(0, 3, dtype=f32)), {}), tag="k0")

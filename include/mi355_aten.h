@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define MI355_ABI_VERSION 1
+#define MI355_ABI_VERSION 2
 #define MI355_MAX_DIMS 8
 
 typedef enum mi355_dtype {
@@ -148,15 +148,22 @@ int mi355_layer_norm(const void* x, int dtype, const void* weight, const void* b
 
 /* ---- matrix multiply -------------------------------------------------------------- */
 
+/* Bytes of scratch mi355_gemm can use for a problem of this size and dtype (0 = none).  The
+ * scratch holds fp32 partial products when a problem with few output tiles and a long K is
+ * split along K over the chip; it only has to live until the kernels of that call have run. */
+int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype);
+
 /* out[M,N] = beta * c + alpha * (a[M,K] @ b[K,N]), fp32 accumulate, out dense row-major
- * in `dtype` (bf16 / f16 via MFMA; f32).  a, b, c carry explicit (row, col) element
+ * in `dtype` (bf16 / f16 / f32 via MFMA).  a, b, c carry explicit (row, col) element
  * strides so transposed operands and a broadcast bias (c_rs = 0, c_cs = 1) need no copy.
  * c may be NULL (then beta is ignored); beta == 0 never reads c.  K == 0 is accepted.
+ * workspace: device memory, 16-byte aligned, of at least mi355_gemm_workspace_bytes() bytes,
+ * or NULL / smaller — then the call is not split along K (same result, slower on skinny shapes).
  * Slots: mm__default (op_map.py:739), addmm__default (op_map.py:270). */
 int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs,
                int64_t b_cs, const void* c, int64_t c_rs, int64_t c_cs, void* out,
                int64_t M, int64_t N, int64_t K, double alpha, double beta, int dtype,
-               void* stream);
+               void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- indexing --------------------------------------------------------------------- */
 

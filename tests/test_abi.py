@@ -28,7 +28,7 @@ def header_enum(name):
 def test_header_declares_the_expected_entry_points():
     fns = declared_functions()
     assert "mi355_gemm" in fns and "mi355_softmax" in fns and "mi355_index_select" in fns
-    assert len(fns) == 13
+    assert len(fns) == 14
 
 
 def test_every_declared_symbol_is_exported_and_bound():
@@ -69,7 +69,7 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert rc == -1 and b"bad extents" in lib.mi355_last_error()
     with pytest.raises(RuntimeError, match="bad extents"):
         _lib.check(rc)
-    assert lib.mi355_gemm(None, 1, 1, None, 1, 1, None, 0, 0, None, 0, 8, 8, 1.0, 0.0, _lib.BF16, None) == 0
+    assert lib.mi355_gemm(None, 1, 1, None, 1, 1, None, 0, 0, None, 0, 8, 8, 1.0, 0.0, _lib.BF16, None, 0, None) == 0
 
 
 def test_reduce_workspace_plan():
