@@ -73,7 +73,64 @@ template <typename T, int NV, bool VEC, int W, int BLOCK = kRowBlock> struct Row
       }
     }
   }
+
+  // Shifted access (vector layout only) for rows that do not start on a 16-byte boundary: `a`
+  // (0 <= a < V) is how many elements past the previous boundary the row begins.  The lanes
+  // walk the aligned window that starts `a` elements before the row, so every load is a whole
+  // aligned 128-bit vector; elements outside [0, n) — the tail of the previous row, the head
+  // of the next one, or at most 15 bytes beyond either end of the tensor, inside 16-byte
+  // chunks that also hold tensor bytes — are replaced by `pad`.  The row fits when
+  // n + a <= NV * GROUP * V.
+  __device__ __forceinline__ void load_shifted(const T* row, int64_t n, int a, int t, float pad) {
+    static_assert(VEC, "shifted access uses the vector layout");
+    const T* win = row - a;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int64_t w = ((int64_t)k * GROUP + t) * V;
+      if (w < n + a) {
+        const VecN<T, V> x = ld_nt<T, V>(win + w);
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          const int64_t c = w + j - a;
+          v[k][j] = (c >= 0 && c < n) ? static_cast<float>(x.v[j]) : pad;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[k][j] = pad;
+      }
+    }
+  }
+
+  // Counterpart of load_shifted: whole vectors where all V elements belong to the row, single
+  // elements at the two ends (the neighbouring rows are written by other waves).
+  template <typename O, typename Fn>
+  __device__ __forceinline__ void store_shifted(O* row, int64_t n, int a, int t, Fn f) const {
+    O* win = row - a;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int64_t w = ((int64_t)k * GROUP + t) * V;
+      if (w >= n + a) continue;
+      if (w >= a && w + V <= n + a) {
+        VecN<O, V> x;
+#pragma unroll
+        for (int j = 0; j < V; ++j) x.v[j] = static_cast<O>(f(v[k][j], w + j - a));
+        st_nt<O, V>(win + w, x);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          const int64_t c = w + j - a;
+          if (c >= 0 && c < n) row[c] = static_cast<O>(f(v[k][j], c));
+        }
+      }
+    }
+  }
 };
+
+// Elements between the previous 16-byte-per-V-elements boundary and `p` (0 for aligned rows).
+template <typename T> __device__ __forceinline__ int row_misalignment(const T* p) {
+  constexpr int V = 16 / sizeof(T);
+  return (int)((reinterpret_cast<uintptr_t>(p) / sizeof(T)) % V);
+}
 
 // All-reduce over the W waves of a row group.  `smem` has one slot per wave of the block and
 // must not be reused by the caller before the next __syncthreads().  Every thread of the
@@ -96,9 +153,10 @@ __device__ __forceinline__ T group_allreduce(T v, Op op, T* smem) {
 }
 
 // Picks (NV, W) for rows of n elements of T and calls body(NV, W, VEC) with integral
-// constants; false when the row does not fit 16 slabs over 4 waves.  Aligned rows get at most
+// constants; false when the row does not fit (16 slabs over 4 waves, or 64 values per lane over
+// max_w waves).  Aligned rows get at most
 // 32 values per lane (W grows instead); unaligned rows use one wave and the scalar layout.
-template <typename T, typename Body> inline bool dispatch_row_tile(int64_t n, bool vec, Body body) {
+template <typename T, typename Body> inline bool dispatch_row_tile(int64_t n, bool vec, Body body, int max_w = 4) {
   constexpr int V = 16 / sizeof(T);
   using std::integral_constant;
 #define MI355_ROW(NV_, W_, VEC_)                                                              \
@@ -126,6 +184,11 @@ template <typename T, typename Body> inline bool dispatch_row_tile(int64_t n, bo
   if (n <= 32 * kWave * 2) MI355_ROW(NV32, 2, true)
   const int64_t unit4 = V * kWave * 4;
   if (n <= NV32 * unit4) MI355_ROW(NV32, 4, true)
+  // Callers whose kernels take 512- and 1024-thread blocks (max_w 8 / 16) keep 32 values per
+  // lane up to 32 K elements and go to 64 per lane only beyond that.
+  if (max_w >= 8 && n <= 32 * kWave * 8) MI355_ROW(NV32, 8, true)
+  if (max_w >= 16 && n <= 32 * kWave * 16) MI355_ROW(NV32, 16, true)
+  if (max_w >= 16 && n <= 64 * kWave * 16) MI355_ROW(2 * NV32, 16, true)
   if (NV32 < 8 && n <= 8 * unit4) MI355_ROW(8, 4, true)
   if (n <= 16 * unit4) MI355_ROW(16, 4, true)
 #undef MI355_ROW

@@ -17,18 +17,28 @@ namespace mi355 {
 
 constexpr int kSmBlock = kRowBlock;
 
-template <typename T, typename O, int NV, bool VEC, int W, bool LOG>
-__global__ __launch_bounds__(kSmBlock) void softmax_tile_kernel(const T* __restrict__ x, O* __restrict__ y,
-                                                               int64_t rows, int64_t n) {
-  using Tile = RowTile<T, NV, VEC, W>;
+// SHIFT: rows are not 16-byte aligned (odd row length); see RowTile::load_shifted.
+constexpr int sm_tile_block(int w) { return w <= 4 ? kSmBlock : kWave * w; }  // rows over 8 / 16 waves: one row per block
+
+template <typename T, typename O, int NV, bool VEC, int W, bool LOG, bool SHIFT>
+__global__ __launch_bounds__(sm_tile_block(W)) void softmax_tile_kernel(const T* __restrict__ x, O* __restrict__ y,
+                                                                       int64_t rows, int64_t n) {
+  constexpr int BLOCK = sm_tile_block(W);
+  using Tile = RowTile<T, NV, VEC, W, BLOCK>;
   constexpr int V = Tile::V;
-  __shared__ float red_max[kSmBlock / kWave], red_sum[kSmBlock / kWave];
+  __shared__ float red_max[BLOCK / kWave], red_sum[BLOCK / kWave];
   const int t = threadIdx.x % Tile::GROUP;
   int64_t row = (int64_t)blockIdx.x * Tile::ROWS_PER_BLOCK + threadIdx.x / Tile::GROUP;
   const bool active = row < rows;  // inactive groups still walk through the barriers
   if (!active) row = rows - 1;
   Tile tile;
-  tile.load(x + row * n, n, t, -INFINITY);
+  int a = 0;
+  if constexpr (SHIFT) {
+    a = row_misalignment(x + row * n);
+    tile.load_shifted(x + row * n, n, a, t, -INFINITY);
+  } else {
+    tile.load(x + row * n, n, t, -INFINITY);
+  }
   float m = -INFINITY;
 #pragma unroll
   for (int k = 0; k < NV; ++k)
@@ -47,13 +57,11 @@ __global__ __launch_bounds__(kSmBlock) void softmax_tile_kernel(const T* __restr
     }
   // Padding lanes hold exp(-inf - m) = 0 unless m is -inf/NaN, where the row is NaN anyway.
   s = group_allreduce<W>(s, SumOp(), red_sum);
-  if constexpr (LOG) {
-    const float ls = __logf(s);
-    if (active) tile.store(y + row * n, n, t, [ls](float d, int64_t) { return d - ls; });
-  } else {
-    const float inv = 1.f / s;
-    if (active) tile.store(y + row * n, n, t, [inv](float e, int64_t) { return e * inv; });
-  }
+  if (!active) return;
+  const float ls = __logf(s), inv = 1.f / s;
+  auto fin = [ls, inv](float v, int64_t) { return LOG ? v - ls : v * inv; };
+  if constexpr (SHIFT) tile.store_shifted(y + row * n, n, a, t, fin);
+  else tile.store(y + row * n, n, t, fin);
 }
 
 // Online (max, sum) pair in the accumulation type A (float; double for f64 input); see the
@@ -97,42 +105,61 @@ template <typename A> __device__ __forceinline__ MS<A> ms_wave_reduce(MS<A> a) {
   return a;
 }
 
-template <typename T, typename O, bool VEC, bool LOG>
-__global__ __launch_bounds__(kSmBlock) void softmax_block_kernel(const T* __restrict__ x, O* __restrict__ y,
-                                                                int64_t n) {
+// MODE 0: scalar accesses; 1: rows 16-byte aligned, vector accesses; 2: vector accesses over the
+// aligned window around a misaligned row (as RowTile::load_shifted): interior vectors whole,
+// the two end vectors element by element.
+template <typename T, typename O, int MODE, bool LOG, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void softmax_block_kernel(const T* __restrict__ x, O* __restrict__ y,
+                                                             int64_t n) {
   using A = typename SmAcc<T>::type;
   constexpr int V = Vec<T>::N;
-  __shared__ MS<A> smem[kSmBlock / kWave];
+  __shared__ MS<A> smem[BLOCK / kWave];
   const T* row = x + (int64_t)blockIdx.x * n;
   O* out = y + (int64_t)blockIdx.x * n;
-  MS<A> a{-INFINITY, A(0)};
-  if constexpr (VEC) {
-    for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kSmBlock * V) {
-      const Vec<T> t = load_vec(row + c);
+  const int a = MODE == 2 ? row_misalignment(row) : 0;
+  const T* win = row - a;
+  O* owin = out - a;
+  const int64_t total = n + a;  // window extent in elements
+  MS<A> acc{-INFINITY, A(0)};
+  if constexpr (MODE != 0) {
+    for (int64_t w = (int64_t)threadIdx.x * V; w < total; w += (int64_t)BLOCK * V) {
+      const Vec<T> t = load_vec(win + w);
+      if (MODE == 1 || (w >= a && w + V <= total)) {
 #pragma unroll
-      for (int j = 0; j < V; ++j) ms_update(a, static_cast<A>(t.v[j]));
+        for (int j = 0; j < V; ++j) ms_update(acc, static_cast<A>(t.v[j]));
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          if (w + j >= a && w + j < total) ms_update(acc, static_cast<A>(t.v[j]));
+      }
     }
   } else {
-    for (int64_t c = threadIdx.x; c < n; c += kSmBlock) ms_update(a, static_cast<A>(row[c]));
+    for (int64_t c = threadIdx.x; c < n; c += BLOCK) ms_update(acc, static_cast<A>(row[c]));
   }
-  a = ms_wave_reduce(a);
-  if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = a;
+  acc = ms_wave_reduce(acc);
+  if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = acc;
   __syncthreads();
-  a = smem[0];
+  acc = smem[0];
 #pragma unroll
-  for (int w = 1; w < kSmBlock / kWave; ++w) a = ms_combine(a, smem[w]);
-  const A m = a.m, inv = A(1) / a.s, ls = sm_log(a.s);
+  for (int w = 1; w < BLOCK / kWave; ++w) acc = ms_combine(acc, smem[w]);
+  const A m = acc.m, inv = A(1) / acc.s, ls = sm_log(acc.s);
   auto fin = [=](A v) { return LOG ? (v - m) - ls : sm_exp(v - m) * inv; };
-  if constexpr (VEC) {
-    for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kSmBlock * V) {
-      const Vec<T> t = load_vec(row + c);
-      VecN<O, V> r;
+  if constexpr (MODE != 0) {
+    for (int64_t w = (int64_t)threadIdx.x * V; w < total; w += (int64_t)BLOCK * V) {
+      const Vec<T> t = load_vec(win + w);
+      if (MODE == 1 || (w >= a && w + V <= total)) {
+        VecN<O, V> r;
 #pragma unroll
-      for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(fin(static_cast<A>(t.v[j])));
-      st<O, V>(out + c, r);
+        for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(fin(static_cast<A>(t.v[j])));
+        st<O, V>(owin + w, r);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          if (w + j >= a && w + j < total) owin[w + j] = static_cast<O>(fin(static_cast<A>(t.v[j])));
+      }
     }
   } else {
-    for (int64_t c = threadIdx.x; c < n; c += kSmBlock)
+    for (int64_t c = threadIdx.x; c < n; c += BLOCK)
       out[c] = static_cast<O>(fin(static_cast<A>(row[c])));
   }
 }
@@ -168,21 +195,39 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
     return check_launch("mi355_softmax(cols)");
   }
   const bool vec = n % V == 0 && aligned16(x) && (reinterpret_cast<uintptr_t>(y) % (sizeof(O) * V)) == 0;
+  // Rows that start off a 16-byte boundary (odd n, offset views) still take the vector layout,
+  // shifted per row, when input and output rows are misaligned by the same number of elements.
+  const bool shift = !vec && V > 1 &&
+                     (reinterpret_cast<uintptr_t>(x) / sizeof(T)) % V == (reinterpret_cast<uintptr_t>(y) / sizeof(O)) % V;
   bool done = false;
   if constexpr (!std::is_same<T, double>::value)  // f64 rows take the block kernel (double accumulation)
   if (outer < (int64_t(1) << 31)) {
-    done = dispatch_row_tile<T>(n, vec, [&](auto nv, auto w, auto v) {
+    done = dispatch_row_tile<T>(shift ? n + V - 1 : n, vec || shift, [&](auto nv, auto w, auto v) {
       constexpr int NV = decltype(nv)::value, W = decltype(w)::value;
       constexpr bool VEC = decltype(v)::value;
-      constexpr int rpb = kSmBlock / (kWave * W);
+      constexpr int block = sm_tile_block(W);
+      constexpr int rpb = block / (kWave * W);
       const unsigned nblk = (unsigned)((outer + rpb - 1) / rpb);
-      hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, VEC, W, LOG>), dim3(nblk), dim3(kSmBlock), 0, st, x, y, outer, n);
-    });
+      if constexpr (VEC) {
+        if (shift) {
+          hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, true, W, LOG, true>), dim3(nblk), dim3(block), 0, st, x, y, outer, n);
+          return;
+        }
+      }
+      hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, VEC, W, LOG, false>), dim3(nblk), dim3(block), 0, st, x, y, outer, n);
+    }, 16);
   }
   if (!done) {
     MI355_REQUIRE(outer < (int64_t(1) << 31), "mi355_softmax: too many rows (%lld)", (long long)outer);
-    if (vec) hipLaunchKernelGGL((softmax_block_kernel<T, O, true, LOG>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
-    else hipLaunchKernelGGL((softmax_block_kernel<T, O, false, LOG>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
+    // Rows this long get a 1024-thread block each: more loads in flight per row.
+    const bool big = n >= 32768;
+#define MI355_SM_BLOCK(MODE_)                                                                                         \
+  if (big) hipLaunchKernelGGL((softmax_block_kernel<T, O, MODE_, LOG, 1024>), dim3((unsigned)outer), dim3(1024), 0, st, x, y, n); \
+  else hipLaunchKernelGGL((softmax_block_kernel<T, O, MODE_, LOG, kSmBlock>), dim3((unsigned)outer), dim3(kSmBlock), 0, st, x, y, n);
+    if (vec) { MI355_SM_BLOCK(1) }
+    else if (shift) { MI355_SM_BLOCK(2) }
+    else { MI355_SM_BLOCK(0) }
+#undef MI355_SM_BLOCK
   }
   return check_launch("mi355_softmax");
 }

@@ -328,6 +328,13 @@ def edge_cases() -> List[Case]:
     add(aten._log_softmax.default, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), -1, False), {}), tag="empty")
     add(aten._log_softmax.default, lambda d: (_to(d, normal((37, 129), bf16, 0, 2, seed=1), -1, True), {}), tag="half_to_float")
 
+    # odd row lengths: rows start off 16-byte boundaries (shifted vector access, all row tile widths)
+    add(aten._softmax.default, lambda d: (_to(d, normal((300, 2049), f16, 0, 2, seed=1), -1, False), {}), tag="odd_2049_f16")
+    add(aten._softmax.default, lambda d: (_to(d, normal((33, 1001), f32, 0, 2, seed=1), -1, False), {}), tag="odd_1001_f32")
+    add(aten._softmax.default, lambda d: (_to(d, normal((64, 197), f16, 0, 2, seed=1), -1, True), {}), tag="odd_197_half_to_float")
+    add(aten._softmax.default, lambda d: (_to(d, normal((9, 16385), bf16, 0, 2, seed=1), -1, False), {}), tag="odd_16385_bf16")
+    add(aten._log_softmax.default, lambda d: (_to(d, normal((5, 50257), f16, 0, 2, seed=1), -1, False), {}), tag="odd_50257_f16")
+    add(aten._log_softmax.default, lambda d: (_to(d, normal((3, 40001), f32, 0, 2, seed=1), -1, False), {}), tag="odd_40001_f32")
     f64 = torch.float64
     add(aten._softmax.default, lambda d: (_to(d, normal((37, 129), f64, 0, 2, seed=1), -1, False), {}), tag="last_f64")
     add(aten._softmax.default, lambda d: (_to(d, normal((5, 30, 7), f64, seed=1), 1, False), {}), tag="mid_f64")
