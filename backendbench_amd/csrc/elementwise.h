@@ -83,12 +83,26 @@ __device__ __forceinline__ VecN<typename F::out_t, V> ew_apply(const F& f, const
 constexpr int kEwBlock = 256;
 constexpr int kEwUnroll = 4;
 
+template <typename T, int V>
+__device__ __forceinline__ VecN<T, V> ld_or_splat(const T* p, bool splat) {
+  if (V == 1 || splat) {
+    VecN<T, V> r;
+    const T s = *p;
+#pragma unroll
+    for (int j = 0; j < V; ++j) r.v[j] = s;
+    return r;
+  }
+  return ld<T, V>(p);
+}
+
 // One block = one contiguous tile of kEwUnroll x 256 vectors per operand (16 KB each for
 // 128-bit vectors): all loads of the tile are issued before the first store, and the tile is a
 // single DRAM-friendly span — a grid-stride walk with the same number of loads in flight
 // measured 10-25 % slower on this chip.
-template <typename F>
-__global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_t n) {
+// SC: some inputs are single values broadcast over the whole output (bit t of scalar_mask): they
+// are read once per thread and never indexed.
+template <typename F, bool SC>
+__global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_t n, uint32_t scalar_mask) {
   using TO = typename F::out_t;
   using T0 = typename F::in0_t;
   using T1 = typename F::in1_t;
@@ -99,6 +113,15 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_
   const T1* b = static_cast<const T1*>(p.in[1]);
   const T2* c = static_cast<const T2*>(p.in[2]);
   TO* o = static_cast<TO*>(p.out);
+  const bool sa = SC && (scalar_mask & 1u), sb = SC && NIN > 1 && (scalar_mask & 2u), sc = SC && NIN > 2 && (scalar_mask & 4u);
+  VecN<T0, V> ka;
+  VecN<T1, V> kb;
+  VecN<T2, V> kc;
+  if constexpr (SC) {
+    if (sa) ka = ld_or_splat<T0, V>(a, true);
+    if constexpr (NIN > 1) if (sb) kb = ld_or_splat<T1, V>(b, true);
+    if constexpr (NIN > 2) if (sc) kc = ld_or_splat<T2, V>(c, true);
+  }
 
   const int64_t nvec = n / V;
   constexpr int64_t TILE = (int64_t)kEwBlock * kEwUnroll;
@@ -111,9 +134,9 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_
 #pragma unroll
       for (int u = 0; u < kEwUnroll; ++u) {
         const int64_t e = (i0 + u * kEwBlock) * V;
-        va[u] = ld_nt<T0, V>(a + e);
-        if constexpr (NIN > 1) vb[u] = ld_nt<T1, V>(b + e);
-        if constexpr (NIN > 2) vc[u] = ld_nt<T2, V>(c + e);
+        va[u] = sa ? ka : ld_nt<T0, V>(a + e);
+        if constexpr (NIN > 1) vb[u] = sb ? kb : ld_nt<T1, V>(b + e);
+        if constexpr (NIN > 2) vc[u] = sc ? kc : ld_nt<T2, V>(c + e);
       }
 #pragma unroll
       for (int u = 0; u < kEwUnroll; ++u) {
@@ -123,11 +146,11 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_
     } else {
       for (int64_t i = i0; i < nvec; i += kEwBlock) {
         const int64_t e = i * V;
-        VecN<T0, V> va = ld_nt<T0, V>(a + e);
+        VecN<T0, V> va = sa ? ka : ld_nt<T0, V>(a + e);
         VecN<T1, V> vb;
         VecN<T2, V> vc;
-        if constexpr (NIN > 1) vb = ld_nt<T1, V>(b + e);
-        if constexpr (NIN > 2) vc = ld_nt<T2, V>(c + e);
+        if constexpr (NIN > 1) vb = sb ? kb : ld_nt<T1, V>(b + e);
+        if constexpr (NIN > 2) vc = sc ? kc : ld_nt<T2, V>(c + e);
         st_nt<TO, V>(o + e, ew_apply<F, V>(f, va, vb, vc));
       }
     }
@@ -136,11 +159,11 @@ __global__ __launch_bounds__(kEwBlock) void ew_flat_kernel(F f, EwPtrs p, int64_
   if (blockIdx.x == 0) {
     const int64_t e = nvec * V + threadIdx.x;
     if (e < n) {
-      T1 sb{};
-      T2 sc{};
-      if constexpr (NIN > 1) sb = b[e];
-      if constexpr (NIN > 2) sc = c[e];
-      o[e] = f(a[e], sb, sc);
+      T1 tb{};
+      T2 tc{};
+      if constexpr (NIN > 1) tb = b[sb ? 0 : e];
+      if constexpr (NIN > 2) tc = c[sc ? 0 : e];
+      o[e] = f(a[sa ? 0 : e], tb, tc);
     }
   }
 }
@@ -189,17 +212,6 @@ template <int NT> struct StridedArgs {
   int64_t strides[NT][MI355_MAX_DIMS];  // element strides; [NT-1] is the output
 };
 
-template <typename T, int V>
-__device__ __forceinline__ VecN<T, V> ld_or_splat(const T* p, bool splat) {
-  if (V == 1 || splat) {
-    VecN<T, V> r;
-    const T s = *p;
-#pragma unroll
-    for (int j = 0; j < V; ++j) r.v[j] = s;
-    return r;
-  }
-  return ld<T, V>(p);
-}
 
 // One work item = V consecutive elements of the innermost dim (V == 1: one element).  A block
 // takes U * kEwBlock consecutive work items, U per thread: the U index splits and loads are all
@@ -290,18 +302,35 @@ int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_t
   p.out = out->data;
   const int max_blocks = kNumCU * 8;
 
-  if (same_dense_layout(ts, NT)) {
+  // Inputs that are one value broadcast over the whole output (0-d operands, expanded scalars)
+  // do not constrain the layout: the flat kernel reads them once.
+  uint32_t scalar_mask = 0;
+  const mi355_tensor* laid[NT];
+  int nlaid = 0;
+  for (int t = 0; t < NIN; ++t) {
+    bool scalar = n > 1;
+    for (int i = 0; i < ins[t]->ndim && scalar; ++i)
+      if (ins[t]->sizes[i] > 1 && ins[t]->strides[i] != 0) scalar = false;
+    if (scalar) scalar_mask |= 1u << t;
+    else laid[nlaid++] = ins[t];
+  }
+  laid[nlaid++] = out;
+  if (same_dense_layout(laid, nlaid)) {
     bool vec_ok = (reinterpret_cast<uintptr_t>(out->data) % (esz[3] * V)) == 0;
     for (int t = 0; t < NIN; ++t)
-      vec_ok = vec_ok && (reinterpret_cast<uintptr_t>(ins[t]->data) % (esz[t] * V)) == 0;
+      if (!(scalar_mask & (1u << t)))
+        vec_ok = vec_ok && (reinterpret_cast<uintptr_t>(ins[t]->data) % (esz[t] * V)) == 0;
     if (vec_ok) {
       const int grid = grid_for((n + V - 1) / V, kEwBlock * kEwUnroll, 1 << 30);
-      hipLaunchKernelGGL(ew_flat_kernel<F>, dim3(grid), dim3(kEwBlock), 0, stream, f, p, n);
-    } else {
+      if (scalar_mask) hipLaunchKernelGGL((ew_flat_kernel<F, true>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, n, scalar_mask);
+      else hipLaunchKernelGGL((ew_flat_kernel<F, false>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, n, 0u);
+      return check_launch(name);
+    }
+    if (!scalar_mask) {
       const int grid = grid_for(n, kEwBlock, max_blocks);
       hipLaunchKernelGGL(ew_flat_scalar_kernel<F>, dim3(grid), dim3(kEwBlock), 0, stream, f, p, n);
+      return check_launch(name);
     }
-    return check_launch(name);
   }
 
   // Output stride for broadcast-free iteration must be real (no stride-0 output dims).
