@@ -25,7 +25,7 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
                                                               int64_t rows, int64_t n, float eps) {
   using Tile = RowTile<T, NV, VEC, W, BLOCK>;
   constexpr int V = Tile::V;
-  constexpr bool STAGE = VEC && BLOCK > kLnBlock;
+  constexpr bool STAGE = VEC && BLOCK > kLnBlock && W <= 4;  // rows over 8 / 16 waves: one row per block, nothing to share
   extern __shared__ __attribute__((aligned(32))) unsigned char ln_smem[];
   __shared__ float red_a[BLOCK / kWave], red_b[BLOCK / kWave];
   const Wt* gs = w;
@@ -191,8 +191,13 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
   done = dispatch_row_tile<T>(N, vec, [&](auto nv, auto wv, auto v) {
     constexpr int NV = decltype(nv)::value, WG = decltype(wv)::value;
     constexpr bool VEC = decltype(v)::value;
+    if constexpr (WG >= 8) {  // rows of 8 K - 64 K elements: a 512- or 1024-thread block per row
+      constexpr int BLK = kWave * WG;
+      hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, VEC, WG, BLK>), dim3((unsigned)M), dim3(BLK), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+      return;
+    }
     constexpr int BIG = 1024;
-    constexpr int rpb_big = BIG / (kWave * WG), rpb = kLnBlock / (kWave * WG);
+    constexpr int rpb_big = WG >= 8 ? 1 : BIG / (kWave * WG), rpb = WG >= 8 ? 1 : kLnBlock / (kWave * WG);
     // Enough rows to fill the chip with 1024-thread blocks: share gamma/beta through LDS.
     if (VEC && has_params && param_bytes <= 48 * 1024 && M >= (int64_t)rpb_big * 2 * kNumCU) {
       const unsigned nblk = (unsigned)((M + rpb_big - 1) / rpb_big);
@@ -201,7 +206,7 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
       const unsigned nblk = (unsigned)((M + rpb - 1) / rpb);
       hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, VEC, WG, kLnBlock>), dim3(nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
     }
-  });
+  }, 16);
   if (!done) {
     if (vec) hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, true>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, (float)eps);
     else hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, false>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, (float)eps);

@@ -339,6 +339,10 @@ def edge_cases() -> List[Case]:
     add(aten._softmax.default, lambda d: (_to(d, normal((37, 129), f64, 0, 2, seed=1), -1, False), {}), tag="last_f64")
     add(aten._softmax.default, lambda d: (_to(d, normal((5, 30, 7), f64, seed=1), 1, False), {}), tag="mid_f64")
     add(aten._log_softmax.default, lambda d: (_to(d, normal((3, 5000), f64, 0, 2, seed=1), -1, False), {}), tag="long_rows_f64")
+    # long rows: 8- and 16-wave register tiles, then the two-pass block kernel
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((5, 12288), bf16, 1, 2, seed=1), [12288], normal((12288,), bf16, 1, 0.1, seed=2), normal((12288,), bf16, 0, 0.1, seed=3), 1e-5), {}), tag="row12288_bf16")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((3, 40000), f32, -2, 3, seed=1), [40000], normal((40000,), f32, 1, 0.1, seed=2), None, 1e-5), {}), tag="row40000_f32")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((2, 70000), f16, 0, 1, seed=1), [70000], None, normal((70000,), f16, 0, 0.1, seed=3), 1e-5), {}), tag="row70000_f16")
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((33, 300), f64, 3, 2, seed=1), [300], normal((300,), f64, 1, 0.1, seed=2), normal((300,), f64, 0, 0.1, seed=3), 1e-5), {}), tag="f64")
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((4, 6, 10), f64, seed=1), [6, 10], None, None, 1e-5), {}), tag="f64_no_affine_2d")
 
