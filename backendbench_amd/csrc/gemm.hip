@@ -519,7 +519,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma_kernel(GemmArgs g) {
 }
 
 // ---------------------------------------------------------------- MFMA kernel, full-line A fills
-// Row-major ("NN") B and K % 64 == 0.  As gemm_mfma_dma_kernel, except that the A panel is
+// K % 64 == 0, either B layout.  As gemm_mfma_dma_kernel, except that the A panel is
 // fetched 64 k (one whole 128-byte line per row) at a time: with 32-k steps every line of A is
 // requested twice, 64 bytes each, which halves the useful width of each L2 request and was
 // measured to hold the A stream to ~13.5 TB/s chip-wide against ~21.5 TB/s for whole lines.
@@ -544,7 +544,7 @@ __device__ __forceinline__ int swz_k64(int r, int c) {
   return r * 128 + ((c ^ (((r >> 1) & 1) | ((r >> 2) & 6))) << 4);
 }
 
-template <typename T>
+template <typename T, bool B_NN>
 __global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using frag_t = typename Mfma<T>::frag;
@@ -572,11 +572,19 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    const int k = 2 * (wave + 8 * i) + (lane >> 5), pos = lane & 31;
-    const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
-    int gn = bn + u * 8;
-    gn = gn < g.N ? gn : 0;
-    b_src[i] = B + (int64_t)k * g.ldb + gn;
+    if constexpr (B_NN) {
+      const int k = 2 * (wave + 8 * i) + (lane >> 5), pos = lane & 31;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gn = bn + u * 8;
+      gn = gn < g.N ? gn : 0;
+      b_src[i] = B + (int64_t)k * g.ldb + gn;
+    } else {  // K-contiguous B ([N][K]): 64-byte rows per step, as the A panel of gemm_mfma_dma_kernel
+      const int r = 16 * (wave + 8 * i) + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gn = bn + r;
+      gn = gn < g.N ? gn : g.N - 1;
+      b_src[i] = B + (int64_t)gn * g.ldb + c * 8;
+    }
   }
   // a_slot: byte offset of the A slot to fill; t: first of the two steps it will hold.
   auto request_a = [&](int t, uint32_t a_slot) {
@@ -588,7 +596,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
     const uint32_t stage = lds_base + kBRing64 + (uint32_t)(t & 3) * kPanel3;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
-      lds_dma16(stage + (uint32_t)(wave + 8 * i) * 1024u, b_src[i] + (int64_t)t * BK3 * g.ldb);
+      lds_dma16(stage + (uint32_t)(wave + 8 * i) * 1024u, b_src[i] + (B_NN ? (int64_t)t * BK3 * g.ldb : (int64_t)t * BK3));
   };
 
   const int fr = lane & 31, fg = lane >> 5;
@@ -603,11 +611,15 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
       fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 128 + i * 32 + fr, half * 4 + ks * 2 + fg));
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int k = ks * 16 + tr_k;
-      const int n = wn * 64 + j * 32 + tr_n;
-      const s16x4 lo = lds_read_tr(pb + swz_n(k, n >> 3) + ((n & 7) << 1));
-      const s16x4 hi = lds_read_tr(pb + swz_n(k + 4, n >> 3) + ((n & 7) << 1));
-      fb[j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      if constexpr (B_NN) {
+        const int k = ks * 16 + tr_k;
+        const int n = wn * 64 + j * 32 + tr_n;
+        const s16x4 lo = lds_read_tr(pb + swz_n(k, n >> 3) + ((n & 7) << 1));
+        const s16x4 hi = lds_read_tr(pb + swz_n(k + 4, n >> 3) + ((n & 7) << 1));
+        fb[j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      } else {
+        fb[j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * 64 + j * 32 + fr, ks * 2 + fg));
+      }
     }
   };
 
@@ -1132,8 +1144,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         threads = 256;
       } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
-      } else if (!b_nt && K % 64 == 0) {
-        kern = (const void*)gemm_mfma_dma64_kernel<T>;
+      } else if (K % 64 == 0) {
+        kern = b_nt ? (const void*)gemm_mfma_dma64_kernel<T, false> : (const void*)gemm_mfma_dma64_kernel<T, true>;
         lds_bytes = kGemmLds64;
       } else {
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
