@@ -55,14 +55,30 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
     for (int j = 0; j < V; ++j) s += tile.v[k][j];
   const float inv_n = 1.f / (float)n;
   const float mean = group_allreduce<W>(s, SumOp(), red_a) * inv_n;
+  // Centre the tile in place (the output needs v - mean again) and accumulate the second moment.
+  // In the vector layout a 128-bit slab is wholly inside or wholly outside the row, so the
+  // padding test is made once per slab, not per element.
   float q = 0.f;
 #pragma unroll
-  for (int k = 0; k < NV; ++k)
+  for (int k = 0; k < NV; ++k) {
+    if constexpr (VEC) {
+      if (Tile::col(k, 0, t) < n) {
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-      const float d = Tile::col(k, j, t) < n ? tile.v[k][j] - mean : 0.f;
-      q += d * d;
+        for (int j = 0; j < V; ++j) {
+          const float d = tile.v[k][j] - mean;
+          tile.v[k][j] = d;
+          q += d * d;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const float d = Tile::col(k, j, t) < n ? tile.v[k][j] - mean : 0.f;
+        tile.v[k][j] = d;
+        q += d * d;
+      }
     }
+  }
   const float var = group_allreduce<W>(q, SumOp(), red_b) * inv_n;
   const float rstd = rsqrtf(var + eps);
   if (!active) return;
@@ -72,27 +88,39 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
   }
   T* out = y + row * n;
   if constexpr (VEC) {
+    // The weight / bias null tests are made once, outside the unrolled loops: inside, the
+    // compiler turns them into a branch per element.
+    auto emit = [&](auto has_w, auto has_b) {
+      constexpr bool HW = decltype(has_w)::value, HB = decltype(has_b)::value;
 #pragma unroll
-    for (int k = 0; k < NV; ++k) {
-      const int64_t c = Tile::col(k, 0, t);
-      if (c < n) {
-        VecN<Wt, V> g, be;
-        if (w) g = ld<Wt, V>(gs + c);
-        if (b) be = ld<Wt, V>(bs + c);
-        VecN<T, V> r;
+      for (int k = 0; k < NV; ++k) {
+        const int64_t c = Tile::col(k, 0, t);
+        if (c < n) {
+          VecN<Wt, V> g, be;
+          if constexpr (HW) g = ld<Wt, V>(gs + c);
+          if constexpr (HB) be = ld<Wt, V>(bs + c);
+          VecN<T, V> r;
 #pragma unroll
-        for (int j = 0; j < V; ++j) {
-          float f = (tile.v[k][j] - mean) * rstd;
-          if (w) f *= static_cast<float>(g.v[j]);
-          if (b) f += static_cast<float>(be.v[j]);
-          r.v[j] = static_cast<T>(f);
+          for (int j = 0; j < V; ++j) {
+            float f = tile.v[k][j] * rstd;
+            if constexpr (HW && HB) f = f * static_cast<float>(g.v[j]) + static_cast<float>(be.v[j]);
+            else if constexpr (HW) f *= static_cast<float>(g.v[j]);
+            else if constexpr (HB) f += static_cast<float>(be.v[j]);
+            r.v[j] = static_cast<T>(f);
+          }
+          st_nt<T, V>(out + c, r);
         }
-        st_nt<T, V>(out + c, r);
       }
-    }
+    };
+    using std::true_type;
+    using std::false_type;
+    if (w && b) emit(true_type(), true_type());
+    else if (w) emit(true_type(), false_type());
+    else if (b) emit(false_type(), true_type());
+    else emit(false_type(), false_type());
   } else {
-    tile.store(out, n, t, [=](float v, int64_t c) {
-      float r = (v - mean) * rstd;
+    tile.store(out, n, t, [=](float d, int64_t c) {
+      float r = d * rstd;
       if (w) r *= static_cast<float>(w[c]);
       if (b) r += static_cast<float>(b[c]);
       return r;
