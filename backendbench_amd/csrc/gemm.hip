@@ -1016,23 +1016,24 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
                                                           const T* __restrict__ C, int64_t c_rs, int64_t c_cs,
                                                           T* __restrict__ D, int64_t M, int64_t N, int64_t K,
                                                           float alpha, float beta) {
-  __shared__ float As[GK][GT + 1], Bs[GK][GT + 1];
+  using Acc = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+  __shared__ Acc As[GK][GT + 1], Bs[GK][GT + 1];
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
   const int64_t bm = (int64_t)blockIdx.y * GT, bn = (int64_t)blockIdx.x * GT;
-  float acc[4][4] = {};
+  Acc acc[4][4] = {};
   for (int64_t k0 = 0; k0 < K; k0 += GK) {
     for (int e = threadIdx.x; e < GT * GK; e += 256) {
       const int r = e / GK, kk = e % GK;
       const int64_t m = bm + r, k = k0 + kk;
-      As[kk][r] = (m < M && k < K) ? static_cast<float>(A[m * a_rs + k * a_cs]) : 0.f;
+      As[kk][r] = (m < M && k < K) ? static_cast<Acc>(A[m * a_rs + k * a_cs]) : Acc(0);
       const int kk2 = e / GT, c = e % GT;
       const int64_t n = bn + c, k2 = k0 + kk2;
-      Bs[kk2][c] = (n < N && k2 < K) ? static_cast<float>(B[k2 * b_rs + n * b_cs]) : 0.f;
+      Bs[kk2][c] = (n < N && k2 < K) ? static_cast<Acc>(B[k2 * b_rs + n * b_cs]) : Acc(0);
     }
     __syncthreads();
 #pragma unroll
     for (int kk = 0; kk < GK; ++kk) {
-      float av[4], bv[4];
+      Acc av[4], bv[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
 #pragma unroll
@@ -1051,8 +1052,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
     for (int j = 0; j < 4; ++j) {
       const int64_t n = bn + tx * 4 + j;
       if (n >= N) continue;
-      float v = alpha * acc[i][j];
-      if (use_c) v += beta * static_cast<float>(C[m * c_rs + n * c_cs]);
+      Acc v = (Acc)alpha * acc[i][j];
+      if (use_c) v += (Acc)beta * static_cast<Acc>(C[m * c_rs + n * c_cs]);
       D[m * N + n] = static_cast<T>(v);
     }
   }
@@ -1248,6 +1249,7 @@ extern "C" int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void*
     case MI355_BF16: return run_gemm<bf16_t>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
     case MI355_F16: return run_gemm<f16_t>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
     case MI355_F32: return run_gemm<float>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
+    case MI355_F64: return run_gemm<double>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
     default: return set_error(MI355_ERR_UNSUPPORTED, "mi355_gemm: unsupported dtype %s", dtype_name(dtype));
   }
 }

@@ -219,7 +219,7 @@ def _layer_norm(d):
 
 
 def _mm(d):
-    dt = d.r.choice([torch.bfloat16, torch.float16, torch.float32, torch.bfloat16])
+    dt = d.r.choice([torch.bfloat16, torch.float16, torch.float32, torch.bfloat16, torch.float64])
     m, k, n = (d.r.choice([0, 1, 3, 8, 33, 64, 130, 264, 300]) for _ in range(3))
     if d.r.random() < 0.4:   # MFMA-path shapes: multiples of 8, larger
         m, k, n = d.r.choice([128, 256, 264, 520]), d.r.choice([32, 64, 96, 128, 200, 320]), d.r.choice([128, 136, 256, 512])
