@@ -79,3 +79,22 @@ def test_reduce_workspace_plan():
     ws = lib.mi355_reduce_workspace_bytes(_lib.SUM, _lib.F32, 1, 1 << 24, 1)              # one long row: split
     assert ws > 0 and ws % 4 == 0
     assert lib.mi355_reduce_workspace_bytes(_lib.ARGMAX, _lib.F32, 1, 1 << 24, 1) == ws * 4
+
+
+def test_workspace_planners_run_on_the_host():
+    """The two *_workspace_bytes entry points are pure host arithmetic: callable without a GPU,
+    zero for shapes that are never split, and sized as splits x outputs x state otherwise."""
+    lib = _lib.load()
+    # reductions: many short rows need no scratch; one long row is split and needs 4-byte states
+    assert lib.mi355_reduce_workspace_bytes(_lib.SUM, _lib.BF16, 8192, 4096, 1) == 0
+    one_row = lib.mi355_reduce_workspace_bytes(_lib.SUM, _lib.F32, 1, 1 << 24, 1)
+    assert one_row > 0 and one_row % 4 == 0 and one_row <= 4 * 4096
+    arg = lib.mi355_reduce_workspace_bytes(_lib.ARGMAX, _lib.F32, 1, 1 << 24, 1)
+    assert arg == 4 * one_row        # (value, int64 index) states are 16 bytes
+    assert lib.mi355_reduce_workspace_bytes(_lib.SUM, _lib.F32, 0, 16, 1) == 0
+    # GEMM: large outputs are never split along K; a skinny one is, in whole fp32 planes of M x N
+    assert lib.mi355_gemm_workspace_bytes(4096, 4096, 11008, _lib.BF16) == 0
+    skinny = lib.mi355_gemm_workspace_bytes(16, 4096, 4096, _lib.BF16)
+    assert skinny > 0 and skinny % (16 * 4096 * 4) == 0 and skinny // (16 * 4096 * 4) <= 64
+    assert lib.mi355_gemm_workspace_bytes(16, 4096, 4096, _lib.I32) == 0     # no integer GEMM
+    assert lib.mi355_gemm_workspace_bytes(16, 4096, 32, _lib.BF16) == 0      # K too short to split

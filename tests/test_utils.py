@@ -159,3 +159,55 @@ def test_our_entry_points_pass_the_stream_scan(repo_root):
     assert len(backend.compiled_kernels) == 43
     for impl in backend.compiled_kernels.values():
         assert not uses_cuda_stream(impl)
+
+
+def test_python_side_broadcasting_matches_torch():
+    """The wrappers broadcast shapes and strides themselves (torch.broadcast_shapes and expand()
+    cost more host time than a kernel launch): same results as torch on random shapes."""
+    import random
+
+    import torch
+
+    from backendbench_amd import _lib
+    from backendbench_amd.ops.elementwise import _broadcast_shape, _clamp_dtype, _desc_as
+
+    rng = random.Random(0)
+    for _ in range(300):
+        full = [rng.choice([1, 2, 3, 5]) for _ in range(rng.randint(0, 4))]
+        shapes = []
+        for _ in range(rng.randint(2, 3)):
+            s = [1 if rng.random() < 0.3 else v for v in full]
+            shapes.append(s[rng.randint(0, len(s)):] if rng.random() < 0.4 else s)
+        want = torch.broadcast_shapes(*shapes)
+        assert _broadcast_shape(*[torch.Size(s) for s in shapes]) == want
+        t = torch.empty(shapes[0])
+        ours = _lib.TensorDesc.from_buffer_copy(_desc_as(t, want))
+        ref = _lib.TensorDesc.from_buffer_copy(_lib.desc(t.expand(want)))
+        assert (ours.data, ours.dtype, ours.ndim, list(ours.sizes)) == (ref.data, ref.dtype, ref.ndim, list(ref.sizes))
+        for size, a, b in zip(ours.sizes, ours.strides, ref.strides):   # strides of size-1 dims never matter
+            assert size <= 1 or a == b
+    with pytest.raises(RuntimeError):
+        _broadcast_shape(torch.Size([2, 3]), torch.Size([4, 3]))
+    assert torch.broadcast_shapes((0, 3), (1, 3)) == _broadcast_shape(torch.Size([0, 3]), torch.Size([1, 3]))
+    for dt in (torch.float32, torch.bfloat16, torch.int32, torch.int64, torch.uint8):
+        for bounds in ((1, None), (None, 2.5), (0.5, 1), (1, 2)):
+            t = torch.zeros(3, dtype=dt)
+            assert _clamp_dtype(t, bounds) == torch.clamp(t, *bounds).dtype
+
+
+def test_packed_descriptor_layout():
+    import ctypes
+
+    import torch
+
+    from backendbench_amd import _lib
+
+    t = torch.empty(4, 6, 8)[:, ::2, 1:]
+    d = _lib.TensorDesc.from_buffer_copy(_lib.desc(t))
+    assert d.data == t.data_ptr() and d.dtype == _lib.F32 and d.ndim == 3
+    assert list(d.sizes)[:3] == [4, 3, 7] and list(d.strides)[:3] == [48, 16, 1]
+    assert list(d.sizes)[3:] == [0] * 5 and ctypes.sizeof(d) == len(_lib.desc(t))
+    with pytest.raises(NotImplementedError):
+        _lib.desc(torch.empty(2, dtype=torch.complex64))
+    with pytest.raises(NotImplementedError):
+        _lib.desc(torch.empty([1] * 9))
