@@ -5,8 +5,9 @@
 //          max and sum by wave all-reduce (+ one LDS exchange between waves), one HBM write;
 //   block  inner == 1, longer rows: 256 threads keep an online (max, sum) pair in one
 //          pass, combine through LDS, then re-read the row (L2) to normalise;
-//   cols   inner > 1: one thread per (outer, inner) column, coalesced along inner,
-//          online pass then normalise pass.
+//   cols   inner > 1: lanes along inner (128-bit accesses and the softmax axis split over 8
+//          row groups when inner allows, else one thread per column), online pass then
+//          normalise pass.
 // exp(x - max) carries the special values: a +inf or NaN in the row, or a row of -inf,
 // turns the whole row into NaN, as ATen does.
 #include <type_traits>
@@ -184,12 +185,71 @@ __global__ __launch_bounds__(kSmBlock) void softmax_cols_kernel(const T* __restr
   }
 }
 
+// inner > 1 with 128-bit accesses along inner: block = (64, R).  Lane tx owns V consecutive
+// columns, the R row groups split the softmax axis; their online (max, sum) pairs meet in LDS,
+// then every thread normalises the rows it read (second read from L2).  inner % V == 0 and
+// 16-byte aligned operands.  grid = (ceil(inner / (64 V)), outer).
+constexpr int kSmColsR = 8;
+template <typename T, typename O, bool LOG>
+__global__ __launch_bounds__(kWave * kSmColsR) void softmax_cols_vec_kernel(const T* __restrict__ x, O* __restrict__ y,
+                                                                          int64_t n, int64_t inner) {
+  using A = typename SmAcc<T>::type;
+  constexpr int V = Vec<T>::N, R = kSmColsR;
+  __shared__ MS<A> smem[R][V][kWave];
+  const int tx = threadIdx.x, ty = threadIdx.y;
+  const int64_t col = ((int64_t)blockIdx.x * kWave + tx) * V;
+  const bool live = col < inner;
+  const T* p = x + (int64_t)blockIdx.y * n * inner + col;
+  O* q = y + (int64_t)blockIdx.y * n * inner + col;
+  MS<A> acc[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) acc[j] = {-INFINITY, A(0)};
+  if (live) {
+    for (int64_t r = ty; r < n; r += R) {
+      const Vec<T> t = load_vec(p + r * inner);
+#pragma unroll
+      for (int j = 0; j < V; ++j) ms_update(acc[j], static_cast<A>(t.v[j]));
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < V; ++j) smem[ty][j][tx] = acc[j];
+  __syncthreads();
+  if (!live) return;
+  A m[V], inv[V], ls[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    MS<A> a = smem[0][j][tx];
+#pragma unroll
+    for (int k = 1; k < R; ++k) a = ms_combine(a, smem[k][j][tx]);
+    m[j] = a.m;
+    inv[j] = A(1) / a.s;
+    ls[j] = sm_log(a.s);
+  }
+  for (int64_t r = ty; r < n; r += R) {
+    const Vec<T> t = load_vec(p + r * inner);
+    VecN<O, V> o;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const A v = static_cast<A>(t.v[j]);
+      o.v[j] = static_cast<O>(LOG ? (v - m[j]) - ls[j] : sm_exp(v - m[j]) * inv[j]);
+    }
+    st<O, V>(q + r * inner, o);
+  }
+}
+
 template <typename T, typename O, bool LOG>
 static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64_t inner, hipStream_t st) {
   const T* x = static_cast<const T*>(xv);
   O* y = static_cast<O*>(yv);
   constexpr int V = Vec<T>::N;
   if (inner > 1) {
+    if (V > 1 && inner % V == 0 && n >= 4 * kSmColsR && aligned16(x) &&
+        reinterpret_cast<uintptr_t>(y) % (sizeof(O) * V) == 0 && outer < 65536) {
+      const int64_t xb = (inner + kWave * V - 1) / (kWave * V);
+      MI355_REQUIRE(xb < (int64_t(1) << 31), "mi355_softmax: inner extent too large");
+      hipLaunchKernelGGL((softmax_cols_vec_kernel<T, O, LOG>), dim3((unsigned)xb, (unsigned)outer), dim3(kWave, kSmColsR), 0, st, x, y, n, inner);
+      return check_launch("mi355_softmax(cols, vector)");
+    }
     const int grid = grid_for(outer * inner, kSmBlock, kNumCU * 16);
     hipLaunchKernelGGL((softmax_cols_kernel<T, O, LOG>), dim3(grid), dim3(kSmBlock), 0, st, x, y, outer, n, inner);
     return check_launch("mi355_softmax(cols)");

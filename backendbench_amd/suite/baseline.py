@@ -328,6 +328,11 @@ def edge_cases() -> List[Case]:
     add(aten._log_softmax.default, lambda d: (_to(d, torch.empty(0, 128, dtype=f16), -1, False), {}), tag="empty")
     add(aten._log_softmax.default, lambda d: (_to(d, normal((37, 129), bf16, 0, 2, seed=1), -1, True), {}), tag="half_to_float")
 
+    # softmax axis is not the last one, inner extent a multiple of the vector width
+    add(aten._softmax.default, lambda d: (_to(d, normal((4, 100, 64), f16, 0, 2, seed=1), 1, False), {}), tag="mid_vec_f16")
+    add(aten._softmax.default, lambda d: (_to(d, normal((3, 40, 8, 16), f32, 0, 2, seed=1), 1, False), {}), tag="mid_vec_f32")
+    add(aten._softmax.default, lambda d: (_to(d, normal((64, 256), bf16, 0, 2, seed=1), 0, True), {}), tag="dim0_half_to_float")
+    add(aten._log_softmax.default, lambda d: (_to(d, poison(normal((2, 33, 520), f16, 0, 2, seed=1), 0.01, 4), 1, False), {}), tag="mid_vec_naninf")
     # odd row lengths: rows start off 16-byte boundaries (shifted vector access, all row tile widths)
     add(aten._softmax.default, lambda d: (_to(d, normal((300, 2049), f16, 0, 2, seed=1), -1, False), {}), tag="odd_2049_f16")
     add(aten._softmax.default, lambda d: (_to(d, normal((33, 1001), f32, 0, 2, seed=1), -1, False), {}), tag="odd_1001_f32")
