@@ -1059,10 +1059,11 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
   }
 }
 
-// Split-K plan for problems with few 128x128 tiles and a long K: how many splits, and the k
-// extent of each (a multiple of the kernel's k step).  Splits are added until the launch has
-// about two workgroups per CU, each split keeps at least eight k steps, and the fp32 partials
-// (written and read once) stay below a small multiple of the bytes of A and B.
+// Split-K plan for problems with fewer 128x128 tiles than CUs and a long K: how many splits,
+// and the k extent of each (a multiple of the kernel's k step).  The split count minimises a
+// small cost model fitted to this chip: a 128x128 workgroup alone on a CU spends ~12.8 ns per k
+// (fp32: ~70 ns), two on a CU ~0.7 of that each, and a split adds a finishing launch (~3 us)
+// plus the fp32 partial planes written and read once at ~4 TB/s.  Each split keeps >= 8 k steps.
 struct SplitPlan {
   int nsplit, ksplit;
 };
@@ -1070,17 +1071,26 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   const int bk = elem_size == 4 ? FBK : BK3;
   const int64_t tiles = ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN);
   SplitPlan p{1, (int)K};
-  if (tiles >= kNumCU / 2 || K % bk != 0) return p;
-  int64_t ns = (2 * kNumCU + tiles - 1) / tiles;
-  const int64_t by_k = K / (8 * bk);
-  if (ns > by_k) ns = by_k;
-  if (ns > 64) ns = 64;
-  // fp32 MFMAs run at a sixteenth of the half-precision rate, so fp32 problems can afford more
-  // partial traffic per operand byte before the split stops paying.
-  const int64_t budget = (M * K + K * N) * elem_size * (elem_size == 4 ? 4 : 2);
-  while (ns > 1 && ns * M * N * 8 > budget) --ns;
-  if (ns <= 1) return p;
-  int64_t ks = (K + ns - 1) / ns;
+  if (tiles >= kNumCU || K % bk != 0) return p;
+  const double ns_per_k = elem_size == 4 ? 70.0 : 12.8;
+  const int64_t max_ns = K / (8 * bk) < 64 ? K / (8 * bk) : 64;
+  double best = 0;
+  int64_t best_ns = 1;
+  for (int64_t ns = 1; ns <= max_ns; ++ns) {
+    int64_t ks = (K + ns - 1) / ns;
+    ks = (ks + bk - 1) / bk * bk;
+    const int64_t real_ns = (K + ks - 1) / ks;
+    if (real_ns != ns) continue;  // this count rounds to one already tried
+    const int64_t per_cu = (tiles * ns + kNumCU - 1) / kNumCU;
+    double t = (double)per_cu * (per_cu >= 2 ? 0.7 : 1.0) * (double)ks * ns_per_k;
+    if (ns > 1) t += 3000.0 + (double)ns * (double)M * (double)N * 8.0 / 4000.0;  // ns; 4 TB/s = 4000 B/ns
+    if (ns == 1 || t < best) {
+      best = t;
+      best_ns = ns;
+    }
+  }
+  if (best_ns <= 1) return p;
+  int64_t ks = (K + best_ns - 1) / best_ns;
   ks = (ks + bk - 1) / bk * bk;
   p.ksplit = (int)ks;
   p.nsplit = (int)((K + ks - 1) / ks);

@@ -6,7 +6,7 @@ from .. import _lib
 from ._common import cast, device_managed, launch, new_dense
 
 _GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32, torch.float64)
-_SPLITK_MAX_OUT = 128 * 128 * 128  # the planner never splits problems with 128 or more 128x128 tiles
+_SPLITK_MAX_OUT = 128 * 128 * 256  # the planner never splits problems with 256 or more 128x128 tiles
 _ws_fn = None
 
 
