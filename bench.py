@@ -3,8 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Prints ONE JSON line.  A "step" is one pass of the headline row-op workload
-(BASELINE.json configs[1]): `_softmax`, `native_layer_norm`, `sum` and `amax` over the last
+Prints ONE JSON line.  A "step" is one pass of the headline row-op workload (the second of
+the five benchmark configurations): `_softmax`, `native_layer_norm`, `sum` and `amax` over the last
 dim of a bf16 [8192, 4096] tensor, each called once through the drop-in boundary
 (DirectoryBackend -> `<folder>_kernel_impl` -> ctypes -> libmi355_aten.so).  Inputs are
 resident in HBM before the clock starts; consecutive steps walk a pool of input copies larger
