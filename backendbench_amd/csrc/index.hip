@@ -148,14 +148,15 @@ __global__ __launch_bounds__(kIxBlock) void gather_kernel(const U* __restrict__ 
   }
 }
 
-// Gather along the last dim of a dense [rows, len] source with a dense [rows, n_idx] index:
+// Gather along the last dim of a dense [rows, len] source with a dense [rows, n_idx] index (or
+// one [n_idx] index shared by all rows: index_select along the last dim):
 // one block stages (its share of) the source row in LDS with coalesced 128-bit loads, then
 // resolves four indices per thread per step from LDS — the index stream and the output stay
 // fully coalesced and no random access leaves the CU.  grid = (splits, rows).
 template <typename U>
 __global__ __launch_bounds__(kIxBlock) void gather_rows_lds_kernel(const U* __restrict__ src, const int64_t* __restrict__ index,
                                                                   U* __restrict__ out, int64_t len, int64_t n_idx,
-                                                                  int64_t per_split, int32_t* err) {
+                                                                  int64_t idx_row_stride, int64_t per_split, int32_t* err) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   U* row = reinterpret_cast<U*>(smem_raw);
   const int64_t r = blockIdx.y;
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(kIxBlock) void gather_rows_lds_kernel(const U* __re
   __syncthreads();
   const int64_t j0 = (int64_t)blockIdx.x * per_split;
   const int64_t j1 = j0 + per_split < n_idx ? j0 + per_split : n_idx;
-  const int64_t* ix = index + r * n_idx;
+  const int64_t* ix = index + r * idx_row_stride;  // 0: every row uses the same indices (index_select)
   U* o = out + r * n_idx;
   const bool vec = n_idx % 4 == 0 && per_split % 4 == 0 && (reinterpret_cast<uintptr_t>(ix) & 15) == 0 &&
                    (reinterpret_cast<uintptr_t>(o) % (4 * sizeof(U))) == 0;
@@ -240,7 +241,7 @@ static int run_gather(const mi355_tensor* src, int dim, const mi355_tensor* inde
       splits = (n_idx + per_split - 1) / per_split;
       hipLaunchKernelGGL((gather_rows_lds_kernel<U>), dim3((unsigned)splits, (unsigned)rows), dim3(kIxBlock),
                          (size_t)(len * sizeof(U)), st, (const U*)src->data, (const int64_t*)index->data,
-                         (U*)out->data, len, n_idx, per_split, err);
+                         (U*)out->data, len, n_idx, n_idx, per_split, err);
       return check_launch("mi355_gather(lds)");
     }
   }
@@ -273,6 +274,30 @@ extern "C" int mi355_index_select(const void* src, int elem_size, int64_t outer,
   MI355_REQUIRE(index != nullptr && out != nullptr, "mi355_index_select: NULL data pointer");
   MI355_REQUIRE(src != nullptr || n_src == 0, "mi355_index_select: NULL src");
   hipStream_t st = static_cast<hipStream_t>(stream);
+  // Selecting single elements along the last dim: stage each source row in LDS and resolve the
+  // (shared) indices there instead of issuing one scattered global read per element.
+  if (inner == 1 && idx_dtype == MI355_I64 && n_src * elem_size <= 64 * 1024 && outer < 65536 && n_idx >= n_src / 8 &&
+      n_src > 0) {
+    int64_t splits = 1;
+    if (outer < 512) {
+      splits = n_idx / 4096;
+      if (splits < 1) splits = 1;
+      if (splits > 64) splits = 64;
+    }
+    int64_t per_split = (n_idx + splits - 1) / splits;
+    per_split = (per_split + 3) / 4 * 4;
+    splits = (n_idx + per_split - 1) / per_split;
+    const dim3 grid((unsigned)splits, (unsigned)outer);
+    const size_t lds = (size_t)(n_src * elem_size);
+    const int64_t* ix = static_cast<const int64_t*>(index);
+    switch (elem_size) {
+      case 1: hipLaunchKernelGGL((gather_rows_lds_kernel<uint8_t>), grid, dim3(kIxBlock), lds, st, (const uint8_t*)src, ix, (uint8_t*)out, n_src, n_idx, (int64_t)0, per_split, err_flag); break;
+      case 2: hipLaunchKernelGGL((gather_rows_lds_kernel<uint16_t>), grid, dim3(kIxBlock), lds, st, (const uint16_t*)src, ix, (uint16_t*)out, n_src, n_idx, (int64_t)0, per_split, err_flag); break;
+      case 4: hipLaunchKernelGGL((gather_rows_lds_kernel<uint32_t>), grid, dim3(kIxBlock), lds, st, (const uint32_t*)src, ix, (uint32_t*)out, n_src, n_idx, (int64_t)0, per_split, err_flag); break;
+      default: hipLaunchKernelGGL((gather_rows_lds_kernel<uint64_t>), grid, dim3(kIxBlock), lds, st, (const uint64_t*)src, ix, (uint64_t*)out, n_src, n_idx, (int64_t)0, per_split, err_flag); break;
+    }
+    return check_launch("mi355_index_select(lds)");
+  }
   const int64_t row_bytes = inner * elem_size;
   const uintptr_t align = reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(out) | (uintptr_t)row_bytes;
   if (align % 16 == 0) return run_index_select<U128>(src, index, idx_dtype, out, outer, n_src, n_idx, row_bytes / 16, err_flag, st);

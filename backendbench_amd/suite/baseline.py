@@ -410,6 +410,9 @@ def edge_cases() -> List[Case]:
         add(aten.gather.default, lambda d, src=src: (_to(d, src((20, 64)), 1, randint((20, 64), 64, 3)), {}), exact=True, tag=f"dim1_{t}")
         add(aten.gather.default, lambda d, src=src: (_to(d, src((20, 64)), 0, randint((11, 33), 20, 3)), {}), exact=True, tag=f"dim0_{t}")
     add(aten.index_select.default, lambda d: (_to(d, normal((300, 4096), bf16, seed=1), 0, randint((100,), 300, 3)), {}), exact=True, tag="rows8k")
+    for dt, t in ((f16, "f16"), (f32, "f32"), (torch.float64, "f64"), (torch.uint8, "u8")):   # single elements along the last dim: LDS-staged rows
+        add(aten.index_select.default, lambda d, dt=dt: ([(normal((37, 1000), f32, 0, 50, seed=1).to(dt)).to(d), -1, randint((300,), 1000, 3).to(d)], {}), exact=True, tag=f"last_lds_{t}")
+    add(aten.index_select.default, lambda d: (_to(d, normal((3, 5, 4099), bf16, seed=1), 2, randint((9001,), 4099, 3)), {}), exact=True, tag="last_lds_split")
     add(aten.index_select.default, lambda d: (_to(d, normal((300, 33), bf16, seed=1), 0, randint((100,), 300, 3)), {}), exact=True, tag="odd_row_bytes")
     add(aten.index_select.default, lambda d: ([normal((64, 50), f32, seed=1).to(d).t(), 0, randint((33,), 50, 3).to(d)], {}), exact=True, tag="transposed_src")
     add(aten.index_select.default, lambda d: (_to(d, normal((50, 64), f32, seed=1), 0, torch.tensor(7)), {}), exact=True, tag="0d_index")

@@ -159,6 +159,8 @@ def test_error_behaviour_matches_the_oracle(backend, monkeypatch):
             backend[aten.index_select.default](table, 0, idx)
         with pytest.raises(IndexError):
             backend[aten.embedding.default](table, idx)
+    with pytest.raises(IndexError):   # selecting along the last dim goes through the LDS-staged kernel
+        backend[aten.index_select.default](table, 1, torch.tensor([0, 6, 2], device="cuda"))
     with pytest.raises((RuntimeError, IndexError)):
         backend[aten.gather.default](table, 1, torch.tensor([[-1]], device="cuda"))
     # a good call after a bad one is clean again
