@@ -843,6 +843,146 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
   else store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
 }
 
+// Variant of gemm_mfma_small_kernel for launches with at most one workgroup per CU: nothing else
+// hides a workgroup's barrier and LDS latencies there, so it takes two tiles per barrier (16
+// MFMAs per wave between synchronisations instead of 8) from a ring of eight stages (128 KB).
+template <typename T, bool B_NN, bool SPLIT>
+__global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
+  constexpr int S = 8;  // ring depth: two tiles per barrier, requested three pairs ahead
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  using frag_t = typename Mfma<T>::frag;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  const int bm = tm * SBM, bn = tn * SBN;
+  const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
+  const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
+  const T* A = static_cast<const T*>(g.a) + kbeg;
+  const T* B = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  // Region q = wave + 4 i (i < 2) of a panel is LDS bytes [q * 1024, q * 1024 + 1024).
+  const T* a_src[2];
+  const T* b_src[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = wave + 4 * i;
+    {  // K-contiguous A panel: region q = rows 16q .. 16q+15, 4 chunks per row
+      const int r = 16 * q + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gr = bm + r;
+      gr = gr < g.M ? gr : g.M - 1;
+      a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+    }
+    if constexpr (!B_NN) {
+      const int r = 16 * q + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gn = bn + r;
+      gn = gn < g.N ? gn : g.N - 1;
+      b_src[i] = B + (int64_t)gn * g.ldb + c * 8;
+    } else {  // N-contiguous B panel: region q = k rows 4q .. 4q+3, 16 units per row
+      const int k = 4 * q + (lane >> 4), pos = lane & 15;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gn = bn + u * 8;
+      gn = gn < g.N ? gn : 0;
+      b_src[i] = B + (int64_t)k * g.ldb + gn;
+    }
+  }
+  auto request_tile = [&](int t) {
+    const uint32_t stage = lds_base + (uint32_t)(t % S) * kSStage;
+    const int64_t k0 = (int64_t)t * BK3;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
+      lds_dma16(stage + region, a_src[i] + k0);
+      if constexpr (!B_NN) lds_dma16(stage + kSPanel + region, b_src[i] + k0);
+      else lds_dma16(stage + kSPanel + region, b_src[i] + k0 * g.ldb);
+    }
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  const int tr_k = fg * 8 + ((lane & 15) >> 2);
+  const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  auto read_frags = [&](int t, int ks, frag_t (&fa)[2], frag_t (&fb)[2]) {
+    const unsigned char* pa = lds + (t % S) * kSStage;
+    const unsigned char* pb = pa + kSPanel;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k32(wm * 64 + i * 32 + fr, ks * 2 + fg));
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if constexpr (!B_NN) {
+        fb[j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * 64 + j * 32 + fr, ks * 2 + fg));
+      } else {
+        const int k = ks * 16 + tr_k;
+        const int n = wn * 64 + j * 32 + tr_n;
+        const s16x4 lo = lds_read_tr(pb + swz_n128(k, n >> 3) + ((n & 7) << 1));
+        const s16x4 hi = lds_read_tr(pb + swz_n128(k + 4, n >> 3) + ((n & 7) << 1));
+        fb[j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto mma = [&](frag_t (&fa)[2], frag_t (&fb)[2]) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+  };
+
+  // Two 32-k tiles per barrier.  Pair p = tiles 2p, 2p+1; tiles 2p+6, 2p+7 are requested at its
+  // start into the slots pair p-1 left.  The first fragments of tile 2p+2 are read before the
+  // barrier that ends pair p, so at the end of pair p every tile up to 2p+4 must have landed:
+  // the twelve loads of tiles 2p+5 .. 2p+7 may still fly.  K % 64 == 0.
+  const int nk = (kend - kbeg) / BK3;
+  for (int t = 0; t < 6 && t < nk; ++t) request_tile(t);
+  if (nk >= 6) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  frag_t fa0[2], fb0[2], fa1[2], fb1[2];
+  read_frags(0, 0, fa0, fb0);
+  int t0 = 0;
+  for (; t0 + 7 < nk; t0 += 2) {
+    request_tile(t0 + 6);
+    request_tile(t0 + 7);
+    read_frags(t0, 1, fa1, fb1);
+    mma(fa0, fb0);
+    read_frags(t0 + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    read_frags(t0 + 1, 1, fa1, fb1);
+    mma(fa0, fb0);
+    read_frags(t0 + 2, 0, fa0, fb0);
+    mma(fa1, fb1);
+    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    __syncthreads();
+  }
+  for (; t0 < nk; t0 += 2) {  // drain: nothing left to request
+    read_frags(t0, 1, fa1, fb1);
+    mma(fa0, fb0);
+    read_frags(t0 + 1, 0, fa0, fb0);
+    mma(fa1, fb1);
+    read_frags(t0 + 1, 1, fa1, fb1);
+    mma(fa0, fb0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (t0 + 2 < nk) read_frags(t0 + 2, 0, fa0, fb0);
+    mma(fa1, fb1);
+  }
+  __syncthreads();  // the epilogue reuses the ring
+
+  if constexpr (SPLIT) store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
+  else store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
+}
+
 // ---------------------------------------------------------------- MFMA kernel, fp32
 // v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate; 157 TFLOP/s dense peak).  Same shape as the
 // 128x128 half-precision kernel in bytes: four waves (2x2) of 64x64, 16-k steps (64-byte rows),
@@ -1142,16 +1282,23 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
         nblocks = (int64_t)g.tiles_m * g.tiles_n;
         const SplitPlan sp = plan_splitk(M, N, K, sizeof(T));
-        if (sp.nsplit > 1 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 &&
-            reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+        const bool split = sp.nsplit > 1 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 &&
+                           reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+        if (split) {
           nsplit = sp.nsplit;
           g.ws = static_cast<float*>(workspace);
           g.ksplit = sp.ksplit;
-          kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, true> : (const void*)gemm_mfma_small_kernel<T, true, true>;
-        } else {
-          kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, false> : (const void*)gemm_mfma_small_kernel<T, true, false>;
         }
-        lds_bytes = kSmallLds;
+        // At most one workgroup per CU and whole pairs of tiles per split: two tiles per barrier.
+        const bool pairs = nblocks * nsplit <= kNumCU && K % 64 == 0 && (!split || sp.ksplit % 64 == 0);
+        lds_bytes = pairs ? 8 * kSStage : kSmallLds;
+        if (pairs) {
+          if (split) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, true> : (const void*)gemm_mfma_small2_kernel<T, true, true>;
+          else kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, false> : (const void*)gemm_mfma_small2_kernel<T, true, false>;
+        } else {
+          if (split) kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, true> : (const void*)gemm_mfma_small_kernel<T, true, true>;
+          else kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, false> : (const void*)gemm_mfma_small_kernel<T, true, false>;
+        }
         threads = 256;
       } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
@@ -1162,7 +1309,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
       }
       // More than 64 KB of dynamic LDS needs the attribute once per kernel and process.
-      static thread_local const void* attr_done[12] = {};
+      static thread_local const void* attr_done[16] = {};
       bool seen = false;
       for (const void* k : attr_done) seen = seen || k == kern;
       if (!seen) {
