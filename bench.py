@@ -49,6 +49,9 @@ def parse():
     ap.add_argument("--ops", default="all", help="comma-separated substrings of per-op rows to time, or 'none'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy")
+    ap.add_argument("--fill", default=None, choices=["zeros", "ones", "sign"],
+                    help="with --only-op: overwrite the floating-point inputs with zeros, ones or values from "
+                         "{-1, 0, 1} (shows how far a kernel's time depends on the data through the power/clock envelope)")
     return ap.parse_args()
 
 
@@ -92,8 +95,16 @@ def main():
             case = by_key[args.only_op]
             a, kw = case.make(dev)
             f, work = impl_of(case), case.work
+            if args.fill:
+                for t in a:
+                    if isinstance(t, torch.Tensor) and t.dtype.is_floating_point:
+                        if args.fill == "sign":
+                            t.copy_(torch.randint(-1, 2, t.shape, device=t.device).to(t.dtype))
+                        else:
+                            t.fill_(0.0 if args.fill == "zeros" else 1.0)
         ms, how = graph_bench(f, a, kw)
-        print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "work": work, "timing": how}))
+        print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "work": work, "timing": how,
+                          **({"fill": args.fill} if args.fill else {})}))
         return
 
     # ------------------------------------------------------------ headline step loop (C2)
