@@ -466,3 +466,29 @@ def test_trace_replay_scores_every_op_correct(backend):
               + " ".join(f"{r.speedup:.2f}" for r in pr), flush=True)
         seen += 1
     assert seen == 20
+
+
+def test_tensors_beyond_2_to_31_elements(backend):
+    """Element counts and byte offsets past 2^31 / 2^32: the kernels index with 64 bits."""
+    announce("tensors beyond 2^31 elements")
+    n = (1 << 31) + 4096 + 3
+    g = torch.Generator().manual_seed(11)
+    x = torch.randint(-100, 100, (n,), generator=g, dtype=torch.int8)
+    xg = x.cuda()
+    y = backend[aten.relu.default](xg)
+    torch.cuda.synchronize()
+    assert torch.equal(y[-(1 << 20):].cpu(), torch.relu(x[-(1 << 20):])) and torch.equal(y[: 1 << 20].cpu(), torch.relu(x[: 1 << 20]))
+    mid = (1 << 31) - 512
+    assert torch.equal(y[mid: mid + 1024].cpu(), torch.relu(x[mid: mid + 1024]))
+    s = backend[aten.sum.default](xg)
+    assert s.dtype == torch.int64 and int(s.item()) == int(x.sum(dtype=torch.int64).item())
+    del y, xg
+    # rows whose byte offset exceeds 2^32
+    table = torch.empty(70000, 16384, dtype=torch.float32, device="cuda")
+    rows = torch.tensor([69999, 0, 65537, 33000, 69998], device="cuda")
+    table[rows] = torch.arange(5, dtype=torch.float32, device="cuda")[:, None] + 1
+    out = backend[aten.index_select.default](table, 0, rows)
+    emb = backend[aten.embedding.default](table, rows.view(5, 1))
+    torch.cuda.synchronize()
+    want = (torch.arange(5, dtype=torch.float32)[:, None] + 1).expand(5, 16384)
+    assert torch.equal(out.cpu(), want) and torch.equal(emb.cpu().view(5, 16384), want)
