@@ -632,9 +632,9 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
   auto mma = [&](frag_t (&fa)[4], frag_t (&fb)[2]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
+      for (int i = 0; i < 4; ++i) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
   };
   auto next_slot = [](uint32_t s) { return s + kASlot64 == (uint32_t)kBRing64 ? 0u : s + kASlot64; };
 
