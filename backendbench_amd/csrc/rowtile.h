@@ -16,8 +16,10 @@ namespace mi355 {
 
 constexpr int kRowBlock = 256;  // threads per block of every row-tile kernel
 
-template <typename T, int NV, bool VEC, int W, int BLOCK = kRowBlock> struct RowTile {
-  static constexpr int V = 16 / sizeof(T);
+// VB: bytes per lane and access (16; 8 when the output element is twice as wide as the input
+// element, so that the output side still moves whole 16-byte pieces per lane).
+template <typename T, int NV, bool VEC, int W, int BLOCK = kRowBlock, int VB = 16> struct RowTile {
+  static constexpr int V = VB / sizeof(T);
   static constexpr int GROUP = kWave * W;        // lanes cooperating on one row
   static constexpr int ROWS_PER_BLOCK = BLOCK / GROUP;
   float v[NV][V];
@@ -126,9 +128,8 @@ template <typename T, int NV, bool VEC, int W, int BLOCK = kRowBlock> struct Row
   }
 };
 
-// Elements between the previous 16-byte-per-V-elements boundary and `p` (0 for aligned rows).
-template <typename T> __device__ __forceinline__ int row_misalignment(const T* p) {
-  constexpr int V = 16 / sizeof(T);
+// Elements between the previous V-element boundary and `p` (0 for aligned rows).
+template <typename T, int V = 16 / sizeof(T)> __device__ __forceinline__ int row_misalignment(const T* p) {
   return (int)((reinterpret_cast<uintptr_t>(p) / sizeof(T)) % V);
 }
 
@@ -156,8 +157,9 @@ __device__ __forceinline__ T group_allreduce(T v, Op op, T* smem) {
 // constants; false when the row does not fit (16 slabs over 4 waves, or 64 values per lane over
 // max_w waves).  Aligned rows get at most
 // 32 values per lane (W grows instead); unaligned rows use one wave and the scalar layout.
-template <typename T, typename Body> inline bool dispatch_row_tile(int64_t n, bool vec, Body body, int max_w = 4) {
-  constexpr int V = 16 / sizeof(T);
+template <typename T, typename Body, int VB = 16>
+inline bool dispatch_row_tile(int64_t n, bool vec, Body body, int max_w = 4, std::integral_constant<int, VB> = {}) {
+  constexpr int V = VB / sizeof(T);
   using std::integral_constant;
 #define MI355_ROW(NV_, W_, VEC_)                                                              \
   {                                                                                           \

@@ -21,11 +21,11 @@ constexpr int kSmBlock = kRowBlock;
 // SHIFT: rows are not 16-byte aligned (odd row length); see RowTile::load_shifted.
 constexpr int sm_tile_block(int w) { return w <= 4 ? kSmBlock : kWave * w; }  // rows over 8 / 16 waves: one row per block
 
-template <typename T, typename O, int NV, bool VEC, int W, bool LOG, bool SHIFT>
+template <typename T, typename O, int NV, bool VEC, int W, bool LOG, bool SHIFT, int VB>
 __global__ __launch_bounds__(sm_tile_block(W)) void softmax_tile_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                        int64_t rows, int64_t n) {
   constexpr int BLOCK = sm_tile_block(W);
-  using Tile = RowTile<T, NV, VEC, W, BLOCK>;
+  using Tile = RowTile<T, NV, VEC, W, BLOCK, VB>;
   constexpr int V = Tile::V;
   __shared__ float red_max[BLOCK / kWave], red_sum[BLOCK / kWave];
   const int t = threadIdx.x % Tile::GROUP;
@@ -35,7 +35,7 @@ __global__ __launch_bounds__(sm_tile_block(W)) void softmax_tile_kernel(const T*
   Tile tile;
   int a = 0;
   if constexpr (SHIFT) {
-    a = row_misalignment(x + row * n);
+    a = row_misalignment<T, V>(x + row * n);
     tile.load_shifted(x + row * n, n, a, t, -INFINITY);
   } else {
     tile.load(x + row * n, n, t, -INFINITY);
@@ -259,23 +259,32 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
   // shifted per row, when input and output rows are misaligned by the same number of elements.
   const bool shift = !vec && V > 1 &&
                      (reinterpret_cast<uintptr_t>(x) / sizeof(T)) % V == (reinterpret_cast<uintptr_t>(y) / sizeof(O)) % V;
+  // Register tiles.  When the output element is wider than the input element (half_to_float)
+  // a lane takes 8 input bytes per access, so that its output is one 16-byte piece and every
+  // store instruction of a wave covers whole lines.
+  constexpr int VB = sizeof(O) > sizeof(T) ? 8 : 16;
+  constexpr int TV = VB / sizeof(T);
+  const bool tvec = TV == V ? vec : (n % TV == 0 && reinterpret_cast<uintptr_t>(x) % VB == 0 && aligned16(y));
+  const bool tshift = TV == V ? shift
+                              : (!tvec && (reinterpret_cast<uintptr_t>(x) / sizeof(T)) % TV ==
+                                              (reinterpret_cast<uintptr_t>(y) / sizeof(O)) % TV);
   bool done = false;
   if constexpr (!std::is_same<T, double>::value)  // f64 rows take the block kernel (double accumulation)
   if (outer < (int64_t(1) << 31)) {
-    done = dispatch_row_tile<T>(shift ? n + V - 1 : n, vec || shift, [&](auto nv, auto w, auto v) {
+    done = dispatch_row_tile<T>(tshift ? n + TV - 1 : n, tvec || tshift, [&](auto nv, auto w, auto v) {
       constexpr int NV = decltype(nv)::value, W = decltype(w)::value;
       constexpr bool VEC = decltype(v)::value;
       constexpr int block = sm_tile_block(W);
       constexpr int rpb = block / (kWave * W);
       const unsigned nblk = (unsigned)((outer + rpb - 1) / rpb);
       if constexpr (VEC) {
-        if (shift) {
-          hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, true, W, LOG, true>), dim3(nblk), dim3(block), 0, st, x, y, outer, n);
+        if (tshift) {
+          hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, true, W, LOG, true, VB>), dim3(nblk), dim3(block), 0, st, x, y, outer, n);
           return;
         }
       }
-      hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, VEC, W, LOG, false>), dim3(nblk), dim3(block), 0, st, x, y, outer, n);
-    }, 16);
+      hipLaunchKernelGGL((softmax_tile_kernel<T, O, NV, VEC, W, LOG, false, VB>), dim3(nblk), dim3(block), 0, st, x, y, outer, n);
+    }, 16, std::integral_constant<int, VB>());
   }
   if (!done) {
     MI355_REQUIRE(outer < (int64_t(1) << 31), "mi355_softmax: too many rows (%lld)", (long long)outer);
