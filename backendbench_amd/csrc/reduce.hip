@@ -106,39 +106,52 @@ __device__ __forceinline__ void write_final(O* out, int64_t at, const typename R
 // ---------------------------------------------------------------- kernels
 constexpr int kRedBlock = 256;
 
-// Accumulate x[base + lo .. base + hi) striding by `nthr` lanes starting at `tid`.
-template <typename T, typename R, bool VEC>
+// Accumulate row[lo .. hi) striding by `nthr` lanes starting at `tid`.
+//   MODE 0  scalar accesses;
+//   MODE 1  row 16-byte aligned, lo and hi multiples of V (the planner guarantees it): vectors;
+//   MODE 2  misaligned row (odd row length, offset view): vectors over the aligned window that
+//           starts `a` elements before the row; [lo, hi) are window positions (multiples of V
+//           except the last hi), elements outside the row are skipped.  The window may reach up
+//           to 15 bytes outside the row, inside 16-byte pieces that also hold row bytes.
+template <typename T, typename R, int MODE>
 __device__ __forceinline__ void accumulate_span(typename R::State& st, const T* row, int64_t lo, int64_t hi,
-                                                int tid, int nthr) {
+                                                int tid, int nthr, int a = 0, int64_t red = 0) {
   using A = typename R::acc_t;
-  if constexpr (VEC) {
+  if constexpr (MODE != 0) {
     constexpr int V = Vec<T>::N;
-    // lo and hi are multiples of V (the planner guarantees it on the VEC path).
+    const T* win = row - a;
+    const int64_t total = red + a;  // MODE 2 only
+    auto take = [&](const Vec<T>& v, int64_t w) {
+      if (MODE == 1 || (w >= a && w + V <= total)) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) R::acc(st, (A)v.v[j], w + j - a);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j)
+          if (w + j >= a && w + j < total) R::acc(st, (A)v.v[j], w + j - a);
+      }
+    };
     int64_t i = lo + (int64_t)tid * V;
     const int64_t step = (int64_t)nthr * V;
     for (; i + 3 * step < hi; i += 4 * step) {
-      Vec<T> v0 = load_vec_nt(row + i), v1 = load_vec_nt(row + i + step), v2 = load_vec_nt(row + i + 2 * step),
-             v3 = load_vec_nt(row + i + 3 * step);
-#pragma unroll
-      for (int j = 0; j < V; ++j) R::acc(st, (A)v0.v[j], i + j);
-#pragma unroll
-      for (int j = 0; j < V; ++j) R::acc(st, (A)v1.v[j], i + step + j);
-#pragma unroll
-      for (int j = 0; j < V; ++j) R::acc(st, (A)v2.v[j], i + 2 * step + j);
-#pragma unroll
-      for (int j = 0; j < V; ++j) R::acc(st, (A)v3.v[j], i + 3 * step + j);
+      Vec<T> v0 = load_vec_nt(win + i), v1 = load_vec_nt(win + i + step), v2 = load_vec_nt(win + i + 2 * step),
+             v3 = load_vec_nt(win + i + 3 * step);
+      take(v0, i);
+      take(v1, i + step);
+      take(v2, i + 2 * step);
+      take(v3, i + 3 * step);
     }
-    for (; i < hi; i += step) {
-      Vec<T> v = load_vec_nt(row + i);
-#pragma unroll
-      for (int j = 0; j < V; ++j) R::acc(st, (A)v.v[j], i + j);
-    }
+    for (; i < hi; i += step) take(load_vec_nt(win + i), i);
   } else {
     for (int64_t i = lo + tid; i < hi; i += nthr) R::acc(st, (A)row[i], i);
   }
 }
 
-template <typename T, typename O, typename R, int FIN, bool VEC>
+template <typename T> __device__ __forceinline__ int reduce_row_misalignment(const T* p) {
+  return (int)((reinterpret_cast<uintptr_t>(p) / sizeof(T)) % Vec<T>::N);
+}
+
+template <typename T, typename O, typename R, int FIN, int MODE>
 __global__ __launch_bounds__(kRedBlock) void rows_wave_kernel(const T* __restrict__ x, O* __restrict__ out,
                                                              int64_t outer, int64_t red, double divisor) {
   const int lane = threadIdx.x % kWave;
@@ -146,23 +159,29 @@ __global__ __launch_bounds__(kRedBlock) void rows_wave_kernel(const T* __restric
   const int64_t nwaves = (int64_t)gridDim.x * (kRedBlock / kWave);
   for (int64_t row = wave0; row < outer; row += nwaves) {
     typename R::State st = R::init();
-    accumulate_span<T, R, VEC>(st, x + row * red, 0, red, lane, kWave);
+    const T* r = x + row * red;
+    const int a = MODE == 2 ? reduce_row_misalignment(r) : 0;
+    accumulate_span<T, R, MODE>(st, r, 0, red + a, lane, kWave, a, red);
     st = wave_reduce(st, (R*)nullptr);
     if (lane == 0) write_final<R, O, FIN>(out, row, st, divisor);
   }
 }
 
 // grid = (nsplit, outer).  PARTIAL: writes State to ws[row * nsplit + split].
-template <typename T, typename O, typename R, int FIN, bool VEC, bool PARTIAL>
+template <typename T, typename O, typename R, int FIN, int MODE, bool PARTIAL>
 __global__ __launch_bounds__(kRedBlock) void rows_block_kernel(const T* __restrict__ x, O* __restrict__ out,
                                                               typename R::State* __restrict__ ws, int64_t red,
                                                               int64_t chunk, double divisor) {
   __shared__ typename R::State smem[kRedBlock / kWave];
   const int64_t row = blockIdx.y;
+  const T* r = x + row * red;
+  const int a = MODE == 2 ? reduce_row_misalignment(r) : 0;
+  const int64_t total = red + a;  // window extent (= red unless MODE 2)
   const int64_t lo = (int64_t)blockIdx.x * chunk;
-  const int64_t hi = lo + chunk < red ? lo + chunk : red;
+  // the last split also takes the few window positions the misalignment adds
+  const int64_t hi = (blockIdx.x + 1 == gridDim.x || lo + chunk > total) ? total : lo + chunk;
   typename R::State st = R::init();
-  accumulate_span<T, R, VEC>(st, x + row * red, lo, hi, threadIdx.x, kRedBlock);
+  if (lo < hi) accumulate_span<T, R, MODE>(st, r, lo, hi, threadIdx.x, kRedBlock, a, red);
   st = block_reduce_state<R>(st, smem);
   if (threadIdx.x == 0) {
     if constexpr (PARTIAL) ws[row * gridDim.x + blockIdx.x] = st;
@@ -372,8 +391,9 @@ static int run_reduce(const void* xv, int64_t outer, int64_t red, int64_t inner,
     case ROWS_WAVE: {
       const bool vec = aligned16(x) && red % V == 0;
       const int grid = grid_for(outer, kRedBlock / kWave, kNumCU * 16);
-      if (vec) hipLaunchKernelGGL((rows_wave_kernel<T, O, R, FIN, true>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
-      else hipLaunchKernelGGL((rows_wave_kernel<T, O, R, FIN, false>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      if (vec) hipLaunchKernelGGL((rows_wave_kernel<T, O, R, FIN, 1>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      else if (V > 1) hipLaunchKernelGGL((rows_wave_kernel<T, O, R, FIN, 2>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      else hipLaunchKernelGGL((rows_wave_kernel<T, O, R, FIN, 0>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
       break;
     }
     case ROWS_BLOCK: {
@@ -385,13 +405,13 @@ static int run_reduce(const void* xv, int64_t outer, int64_t red, int64_t inner,
         const T* xr = x + r0 * red;
         O* outr = out + r0;
         State* wsr = ws ? ws + r0 * p.nsplit : nullptr;
-        if (p.nsplit > 1) {
-          if (vec) hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, true, true>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
-          else hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, false, true>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
-        } else {
-          if (vec) hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, true, false>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
-          else hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, false, false>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
-        }
+#define MI355_ROWS_BLOCK(MODE_)                                                                                          \
+  if (p.nsplit > 1) hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, MODE_, true>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor); \
+  else hipLaunchKernelGGL((rows_block_kernel<T, O, R, FIN, MODE_, false>), grid, dim3(kRedBlock), 0, st, xr, outr, wsr, red, p.chunk, divisor);
+        if (vec) { MI355_ROWS_BLOCK(1) }
+        else if (V > 1) { MI355_ROWS_BLOCK(2) }
+        else { MI355_ROWS_BLOCK(0) }
+#undef MI355_ROWS_BLOCK
       }
       break;
     }

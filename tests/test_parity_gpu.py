@@ -492,3 +492,35 @@ def test_tensors_beyond_2_to_31_elements(backend):
     torch.cuda.synchronize()
     want = (torch.arange(5, dtype=torch.float32)[:, None] + 1).expand(5, 16384)
     assert torch.equal(out.cpu(), want) and torch.equal(emb.cpu().view(5, 16384), want)
+
+
+@pytest.mark.parametrize("n", [2049, 197, 50257, 8193])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_misaligned_rows_see_exactly_their_own_elements(backend, n, dtype):
+    """Odd row lengths put rows off 16-byte boundaries; the row kernels then read the aligned
+    window around each row.  Markers on the first and last element of alternating rows make
+    any element dropped at a row's ends, or leaked in from a neighbouring row, change the result."""
+    announce(f"row boundaries n={n} {dtype}")
+    rows = 64 if n > 20000 else 300
+    g = torch.Generator().manual_seed(n)
+    x = -torch.rand(rows, n, generator=g)            # everything in (-1, 0]
+    x[0::2, -1] = 500.0                               # even rows: the maximum is the last element
+    x[1::4, 0] = 900.0                                # some odd rows: the maximum is the first element
+    x = x.to(dtype)
+    xg = x.cuda()
+    for op, args in ((aten.amax.default, [[-1]]), (aten.argmax.default, [-1]), (aten.sum.dim_IntList, [[-1]]),
+                     (aten._softmax.default, [-1, False]), (aten._log_softmax.default, [-1, False])):
+        got = backend[op](xg, *args)
+        torch.cuda.synchronize()
+        ref = aten_cpu.reference(op, [x, *args])
+        assert ev.allclose(ref, got.cpu(), exact=op is aten.argmax.default), f"{op.__name__} n={n}"
+    w = torch.rand(n, generator=g).to(dtype)
+    got = backend[aten.native_layer_norm.default](xg, [n], w.cuda(), None, 1e-5)
+    ref = aten_cpu.reference(aten.native_layer_norm.default, [x, [n], w, None, 1e-5])
+    assert ev.allclose(ref, tuple(t.cpu() for t in got)), f"layer_norm n={n}"
+    # the same through a view that starts one element into its storage
+    flat = torch.cat([torch.zeros(1, dtype=dtype), x.reshape(-1)]).cuda()
+    view = flat[1:].view(rows, n)
+    assert view.data_ptr() % 16 != 0
+    assert ev.allclose(aten_cpu.reference(aten.amax.default, [x, [-1]]), backend[aten.amax.default](view, [-1]).cpu())
+    assert ev.allclose(aten_cpu.reference(aten._softmax.default, [x, -1, False]), backend[aten._softmax.default](view, -1, False).cpu())
