@@ -69,6 +69,7 @@ struct GemmArgs {
   float alpha, beta;
   int32_t tiles_m, tiles_n;
   int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
+  int32_t out_vec;  // out rows start on 16-byte boundaries (N a multiple of the vector width): vector stores
   // Split-K (128x128 kernels only): blockIdx.y = split, which covers k in [split * ksplit,
   // min(K, (split + 1) * ksplit)) and writes its raw fp32 tile to ws[split][M][N].
   float* ws;
@@ -183,17 +184,21 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int nl = j * 32 + q * 8 + fg * 4;
-        int n = n0 + nl;
-        n = n + 4 <= g.N ? n : 0;  // out-of-range columns are computed on valid addresses and never stored
+        const int n = n0 + nl;
+        // Columns past N are computed on valid addresses and never stored.
         float cv[4] = {0.f, 0.f, 0.f, 0.f};
         if (use_c) {
-          if (g.c_vec) {
-            const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (int64_t)mc * g.c_rs + n);
+          if (g.c_vec) {  // N % 4 == 0: a group of four columns is wholly inside or wholly outside
+            const int nv = n + 4 <= g.N ? n : 0;
+            const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (int64_t)mc * g.c_rs + nv);
 #pragma unroll
             for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(t.v[e]);
           } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(C[(int64_t)mc * g.c_rs + (int64_t)(n + e) * g.c_cs]);
+            for (int e = 0; e < 4; ++e) {
+              const int ne = n + e < g.N ? n + e : g.N - 1;
+              cv[e] = static_cast<float>(C[(int64_t)mc * g.c_rs + (int64_t)ne * g.c_cs]);
+            }
           }
         }
         VecN4<T> r;
@@ -215,7 +220,16 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
     const int row = chunk >> 3, s = chunk & 7;
     const u32x4 v = *reinterpret_cast<const u32x4*>(slab + row * 128 + ((s ^ ((row >> 1) & 7)) << 4));
     const int m = m0 + row, n = n0 + s * 8;
-    if (m < g.M && n < g.N) *reinterpret_cast<u32x4*>(D + (int64_t)m * g.N + n) = v;  // N % 8 == 0 on this path
+    if (m >= g.M || n >= g.N) continue;
+    if (g.out_vec) {
+      *reinterpret_cast<u32x4*>(D + (int64_t)m * g.N + n) = v;
+    } else {  // N not a multiple of 8 (e.g. a 50257-wide vocabulary): rows are misaligned, element stores
+      struct alignas(16) Elems { T v[8]; };
+      const Elems ev = __builtin_bit_cast(Elems, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if (n + e < g.N) D[(int64_t)m * g.N + n + e] = ev.v[e];
+    }
   }
 }
 
@@ -1135,15 +1149,22 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = bn + wn * 64 + j * 32 + q * 8 + fg * 4;
-        if (n >= g.N) continue;  // N % 4 == 0: a vector is all-in or all-out
+        if (n >= g.N) continue;
         f32x4 r;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float v = g.alpha * acc[i][j][q * 4 + e];
-          if (use_c) v += g.beta * C[(int64_t)m * g.c_rs + (int64_t)(n + e) * g.c_cs];
+          const int ne = n + e < g.N ? n + e : g.N - 1;
+          if (use_c) v += g.beta * C[(int64_t)m * g.c_rs + (int64_t)ne * g.c_cs];
           r[e] = v;
         }
-        *reinterpret_cast<f32x4*>(D + (int64_t)m * g.N + n) = r;
+        if (g.out_vec) {
+          *reinterpret_cast<f32x4*>(D + (int64_t)m * g.N + n) = r;
+        } else {  // N % 4 != 0: misaligned rows, element stores
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < g.N) D[(int64_t)m * g.N + n + e] = r[e];
+        }
       }
   }
 }
@@ -1257,14 +1278,17 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     const bool fits = M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
     // Tiny problems are cheaper on the generic kernel than on a mostly empty 256x256 tile.
     const bool worth = M * N >= 128 * 128 && K >= 32;
-    if (a_ok && (b_nt || b_nn) && K % 8 == 0 && N % 8 == 0 && fits && worth && K > 0 &&
-        aligned16(out)) {
+    // Row-major B needs N % 8 == 0 (its rows must start on 16-byte boundaries); transposed B takes
+    // any N — a 50257-wide vocabulary projection stores its misaligned output rows element-wise.
+    const bool b_nn_ok = b_nn && N % 8 == 0;
+    if (a_ok && (b_nt || b_nn_ok) && K % 8 == 0 && fits && worth && K > 0) {
       GemmArgs g{};
       g.a = a; g.b = b; g.c = c; g.out = out;
       g.lda = a_rs;
       g.ldb = b_nt ? b_cs : b_rs;
       g.c_rs = c_rs; g.c_cs = c_cs;
-      g.c_vec = c != nullptr && c_cs == 1 && c_rs % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 8 == 0;
+      g.c_vec = c != nullptr && c_cs == 1 && c_rs % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 8 == 0 && N % 4 == 0;
+      g.out_vec = N % 8 == 0 && aligned16(out);
       g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
       g.alpha = (float)alpha; g.beta = (float)beta;
       g.tiles_m = (int32_t)((M + BM - 1) / BM);
@@ -1282,8 +1306,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
         nblocks = (int64_t)g.tiles_m * g.tiles_n;
         const SplitPlan sp = plan_splitk(M, N, K, sizeof(T));
-        const bool split = sp.nsplit > 1 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 &&
-                           reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+        const bool split = sp.nsplit > 1 && N % 4 == 0 && workspace != nullptr &&
+                           workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
         if (split) {
           nsplit = sp.nsplit;
           g.ws = static_cast<float*>(workspace);
@@ -1332,12 +1356,14 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     const bool b_nt = b_rs == 1 && b_cs % 4 == 0 && aligned16(b);
     const bool b_nn = b_cs == 1 && b_rs % 4 == 0 && aligned16(b);
     const bool fits = M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
-    if (a_ok && (b_nt || b_nn) && K % FBK == 0 && K > 0 && N % 4 == 0 && fits && M * N >= 64 * 64 && aligned16(out)) {
+    const bool b_nn_ok = b_nn && N % 4 == 0;
+    if (a_ok && (b_nt || b_nn_ok) && K % FBK == 0 && K > 0 && fits && M * N >= 64 * 64) {
       GemmArgs g{};
       g.a = a; g.b = b; g.c = c; g.out = out;
       g.lda = a_rs;
       g.ldb = b_nt ? b_cs : b_rs;
       g.c_rs = c_rs; g.c_cs = c_cs;
+      g.out_vec = N % 4 == 0 && aligned16(out);
       g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
       g.alpha = (float)alpha; g.beta = (float)beta;
       g.tiles_m = (int32_t)((M + SBM - 1) / SBM);
@@ -1346,7 +1372,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       MI355_REQUIRE(nblocks < (int64_t(1) << 31), "mi355_gemm: too many tiles");
       int nsplit = 1;
       const SplitPlan sp = plan_splitk(M, N, K, 4);
-      if (sp.nsplit > 1 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 &&
+      if (sp.nsplit > 1 && N % 4 == 0 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 &&
           reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
         nsplit = sp.nsplit;
         g.ws = static_cast<float*>(workspace);

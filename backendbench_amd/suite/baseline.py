@@ -384,6 +384,12 @@ def edge_cases() -> List[Case]:
     add(aten.mm.default, lambda d: (_to(d, torch.eye(128, dtype=f32), normal((128, 128), f32, seed=2)), {}), exact=True, tag="f32_identity")
     add(aten.mm.default, lambda d: (_to(d, normal((70, 90), torch.float64, seed=1), normal((90, 50), torch.float64, 0, 0.1, seed=2)), {}), tag="f64")
     add(aten.addmm.default, lambda d: (_to(d, normal((50,), torch.float64, seed=3), normal((70, 90), torch.float64, seed=1), normal((90, 50), torch.float64, 0, 0.1, seed=2)), {"beta": 0.5}), tag="f64")
+    # output width not a multiple of the vector width (transposed B, e.g. a 50257-wide vocabulary): element stores
+    add(aten.mm.default, lambda d: ([normal((300, 96), bf16, seed=1).to(d), normal((261, 96), bf16, 0, 0.1, seed=2).to(d).t()], {}), tag="odd_n_bf16")
+    add(aten.mm.default, lambda d: ([normal((300, 96), f32, seed=1).to(d), normal((261, 96), f32, 0, 0.1, seed=2).to(d).t()], {}), tag="odd_n_f32")
+    add(aten.addmm.default, lambda d: ([normal((263,), f16, seed=3).to(d), normal((300, 128), f16, seed=1).to(d), normal((263, 128), f16, 0, 0.1, seed=2).to(d).t()], {"beta": 0.5}), tag="odd_n_bias_f16")
+    add(aten.addmm.default, lambda d: ([normal((300, 263), f32, seed=3).to(d), normal((300, 128), f32, seed=1).to(d), normal((263, 128), f32, 0, 0.1, seed=2).to(d).t()], {"alpha": 2.0}), tag="odd_n_full_c_f32")
+    add(aten.mm.default, lambda d: ([normal((64, 768), f16, seed=1).to(d), normal((50257, 768), f16, 0, 0.05, seed=2).to(d).t()], {}), tag="vocab_50257_f16")
     # skinny problems with a long K: split along K over the chip, fp32 partials, finishing pass
     add(aten.mm.default, lambda d: (_to(d, normal((16, 2048), bf16, seed=1), normal((2048, 1024), bf16, 0, 0.05, seed=2)), {}), tag="splitk_bf16")
     add(aten.mm.default, lambda d: (_to(d, normal((40, 2144), f16, seed=1), normal((2144, 520), f16, 0, 0.05, seed=2)), {}), tag="splitk_ragged_f16")
