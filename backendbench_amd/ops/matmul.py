@@ -3,7 +3,7 @@
 import torch
 
 from .. import _lib
-from ._common import cast, device_managed, launch, new_dense
+from ._common import cast, dense, device_managed, launch, new_dense
 
 _GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32, torch.float64)
 _SPLITK_MAX_OUT = 128 * 128 * 256  # the planner never splits problems with 256 or more 128x128 tiles
@@ -40,6 +40,14 @@ def _gemm(a, b, c, alpha, beta):
     else:
         c_ptr, c_rs, c_cs = None, 0, 0
     code = _lib.dtype_code(a.dtype)
+    # The MFMA kernels want K-contiguous rows of A and a row-major or K-contiguous B.  Any other
+    # layout (a transposed left operand, sliced views) is densified once with the copy kernel: one
+    # pass over the operand, instead of the whole product on the FMA fallback.
+    if M * N >= 64 * 64 and K >= 16 and a.dtype != torch.float64:
+        if a.stride(1) != 1 and M > 1 and K > 1:
+            a = dense(a)
+        if b.stride(1) != 1 and b.stride(0) != 1 and K > 1 and N > 1:
+            b = dense(b)
     ws, ws_bytes = None, 0
     if M * N < _SPLITK_MAX_OUT:  # only skinny / small outputs are ever split along K
         ws_bytes = _workspace_bytes()(M, N, K, code)

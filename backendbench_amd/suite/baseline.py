@@ -384,6 +384,8 @@ def edge_cases() -> List[Case]:
     add(aten.mm.default, lambda d: (_to(d, torch.eye(128, dtype=f32), normal((128, 128), f32, seed=2)), {}), exact=True, tag="f32_identity")
     add(aten.mm.default, lambda d: (_to(d, normal((70, 90), torch.float64, seed=1), normal((90, 50), torch.float64, 0, 0.1, seed=2)), {}), tag="f64")
     add(aten.addmm.default, lambda d: (_to(d, normal((50,), torch.float64, seed=3), normal((70, 90), torch.float64, seed=1), normal((90, 50), torch.float64, 0, 0.1, seed=2)), {"beta": 0.5}), tag="f64")
+    add(aten.mm.default, lambda d: ([normal((512, 700), bf16, seed=1).to(d)[:, ::2], normal((350, 264), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_strided_cols")
+    add(aten.mm.default, lambda d: ([normal((256, 320), bf16, seed=1).to(d), normal((320, 600), bf16, 0, 0.05, seed=2).to(d)[:, ::2]], {}), tag="b_strided_cols")
     # output width not a multiple of the vector width (transposed B, e.g. a 50257-wide vocabulary): element stores
     add(aten.mm.default, lambda d: ([normal((300, 96), bf16, seed=1).to(d), normal((261, 96), bf16, 0, 0.1, seed=2).to(d).t()], {}), tag="odd_n_bf16")
     add(aten.mm.default, lambda d: ([normal((300, 96), f32, seed=1).to(d), normal((261, 96), f32, 0, 0.1, seed=2).to(d).t()], {}), tag="odd_n_f32")
