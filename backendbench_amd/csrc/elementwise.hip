@@ -132,6 +132,55 @@ template <typename S> static int copy_from(const mi355_tensor* src, const mi355_
   }
 }
 
+// ---- transposing copy ------------------------------------------------------------
+// dst[b][m][n] = src[b][n][m] for same-width elements when the source is unit-stride along m
+// and the destination along n (a transposed view made dense, per batch).  64 x 64 tiles go
+// through LDS so that both the reads and the writes of a wave are contiguous; the strided
+// elementwise kernel reads such a source one scattered element per lane.
+// grid = (ceil(N / 64), ceil(M / 64), batch), block = 256.
+template <typename U>
+__global__ __launch_bounds__(256) void transpose_copy_kernel(const U* __restrict__ src, U* __restrict__ dst, int64_t M,
+                                                            int64_t N, int64_t src_n_stride, int64_t dst_m_stride,
+                                                            int64_t src_b_stride, int64_t dst_b_stride) {
+  __shared__ U tile[64][65];
+  const int64_t n0 = (int64_t)blockIdx.x * 64, m0 = (int64_t)blockIdx.y * 64;
+  const U* s = src + (int64_t)blockIdx.z * src_b_stride;
+  U* d = dst + (int64_t)blockIdx.z * dst_b_stride;
+  const int c = threadIdx.x % 64, r4 = threadIdx.x / 64;
+#pragma unroll
+  for (int p = 0; p < 16; ++p) {  // row n0 + r of the source view: 64 consecutive m
+    const int r = p * 4 + r4;
+    if (n0 + r < N && m0 + c < M) tile[r][c] = s[(n0 + r) * src_n_stride + m0 + c];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int p = 0; p < 16; ++p) {  // row m0 + r of the destination: 64 consecutive n
+    const int r = p * 4 + r4;
+    if (m0 + r < M && n0 + c < N) d[(m0 + r) * dst_m_stride + n0 + c] = tile[c][r];
+  }
+}
+
+// True (and the copy enqueued) when src -> dst is such a transposition.
+template <typename U>
+static bool try_transpose_copy(const mi355_tensor* src, const mi355_tensor* dst, hipStream_t st, int* rc) {
+  const int64_t* strides[2] = {src->strides, dst->strides};
+  const Dims<2> d = collapse_dims<2>(dst->ndim, dst->sizes, strides);
+  if (d.ndim != 2 && d.ndim != 3) return false;
+  const int im = d.ndim - 2, in = d.ndim - 1;
+  const int64_t M = d.sizes[im], N = d.sizes[in];
+  // destination row-major over (m, n), source unit-stride along m
+  if (d.strides[1][in] != 1 || d.strides[0][im] != 1 || d.strides[0][in] < M || d.strides[1][im] < N) return false;
+  if (M < 16 || N < 16) return false;
+  const int64_t batch = d.ndim == 3 ? d.sizes[0] : 1;
+  if (batch > 65535 || (M + 63) / 64 > 65535) return false;
+  const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)batch);
+  hipLaunchKernelGGL((transpose_copy_kernel<U>), grid, dim3(256), 0, st, (const U*)src->data, (U*)dst->data, M, N,
+                     d.strides[0][in], d.strides[1][im], d.ndim == 3 ? d.strides[0][0] : 0,
+                     d.ndim == 3 ? d.strides[1][0] : 0);
+  *rc = check_launch("mi355_copy(transpose)");
+  return true;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -221,6 +270,16 @@ extern "C" int mi355_copy(const mi355_tensor* src, const mi355_tensor* dst, void
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (src->dtype == dst->dtype) {  // same dtype: move raw bits by element width
     const mi355_tensor* ins[1] = {src};
+    if (same_shape(src, dst) && numel(dst) > 0) {
+      bool done = false;
+      switch (dtype_size(src->dtype)) {
+        case 1: done = try_transpose_copy<uint8_t>(src, dst, st, &rc); break;
+        case 2: done = try_transpose_copy<uint16_t>(src, dst, st, &rc); break;
+        case 4: done = try_transpose_copy<uint32_t>(src, dst, st, &rc); break;
+        case 8: done = try_transpose_copy<uint64_t>(src, dst, st, &rc); break;
+      }
+      if (done) return rc;
+    }
     switch (dtype_size(src->dtype)) {
       case 1: return launch_elementwise(CastF<uint8_t, uint8_t>{}, ins, dst, st, "mi355_copy");
       case 2: return launch_elementwise(CastF<uint16_t, uint16_t>{}, ins, dst, st, "mi355_copy");

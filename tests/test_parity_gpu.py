@@ -580,3 +580,26 @@ def test_transformers_model_under_the_dispatcher_override(backend, family):
         err = (ours.float() - plain.float()).abs().max().item()
         scale = plain.float().abs().max().item()
         assert err <= tol * max(scale, 1.0), f"{family}/{dtype}: max abs diff {err} at scale {scale}"
+
+
+def test_transposing_copy_matches_contiguous(backend):
+    """`dense()` of transposed views (the copy every wrapper makes of an operand it cannot take
+    as is) goes through the LDS-tiled transposing copy: bit-exact against torch's contiguous()."""
+    from backendbench_amd.ops._common import copy_into, dense
+
+    announce("transposing copy")
+    g = torch.Generator().manual_seed(5)
+    for dtype in (torch.float16, torch.float32, torch.int8, torch.int64, torch.bool):
+        for shape in ((64, 64), (100, 37), (1000, 513), (17, 4096), (3, 130, 70), (2, 5, 65, 129)):
+            base = torch.randint(-100, 100, shape, generator=g).to(dtype).cuda()
+            view = base.transpose(-1, -2)
+            assert not view.is_contiguous()
+            assert torch.equal(dense(view), view.contiguous()), (dtype, shape)
+        wide = torch.randint(-100, 100, (300, 512), generator=g).to(dtype).cuda()
+        view = wide[:, 7:200].t()                       # source rows longer than the part copied
+        assert torch.equal(dense(view), view.contiguous()), dtype
+        dst = torch.zeros(193, 400, dtype=dtype, device="cuda")[:, :300]   # destination rows longer too
+        assert torch.equal(copy_into(dst, view), view)
+    # a permutation that is not a (batched) 2-D transposition keeps using the strided kernel
+    x = torch.randn(6, 7, 40, 50, generator=g).cuda().permute(3, 0, 2, 1)
+    assert torch.equal(dense(x), x.contiguous())
