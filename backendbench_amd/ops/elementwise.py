@@ -10,7 +10,7 @@ import math
 import torch
 
 from .. import _lib
-from ._common import cast, copy_into, device_managed, launch, new_dense
+from ._common import cast, copy_into, dense, device_managed, launch, new_dense
 
 
 def _out_like_inputs(shape, dtype, inputs):
@@ -29,6 +29,22 @@ def _out_like_inputs(shape, dtype, inputs):
         if lead.is_contiguous() or out.stride() == lead.stride():  # preserve_format: dense permutations survive
             return out
     return new_dense(shape, dtype, inputs[0].device)
+
+
+def _align_layouts(shape, tensors):
+    """Full-shape operands that disagree on layout run on the strided kernel, where the odd one is
+    read one scattered element per lane.  When some operand is row-major and another is its
+    (batched) transpose, the transpose is made dense first with the tiled transposing copy: two
+    coalesced passes instead of one scattered pass."""
+    full = [t for t in tensors if t.shape == shape]
+    if len(full) < 2 or len(shape) < 2 or not any(t.is_contiguous() for t in full):
+        return tensors
+    out = []
+    for t in tensors:
+        if t.shape == shape and not t.is_contiguous() and t.transpose(-1, -2).is_contiguous():
+            t = dense(t)
+        out.append(t)
+    return out
 
 
 def _broadcast_shape(*shapes):
@@ -88,6 +104,8 @@ def _binary(op, a, b, alpha=1):
     shape = a.shape if a.shape == b.shape else _broadcast_shape(a.shape, b.shape)
     a = cast(a, dtype)
     b = cast(b, dtype)
+    if a.stride() != b.stride():
+        a, b = _align_layouts(shape, (a, b))
     out = _out_like_inputs(shape, dtype, (a, b))
     if out.numel() == 0:
         return out
@@ -282,6 +300,8 @@ def where(condition, self, other):
         shape = _broadcast_shape(condition.shape, self.shape, other.shape)
     a = cast(self, dtype)
     b = cast(other, dtype)
+    if not (condition.stride() == a.stride() == b.stride()):
+        condition, a, b = _align_layouts(shape, (condition, a, b))
     out = _out_like_inputs(shape, dtype, (condition, a, b))
     if out.numel() == 0:
         return out

@@ -27,11 +27,38 @@ def _norm_dims(dim, ndim):
     return dims
 
 
+def _memory_view3(x, dims):
+    """(outer, red, inner) when `x` is a permuted dense tensor whose reduced dims are adjacent *in
+    memory* and whose kept dims lie in memory in their logical order (e.g. the last dim of a
+    transposed matrix): the reduction then runs on the memory as it is, no copy.  None otherwise."""
+    live = [d for d in range(x.dim()) if x.shape[d] != 1]
+    order = sorted(live, key=lambda d: -x.stride(d))          # outermost in memory first
+    expect = 1
+    for d in reversed(order):
+        if x.stride(d) != expect:
+            return None
+        expect *= x.shape[d]
+    red_pos = [i for i, d in enumerate(order) if d in dims]
+    if not red_pos or red_pos != list(range(red_pos[0], red_pos[-1] + 1)):
+        return None
+    kept = [d for d in order if d not in dims]
+    if kept != sorted(kept):
+        return None
+    outer = prod(x.shape[d] for d in order[: red_pos[0]])
+    red = prod(x.shape[d] for d in order[red_pos[0] : red_pos[-1] + 1])
+    inner = prod(x.shape[d] for d in order[red_pos[-1] + 1 :])
+    return outer, red, inner
+
+
 def _view3(x, dims):
     """(dense tensor, outer, red, inner) with the dims in `dims` reduced."""
     nd = x.dim()
     if nd == 0:
         return dense(x), 1, 1, 1
+    if not x.is_contiguous():
+        mem = _memory_view3(x, dims)
+        if mem is not None:
+            return (x,) + mem
     adjacent = dims == list(range(dims[0], dims[-1] + 1))
     if adjacent:
         xd = dense(x)
