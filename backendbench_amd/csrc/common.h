@@ -153,8 +153,7 @@ struct SumOp {
 struct MaxNanOp {
   template <typename T> __device__ __forceinline__ T operator()(T a, T b) const {
     if constexpr (IsFloat<T>::value) {
-      if (a == b) return __builtin_signbit(a) ? b : a;  // +0 above -0 (IEEE 754-2019), whatever the order
-      return (is_nan(a) || a > b) ? a : b;                // b NaN: a > b false -> b
+      return (is_nan(a) || a > b) ? a : b;  // b NaN: a > b false -> b
     } else {
       return a > b ? a : b;
     }

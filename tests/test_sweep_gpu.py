@@ -279,7 +279,7 @@ SWEEP = {
     aten.sum.default: (_full_reduce(True), False),
     aten.mean.dim: (_mean_dim, False),
     aten.mean.default: (_full_reduce(False), False),
-    aten.amax.default: (_amax, False),   # sign of a zero maximum depends on ATen's reduction order; ours is +0 when any +0 ties
+    aten.amax.default: (_amax, False),   # the sign of a zero maximum depends on the reduction order, in ATen as here
     aten.argmax.default: (_argmax, True),
     aten._softmax.default: (_softmax, False),
     aten._log_softmax.default: (_softmax, False),
