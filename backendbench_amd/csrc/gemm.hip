@@ -14,6 +14,7 @@
 //              gemm_mfma_kernel      K tail: global -> registers -> LDS with zero fill.
 //   generic  any strides, bf16 / f16 / f32: 64x64 LDS tile, FMA inner loop.  Correctness
 //            path for shapes the MFMA kernel does not take.
+#include <stdlib.h>
 #include <type_traits>
 
 #include "common.h"
@@ -166,8 +167,9 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
 // 16 KB slice of the (now idle) LDS ring, and reads it back row-major: every global store
 // instruction then writes 8 complete 128-byte rows.  Must be called by all waves after the
 // last barrier of the main loop (the ring is no longer read).
-template <typename T, int MI>
-__device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x16 (&acc)[MI][2], unsigned char* lds,
+// A wave with more than two 32-column blocks (NJ > 2) calls this once per pair of blocks, J0 = 0, 2, ...
+template <typename T, int MI, int J0 = 0, int NJ>
+__device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x16 (&acc)[MI][NJ], unsigned char* lds,
                                                   int wave, int lane, int m0, int n0) {
   const int fr = lane & 31, fg = lane >> 5;
   const T* C = static_cast<const T*>(g.c);
@@ -204,7 +206,7 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
         VecN4<T> r;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float v = g.alpha * acc[i][j][q * 4 + e];
+          const float v = g.alpha * acc[i][J0 + j][q * 4 + e];
           r.v[e] = static_cast<T>(use_c ? v + g.beta * cv[e] : v);
         }
         const int slot = (j * 4 + q) ^ ((row >> 1) & 7);
@@ -716,6 +718,222 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
   }
 
   store_tile_result<T, 4>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
+}
+
+// ---------------------------------------------------------------- MFMA kernel, four waves of 128x128
+// Same LDS layout, fills and step structure as gemm_mfma_dma64_kernel, with the 256x256 tile
+// split over four waves (2x2, one per SIMD) instead of eight: each wave owns 128x128 = 4x4 MFMA
+// blocks (256 fp32 accumulators) and reads 4 + 4 fragments for 16 MFMAs per 16-k sub-step, where
+// the eight-wave form reads 4 + 2 for 8 — one third fewer LDS fragment bytes per flop.  Every
+// lane issues twice the fills (A: region q = wave + 4 i, i < 8; B: q = wave + 4 i, i < 4).
+template <typename T, bool B_NN>
+__global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  using frag_t = typename Mfma<T>::frag;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  const int bm = tm * BM, bn = tn * BN;
+  const T* A = static_cast<const T*>(g.a);
+  const T* B = static_cast<const T*>(g.b);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  const T* a_src[8];
+  const T* b_src[4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int r = 8 * (wave + 4 * i) + (lane >> 3), slot = lane & 7;
+    const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
+    int gr = bm + r;
+    gr = gr < g.M ? gr : g.M - 1;
+    a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if constexpr (B_NN) {
+      const int k = 2 * (wave + 4 * i) + (lane >> 5), pos = lane & 31;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gn = bn + u * 8;
+      gn = gn < g.N ? gn : 0;
+      b_src[i] = B + (int64_t)k * g.ldb + gn;
+    } else {
+      const int r = 16 * (wave + 4 * i) + (lane >> 2), slot = lane & 3;
+      const int c = slot ^ ((r >> 2) & 3);
+      int gn = bn + r;
+      gn = gn < g.N ? gn : g.N - 1;
+      b_src[i] = B + (int64_t)gn * g.ldb + c * 8;
+    }
+  }
+  // Fill requests: A request i (0..7) of the slot at byte offset a_slot, holding steps t, t+1;
+  // B request i (0..3) of step t.
+  auto request_a = [&](int i, int t, uint32_t a_slot) {
+    lds_dma16(lds_base + a_slot + (uint32_t)(wave + 4 * i) * 1024u, a_src[i] + (int64_t)t * BK3);
+  };
+  auto request_b = [&](int i, int t) {
+    lds_dma16(lds_base + kBRing64 + (uint32_t)(t & 3) * kPanel3 + (uint32_t)(wave + 4 * i) * 1024u,
+              b_src[i] + (B_NN ? (int64_t)t * BK3 * g.ldb : (int64_t)t * BK3));
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  const int tr_k = fg * 8 + ((lane & 15) >> 2);
+  const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  // The LDS reads of step t (A in half `half` of a_slot) into one register set, with this step's
+  // eight fill requests threaded behind the reads of the second sub-step in program order — A
+  // request a_first .. a_first+3 of the slot fill_slot (steps ta, ta+1), then the four B requests
+  // of step tb — so that the fills leave the wave one at a time over the second half of the step
+  // instead of as a burst behind the barrier (the burst form ran the all-zero GEMM 20 % slower).
+  auto io_step = [&](int t, uint32_t a_slot, int half, frag_t (&xa)[2][4], frag_t (&xb)[2][4], bool fill_a, int ta,
+                     uint32_t fill_slot, int a_first, bool fill_b, int tb) __attribute__((always_inline)) {
+    const unsigned char* pa = lds + a_slot;
+    const unsigned char* pb = lds + kBRing64 + (t & 3) * kPanel3;
+    auto fill = [&](int q) __attribute__((always_inline)) {
+      if (q < 4) {
+        if (fill_a) request_a(a_first + q, ta, fill_slot);
+      } else if (fill_b) {
+        request_b(q - 4, tb);
+      }
+    };
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        xa[ks][i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 128 + i * 32 + fr, half * 4 + ks * 2 + fg));
+        if (ks == 1) fill(i);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if constexpr (B_NN) {
+          const int k = ks * 16 + tr_k;
+          const int n = wn * 128 + j * 32 + tr_n;
+          const s16x4 lo = lds_read_tr(pb + swz_n(k, n >> 3) + ((n & 7) << 1));
+          const s16x4 hi = lds_read_tr(pb + swz_n(k + 4, n >> 3) + ((n & 7) << 1));
+          xb[ks][j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        } else {
+          xb[ks][j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * 128 + j * 32 + fr, ks * 2 + fg));
+        }
+        if (ks == 1) fill(4 + j);
+      }
+    }
+  };
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto mma_step = [&](frag_t (&xa)[2][4], frag_t (&xb)[2][4]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i][j] = Mfma<T>::run(xb[ks][j], xa[ks][i], acc[i][j]);
+  };
+  auto next_slot = [](uint32_t s) { return s + kASlot64 == (uint32_t)kBRing64 ? 0u : s + kASlot64; };
+
+  // One step = 32 MFMAs.  The LDS reads are spread over the step (16 reads: one behind every
+  // second MFMA; 24 reads with a row-major B: twenty pairs MFMA/read, then every second), and
+  // nothing moves across the end of the step (the compiler would otherwise sink MFMAs below the
+  // barrier and leave the wait for the last read directly behind it).
+#define MI355_MD __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+#define MI355_MDM MI355_MD __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#define MI355_X4(X) X X X X
+#define MI355_W4_SCHEDULE                                                     \
+  if constexpr (B_NN) {                                                       \
+    MI355_X4(MI355_X4(MI355_MD)) MI355_X4(MI355_MD) MI355_X4(MI355_MDM)       \
+  } else {                                                                    \
+    MI355_X4(MI355_MDM) MI355_X4(MI355_MDM) MI355_X4(MI355_MDM) MI355_X4(MI355_MDM) \
+  }                                                                           \
+  __builtin_amdgcn_sched_group_barrier(0x008, 32, 0);                         \
+  __builtin_amdgcn_sched_barrier(0);
+
+  // Fragments are read one whole step ahead: while the MFMAs of step t run from one register
+  // set, the LDS reads of step t+1 fill the other, so no MFMA of a step waits for LDS.  A panel
+  // is therefore read during the step before its own and is free from the barrier that ends
+  // that step.  Every step issues eight fills per lane: step t refills the B slot of step t
+  // with step t+4; the A slot that held steps u, u+1 (u even) is refilled with steps u+6, u+7,
+  // requests 0-3 in step u+1 and 4-7 in step u+2.  At the barrier that ends step t the panels of
+  // step t+2 must have landed, all requested in step t-2 or earlier: only the 16 loads of steps
+  // t-1 and t may still fly.
+  const int nk = g.K / BK3;  // even: K % 64 == 0
+#pragma unroll
+  for (int i = 0; i < 8; ++i) request_a(i, 0, 0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) request_b(i, 0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) request_b(i, 1);
+  if (nk > 2) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) request_a(i, 2, kASlot64);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) request_b(i, 2);
+    if (nk > 4) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) request_a(i, 4, 2 * kASlot64);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) request_b(i, 3);
+  }
+  if (nk > 4) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");  // steps 0 and 1 are in
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  frag_t fa[2][2][4], fb[2][2][4];
+  uint32_t cur = 0;  // A slot of steps t, t+1 (t even)
+  io_step(0, cur, 0, fa[0], fb[0], false, 0, 0u, 0, false, 0);
+  __syncthreads();  // every wave has its fragments of step 0: the B slot of step 0 may be refilled
+  int t = 0;
+  for (; t + 7 < nk; t += 2) {
+    const uint32_t nxt = next_slot(cur);
+    // even step t
+    io_step(t + 1, cur, 1, fa[1], fb[1], true, t + 4, next_slot(nxt), 4, true, t + 4);
+    mma_step(fa[0], fb[0]);
+    MI355_W4_SCHEDULE
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    __syncthreads();
+    // odd step t+1
+    io_step(t + 2, nxt, 0, fa[0], fb[0], true, t + 6, cur, 0, true, t + 5);
+    mma_step(fa[1], fb[1]);
+    MI355_W4_SCHEDULE
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    __syncthreads();
+    cur = nxt;
+  }
+#undef MI355_W4_SCHEDULE
+#undef MI355_X4
+#undef MI355_MDM
+#undef MI355_MD
+  // Last steps: the requests thin out.  fills(s) = loads that step s issues; the barrier that
+  // ends step s lets exactly those of steps s-1 and s fly, as in the steady state.
+  auto fills = [nk](int s) { return (s & 1) ? 4 * (s + 4 < nk) + 4 * (s + 5 < nk) : 8 * (s + 4 < nk); };
+  auto wait_fills = [](int n) {
+    switch (n) {
+      case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+      case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+      case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+      case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+  };
+  for (; t < nk; t += 2) {
+    const uint32_t nxt = next_slot(cur);
+    io_step(t + 1, cur, 1, fa[1], fb[1], t + 4 < nk, t + 4, next_slot(nxt), 4, t + 4 < nk, t + 4);
+    mma_step(fa[0], fb[0]);
+    wait_fills(fills(t - 1) + fills(t));
+    __syncthreads();
+    if (t + 2 < nk) io_step(t + 2, nxt, 0, fa[0], fb[0], t + 6 < nk, t + 6, cur, 0, t + 5 < nk, t + 5);
+    mma_step(fa[1], fb[1]);
+    wait_fills(fills(t) + fills(t + 1));
+    __syncthreads();
+    cur = nxt;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing is in flight: the last two steps issue no fills)
+
+  store_tile_result<T, 4, 0>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 128);
+  store_tile_result<T, 4, 2>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 128 + 64);
 }
 
 // ---------------------------------------------------------------- MFMA kernel, 128x128 tiles
@@ -1327,7 +1545,16 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
       } else if (K % 64 == 0) {
-        kern = b_nt ? (const void*)gemm_mfma_dma64_kernel<T, false> : (const void*)gemm_mfma_dma64_kernel<T, true>;
+        // Four waves of 128x128 run the steady state 3-5 % faster and pay ~2 us more per tile
+        // (two-pass epilogue), which evens out near K = 2048.  MI355_GEMM_WAVES=4|8 forces one form.
+        const char* forced = getenv("MI355_GEMM_WAVES");
+        const bool w4 = forced != nullptr ? forced[0] == '4' : K >= 2048;
+        if (w4) {
+          kern = b_nt ? (const void*)gemm_mfma_w4_kernel<T, false> : (const void*)gemm_mfma_w4_kernel<T, true>;
+          threads = 256;
+        } else {
+          kern = b_nt ? (const void*)gemm_mfma_dma64_kernel<T, false> : (const void*)gemm_mfma_dma64_kernel<T, true>;
+        }
         lds_bytes = kGemmLds64;
       } else {
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;

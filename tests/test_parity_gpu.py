@@ -134,6 +134,35 @@ def test_headline_gemm_full_size(backend, key):
         assert ev.allclose((2 * plain.float()).to(plain.dtype).cpu(), doubled.cpu())
 
 
+@pytest.mark.parametrize("waves", ["4", "8"])
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch):
+    """The 256x256-tile kernels only run when a problem has enough tiles to fill the chip, so the
+    small K-step cases of the edge suite never reach them.  A [3500, K] x [K, 3600] product has
+    14 x 15 tiles (ragged last row and column of tiles); K walks through every prologue / steady /
+    drain length of the 64-k pipelines, the 32-k ring (K % 64 == 32) and the zero-filled K tail.
+    Small-integer operands make the fp32 accumulation exact, so the sampled rows must be
+    bit-equal to the oracle's.  MI355_GEMM_WAVES forces one of the two 64-k kernels (eight waves of
+    128x64 or four of 128x128), which otherwise split the K range between them."""
+    announce(f"large-tile GEMM K loop lengths, {layout}, {waves} waves")
+    monkeypatch.setenv("MI355_GEMM_WAVES", waves)
+    g = torch.Generator().manual_seed(5)
+    M, N = 3500, 3600
+    rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 127, 128, 255, 256, 3327, 3328, 3499])]))
+    for K in (64, 128, 192, 256, 320, 384, 448, 512, 576, 640, 704, 1024, 2048, 2112, 96, 160, 288, 72, 200):
+        a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+        if layout == "nt":
+            b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
+        else:
+            b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
+        out = backend[aten.mm.default](a, b)
+        ref = aten_cpu.reference(aten.mm.default, [a[rows.cuda()], b])
+        assert ev.bit_equal(ref, out[rows.cuda()].cpu()), (layout, K)
+        bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
+        out2 = backend[aten.addmm.default](bias, a, b)
+        assert ev.bit_equal((out.float() + bias.float()).to(torch.bfloat16), out2), (layout, K, "bias")
+
+
 def test_cpu_tensors_round_trip_through_the_gpu(backend):
     """The smoke suite hands CPU tensors (BackendBench/suite/smoke.py:25,30): the result must
     come back on the CPU and match ATen."""
