@@ -175,45 +175,69 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
   const T* C = static_cast<const T*>(g.c);
   const bool use_c = C != nullptr && g.beta != 0.f;
   unsigned char* slab = lds + wave * (MI * 32 * 128);  // MI * 32 rows x 128 bytes
-  // 16-byte slot s of row r lives at slot s ^ ((r/2) % 8): two-way conflicts at most on both sides
+  // A bias row (c broadcast along m: the Linear-layer addmm) is the same for every row of the
+  // tile: its 8 groups of four columns are loaded once, scaled by beta, and reused for all rows.
+  const bool row_bias = use_c && g.c_vec && g.c_rs == 0;
+  float bias[2][4][4];
+  if (row_bias) {
 #pragma unroll
-  for (int i = 0; i < MI; ++i) {
-    const int row = i * 32 + fr;
-    const int m = m0 + row;
-    const int mc = m < g.M ? m : g.M - 1;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int nl = j * 32 + q * 8 + fg * 4;
-        const int n = n0 + nl;
-        // Columns past N are computed on valid addresses and never stored.
-        float cv[4] = {0.f, 0.f, 0.f, 0.f};
-        if (use_c) {
-          if (g.c_vec) {  // N % 4 == 0: a group of four columns is wholly inside or wholly outside
-            const int nv = n + 4 <= g.N ? n : 0;
-            const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (int64_t)mc * g.c_rs + nv);
+        const int n = n0 + j * 32 + q * 8 + fg * 4;
+        const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (n + 4 <= g.N ? n : 0));
 #pragma unroll
-            for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(t.v[e]);
+        for (int e = 0; e < 4; ++e) bias[j][q][e] = g.beta * static_cast<float>(t.v[e]);
+      }
+  }
+  // 16-byte slot s of row r lives at slot s ^ ((r/2) % 8): two-way conflicts at most on both sides
+  auto stage = [&](auto ROW_BIAS) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const int row = i * 32 + fr;
+      const int m = m0 + row;
+      const int mc = m < g.M ? m : g.M - 1;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int nl = j * 32 + q * 8 + fg * 4;
+          const int n = n0 + nl;
+          VecN4<T> r;
+          if constexpr (decltype(ROW_BIAS)::value) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r.v[e] = static_cast<T>(g.alpha * acc[i][J0 + j][q * 4 + e] + bias[j][q][e]);
           } else {
+            // Columns past N are computed on valid addresses and never stored.
+            float cv[4] = {0.f, 0.f, 0.f, 0.f};
+            if (use_c) {
+              if (g.c_vec) {  // N % 4 == 0: a group of four columns is wholly inside or wholly outside
+                const int nv = n + 4 <= g.N ? n : 0;
+                const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (int64_t)mc * g.c_rs + nv);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(t.v[e]);
+              } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  const int ne = n + e < g.N ? n + e : g.N - 1;
+                  cv[e] = static_cast<float>(C[(int64_t)mc * g.c_rs + (int64_t)ne * g.c_cs]);
+                }
+              }
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              const int ne = n + e < g.N ? n + e : g.N - 1;
-              cv[e] = static_cast<float>(C[(int64_t)mc * g.c_rs + (int64_t)ne * g.c_cs]);
+              const float v = g.alpha * acc[i][J0 + j][q * 4 + e];
+              r.v[e] = static_cast<T>(use_c ? v + g.beta * cv[e] : v);
             }
           }
+          const int slot = (j * 4 + q) ^ ((row >> 1) & 7);
+          *reinterpret_cast<VecN4<T>*>(slab + row * 128 + slot * 16 + fg * 8) = r;
         }
-        VecN4<T> r;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float v = g.alpha * acc[i][J0 + j][q * 4 + e];
-          r.v[e] = static_cast<T>(use_c ? v + g.beta * cv[e] : v);
-        }
-        const int slot = (j * 4 + q) ^ ((row >> 1) & 7);
-        *reinterpret_cast<VecN4<T>*>(slab + row * 128 + slot * 16 + fg * 8) = r;
       }
     }
-  }
+  };
+  if (row_bias) stage(std::true_type{});
+  else stage(std::false_type{});
   // same wave wrote and reads: LDS operations of a wave complete in order
   T* D = static_cast<T*>(g.out);
 #pragma unroll
