@@ -1,19 +1,23 @@
 // mm / addmm:  out[M,N] = beta * c + alpha * (a[M,K] @ b[K,N]),  fp32 accumulate.
 //
 //   mfma     bf16 / f16, a K-contiguous, b either K-contiguous ("NT", e.g. weight.t()) or
-//            N-contiguous ("NN", row-major), 16-byte aligned rows.  256x256x32 block tile,
-//            eight wave64 (2x4, two per SIMD), each wave 128x64 = 4x2 v_mfma_f32_32x32x16
-//            tiles with 128 fp32 accumulators; a four-stage 128 KB LDS ring, swizzled so
-//            that the fills and the fragment reads are bank-conflict free.  A row-major B
-//            stays N-contiguous in LDS and is transposed by the LDS read itself
-//            (ds_read_b64_tr_b16).  Block -> tile map groups tiles per XCD so that one L2
-//            serves neighbouring tiles.  Two fill paths:
-//              gemm_mfma_dma_kernel  K % 32 == 0: panels go global -> LDS directly
-//                                    (global_load_lds_dwordx4), three tiles ahead; MFMAs and
-//                                    LDS reads of a wave are interleaved one to one;
-//              gemm_mfma_kernel      K tail: global -> registers -> LDS with zero fill.
-//   generic  any strides, bf16 / f16 / f32: 64x64 LDS tile, FMA inner loop.  Correctness
-//            path for shapes the MFMA kernel does not take.
+//            N-contiguous ("NN", row-major), 16-byte aligned rows.  256x256 block tile, 32-k steps,
+//            v_mfma_f32_32x32x16, LDS panels swizzled so that the fills and the fragment reads
+//            are bank-conflict free.  A row-major B stays N-contiguous in LDS and is transposed
+//            by the LDS read itself (ds_read_b64_tr_b16).  Block -> tile map groups tiles per
+//            XCD so that one L2 serves neighbouring tiles.  By K:
+//              gemm_mfma_w4_kernel     K % 64 == 0, K >= 2048: four waves of 128x128, fragments
+//                                      read a step ahead, fills issued one at a time;
+//              gemm_mfma_dma64_kernel  K % 64 == 0: eight waves of 128x64 (two per SIMD), A
+//                                      fetched in whole 128-byte lines;
+//              gemm_mfma_dma_kernel    K % 32 == 0: as above with a ring of 32-k stages; all three
+//                                      fill LDS directly (global_load_lds_dwordx4);
+//              gemm_mfma_kernel        K tail: global -> registers -> LDS with zero fill.
+//            Problems with few tiles run on 128x128 tiles (two workgroups per CU), split along
+//            K over the chip when the caller provides a workspace.
+//   mfma f32 v_mfma_f32_32x32x2_f32, 128x128 tiles.
+//   generic  any strides and dtypes (f64 accumulates in f64): 64x64 LDS tile, FMA inner loop.
+//            Correctness path for shapes the MFMA kernels do not take.
 #include <stdlib.h>
 #include <type_traits>
 
