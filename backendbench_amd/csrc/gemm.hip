@@ -244,21 +244,26 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
   else stage(std::false_type{});
   // same wave wrote and reads: LDS operations of a wave complete in order
   T* D = static_cast<T*>(g.out);
+  if (g.out_vec) {
 #pragma unroll
-  for (int t = 0; t < MI * 4; ++t) {
-    const int chunk = t * kWave + lane;  // MI * 256 chunks of 16 bytes, 8 per row
-    const int row = chunk >> 3, s = chunk & 7;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(slab + row * 128 + ((s ^ ((row >> 1) & 7)) << 4));
-    const int m = m0 + row, n = n0 + s * 8;
-    if (m >= g.M || n >= g.N) continue;
-    if (g.out_vec) {
+    for (int t = 0; t < MI * 4; ++t) {
+      const int chunk = t * kWave + lane;  // MI * 256 chunks of 16 bytes, 8 per row
+      const int row = chunk >> 3, s = chunk & 7;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(slab + row * 128 + ((s ^ ((row >> 1) & 7)) << 4));
+      const int m = m0 + row, n = n0 + s * 8;
+      if (m >= g.M || n >= g.N) continue;
       *reinterpret_cast<u32x4*>(D + (int64_t)m * g.N + n) = v;
-    } else {  // N not a multiple of 8 (e.g. a 50257-wide vocabulary): rows are misaligned, element stores
-      struct alignas(16) Elems { T v[8]; };
-      const Elems ev = __builtin_bit_cast(Elems, v);
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        if (n + e < g.N) D[(int64_t)m * g.N + n + e] = ev.v[e];
+    }
+  } else {
+    // N not a multiple of 8 (e.g. a 50257-wide vocabulary): the rows of out start at any 2-byte
+    // offset.  One row per store instruction, lane l writes column l: the 64 element stores of an
+    // instruction fall into the same one or two 128-byte lines.
+    const int n = n0 + lane;
+    const int rows = g.M - m0 < MI * 32 ? g.M - m0 : MI * 32;
+#pragma unroll 8
+    for (int row = 0; row < rows; ++row) {
+      const T v = *reinterpret_cast<const T*>(slab + row * 128 + (((lane >> 3) ^ ((row >> 1) & 7)) << 4) + ((lane & 7) << 1));
+      if (n < g.N) D[(int64_t)(m0 + row) * g.N + n] = v;
     }
   }
 }
