@@ -1113,7 +1113,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
 // MFMAs per wave between synchronisations instead of 8) from a ring of eight stages (128 KB).
 template <typename T, bool B_NN, bool SPLIT>
 __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
-  constexpr int S = 8;  // ring depth: two tiles per barrier, requested three pairs ahead
+  constexpr int S = 5;  // ring depth in 64-k pairs
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using frag_t = typename Mfma<T>::frag;
   const int tid = threadIdx.x, lane = tid % kWave;
@@ -1128,26 +1128,28 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   const T* B = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
-  // Region q = wave + 4 i (i < 2) of a panel is LDS bytes [q * 1024, q * 1024 + 1024).
-  const T* a_src[2];
-  const T* b_src[2];
+  // A pair slot (32 KB) holds 64 k of A (128 rows of 128 B, swz_k64) and of B (the same for a
+  // K-contiguous B; 64 k-rows of 256 B, swz_n128, for a row-major one), so every request fetches
+  // whole 128-byte lines.  Region q = wave + 4 i (i < 4) of a panel is its bytes [1024 q, 1024 q + 1024).
+  constexpr int kPairPanel = SBM * 64 * 2;  // 16 KB
+  constexpr int kPairSlot = 2 * kPairPanel;
+  const T* a_src[4];
+  const T* b_src[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < 4; ++i) {
     const int q = wave + 4 * i;
-    {  // K-contiguous A panel: region q = rows 16q .. 16q+15, 4 chunks per row
-      const int r = 16 * q + (lane >> 2), slot = lane & 3;
-      const int c = slot ^ ((r >> 2) & 3);
+    const int r = 8 * q + (lane >> 3), slot = lane & 7;
+    const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
+    {
       int gr = bm + r;
       gr = gr < g.M ? gr : g.M - 1;
       a_src[i] = A + (int64_t)gr * g.lda + c * 8;
     }
     if constexpr (!B_NN) {
-      const int r = 16 * q + (lane >> 2), slot = lane & 3;
-      const int c = slot ^ ((r >> 2) & 3);
       int gn = bn + r;
       gn = gn < g.N ? gn : g.N - 1;
       b_src[i] = B + (int64_t)gn * g.ldb + c * 8;
-    } else {  // N-contiguous B panel: region q = k rows 4q .. 4q+3, 16 units per row
+    } else {  // region q = k rows 4q .. 4q+3, 16 units per row
       const int k = 4 * q + (lane >> 4), pos = lane & 15;
       const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
       int gn = bn + u * 8;
@@ -1155,41 +1157,24 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
       b_src[i] = B + (int64_t)k * g.ldb + gn;
     }
   }
-  auto request_tile = [&](int t) {
-    const uint32_t stage = lds_base + (uint32_t)(t % S) * kSStage;
-    const int64_t k0 = (int64_t)t * BK3;
+  // Fill request f (0..7) of pair q: the four regions of A, then the four of B.
+  auto request = [&](int f, int q) {
+    const uint32_t slot = lds_base + (uint32_t)(q % S) * kPairSlot;
+    const int64_t k0 = (int64_t)q * 64;
+    const int i = f & 3;
+    const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
+    if (f < 4) lds_dma16(slot + region, a_src[i] + k0);
+    else if constexpr (!B_NN) lds_dma16(slot + kPairPanel + region, b_src[i] + k0);
+    else lds_dma16(slot + kPairPanel + region, b_src[i] + k0 * g.ldb);
+  };
+  auto request_pair = [&](int q) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
-      lds_dma16(stage + region, a_src[i] + k0);
-      if constexpr (!B_NN) lds_dma16(stage + kSPanel + region, b_src[i] + k0);
-      else lds_dma16(stage + kSPanel + region, b_src[i] + k0 * g.ldb);
-    }
+    for (int f = 0; f < 8; ++f) request(f, q);
   };
 
   const int fr = lane & 31, fg = lane >> 5;
   const int tr_k = fg * 8 + ((lane & 15) >> 2);
   const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
-  auto read_frags = [&](int t, int ks, frag_t (&fa)[2], frag_t (&fb)[2]) {
-    const unsigned char* pa = lds + (t % S) * kSStage;
-    const unsigned char* pb = pa + kSPanel;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-      fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k32(wm * 64 + i * 32 + fr, ks * 2 + fg));
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      if constexpr (!B_NN) {
-        fb[j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * 64 + j * 32 + fr, ks * 2 + fg));
-      } else {
-        const int k = ks * 16 + tr_k;
-        const int n = wn * 64 + j * 32 + tr_n;
-        const s16x4 lo = lds_read_tr(pb + swz_n128(k, n >> 3) + ((n & 7) << 1));
-        const s16x4 hi = lds_read_tr(pb + swz_n128(k + 4, n >> 3) + ((n & 7) << 1));
-        fb[j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-      }
-    }
-  };
-
   f32x16 acc[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -1197,52 +1182,110 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  auto mma = [&](frag_t (&fa)[2], frag_t (&fb)[2]) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
-  };
-
-  // Two 32-k tiles per barrier.  Pair p = tiles 2p, 2p+1; tiles 2p+6, 2p+7 are requested at its
-  // start into the slots pair p-1 left.  The first fragments of tile 2p+2 are read before the
-  // barrier that ends pair p, so at the end of pair p every tile up to 2p+4 must have landed:
-  // the twelve loads of tiles 2p+5 .. 2p+7 may still fly.  K % 64 == 0.
-  const int nk = (kend - kbeg) / BK3;
-  for (int t = 0; t < 6 && t < nk; ++t) request_tile(t);
-  if (nk >= 6) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  // One step = one pair of 32-k tiles = 16 MFMAs per wave.  Fragments are read one whole step
+  // ahead: step p computes pair p from one register set while the LDS reads of pair p+1 fill the
+  // other, so no MFMA waits for LDS; pair p is therefore read during step p-1 and its two slots
+  // are free from the barrier that ends that step.  Step p requests pair p+5 into them, its
+  // eight loads issued one at a time behind the LDS reads (a burst behind the barrier stalls the
+  // whole workgroup on its slowest wave).  At the barrier that ends step p the pairs up to p+2
+  // must have landed: the 24 loads of steps p-2 .. p may still fly.  With one workgroup per CU
+  // the kernel is bound by the latency of these fills; four pairs (128 KB) in flight are what the
+  // LDS of a CU can hold.  K % 64 == 0.
+  const int np = (kend - kbeg) / (2 * BK3);
+  for (int q = 0; q < S && q < np; ++q) request_pair(q);
+  if (np >= 5) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");  // pairs 0 and 1 are in
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  frag_t fa0[2], fb0[2], fa1[2], fb1[2];
-  read_frags(0, 0, fa0, fb0);
-  int t0 = 0;
-  for (; t0 + 7 < nk; t0 += 2) {
-    request_tile(t0 + 6);
-    request_tile(t0 + 7);
-    read_frags(t0, 1, fa1, fb1);
-    mma(fa0, fb0);
-    read_frags(t0 + 1, 0, fa0, fb0);
-    mma(fa1, fb1);
-    read_frags(t0 + 1, 1, fa1, fb1);
-    mma(fa0, fb0);
-    read_frags(t0 + 2, 0, fa0, fb0);
-    mma(fa1, fb1);
-    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  frag_t fa[2][4][2], fb[2][4][2];  // [register set][tile of the pair * 2 + 16-k sub-step][block]
+  // LDS reads of pair q into one register set; `after(f)` runs behind fragment group f (0..7).
+  auto read_pair = [&](int q, frag_t (&xa)[4][2], frag_t (&xb)[4][2], auto after) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {  // 16-k sub-step u of the pair: chunks 2u, 2u+1 of the 128-byte rows
+      const unsigned char* pa = lds + (q % S) * kPairSlot;
+      const unsigned char* pb = pa + kPairPanel;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        xa[u][i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 64 + i * 32 + fr, u * 2 + fg));
+      after(2 * u);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if constexpr (!B_NN) {
+          xb[u][j] = *reinterpret_cast<const frag_t*>(pb + swz_k64(wn * 64 + j * 32 + fr, u * 2 + fg));
+        } else {
+          const int k = u * 16 + tr_k;
+          const int n = wn * 64 + j * 32 + tr_n;
+          const s16x4 lo = lds_read_tr(pb + swz_n128(k, n >> 3) + ((n & 7) << 1));
+          const s16x4 hi = lds_read_tr(pb + swz_n128(k + 4, n >> 3) + ((n & 7) << 1));
+          xb[u][j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      }
+      after(2 * u + 1);
+    }
+  };
+  auto mma_pair = [&](frag_t (&xa)[4][2], frag_t (&xb)[4][2]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(xb[u][j], xa[u][i], acc[i][j]);
+  };
+  // The LDS reads go behind the first eight MFMAs of a step (two each, three with a row-major
+  // B), the other eight MFMAs cover the latency of the last read, and nothing moves across the
+  // end of the step.
+#define MI355_MDD                                                                             \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0);
+#define MI355_X4(X) X X X X
+#define MI355_PAIR_SCHEDULE                                                   \
+  MI355_X4(MI355_MDD) MI355_X4(MI355_MDD)                                     \
+  __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);                         \
+  __builtin_amdgcn_sched_barrier(0);
+
+  read_pair(0, fa[0], fb[0], [](int) {});
+  __syncthreads();  // every wave has its fragments of pair 0: its slots may be refilled
+  int p = 0;
+  for (; p + 6 < np; p += 2) {
+    read_pair(p + 1, fa[1], fb[1], [&](int f) { request(f, p + 5); });
+    mma_pair(fa[0], fb[0]);
+    MI355_PAIR_SCHEDULE
+    asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    __syncthreads();
+    read_pair(p + 2, fa[0], fb[0], [&](int f) { request(f, p + 6); });
+    mma_pair(fa[1], fb[1]);
+    MI355_PAIR_SCHEDULE
+    asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
     __syncthreads();
   }
-  for (; t0 < nk; t0 += 2) {  // drain: nothing left to request
-    read_frags(t0, 1, fa1, fb1);
-    mma(fa0, fb0);
-    read_frags(t0 + 1, 0, fa0, fb0);
-    mma(fa1, fb1);
-    read_frags(t0 + 1, 1, fa1, fb1);
-    mma(fa0, fb0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#undef MI355_PAIR_SCHEDULE
+#undef MI355_X4
+#undef MI355_MDD
+  // Last steps: the requests stop at pair np-1; each barrier lets the loads of its last three steps fly.
+  auto fills = [np](int q) { return q + 5 < np ? 8 : 0; };
+  auto wait_fills = [](int n) {
+    if (n == 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else if (n == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else if (n == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+  for (; p < np; p += 2) {
+    if (p + 1 < np) {
+      const bool fill = p + 5 < np;
+      read_pair(p + 1, fa[1], fb[1], [&](int f) { if (fill) request(f, p + 5); });
+    }
+    mma_pair(fa[0], fb[0]);
+    wait_fills(fills(p - 2) + fills(p - 1) + fills(p));
     __syncthreads();
-    if (t0 + 2 < nk) read_frags(t0 + 2, 0, fa0, fb0);
-    mma(fa1, fb1);
+    if (p + 1 < np) {
+      if (p + 2 < np) {
+        const bool fill = p + 6 < np;
+        read_pair(p + 2, fa[0], fb[0], [&](int f) { if (fill) request(f, p + 6); });
+      }
+      mma_pair(fa[1], fb[1]);
+      wait_fills(fills(p - 1) + fills(p) + fills(p + 1));
+      __syncthreads();
+    }
   }
-  __syncthreads();  // the epilogue reuses the ring
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing is in flight: the last steps issue no fills)
 
   if constexpr (SPLIT) store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
   else store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
@@ -1566,7 +1609,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         }
         // At most one workgroup per CU and whole pairs of tiles per split: two tiles per barrier.
         const bool pairs = nblocks * nsplit <= kNumCU && K % 64 == 0 && (!split || sp.ksplit % 64 == 0);
-        lds_bytes = pairs ? 8 * kSStage : kSmallLds;
+        lds_bytes = pairs ? 10 * kSStage : kSmallLds;
         if (pairs) {
           if (split) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, true> : (const void*)gemm_mfma_small2_kernel<T, true, true>;
           else kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, false> : (const void*)gemm_mfma_small2_kernel<T, true, false>;
