@@ -19,6 +19,7 @@
 //   generic  any strides and dtypes (f64 accumulates in f64): 64x64 LDS tile, FMA inner loop.
 //            Correctness path for shapes the MFMA kernels do not take.
 #include <stdlib.h>
+#include <string.h>
 #include <type_traits>
 
 #include "common.h"
@@ -753,14 +754,24 @@ __global__ __launch_bounds__(512) void gemm_mfma_dma64_kernel(GemmArgs g) {
   store_tile_result<T, 4>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 64);
 }
 
+constexpr int SBM = 128, SBN = 128;
+// N-contiguous B panel of the 128-wide tile: 256 B per k row, 64-byte segments rotated by k % 4.
+__device__ __forceinline__ int swz_n128(int k, int u) {
+  return k * (SBN * 2) + ((((u >> 2) ^ (k & 3))) << 6) + ((u & 3) << 4);
+}
+
 // ---------------------------------------------------------------- MFMA kernel, four waves of 128x128
 // Same LDS layout, fills and step structure as gemm_mfma_dma64_kernel, with the 256x256 tile
 // split over four waves (2x2, one per SIMD) instead of eight: each wave owns 128x128 = 4x4 MFMA
 // blocks (256 fp32 accumulators) and reads 4 + 4 fragments for 16 MFMAs per 16-k sub-step, where
 // the eight-wave form reads 4 + 2 for 8 — one third fewer LDS fragment bytes per flop.  Every
 // lane issues twice the fills (A: region q = wave + 4 i, i < 8; B: q = wave + 4 i, i < 4).
-template <typename T, bool B_NN>
+// NJ = 2 is the same kernel on a 256x128 tile (wave tiles of 128x64, half the B panel) for
+// problems that do not fill the chip with 256x256 tiles.
+template <typename T, bool B_NN, int NJ>
 __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
+  static_assert(NJ == 2 || NJ == 4, "wave tile is 128 x 32 NJ");
+  constexpr int BNT = NJ * 64;  // tile width
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using frag_t = typename Mfma<T>::frag;
   const int tid = threadIdx.x, lane = tid % kWave;
@@ -768,13 +779,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   const int wm = wave >> 1, wn = wave & 1;
   int tm, tn;
   tile_coords(g, tm, tn);
-  const int bm = tm * BM, bn = tn * BN;
+  const int bm = tm * BM, bn = tn * BNT;
   const T* A = static_cast<const T*>(g.a);
   const T* B = static_cast<const T*>(g.b);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
   const T* a_src[8];
-  const T* b_src[4];
+  const T* b_src[NJ];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int r = 8 * (wave + 4 * i) + (lane >> 3), slot = lane & 7;
@@ -784,9 +795,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
     a_src[i] = A + (int64_t)gr * g.lda + c * 8;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if constexpr (B_NN) {
+  for (int i = 0; i < NJ; ++i) {
+    if constexpr (B_NN && NJ == 4) {  // 512-byte k-rows (swz_n): region = two k-rows
       const int k = 2 * (wave + 4 * i) + (lane >> 5), pos = lane & 31;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gn = bn + u * 8;
+      gn = gn < g.N ? gn : 0;
+      b_src[i] = B + (int64_t)k * g.ldb + gn;
+    } else if constexpr (B_NN) {  // 256-byte k-rows (swz_n128): region = four k-rows
+      const int k = 4 * (wave + 4 * i) + (lane >> 4), pos = lane & 15;
       const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
       int gn = bn + u * 8;
       gn = gn < g.N ? gn : 0;
@@ -800,7 +817,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
     }
   }
   // Fill requests: A request i (0..7) of the slot at byte offset a_slot, holding steps t, t+1;
-  // B request i (0..3) of step t.
+  // B request i (0..NJ-1) of step t.
   auto request_a = [&](int i, int t, uint32_t a_slot) {
     lds_dma16(lds_base + a_slot + (uint32_t)(wave + 4 * i) * 1024u, a_src[i] + (int64_t)t * BK3);
   };
@@ -817,7 +834,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   // request a_first .. a_first+3 of the slot fill_slot (steps ta, ta+1), then the four B requests
   // of step tb — so that the fills leave the wave one at a time over the second half of the step
   // instead of as a burst behind the barrier (the burst form ran the all-zero GEMM 20 % slower).
-  auto io_step = [&](int t, uint32_t a_slot, int half, frag_t (&xa)[2][4], frag_t (&xb)[2][4], bool fill_a, int ta,
+  auto io_step = [&](int t, uint32_t a_slot, int half, frag_t (&xa)[2][4], frag_t (&xb)[2][NJ], bool fill_a, int ta,
                      uint32_t fill_slot, int a_first, bool fill_b, int tb) __attribute__((always_inline)) {
     const unsigned char* pa = lds + a_slot;
     const unsigned char* pb = lds + kBRing64 + (t & 3) * kPanel3;
@@ -836,33 +853,35 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
         if (ks == 1) fill(i);
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         if constexpr (B_NN) {
           const int k = ks * 16 + tr_k;
-          const int n = wn * 128 + j * 32 + tr_n;
-          const s16x4 lo = lds_read_tr(pb + swz_n(k, n >> 3) + ((n & 7) << 1));
-          const s16x4 hi = lds_read_tr(pb + swz_n(k + 4, n >> 3) + ((n & 7) << 1));
+          const int n = wn * (NJ * 32) + j * 32 + tr_n;
+          const int off_lo = NJ == 4 ? swz_n(k, n >> 3) : swz_n128(k, n >> 3);
+          const int off_hi = NJ == 4 ? swz_n(k + 4, n >> 3) : swz_n128(k + 4, n >> 3);
+          const s16x4 lo = lds_read_tr(pb + off_lo + ((n & 7) << 1));
+          const s16x4 hi = lds_read_tr(pb + off_hi + ((n & 7) << 1));
           xb[ks][j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         } else {
-          xb[ks][j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * 128 + j * 32 + fr, ks * 2 + fg));
+          xb[ks][j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * (NJ * 32) + j * 32 + fr, ks * 2 + fg));
         }
         if (ks == 1) fill(4 + j);
       }
     }
   };
 
-  f32x16 acc[4][4];
+  f32x16 acc[4][NJ];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  auto mma_step = [&](frag_t (&xa)[2][4], frag_t (&xb)[2][4]) __attribute__((always_inline)) {
+  auto mma_step = [&](frag_t (&xa)[2][4], frag_t (&xb)[2][NJ]) __attribute__((always_inline)) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < NJ; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i][j] = Mfma<T>::run(xb[ks][j], xa[ks][i], acc[i][j]);
   };
@@ -871,12 +890,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   // One step = 32 MFMAs.  The LDS reads are spread over the step (16 reads: one behind every
   // second MFMA; 24 reads with a row-major B: twenty pairs MFMA/read, then every second), and
   // nothing moves across the end of the step (the compiler would otherwise sink MFMAs below the
-  // barrier and leave the wait for the last read directly behind it).
+  // barrier and leave the wait for the last read directly behind it).  NJ = 2: 16 MFMAs, 12
+  // reads (16 with a row-major B), all behind the first twelve (eight) MFMAs.
 #define MI355_MD __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
 #define MI355_MDM MI355_MD __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 #define MI355_X4(X) X X X X
+#define MI355_MDD MI355_MD __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
 #define MI355_W4_SCHEDULE                                                     \
-  if constexpr (B_NN) {                                                       \
+  if constexpr (NJ == 2 && B_NN) {                                            \
+    MI355_X4(MI355_MDD) MI355_X4(MI355_MDD)                                   \
+  } else if constexpr (NJ == 2) {                                             \
+    MI355_X4(MI355_MD) MI355_X4(MI355_MD) MI355_X4(MI355_MD)                  \
+  } else if constexpr (B_NN) {                                                \
     MI355_X4(MI355_X4(MI355_MD)) MI355_X4(MI355_MD) MI355_X4(MI355_MDM)       \
   } else {                                                                    \
     MI355_X4(MI355_MDM) MI355_X4(MI355_MDM) MI355_X4(MI355_MDM) MI355_X4(MI355_MDM) \
@@ -890,31 +915,33 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   // that step.  Every step issues eight fills per lane: step t refills the B slot of step t
   // with step t+4; the A slot that held steps u, u+1 (u even) is refilled with steps u+6, u+7,
   // requests 0-3 in step u+1 and 4-7 in step u+2.  At the barrier that ends step t the panels of
-  // step t+2 must have landed, all requested in step t-2 or earlier: only the 16 loads of steps
-  // t-1 and t may still fly.
+  // step t+2 must have landed, all requested in step t-2 or earlier: only the 2 (4 + NJ) loads of
+  // steps t-1 and t may still fly.
   const int nk = g.K / BK3;  // even: K % 64 == 0
 #pragma unroll
   for (int i = 0; i < 8; ++i) request_a(i, 0, 0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) request_b(i, 0);
+  for (int i = 0; i < NJ; ++i) request_b(i, 0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) request_b(i, 1);
+  for (int i = 0; i < NJ; ++i) request_b(i, 1);
   if (nk > 2) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) request_a(i, 2, kASlot64);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) request_b(i, 2);
+    for (int i = 0; i < NJ; ++i) request_b(i, 2);
     if (nk > 4) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) request_a(i, 4, 2 * kASlot64);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) request_b(i, 3);
+    for (int i = 0; i < NJ; ++i) request_b(i, 3);
   }
-  if (nk > 4) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");  // steps 0 and 1 are in
+  // steps 0 and 1 are in when only the 12 + 2 NJ loads behind them still fly
+  if (nk > 4 && NJ == 4) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+  else if (nk > 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  frag_t fa[2][2][4], fb[2][2][4];
+  frag_t fa[2][2][4], fb[2][2][NJ];
   uint32_t cur = 0;  // A slot of steps t, t+1 (t even)
   io_step(0, cur, 0, fa[0], fb[0], false, 0, 0u, 0, false, 0);
   __syncthreads();  // every wave has its fragments of step 0: the B slot of step 0 may be refilled
@@ -925,29 +952,36 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
     io_step(t + 1, cur, 1, fa[1], fb[1], true, t + 4, next_slot(nxt), 4, true, t + 4);
     mma_step(fa[0], fb[0]);
     MI355_W4_SCHEDULE
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    if constexpr (NJ == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
     __syncthreads();
     // odd step t+1
     io_step(t + 2, nxt, 0, fa[0], fb[0], true, t + 6, cur, 0, true, t + 5);
     mma_step(fa[1], fb[1]);
     MI355_W4_SCHEDULE
-    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    if constexpr (NJ == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
     __syncthreads();
     cur = nxt;
   }
 #undef MI355_W4_SCHEDULE
 #undef MI355_X4
+#undef MI355_MDD
 #undef MI355_MDM
 #undef MI355_MD
   // Last steps: the requests thin out.  fills(s) = loads that step s issues; the barrier that
   // ends step s lets exactly those of steps s-1 and s fly, as in the steady state.
-  auto fills = [nk](int s) { return (s & 1) ? 4 * (s + 4 < nk) + 4 * (s + 5 < nk) : 8 * (s + 4 < nk); };
+  auto fills = [nk](int s) { return (s & 1) ? NJ * (s + 4 < nk) + 4 * (s + 5 < nk) : (4 + NJ) * (s + 4 < nk); };
   auto wait_fills = [](int n) {
     switch (n) {
       case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+      case 14: asm volatile("s_waitcnt vmcnt(14)" ::: "memory"); break;
       case 12: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+      case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
       case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+      case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
       case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
       default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
     }
   };
@@ -965,8 +999,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing is in flight: the last two steps issue no fills)
 
-  store_tile_result<T, 4, 0>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 128);
-  store_tile_result<T, 4, 2>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 128 + 64);
+  store_tile_result<T, 4, 0>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * (NJ * 32));
+  if constexpr (NJ == 4) store_tile_result<T, 4, 2>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 128 + 64);
 }
 
 // ---------------------------------------------------------------- MFMA kernel, 128x128 tiles
@@ -974,14 +1008,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
 // corner (2x2 MFMA blocks, 64 accumulators), 32-k steps, a ring of four 16 KB stages
 // (A 128x32 + B 32x128) filled by global_load_lds_dwordx4 three steps ahead exactly as in
 // gemm_mfma_dma_kernel; 64 KB of LDS, so two workgroups share a CU.  K % 32 == 0.
-constexpr int SBM = 128, SBN = 128;
 constexpr int kSPanel = SBM * BK3 * 2;            // 8 KB per operand per stage
 constexpr int kSStage = 2 * kSPanel;              // 16 KB
 constexpr int kSmallLds = kStages3 * kSStage;     // 64 KB
-// N-contiguous B panel of the 128-wide tile: 256 B per k row, 64-byte segments rotated by k % 4.
-__device__ __forceinline__ int swz_n128(int k, int u) {
-  return k * (SBN * 2) + ((((u >> 2) ^ (k & 3))) << 6) + ((u & 3) << 4);
-}
 
 template <typename T, bool B_NN, bool SPLIT>
 __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
@@ -1193,7 +1222,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   // LDS of a CU can hold.  K % 64 == 0.
   const int np = (kend - kbeg) / (2 * BK3);
   for (int q = 0; q < S && q < np; ++q) request_pair(q);
-  if (np >= 5) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");  // pairs 0 and 1 are in
+  // pairs 0 and 1 are in when only the later ones (at most three) still fly
+  if (np >= 5) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+  else if (np == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  else if (np == 3) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   frag_t fa[2][4][2], fb[2][4][2];  // [register set][tile of the pair * 2 + 16-k sub-step][block]
@@ -1594,8 +1626,21 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       int lds_bytes = kGemmLds;
       int threads = 512;
       int nsplit = 1;
-      // Fewer 256x256 tiles than three quarters of the CUs: 128x128 tiles, two workgroups per CU.
-      if (!ktail && nblocks < kNumCU * 3 / 4) {
+      // Too few 256x256 tiles for the chip but between half a round and one round of 256x128
+      // tiles, and a K loop long enough to amortise the one-workgroup-per-CU pipeline: the
+      // four-wave kernel on 256x128 tiles.  MI355_GEMM_TILE=256x128 forces it (a test knob).
+      const int64_t tiles_mid = (int64_t)g.tiles_m * ((N + 127) / 128);
+      const char* forced_tile = getenv("MI355_GEMM_TILE");
+      const bool mid = !ktail && K % 64 == 0 &&
+                       (forced_tile != nullptr ? strcmp(forced_tile, "256x128") == 0
+                                               : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > kNumCU / 2 && tiles_mid <= kNumCU);
+      if (mid) {
+        g.tiles_n = (int32_t)((N + 127) / 128);
+        nblocks = tiles_mid;
+        kern = b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, 2> : (const void*)gemm_mfma_w4_kernel<T, true, 2>;
+        threads = 256;
+        lds_bytes = kGemmLds64;
+      } else if (!ktail && nblocks < kNumCU * 3 / 4) {  // 128x128 tiles, two workgroups per CU
         g.tiles_m = (int32_t)((M + SBM - 1) / SBM);
         g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
         nblocks = (int64_t)g.tiles_m * g.tiles_n;
@@ -1626,7 +1671,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         const char* forced = getenv("MI355_GEMM_WAVES");
         const bool w4 = forced != nullptr ? forced[0] == '4' : K >= 2048;
         if (w4) {
-          kern = b_nt ? (const void*)gemm_mfma_w4_kernel<T, false> : (const void*)gemm_mfma_w4_kernel<T, true>;
+          kern = b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, 4> : (const void*)gemm_mfma_w4_kernel<T, true, 4>;
           threads = 256;
         } else {
           kern = b_nt ? (const void*)gemm_mfma_dma64_kernel<T, false> : (const void*)gemm_mfma_dma64_kernel<T, true>;
@@ -1636,7 +1681,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
       }
       // More than 64 KB of dynamic LDS needs the attribute once per kernel and process.
-      static thread_local const void* attr_done[16] = {};
+      static thread_local const void* attr_done[24] = {};
       bool seen = false;
       for (const void* k : attr_done) seen = seen || k == kern;
       if (!seen) {

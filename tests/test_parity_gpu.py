@@ -134,7 +134,7 @@ def test_headline_gemm_full_size(backend, key):
         assert ev.allclose((2 * plain.float()).to(plain.dtype).cpu(), doubled.cpu())
 
 
-@pytest.mark.parametrize("waves", ["4", "8"])
+@pytest.mark.parametrize("waves", ["4", "8", "256x128"])
 @pytest.mark.parametrize("layout", ["nt", "nn"])
 def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch):
     """The 256x256-tile kernels only run when a problem has enough tiles to fill the chip, so the
@@ -143,9 +143,13 @@ def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch
     drain length of the 64-k pipelines, the 32-k ring (K % 64 == 32) and the zero-filled K tail.
     Small-integer operands make the fp32 accumulation exact, so the sampled rows must be
     bit-equal to the oracle's.  MI355_GEMM_WAVES forces one of the two 64-k kernels (eight waves of
-    128x64 or four of 128x128), which otherwise split the K range between them."""
-    announce(f"large-tile GEMM K loop lengths, {layout}, {waves} waves")
-    monkeypatch.setenv("MI355_GEMM_WAVES", waves)
+    128x64 or four of 128x128), which otherwise split the K range between them; MI355_GEMM_TILE
+    forces the four-wave kernel on 256x128 tiles for every K that is a multiple of 64."""
+    announce(f"large-tile GEMM K loop lengths, {layout}, {waves}")
+    if waves == "256x128":   # the four-wave kernel on 256x128 tiles, otherwise chosen for mid-sized problems
+        monkeypatch.setenv("MI355_GEMM_TILE", waves)
+    else:
+        monkeypatch.setenv("MI355_GEMM_WAVES", waves)
     g = torch.Generator().manual_seed(5)
     M, N = 3500, 3600
     rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 127, 128, 255, 256, 3327, 3328, 3499])]))
