@@ -1011,6 +1011,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
 constexpr int kSPanel = SBM * BK3 * 2;            // 8 KB per operand per stage
 constexpr int kSStage = 2 * kSPanel;              // 16 KB
 constexpr int kSmallLds = kStages3 * kSStage;     // 64 KB
+constexpr int kSmall2Lds = 5 * 2 * SBM * 64 * 2;  // 160 KB: five pairs of (A 128x64 + B 64x128)
 
 template <typename T, bool B_NN, bool SPLIT>
 __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
@@ -1105,41 +1106,105 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
       for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(fb[j], fa[i], acc[i][j]);
   };
 
-  // At the wait point of step `it`, tile it+2 must have landed (its first fragments are read
-  // before the next barrier); only the newest tile's four loads may still be in flight.
+  // Fragments are read one whole step ahead: step `it` computes tile `it` from one register set
+  // while the LDS reads of tile it+1 fill the other, so no MFMA waits for LDS and the slot of
+  // tile `it`, read during step it-1, is free from the barrier that ends that step.  Step `it`
+  // refills it with tile it+4, its four loads issued one at a time behind the LDS reads.  At the
+  // barrier that ends step `it` tile it+2 must have landed: the eight loads of tiles it+3 and
+  // it+4 may still fly.
   const int nk = (kend - kbeg) / BK3;
-  for (int t = 0; t < S - 1 && t < nk; ++t) request_tile(t);
-  if (nk >= S - 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  for (int t = 0; t < S && t < nk; ++t) request_tile(t);
+  // tiles 0 and 1 are in when only the later ones (at most two) still fly
+  if (nk >= 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  else if (nk == 3) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  frag_t fa0[2], fb0[2], fa1[2], fb1[2];
-  read_frags(0, 0, fa0, fb0);
+  frag_t fa[2][2][2], fb[2][2][2];  // [register set][16-k sub-step][block]
+  auto request1 = [&](int f, int t) {  // request f (0..3) of tile t: A regions, then B regions
+    const uint32_t stage = lds_base + (uint32_t)(t % S) * kSStage;
+    const int64_t k0 = (int64_t)t * BK3;
+    const int i = f & 1;
+    const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
+    if (f < 2) lds_dma16(stage + region, a_src[i] + k0);
+    else if constexpr (!B_NN) lds_dma16(stage + kSPanel + region, b_src[i] + k0);
+    else lds_dma16(stage + kSPanel + region, b_src[i] + k0 * g.ldb);
+  };
+  // LDS reads of tile t into one register set; `after(f)` runs behind fragment group f (0..3).
+  auto read_tile = [&](int t, frag_t (&xa)[2][2], frag_t (&xb)[2][2], auto after) __attribute__((always_inline)) {
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      frag_t ta[2], tb[2];
+      read_frags(t, ks, ta, tb);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) { xa[ks][i] = ta[i]; xb[ks][i] = tb[i]; }
+      after(2 * ks);
+      after(2 * ks + 1);
+    }
+  };
+  auto mma_tile = [&](frag_t (&xa)[2][2], frag_t (&xb)[2][2]) __attribute__((always_inline)) {
+    mma(xa[0], xb[0]);
+    mma(xa[1], xb[1]);
+  };
+  // Eight MFMAs per step; the LDS reads go behind the first four (two each, three with a row-major
+  // B), and nothing moves across the end of the step.
+#define MI355_SMALL_SCHEDULE                                                                               \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);                                                       \
+  __builtin_amdgcn_sched_barrier(0);
+  read_tile(0, fa[0], fb[0], [](int) {});
+  __syncthreads();  // every wave has its fragments of tile 0: its slot may be refilled
   int it = 0;
-  for (; it + S - 1 < nk; ++it) {
-    request_tile(it + S - 1);
-    read_frags(it, 1, fa1, fb1);
-    mma(fa0, fb0);
-    read_frags(it + 1, 0, fa0, fb0);
-    mma(fa1, fb1);
-    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  for (; it + 5 < nk; it += 2) {
+    read_tile(it + 1, fa[1], fb[1], [&](int f) { request1(f, it + 4); });
+    mma_tile(fa[0], fb[0]);
+    MI355_SMALL_SCHEDULE
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __syncthreads();
+    read_tile(it + 2, fa[0], fb[0], [&](int f) { request1(f, it + 5); });
+    mma_tile(fa[1], fb[1]);
+    MI355_SMALL_SCHEDULE
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     __syncthreads();
   }
-  for (; it < nk; ++it) {  // drain: nothing left to request
-    read_frags(it, 1, fa1, fb1);
-    mma(fa0, fb0);
-    if (it + 1 < nk) read_frags(it + 1, 0, fa0, fb0);
-    mma(fa1, fb1);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#undef MI355_SMALL_SCHEDULE
+  // Last steps: the requests stop at tile nk-1; each barrier lets the loads of its last two steps fly.
+  auto fills = [nk](int q) { return q + 4 < nk ? 4 : 0; };
+  auto wait_fills = [](int n) {
+    if (n == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if (n == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  };
+  for (; it < nk; it += 2) {
+    if (it + 1 < nk) {
+      const bool fill = it + 4 < nk;
+      read_tile(it + 1, fa[1], fb[1], [&](int f) { if (fill) request1(f, it + 4); });
+    }
+    mma_tile(fa[0], fb[0]);
+    wait_fills(fills(it - 1) + fills(it));
     __syncthreads();
+    if (it + 1 < nk) {
+      if (it + 2 < nk) {
+        const bool fill = it + 5 < nk;
+        read_tile(it + 2, fa[0], fb[0], [&](int f) { if (fill) request1(f, it + 5); });
+      }
+      mma_tile(fa[1], fb[1]);
+      wait_fills(fills(it) + fills(it + 1));
+      __syncthreads();
+    }
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing is in flight: the last steps issue no fills)
 
   if constexpr (SPLIT) store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
   else store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
 }
 
-// Variant of gemm_mfma_small_kernel for launches with at most one workgroup per CU: nothing else
-// hides a workgroup's barrier and LDS latencies there, so it takes two tiles per barrier (16
-// MFMAs per wave between synchronisations instead of 8) from a ring of eight stages (128 KB).
+// The 128x128 tile for launches with at most one workgroup per CU: nothing else hides a
+// workgroup's barrier, LDS and fill latencies there, so it owns the whole 160 KB of LDS (a ring of
+// five 64-k pairs, every request a whole 128-byte line), works in 64-k steps (16 MFMAs per wave
+// between barriers instead of 8) and reads its fragments a step ahead.
 template <typename T, bool B_NN, bool SPLIT>
 __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   constexpr int S = 5;  // ring depth in 64-k pairs
@@ -1652,9 +1717,9 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
           g.ws = static_cast<float*>(workspace);
           g.ksplit = sp.ksplit;
         }
-        // At most one workgroup per CU and whole pairs of tiles per split: two tiles per barrier.
+        // At most one workgroup per CU and whole 64-k pairs per split: the deep-ring kernel.
         const bool pairs = nblocks * nsplit <= kNumCU && K % 64 == 0 && (!split || sp.ksplit % 64 == 0);
-        lds_bytes = pairs ? 10 * kSStage : kSmallLds;
+        lds_bytes = pairs ? kSmall2Lds : kSmallLds;
         if (pairs) {
           if (split) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, true> : (const void*)gemm_mfma_small2_kernel<T, true, true>;
           else kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, false> : (const void*)gemm_mfma_small2_kernel<T, true, false>;
