@@ -167,6 +167,30 @@ def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch
         assert ev.bit_equal((out.float() + bias.float()).to(torch.bfloat16), out2), (layout, K, "bias")
 
 
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+@pytest.mark.parametrize("shape", [(700, 900), (2000, 2500)])
+def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
+    """The 128x128-tile kernels: [700, K] x [K, 900] has 6 x 8 tiles, at most one workgroup per CU
+    (the deep-ring kernel when K is a multiple of 64, split along K once K is long enough for the
+    planner); [2000, K] x [K, 2500] has 16 x 20, more than one per CU (the two-per-CU kernel).  K
+    walks through every prologue / steady / drain length of both pipelines.  Small-integer operands
+    make the fp32 accumulation exact in any order, so the sampled rows must be bit-equal to the
+    oracle's."""
+    M, N = shape
+    announce(f"small-tile GEMM K loop lengths, {layout}, {M}x{N}")
+    g = torch.Generator().manual_seed(6)
+    rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 63, 64, 127, 128, M - 129, M - 128, M - 1])]))
+    for K in (32, 64, 96, 128, 160, 192, 224, 256, 320, 384, 448, 512, 576, 640, 704, 1056, 2080, 4096):
+        a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+        if layout == "nt":
+            b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
+        else:
+            b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
+        out = backend[aten.mm.default](a, b)
+        ref = aten_cpu.reference(aten.mm.default, [a[rows.cuda()], b])
+        assert ev.bit_equal(ref, out[rows.cuda()].cpu()), (layout, shape, K)
+
+
 def test_cpu_tensors_round_trip_through_the_gpu(backend):
     """The smoke suite hands CPU tensors (BackendBench/suite/smoke.py:25,30): the result must
     come back on the CPU and match ATen."""
