@@ -1,7 +1,7 @@
 // mm / addmm:  out[M,N] = beta * c + alpha * (a[M,K] @ b[K,N]),  fp32 accumulate.
 //
-//   mfma     bf16 / f16, a K-contiguous, b either K-contiguous ("NT", e.g. weight.t()) or
-//            N-contiguous ("NN", row-major), 16-byte aligned rows.  256x256 block tile, 32-k steps,
+//   mfma     bf16 / f16, a K-contiguous (or M-contiguous, a transposed view, when K % 64 == 0), b either
+//            K-contiguous ("NT", e.g. weight.t()) or N-contiguous ("NN", row-major), 16-byte aligned rows.  256x256 block tile, 32-k steps,
 //            v_mfma_f32_32x32x16, LDS panels swizzled so that the fills and the fragment reads
 //            are bank-conflict free.  A row-major B stays N-contiguous in LDS and is transposed
 //            by the LDS read itself (ds_read_b64_tr_b16).  Block -> tile map groups tiles per
@@ -768,7 +768,9 @@ __device__ __forceinline__ int swz_n128(int k, int u) {
 // lane issues twice the fills (A: region q = wave + 4 i, i < 8; B: q = wave + 4 i, i < 4).
 // NJ = 2 is the same kernel on a 256x128 tile (wave tiles of 128x64, half the B panel) for
 // problems that do not fill the chip with 256x256 tiles.
-template <typename T, bool B_NN, int NJ>
+// A_T: the left operand is M-contiguous (a transposed view, e.g. x.t() @ dy): its panel stays k-major
+// in LDS like a row-major B and is transposed by the LDS read.
+template <typename T, bool B_NN, int NJ, bool A_T>
 __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   static_assert(NJ == 2 || NJ == 4, "wave tile is 128 x 32 NJ");
   constexpr int BNT = NJ * 64;  // tile width
@@ -788,11 +790,19 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   const T* b_src[NJ];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int r = 8 * (wave + 4 * i) + (lane >> 3), slot = lane & 7;
-    const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
-    int gr = bm + r;
-    gr = gr < g.M ? gr : g.M - 1;
-    a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+    if constexpr (A_T) {  // M-contiguous A: the pair slot holds 64 k-rows of 512 B (swz_n), region = two k-rows
+      const int k = 2 * (wave + 4 * i) + (lane >> 5), pos = lane & 31;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gm = bm + u * 8;
+      gm = gm < g.M ? gm : 0;
+      a_src[i] = A + (int64_t)k * g.lda + gm;
+    } else {
+      const int r = 8 * (wave + 4 * i) + (lane >> 3), slot = lane & 7;
+      const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
+      int gr = bm + r;
+      gr = gr < g.M ? gr : g.M - 1;
+      a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+    }
   }
 #pragma unroll
   for (int i = 0; i < NJ; ++i) {
@@ -819,7 +829,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   // Fill requests: A request i (0..7) of the slot at byte offset a_slot, holding steps t, t+1;
   // B request i (0..NJ-1) of step t.
   auto request_a = [&](int i, int t, uint32_t a_slot) {
-    lds_dma16(lds_base + a_slot + (uint32_t)(wave + 4 * i) * 1024u, a_src[i] + (int64_t)t * BK3);
+    lds_dma16(lds_base + a_slot + (uint32_t)(wave + 4 * i) * 1024u,
+              a_src[i] + (A_T ? (int64_t)t * BK3 * g.lda : (int64_t)t * BK3));
   };
   auto request_b = [&](int i, int t) {
     lds_dma16(lds_base + kBRing64 + (uint32_t)(t & 3) * kPanel3 + (uint32_t)(wave + 4 * i) * 1024u,
@@ -849,7 +860,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
     for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        xa[ks][i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 128 + i * 32 + fr, half * 4 + ks * 2 + fg));
+        if constexpr (A_T) {
+          const int k = half * 32 + ks * 16 + tr_k;
+          const int m = wm * 128 + i * 32 + tr_n;
+          const s16x4 lo = lds_read_tr(pa + swz_n(k, m >> 3) + ((m & 7) << 1));
+          const s16x4 hi = lds_read_tr(pa + swz_n(k + 4, m >> 3) + ((m & 7) << 1));
+          xa[ks][i] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        } else {
+          xa[ks][i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 128 + i * 32 + fr, half * 4 + ks * 2 + fg));
+        }
         if (ks == 1) fill(i);
       }
 #pragma unroll
@@ -897,7 +916,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
 #define MI355_X4(X) X X X X
 #define MI355_MDD MI355_MD __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
 #define MI355_W4_SCHEDULE                                                     \
-  if constexpr (NJ == 2 && B_NN) {                                            \
+  if constexpr (NJ == 4 && A_T && B_NN) {      /* 32 reads, 32 MFMAs */       \
+    MI355_X4(MI355_MDD) MI355_X4(MI355_MDD) MI355_X4(MI355_X4(MI355_MD))      \
+  } else if constexpr (NJ == 4 && A_T) {       /* 24 reads */                 \
+    MI355_X4(MI355_X4(MI355_MD)) MI355_X4(MI355_MD) MI355_X4(MI355_MDM)       \
+  } else if constexpr (NJ == 2 && A_T && B_NN) { /* 24 reads, 16 MFMAs */     \
+    MI355_X4(MI355_MDD) MI355_X4(MI355_MDD) MI355_X4(MI355_MDD)               \
+  } else if constexpr (NJ == 2 && A_T) {       /* 20 reads */                 \
+    MI355_X4(MI355_MDD) MI355_X4(MI355_MDD) MI355_X4(MI355_MD)                \
+  } else if constexpr (NJ == 2 && B_NN) {                                     \
     MI355_X4(MI355_MDD) MI355_X4(MI355_MDD)                                   \
   } else if constexpr (NJ == 2) {                                             \
     MI355_X4(MI355_MD) MI355_X4(MI355_MD) MI355_X4(MI355_MD)                  \
@@ -1013,7 +1040,7 @@ constexpr int kSStage = 2 * kSPanel;              // 16 KB
 constexpr int kSmallLds = kStages3 * kSStage;     // 64 KB
 constexpr int kSmall2Lds = 5 * 2 * SBM * 64 * 2;  // 160 KB: five pairs of (A 128x64 + B 64x128)
 
-template <typename T, bool B_NN, bool SPLIT>
+template <typename T, bool B_NN, bool SPLIT, bool A_T>
 __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
   constexpr int S = kStages3;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -1026,7 +1053,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
   const int bm = tm * SBM, bn = tn * SBN;
   const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
   const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
-  const T* A = static_cast<const T*>(g.a) + kbeg;
+  const T* A = static_cast<const T*>(g.a) + (A_T ? (int64_t)kbeg * g.lda : (int64_t)kbeg);
   const T* B = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
@@ -1036,7 +1063,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int q = wave + 4 * i;
-    {  // K-contiguous A panel: region q = rows 16q .. 16q+15, 4 chunks per row
+    if constexpr (A_T) {  // M-contiguous A panel (swz_n128): region q = k rows 4q .. 4q+3, 16 units per row
+      const int k = 4 * q + (lane >> 4), pos = lane & 15;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gm = bm + u * 8;
+      gm = gm < g.M ? gm : 0;
+      a_src[i] = A + (int64_t)k * g.lda + gm;
+    } else {  // K-contiguous A panel: region q = rows 16q .. 16q+15, 4 chunks per row
       const int r = 16 * q + (lane >> 2), slot = lane & 3;
       const int c = slot ^ ((r >> 2) & 3);
       int gr = bm + r;
@@ -1063,7 +1096,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
-      lds_dma16(stage + region, a_src[i] + k0);
+      lds_dma16(stage + region, a_src[i] + (A_T ? k0 * g.lda : k0));
       if constexpr (!B_NN) lds_dma16(stage + kSPanel + region, b_src[i] + k0);
       else lds_dma16(stage + kSPanel + region, b_src[i] + k0 * g.ldb);
     }
@@ -1076,8 +1109,17 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
     const unsigned char* pa = lds + (t % S) * kSStage;
     const unsigned char* pb = pa + kSPanel;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k32(wm * 64 + i * 32 + fr, ks * 2 + fg));
+    for (int i = 0; i < 2; ++i) {
+      if constexpr (A_T) {
+        const int k = ks * 16 + tr_k;
+        const int m = wm * 64 + i * 32 + tr_n;
+        const s16x4 lo = lds_read_tr(pa + swz_n128(k, m >> 3) + ((m & 7) << 1));
+        const s16x4 hi = lds_read_tr(pa + swz_n128(k + 4, m >> 3) + ((m & 7) << 1));
+        fa[i] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      } else {
+        fa[i] = *reinterpret_cast<const frag_t*>(pa + swz_k32(wm * 64 + i * 32 + fr, ks * 2 + fg));
+      }
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       if constexpr (!B_NN) {
@@ -1125,7 +1167,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
     const int64_t k0 = (int64_t)t * BK3;
     const int i = f & 1;
     const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
-    if (f < 2) lds_dma16(stage + region, a_src[i] + k0);
+    if (f < 2) lds_dma16(stage + region, a_src[i] + (A_T ? k0 * g.lda : k0));
     else if constexpr (!B_NN) lds_dma16(stage + kSPanel + region, b_src[i] + k0);
     else lds_dma16(stage + kSPanel + region, b_src[i] + k0 * g.ldb);
   };
@@ -1148,10 +1190,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
   // Eight MFMAs per step; the LDS reads go behind the first four (two each, three with a row-major
   // B), and nothing moves across the end of the step.
 #define MI355_SMALL_SCHEDULE                                                                               \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0); \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0); \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0); \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 2 + (B_NN ? 1 : 0) + (A_T ? 1 : 0), 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 2 + (B_NN ? 1 : 0) + (A_T ? 1 : 0), 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 2 + (B_NN ? 1 : 0) + (A_T ? 1 : 0), 0); \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 2 + (B_NN ? 1 : 0) + (A_T ? 1 : 0), 0); \
   __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);                                                       \
   __builtin_amdgcn_sched_barrier(0);
   read_tile(0, fa[0], fb[0], [](int) {});
@@ -1205,7 +1247,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
 // workgroup's barrier, LDS and fill latencies there, so it owns the whole 160 KB of LDS (a ring of
 // five 64-k pairs, every request a whole 128-byte line), works in 64-k steps (16 MFMAs per wave
 // between barriers instead of 8) and reads its fragments a step ahead.
-template <typename T, bool B_NN, bool SPLIT>
+template <typename T, bool B_NN, bool SPLIT, bool A_T>
 __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   constexpr int S = 5;  // ring depth in 64-k pairs
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -1218,7 +1260,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   const int bm = tm * SBM, bn = tn * SBN;
   const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
   const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
-  const T* A = static_cast<const T*>(g.a) + kbeg;
+  const T* A = static_cast<const T*>(g.a) + (A_T ? (int64_t)kbeg * g.lda : (int64_t)kbeg);
   const T* B = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
@@ -1234,7 +1276,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
     const int q = wave + 4 * i;
     const int r = 8 * q + (lane >> 3), slot = lane & 7;
     const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
-    {
+    if constexpr (A_T) {  // M-contiguous A: 64 k-rows of 256 B (swz_n128), region q = k rows 4q .. 4q+3
+      const int k = 4 * q + (lane >> 4), pos = lane & 15;
+      const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+      int gm = bm + u * 8;
+      gm = gm < g.M ? gm : 0;
+      a_src[i] = A + (int64_t)k * g.lda + gm;
+    } else {
       int gr = bm + r;
       gr = gr < g.M ? gr : g.M - 1;
       a_src[i] = A + (int64_t)gr * g.lda + c * 8;
@@ -1257,7 +1305,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
     const int64_t k0 = (int64_t)q * 64;
     const int i = f & 3;
     const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
-    if (f < 4) lds_dma16(slot + region, a_src[i] + k0);
+    if (f < 4) lds_dma16(slot + region, a_src[i] + (A_T ? k0 * g.lda : k0));
     else if constexpr (!B_NN) lds_dma16(slot + kPairPanel + region, b_src[i] + k0);
     else lds_dma16(slot + kPairPanel + region, b_src[i] + k0 * g.ldb);
   };
@@ -1301,8 +1349,17 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
       const unsigned char* pa = lds + (q % S) * kPairSlot;
       const unsigned char* pb = pa + kPairPanel;
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
-        xa[u][i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 64 + i * 32 + fr, u * 2 + fg));
+      for (int i = 0; i < 2; ++i) {
+        if constexpr (A_T) {
+          const int k = u * 16 + tr_k;
+          const int m = wm * 64 + i * 32 + tr_n;
+          const s16x4 lo = lds_read_tr(pa + swz_n128(k, m >> 3) + ((m & 7) << 1));
+          const s16x4 hi = lds_read_tr(pa + swz_n128(k + 4, m >> 3) + ((m & 7) << 1));
+          xa[u][i] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        } else {
+          xa[u][i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 64 + i * 32 + fr, u * 2 + fg));
+        }
+      }
       after(2 * u);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
@@ -1331,7 +1388,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   // B), the other eight MFMAs cover the latency of the last read, and nothing moves across the
   // end of the step.
 #define MI355_MDD                                                                             \
-  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, B_NN ? 3 : 2, 0);
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 2 + (B_NN ? 1 : 0) + (A_T ? 1 : 0), 0);
 #define MI355_X4(X) X X X X
 #define MI355_PAIR_SCHEDULE                                                   \
   MI355_X4(MI355_MDD) MI355_X4(MI355_MDD)                                     \
@@ -1672,10 +1729,13 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     // Row-major B needs N % 8 == 0 (its rows must start on 16-byte boundaries); transposed B takes
     // any N — a 50257-wide vocabulary projection stores its misaligned output rows element-wise.
     const bool b_nn_ok = b_nn && N % 8 == 0;
-    if (a_ok && (b_nt || b_nn_ok) && K % 8 == 0 && fits && worth && K > 0) {
+    // An M-contiguous left operand (a transposed view) is taken as it is by the four-wave and the
+    // 128x128 kernels when its k-rows start on 16-byte boundaries and K is a multiple of 64.
+    const bool a_t = !a_ok && a_rs == 1 && a_cs % 8 == 0 && aligned16(a) && M % 8 == 0 && K % 64 == 0;
+    if ((a_ok || a_t) && (b_nt || b_nn_ok) && K % 8 == 0 && fits && worth && K > 0) {
       GemmArgs g{};
       g.a = a; g.b = b; g.c = c; g.out = out;
-      g.lda = a_rs;
+      g.lda = a_t ? a_cs : a_rs;
       g.ldb = b_nt ? b_cs : b_rs;
       g.c_rs = c_rs; g.c_cs = c_cs;
       g.c_vec = c != nullptr && c_cs == 1 && c_rs % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 8 == 0 && N % 4 == 0;
@@ -1691,6 +1751,21 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       int lds_bytes = kGemmLds;
       int threads = 512;
       int nsplit = 1;
+      auto pick_w4 = [&](auto nj) -> const void* {
+        constexpr int NJ = decltype(nj)::value;
+        if (a_t) return b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, NJ, true> : (const void*)gemm_mfma_w4_kernel<T, true, NJ, true>;
+        return b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, NJ, false> : (const void*)gemm_mfma_w4_kernel<T, true, NJ, false>;
+      };
+      auto pick_small = [&](auto deep, auto split_c) -> const void* {
+        constexpr bool SP = decltype(split_c)::value;
+        if constexpr (decltype(deep)::value) {
+          if (a_t) return b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, SP, true> : (const void*)gemm_mfma_small2_kernel<T, true, SP, true>;
+          return b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, SP, false> : (const void*)gemm_mfma_small2_kernel<T, true, SP, false>;
+        } else {
+          if (a_t) return b_nt ? (const void*)gemm_mfma_small_kernel<T, false, SP, true> : (const void*)gemm_mfma_small_kernel<T, true, SP, true>;
+          return b_nt ? (const void*)gemm_mfma_small_kernel<T, false, SP, false> : (const void*)gemm_mfma_small_kernel<T, true, SP, false>;
+        }
+      };
       // Too few 256x256 tiles for the chip but between half a round and one round of 256x128
       // tiles, and a K loop long enough to amortise the one-workgroup-per-CU pipeline: the
       // four-wave kernel on 256x128 tiles.  MI355_GEMM_TILE=256x128 forces it (a test knob).
@@ -1702,7 +1777,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       if (mid) {
         g.tiles_n = (int32_t)((N + 127) / 128);
         nblocks = tiles_mid;
-        kern = b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, 2> : (const void*)gemm_mfma_w4_kernel<T, true, 2>;
+        kern = pick_w4(std::integral_constant<int, 2>{});
         threads = 256;
         lds_bytes = kGemmLds64;
       } else if (!ktail && nblocks < kNumCU * 3 / 4) {  // 128x128 tiles, two workgroups per CU
@@ -1720,13 +1795,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         // At most one workgroup per CU and whole 64-k pairs per split: the deep-ring kernel.
         const bool pairs = nblocks * nsplit <= kNumCU && K % 64 == 0 && (!split || sp.ksplit % 64 == 0);
         lds_bytes = pairs ? kSmall2Lds : kSmallLds;
-        if (pairs) {
-          if (split) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, true> : (const void*)gemm_mfma_small2_kernel<T, true, true>;
-          else kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, false> : (const void*)gemm_mfma_small2_kernel<T, true, false>;
-        } else {
-          if (split) kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, true> : (const void*)gemm_mfma_small_kernel<T, true, true>;
-          else kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, false> : (const void*)gemm_mfma_small_kernel<T, true, false>;
-        }
+        if (pairs) kern = split ? pick_small(std::true_type{}, std::true_type{}) : pick_small(std::true_type{}, std::false_type{});
+        else kern = split ? pick_small(std::false_type{}, std::true_type{}) : pick_small(std::false_type{}, std::false_type{});
         threads = 256;
       } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
@@ -1734,9 +1804,9 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         // Four waves of 128x128 run the steady state 3-5 % faster and pay ~2 us more per tile
         // (two-pass epilogue), which evens out near K = 2048.  MI355_GEMM_WAVES=4|8 forces one form.
         const char* forced = getenv("MI355_GEMM_WAVES");
-        const bool w4 = forced != nullptr ? forced[0] == '4' : K >= 2048;
+        const bool w4 = a_t || (forced != nullptr ? forced[0] == '4' : K >= 2048);  // the eight-wave kernels have no M-contiguous-A form
         if (w4) {
-          kern = b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, 4> : (const void*)gemm_mfma_w4_kernel<T, true, 4>;
+          kern = pick_w4(std::integral_constant<int, 4>{});
           threads = 256;
         } else {
           kern = b_nt ? (const void*)gemm_mfma_dma64_kernel<T, false> : (const void*)gemm_mfma_dma64_kernel<T, true>;
@@ -1746,7 +1816,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
       }
       // More than 64 KB of dynamic LDS needs the attribute once per kernel and process.
-      static thread_local const void* attr_done[24] = {};
+      static thread_local const void* attr_done[48] = {};
       bool seen = false;
       for (const void* k : attr_done) seen = seen || k == kern;
       if (!seen) {

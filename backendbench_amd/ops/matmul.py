@@ -45,7 +45,11 @@ def _gemm(a, b, c, alpha, beta):
     # pass over the operand, instead of the whole product on the FMA fallback.
     if M * N >= 64 * 64 and K >= 16 and a.dtype != torch.float64:
         if a.stride(1) != 1 and M > 1 and K > 1:
-            a = dense(a)
+            # a transposed left operand (x.t() @ dy) goes in as it is when the MFMA kernels take it
+            direct = (a.stride(0) == 1 and a.element_size() == 2 and K % 64 == 0 and M % 8 == 0
+                      and a.stride(1) % 8 == 0 and a.data_ptr() % 16 == 0 and M * N >= 128 * 128)
+            if not direct:
+                a = dense(a)
         if b.stride(1) != 1 and b.stride(0) != 1 and K > 1 and N > 1:
             b = dense(b)
     ws, ws_bytes = None, 0

@@ -135,7 +135,7 @@ def test_headline_gemm_full_size(backend, key):
 
 
 @pytest.mark.parametrize("waves", ["4", "8", "256x128"])
-@pytest.mark.parametrize("layout", ["nt", "nn"])
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
 def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch):
     """The 256x256-tile kernels only run when a problem has enough tiles to fill the chip, so the
     small K-step cases of the edge suite never reach them.  A [3500, K] x [K, 3600] product has
@@ -151,11 +151,14 @@ def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch
     else:
         monkeypatch.setenv("MI355_GEMM_WAVES", waves)
     g = torch.Generator().manual_seed(5)
-    M, N = 3500, 3600
+    M, N = (3504, 3600) if layout[0] == "t" else (3500, 3600)   # an M-contiguous operand needs M % 8 == 0
     rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 127, 128, 255, 256, 3327, 3328, 3499])]))
     for K in (64, 128, 192, 256, 320, 384, 448, 512, 576, 640, 704, 1024, 2048, 2112, 96, 160, 288, 72, 200):
-        a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
-        if layout == "nt":
+        if layout[0] == "t":   # transposed left operand (M-contiguous): taken as it is when K % 64 == 0
+            a = torch.randint(-1, 2, (K, M), generator=g).to(torch.bfloat16).cuda().t()
+        else:
+            a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+        if layout[1] == "t":
             b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
         else:
             b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
@@ -167,10 +170,10 @@ def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch
         assert ev.bit_equal((out.float() + bias.float()).to(torch.bfloat16), out2), (layout, K, "bias")
 
 
-@pytest.mark.parametrize("layout", ["nt", "nn"])
-@pytest.mark.parametrize("shape", [(700, 900), (2000, 2500)])
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
+@pytest.mark.parametrize("shape", [(704, 900), (2000, 2500)])
 def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
-    """The 128x128-tile kernels: [700, K] x [K, 900] has 6 x 8 tiles, at most one workgroup per CU
+    """The 128x128-tile kernels: [704, K] x [K, 900] has 6 x 8 tiles, at most one workgroup per CU
     (the deep-ring kernel when K is a multiple of 64, split along K once K is long enough for the
     planner); [2000, K] x [K, 2500] has 16 x 20, more than one per CU (the two-per-CU kernel).  K
     walks through every prologue / steady / drain length of both pipelines.  Small-integer operands
@@ -181,8 +184,11 @@ def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
     g = torch.Generator().manual_seed(6)
     rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 63, 64, 127, 128, M - 129, M - 128, M - 1])]))
     for K in (32, 64, 96, 128, 160, 192, 224, 256, 320, 384, 448, 512, 576, 640, 704, 1056, 2080, 4096):
-        a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
-        if layout == "nt":
+        if layout[0] == "t":   # transposed left operand (M-contiguous): taken as it is when K % 64 == 0
+            a = torch.randint(-1, 2, (K, M), generator=g).to(torch.bfloat16).cuda().t()
+        else:
+            a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+        if layout[1] == "t":
             b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
         else:
             b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
