@@ -131,6 +131,46 @@ __global__ __launch_bounds__(256) void gemm_splitk_finish_kernel(GemmArgs g, int
   }
 }
 
+// The same for outputs too small to fill the chip with one thread per four columns: four
+// neighbouring lanes share a group of four columns, each sums every fourth partial plane, and
+// two DPP steps combine them.
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_splitk_finish4_kernel(GemmArgs g, int nsplit) {
+  const int64_t quads = (int64_t)g.M * g.N / 4;
+  const T* C = static_cast<const T*>(g.c);
+  const bool use_c = C != nullptr && g.beta != 0.f;
+  T* D = static_cast<T*>(g.out);
+  const int64_t plane = (int64_t)g.M * g.N;
+  const int part = threadIdx.x & 3;
+  const int64_t stride = (int64_t)gridDim.x * 64;
+  const int64_t rounds = (quads + stride - 1) / stride;  // every lane of a wave stays in the loop: the combine below is wave-wide
+  for (int64_t r = 0; r < rounds; ++r) {
+    const int64_t qd = r * stride + (int64_t)blockIdx.x * 64 + (threadIdx.x >> 2);
+    const bool live = qd < quads;
+    const int64_t e0 = live ? qd * 4 : 0;
+    f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (live)
+      for (int sp = part; sp < nsplit; sp += 4) sum += *reinterpret_cast<const f32x4*>(g.ws + sp * plane + e0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = sum[e];
+      v += dpp<0xB1>(v);  // lanes 0<->1, 2<->3
+      v += dpp<0x4E>(v);  // pairs
+      sum[e] = v;
+    }
+    if (!live || part != 0) continue;
+    const int64_t m = e0 / g.N, n = e0 - m * g.N;
+    VecN4<T> out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float v = g.alpha * sum[e];
+      if (use_c) v += g.beta * static_cast<float>(C[m * g.c_rs + (n + e) * g.c_cs]);
+      out.v[e] = static_cast<T>(v);
+    }
+    *reinterpret_cast<VecN4<T>*>(D + e0) = out;
+  }
+}
+
 // Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous
 // band of tile ids, then walk the band in groups of 8 tile-rows so A and B panels repeat
 // in that XCD's L2.
@@ -1709,8 +1749,13 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
 template <typename T>
 static int finish_splitk(const GemmArgs& g, int nsplit, hipStream_t st) {
   const int64_t quads = (int64_t)g.M * g.N / 4;
-  const int grid = grid_for(quads, 256, kNumCU * 8);
-  hipLaunchKernelGGL((gemm_splitk_finish_kernel<T>), dim3(grid), dim3(256), 0, st, g, nsplit);
+  if (quads < (int64_t)kNumCU * 256 * 2 && nsplit >= 4) {  // under two blocks per CU: four lanes per group of columns
+    const int grid = grid_for(quads, 64, kNumCU * 8);
+    hipLaunchKernelGGL((gemm_splitk_finish4_kernel<T>), dim3(grid), dim3(256), 0, st, g, nsplit);
+  } else {
+    const int grid = grid_for(quads, 256, kNumCU * 8);
+    hipLaunchKernelGGL((gemm_splitk_finish_kernel<T>), dim3(grid), dim3(256), 0, st, g, nsplit);
+  }
   return check_launch("mi355_gemm(split-k finish)");
 }
 
