@@ -6,6 +6,8 @@
 //   rows_block   inner == 1, long or few rows: one 256-thread block per (row, split),
 //                wave reduce then LDS combine across the four waves;
 //   rows_thread  inner == 1, red <= 32: one thread per row;
+//   rows_sub     inner == 1, 32 < red <= 128, many rows (pooling over a 7x7 map): sixteen lanes
+//                per row, four rows per wave, DPP reduce inside the 16-lane row;
 //   cols         inner > 1: 64 lanes along inner (coalesced, one 128-bit load each when inner
 //                allows) x 4 along red, LDS combine;
 //   final        second pass over per-split partial states when a launch was split
@@ -74,6 +76,26 @@ template <typename A> __device__ __forceinline__ typename AmaxR<A>::State wave_r
 }
 template <typename A> __device__ __forceinline__ typename ArgmaxR<A>::State wave_reduce(typename ArgmaxR<A>::State s, ArgmaxR<A>*) {
   return wave_reduce_state<ArgmaxR<A>>(s);
+}
+
+// Reduce over the 16 lanes of a DPP row (lanes 16 g .. 16 g + 15): result in all of them.
+template <typename T, typename Op> __device__ __forceinline__ T row16_allreduce(T v, Op op) {
+  v = op(v, dpp<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = op(v, dpp<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = op(v, dpp<0x124>(v));  // row_ror:4
+  v = op(v, dpp<0x128>(v));  // row_ror:8
+  return v;
+}
+template <typename A> __device__ __forceinline__ typename SumR<A>::State row16_reduce(typename SumR<A>::State s, SumR<A>*) {
+  return {row16_allreduce(s.s, SumOp())};
+}
+template <typename A> __device__ __forceinline__ typename AmaxR<A>::State row16_reduce(typename AmaxR<A>::State s, AmaxR<A>*) {
+  return {row16_allreduce(s.s, MaxNanOp())};
+}
+template <typename A> __device__ __forceinline__ typename ArgmaxR<A>::State row16_reduce(typename ArgmaxR<A>::State s, ArgmaxR<A>*) {
+#pragma unroll
+  for (int m = 1; m < 16; m <<= 1) s = ArgmaxR<A>::combine(s, ArgmaxR<A>::shfl_xor(s, m));
+  return s;
 }
 
 // Block reduce of a State (blockDim.x = 256): result valid in thread 0.
@@ -186,6 +208,39 @@ __global__ __launch_bounds__(kRedBlock) void rows_block_kernel(const T* __restri
   if (threadIdx.x == 0) {
     if constexpr (PARTIAL) ws[row * gridDim.x + blockIdx.x] = st;
     else write_final<R, O, FIN>(out, row, st, divisor);
+  }
+}
+
+// Sixteen lanes per row: the wave's four rows are one contiguous span of memory, every lane
+// reads elements j, j + 16, ... of its row.  All lanes of a wave stay in the loop (the DPP
+// reduce is wave-wide); rows past the end accumulate nothing and write nothing.
+// VEC: rows are whole 16-byte vectors on 16-byte boundaries; lane j takes vectors j, j + 16, ...
+template <typename T, typename O, typename R, int FIN, bool VEC>
+__global__ __launch_bounds__(kRedBlock) void rows_sub_kernel(const T* __restrict__ x, O* __restrict__ out,
+                                                            int64_t outer, int64_t red, double divisor) {
+  using A = typename R::acc_t;
+  constexpr int V = Vec<T>::N;
+  const int j = threadIdx.x & 15;
+  const int64_t group0 = ((int64_t)blockIdx.x * kRedBlock + threadIdx.x) >> 4;
+  const int64_t ngroups = (int64_t)gridDim.x * (kRedBlock / 16);
+  const int64_t rounds = (outer + ngroups - 1) / ngroups;
+  for (int64_t r = 0; r < rounds; ++r) {
+    const int64_t row = group0 + r * ngroups;
+    typename R::State st = R::init();
+    if (row < outer) {
+      const T* p = x + row * red;
+      if constexpr (VEC) {
+        for (int64_t i = (int64_t)j * V; i < red; i += 16 * V) {
+          const Vec<T> v = load_vec_nt(p + i);
+#pragma unroll
+          for (int e = 0; e < V; ++e) R::acc(st, (A)v.v[e], i + e);
+        }
+      } else {
+        for (int64_t i = j; i < red; i += 16) R::acc(st, (A)p[i], i);
+      }
+    }
+    st = row16_reduce(st, (R*)nullptr);
+    if (j == 0 && row < outer) write_final<R, O, FIN>(out, row, st, divisor);
   }
 }
 
@@ -323,7 +378,7 @@ __global__ __launch_bounds__(kRedBlock) void final_rows_kernel(const typename R:
 }
 
 // ---------------------------------------------------------------- planning
-enum Kind { ROWS_WAVE, ROWS_BLOCK, ROWS_THREAD, COLS };
+enum Kind { ROWS_WAVE, ROWS_BLOCK, ROWS_THREAD, ROWS_SUB, COLS };
 struct Plan {
   Kind kind;
   int64_t nsplit, chunk;
@@ -334,6 +389,8 @@ static Plan plan_reduce(int64_t outer, int64_t red, int64_t inner, int elem_size
   const int V = 16 / elem_size;
   const int64_t want_blocks = kNumCU * 4;
   if (inner == 1) {
+    if (red <= 8 && outer >= 4096) { p.kind = ROWS_THREAD; return p; }
+    if (red <= 16 * V && outer >= 8192) { p.kind = ROWS_SUB; return p; }  // up to one vector per lane (scalar rows: <= 128)
     if (red <= 32 && outer >= 4096) { p.kind = ROWS_THREAD; return p; }
     if (outer >= 2048 && red <= 16384) { p.kind = ROWS_WAVE; return p; }
     p.kind = ROWS_BLOCK;
@@ -386,6 +443,14 @@ static int run_reduce(const void* xv, int64_t outer, int64_t red, int64_t inner,
     case ROWS_THREAD: {
       const int grid = grid_for(outer, kRedBlock, kNumCU * 16);
       hipLaunchKernelGGL((rows_thread_kernel<T, O, R, FIN>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      break;
+    }
+    case ROWS_SUB: {
+      const int grid = grid_for(outer, kRedBlock / 16, kNumCU * 16);
+      if (aligned16(x) && red % V == 0)
+        hipLaunchKernelGGL((rows_sub_kernel<T, O, R, FIN, true>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      else
+        hipLaunchKernelGGL((rows_sub_kernel<T, O, R, FIN, false>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
       break;
     }
     case ROWS_WAVE: {

@@ -298,6 +298,18 @@ def edge_cases() -> List[Case]:
     add(aten.argmax.default, lambda d: (_to(d, normal((5, 300, 7), f32, seed=1), 1, True), {}), exact=True, tag="mid_keepdim2")
     add(aten.argmax.default, lambda d: (_to(d, torch.zeros(6, 5000, dtype=f32), -1), {}), exact=True, tag="all_ties")
     add(aten.argmax.default, lambda d: (_to(d, (normal((16, 70000), f32, seed=2) * 4).round(), -1), {}), exact=True, tag="many_ties")
+    # many short rows (global average pooling over a 7x7 map): sixteen lanes per row, scalar and
+    # vector forms, a row count that is not a multiple of the four rows a wave holds
+    for red, dt in ((9, f32), (16, f32), (33, bf16), (49, f16), (64, f32), (100, bf16), (128, f16)):
+        t = f"{dt}".split(".")[-1]
+        rows = 8192 + 5
+        add(aten.sum.dim_IntList, lambda d, red=red, dt=dt, rows=rows: (_to(d, normal((rows, red), dt, seed=1), [-1]), {}), tag=f"short_rows_{red}_{t}")
+        add(aten.mean.dim, lambda d, red=red, dt=dt, rows=rows: (_to(d, normal((rows, red), dt, 3.0, seed=2), [-1], True), {}), tag=f"short_rows_{red}_{t}")
+        add(aten.amax.default, lambda d, red=red, dt=dt, rows=rows: (_to(d, poison(normal((rows, red), dt, seed=3), 0.002, 5), [-1]), {}), tag=f"short_rows_{red}_{t}")
+        add(aten.argmax.default, lambda d, red=red, dt=dt, rows=rows: (_to(d, poison((normal((rows, red), dt, seed=4) * 2).round(), 0.002, 6), -1), {}), exact=True, tag=f"short_rows_{red}_{t}")
+    add(aten.mean.dim, lambda d: (_to(d, normal((16, 600, 7, 7), f16, 1.0, seed=1), [-1, -2], True), {}), tag="pool_7x7")
+    add(aten.sum.dim_IntList, lambda d: (_to(d, randint((9000, 40), 100, 1, i32, low=-100), [-1]), {}), exact=True, tag="short_rows_int")
+    add(aten.sum.dim_IntList, lambda d: ([normal((9000 * 64 + 1,), f32, seed=7).to(d)[1:].view(9000, 64), [-1]], {}), tag="short_rows_offset_view")
 
     # ---- _softmax
     for dt in (f32, f16, bf16):
