@@ -377,9 +377,12 @@ int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_t
     for (int k = 0; k < d.ndim; ++k) a.div[k] = make_fastdiv((uint32_t)a.sizes[k]);
   // Large vectorised problems: four work items per thread, so that a block owns 4 * 256 vectors.
   constexpr int kStridedUnroll = 4;
-  if (vec_ok && !wide && total >= (int64_t)kEwBlock * kStridedUnroll * kNumCU * 4) {
+  if (!wide && total >= (int64_t)kEwBlock * kStridedUnroll * kNumCU * 4) {
     const int grid = grid_for(total, kEwBlock * kStridedUnroll, 1 << 30);
-    hipLaunchKernelGGL((ew_strided_kernel<F, V, false, kStridedUnroll>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+    if (vec_ok)
+      hipLaunchKernelGGL((ew_strided_kernel<F, V, false, kStridedUnroll>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
+    else  // an innermost extent that is no multiple of the vector (197 tokens): elements, four in flight per thread
+      hipLaunchKernelGGL((ew_strided_kernel<F, 1, false, kStridedUnroll>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, total);
     return check_launch(name);
   }
   const int grid = grid_for(total, kEwBlock, 1 << 30);

@@ -51,8 +51,15 @@ template <typename A> struct ArgmaxR {
     }
     return v > bv || (v == bv && i < bi);
   }
+  // Every kernel feeds a lane its elements in increasing index order, so an element equal to the
+  // held one never replaces it and the index needs no comparison here.  A lane (or a whole row)
+  // whose elements all equal the initial value keeps i = INT64_MAX; write_final turns that into
+  // index 0, the first of the all-equal row.
   static __device__ __forceinline__ void acc(State& st, A v, int64_t i) {
-    if (better(v, i, st.v, st.i)) { st.v = v; st.i = i; }
+    bool take;
+    if constexpr (IsFloat<A>::value) take = (v != v) ? (st.v == st.v) : (v > st.v);  // v > NaN is false: a held NaN stays
+    else take = v > st.v;
+    if (take) { st.v = v; st.i = i; }
   }
   static __device__ __forceinline__ State combine(State a, State b) {
     return better(b.v, b.i, a.v, a.i) ? b : a;
@@ -74,8 +81,24 @@ template <typename A> __device__ __forceinline__ typename SumR<A>::State wave_re
 template <typename A> __device__ __forceinline__ typename AmaxR<A>::State wave_reduce(typename AmaxR<A>::State s, AmaxR<A>*) {
   return {wave_allreduce(s.s, MaxNanOp())};
 }
+// (value, index) pairs: the four steps inside a 16-lane row move both halves by DPP, only the
+// two steps across rows go through ds_bpermute.
+template <typename A, int CTRL> __device__ __forceinline__ typename ArgmaxR<A>::State argmax_dpp_step(typename ArgmaxR<A>::State s) {
+  const typename ArgmaxR<A>::State o{dpp<CTRL>(s.v), dpp<CTRL>(s.i)};
+  return ArgmaxR<A>::combine(s, o);
+}
+template <typename A> __device__ __forceinline__ typename ArgmaxR<A>::State argmax_row16(typename ArgmaxR<A>::State s) {
+  s = argmax_dpp_step<A, 0xB1>(s);
+  s = argmax_dpp_step<A, 0x4E>(s);
+  s = argmax_dpp_step<A, 0x124>(s);
+  s = argmax_dpp_step<A, 0x128>(s);
+  return s;
+}
 template <typename A> __device__ __forceinline__ typename ArgmaxR<A>::State wave_reduce(typename ArgmaxR<A>::State s, ArgmaxR<A>*) {
-  return wave_reduce_state<ArgmaxR<A>>(s);
+  s = argmax_row16<A>(s);
+  s = ArgmaxR<A>::combine(s, ArgmaxR<A>::shfl_xor(s, 16));
+  s = ArgmaxR<A>::combine(s, ArgmaxR<A>::shfl_xor(s, 32));
+  return s;
 }
 
 // Reduce over the 16 lanes of a DPP row (lanes 16 g .. 16 g + 15): result in all of them.
@@ -93,9 +116,7 @@ template <typename A> __device__ __forceinline__ typename AmaxR<A>::State row16_
   return {row16_allreduce(s.s, MaxNanOp())};
 }
 template <typename A> __device__ __forceinline__ typename ArgmaxR<A>::State row16_reduce(typename ArgmaxR<A>::State s, ArgmaxR<A>*) {
-#pragma unroll
-  for (int m = 1; m < 16; m <<= 1) s = ArgmaxR<A>::combine(s, ArgmaxR<A>::shfl_xor(s, m));
-  return s;
+  return argmax_row16<A>(s);
 }
 
 // Block reduce of a State (blockDim.x = 256): result valid in thread 0.
@@ -117,7 +138,8 @@ template <typename R, typename O, int FIN>
 __device__ __forceinline__ void write_final(O* out, int64_t at, const typename R::State& st, double divisor) {
   using A = typename R::acc_t;
   if constexpr (FIN == FIN_INDEX) {
-    out[at] = (O)(((const typename ArgmaxR<A>::State&)st).i);
+    const int64_t i = ((const typename ArgmaxR<A>::State&)st).i;
+    out[at] = (O)(i == INT64_MAX ? 0 : i);  // nothing beat the initial value: every element equals it
   } else {
     A v = *reinterpret_cast<const A*>(&st);
     if constexpr (FIN == FIN_MEAN) v = v / (A)divisor;
@@ -155,6 +177,23 @@ __device__ __forceinline__ void accumulate_span(typename R::State& st, const T* 
     };
     int64_t i = lo + (int64_t)tid * V;
     const int64_t step = (int64_t)nthr * V;
+    if (hi - lo <= 4 * step) {
+      // A short span (at most four vectors per lane) is one batch under per-lane predicates: one
+      // memory latency for the whole row, whatever its length.
+      if (i < hi) {
+        const bool k1 = i + step < hi, k2 = i + 2 * step < hi, k3 = i + 3 * step < hi;
+        Vec<T> v0 = load_vec_nt(win + i), v1, v2, v3;
+        if (k1) v1 = load_vec_nt(win + i + step);
+        if (k2) v2 = load_vec_nt(win + i + 2 * step);
+        if (k3) v3 = load_vec_nt(win + i + 3 * step);
+        take(v0, i);
+        if (k1) take(v1, i + step);
+        if (k2) take(v2, i + 2 * step);
+        if (k3) take(v3, i + 3 * step);
+      }
+      return;
+    }
+    // Batches of four vectors per lane, all loads of a batch issued before the first is used.
     for (; i + 3 * step < hi; i += 4 * step) {
       Vec<T> v0 = load_vec_nt(win + i), v1 = load_vec_nt(win + i + step), v2 = load_vec_nt(win + i + 2 * step),
              v3 = load_vec_nt(win + i + 3 * step);
@@ -163,7 +202,17 @@ __device__ __forceinline__ void accumulate_span(typename R::State& st, const T* 
       take(v2, i + 2 * step);
       take(v3, i + 3 * step);
     }
-    for (; i < hi; i += step) take(load_vec_nt(win + i), i);
+    // The last batch of a row may be partial (per-lane predicates); its loads go out together as
+    // well, so a short row costs one memory latency, not one per leftover vector.
+    if (i < hi) {
+      const bool k1 = i + step < hi, k2 = i + 2 * step < hi;
+      Vec<T> v0 = load_vec_nt(win + i), v1, v2;
+      if (k1) v1 = load_vec_nt(win + i + step);
+      if (k2) v2 = load_vec_nt(win + i + 2 * step);
+      take(v0, i);
+      if (k1) take(v1, i + step);
+      if (k2) take(v2, i + 2 * step);
+    }
   } else {
     for (int64_t i = lo + tid; i < hi; i += nthr) R::acc(st, (A)row[i], i);
   }
