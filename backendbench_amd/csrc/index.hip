@@ -41,6 +41,20 @@ __global__ __launch_bounds__(kIxBlock) void index_rows_wave_kernel(const U* __re
     const U* s = src + (o * n_src + idx) * row_units;
     // rows are read and written once: streaming (non-temporal) accesses, four loads in flight
     int64_t u = lane;
+    if (row_units <= 4 * kWave) {  // a short row is one batch under per-lane predicates: one memory latency
+      if (u < row_units) {
+        const bool k1 = u + kWave < row_units, k2 = u + 2 * kWave < row_units, k3 = u + 3 * kWave < row_units;
+        U a = __builtin_nontemporal_load(s + u), b, c, d;
+        if (k1) b = __builtin_nontemporal_load(s + u + kWave);
+        if (k2) c = __builtin_nontemporal_load(s + u + 2 * kWave);
+        if (k3) d = __builtin_nontemporal_load(s + u + 3 * kWave);
+        __builtin_nontemporal_store(a, dst + u);
+        if (k1) __builtin_nontemporal_store(b, dst + u + kWave);
+        if (k2) __builtin_nontemporal_store(c, dst + u + 2 * kWave);
+        if (k3) __builtin_nontemporal_store(d, dst + u + 3 * kWave);
+      }
+      continue;
+    }
     for (; u + 3 * kWave < row_units; u += 4 * kWave) {
       const U a = __builtin_nontemporal_load(s + u), b = __builtin_nontemporal_load(s + u + kWave),
               c = __builtin_nontemporal_load(s + u + 2 * kWave), d = __builtin_nontemporal_load(s + u + 3 * kWave);
