@@ -279,6 +279,74 @@ __global__ __launch_bounds__(kEwBlock) void ew_strided_kernel(F f, EwPtrs p,
   }
 }
 
+// Dense row-major output whose innermost extent is no multiple of the vector (a 197-token
+// attention map plus a [B,1,1,197] mask): the strided kernel would fall back to single
+// elements.  Here one work item is V consecutive elements of the flat output: inputs laid out
+// like the output (flat_mask bit t) are read as one aligned vector, the others element by
+// element along a coordinate walk (the innermost index steps, a carry into the outer dims
+// re-splits the flat index: once per row), and the result leaves as one aligned vector store.
+template <typename F, int V>
+__global__ __launch_bounds__(kEwBlock) void ew_dense_out_kernel(F f, EwPtrs p, StridedArgs<F::NIN + 1> a, int64_t n,
+                                                                 uint32_t flat_mask) {
+  using TO = typename F::out_t;
+  using T0 = typename F::in0_t;
+  using T1 = typename F::in1_t;
+  using T2 = typename F::in2_t;
+  constexpr int NIN = F::NIN;
+  constexpr int NT = NIN + 1;
+  const int last = a.ndim - 1;
+  const int64_t items = (n + V - 1) / V;
+  const T0* in0 = static_cast<const T0*>(p.in[0]);
+  const T1* in1 = static_cast<const T1*>(p.in[1]);
+  const T2* in2 = static_cast<const T2*>(p.in[2]);
+  for (int64_t item = (int64_t)blockIdx.x * kEwBlock + threadIdx.x; item < items; item += (int64_t)gridDim.x * kEwBlock) {
+    const int64_t e0 = item * V;
+    const bool full = e0 + V <= n;
+    VecN<T0, V> va;
+    VecN<T1, V> vb;
+    VecN<T2, V> vc;
+    if (full) {
+      if (flat_mask & 1u) va = ld_nt<T0, V>(in0 + e0);
+      if constexpr (NIN > 1) if (flat_mask & 2u) vb = ld_nt<T1, V>(in1 + e0);
+      if constexpr (NIN > 2) if (flat_mask & 4u) vc = ld_nt<T2, V>(in2 + e0);
+    }
+    int64_t off[NT];
+    ew_split_index<F, NT, false>(a, e0, off);
+    int64_t inner = 0;  // index along the innermost dim = e0 % sizes[last]
+    {
+      const FastDiv d = a.div[last];
+      const uint32_t q = (uint32_t)(((uint64_t)__umulhi((uint32_t)e0, d.m) + (uint32_t)e0) >> d.s);
+      inner = (uint32_t)e0 - q * d.d;
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      if (e0 + j < n) {
+        if (!full || !(flat_mask & 1u)) va.v[j] = in0[off[0]];
+        if constexpr (NIN > 1) if (!full || !(flat_mask & 2u)) vb.v[j] = in1[off[1]];
+        if constexpr (NIN > 2) if (!full || !(flat_mask & 4u)) vc.v[j] = in2[off[2]];
+      }
+      if (j + 1 < V) {
+        if (++inner == a.sizes[last]) {
+          inner = 0;
+          ew_split_index<F, NT, false>(a, e0 + j + 1, off);
+        } else {
+#pragma unroll
+          for (int t = 0; t < NIN; ++t) off[t] += a.strides[t][last];
+        }
+      }
+    }
+    const VecN<TO, V> r = ew_apply<F, V>(f, va, vb, vc);
+    TO* o = static_cast<TO*>(p.out) + e0;
+    if (full) {
+      st_nt<TO, V>(o, r);
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; ++j)
+        if (e0 + j < n) o[j] = r.v[j];
+    }
+  }
+}
+
 // ---------------------------------------------------------------- host launcher
 template <typename F>
 int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_tensor* out,
@@ -375,6 +443,26 @@ int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_t
   const bool wide = total >= (int64_t(1) << 31);
   if (!wide)
     for (int k = 0; k < d.ndim; ++k) a.div[k] = make_fastdiv((uint32_t)a.sizes[k]);
+  if (!vec_ok && V > 1 && !wide && n >= 4096) {
+    // dense row-major output on a vector boundary: vector stores over the flat output
+    bool dense_out = reinterpret_cast<uintptr_t>(out->data) % (esz[3] * V) == 0;
+    int64_t expect = 1;
+    for (int k = d.ndim - 1; k >= 0 && dense_out; --k) {
+      dense_out = d.strides[NT - 1][k] == expect;
+      expect *= d.sizes[k];
+    }
+    if (dense_out) {
+      uint32_t flat_mask = 0;
+      for (int t = 0; t < NIN; ++t) {
+        bool same = reinterpret_cast<uintptr_t>(ts[t]->data) % (esz[t] * V) == 0;
+        for (int k = 0; k < d.ndim && same; ++k) same = d.strides[t][k] == d.strides[NT - 1][k];
+        if (same) flat_mask |= 1u << t;
+      }
+      const int grid = grid_for((n + V - 1) / V, kEwBlock, 1 << 30);
+      hipLaunchKernelGGL((ew_dense_out_kernel<F, V>), dim3(grid), dim3(kEwBlock), 0, stream, f, p, a, n, flat_mask);
+      return check_launch(name);
+    }
+  }
   // Large vectorised problems: four work items per thread, so that a block owns 4 * 256 vectors.
   constexpr int kStridedUnroll = 4;
   if (!wide && total >= (int64_t)kEwBlock * kStridedUnroll * kNumCU * 4) {

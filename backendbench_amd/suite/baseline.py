@@ -193,6 +193,16 @@ def edge_cases() -> List[Case]:
     add(aten.add.Tensor, lambda d: (_to(d, normal((33, 65), f32, seed=1), normal((33, 65), f32, seed=2)), {"alpha": 2.5}), tag="alpha")
     add(aten.add.Tensor, lambda d: (_to(d, normal((33, 65), bf16, seed=1), normal((65,), bf16, seed=2)), {"alpha": -1}), tag="alpha_bf16")
     add(aten.add.Tensor, lambda d: (_to(d, randint((12,), 50, 1, i64), randint((12,), 50, 2, i64)), {"alpha": 3}), exact=True, tag="alpha_int")
+    # dense output, innermost extent no multiple of the vector width, one operand broadcast or strided: vector
+    # stores over the flat output, the odd operand gathered along a coordinate walk (attention map + mask at 197 tokens)
+    add(aten.add.Tensor, lambda d: (_to(d, normal((2, 3, 197, 197), f16, seed=1), normal((2, 1, 1, 197), f16, seed=2)), {}), tag="mask_197_f16")
+    add(aten.mul.Tensor, lambda d: (_to(d, poison(normal((33, 131), f32, seed=1), 0.01, 3), normal((131,), f32, seed=2)), {}), tag="row_131_f32")
+    add(aten.add.Tensor, lambda d: (_to(d, normal((3, 1367), bf16, seed=1), normal((1367,), bf16, seed=2)), {"alpha": 0.5}), tag="ragged_tail_bf16")
+    add(aten.where.self, lambda d: (_to(d, normal((5, 1, 77), f32, seed=1) > 0, normal((5, 19, 77), f16, seed=2), normal((1, 19, 1), f16, seed=3)), {}), exact=True, tag="three_way_77")
+    add(aten.maximum.default, lambda d: ([normal((67, 65), f32, seed=1).to(d), normal((65, 67), f32, seed=2).to(d).t()], {}), tag="transposed_odd")
+    add(aten.add.Tensor, lambda d: (_to(d, normal((7, 599), f16, seed=1), normal((7, 599), f32, seed=2)), {}), tag="promote_odd")
+    add(aten.mul.Tensor, lambda d: ([normal((9, 1001), f32, seed=1).to(d)[:, ::2], normal((501,), f32, seed=2).to(d)], {}), tag="strided_cols_odd")
+    add(aten.clamp.Tensor, lambda d: (_to(d, normal((11, 401), f32, seed=1), normal((401,), f32, -0.5, 0.1, seed=2), normal((11, 1), f32, 0.5, 0.1, seed=3)), {}), tag="bounds_broadcast_odd")
 
     # ---- unary: relu / clamp
     for dt in (f32, f16, bf16):
