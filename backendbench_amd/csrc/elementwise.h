@@ -406,9 +406,29 @@ int launch_elementwise(const F& f, const mi355_tensor* const* ins, const mi355_t
     if (out->sizes[i] > 1 && out->strides[i] == 0)
       return set_error(MI355_ERR_INVALID, "%s: output has a broadcast (stride 0) dim", name);
 
+  // Walk the dims in the memory order of the output (largest stride first): a channels-last
+  // output then has its channels innermost, where they are unit-stride, instead of its width.
+  int order[MI355_MAX_DIMS];
+  for (int i = 0; i < out->ndim; ++i) order[i] = i;
+  auto key = [&](int i) { return out->sizes[i] > 1 ? out->strides[i] : INT64_MAX; };  // size-1 dims: anywhere (dropped later)
+  for (int i = 1; i < out->ndim; ++i) {  // stable insertion sort by descending output stride
+    const int v = order[i];
+    int j = i;
+    while (j > 0 && key(order[j - 1]) < key(v)) {
+      order[j] = order[j - 1];
+      --j;
+    }
+    order[j] = v;
+  }
+  int64_t psizes[MI355_MAX_DIMS];
+  int64_t pstrides[NT][MI355_MAX_DIMS];
+  for (int i = 0; i < out->ndim; ++i) {
+    psizes[i] = out->sizes[order[i]];
+    for (int t = 0; t < NT; ++t) pstrides[t][i] = ts[t]->strides[order[i]];
+  }
   const int64_t* strides[NT];
-  for (int t = 0; t < NT; ++t) strides[t] = ts[t]->strides;
-  Dims<NT> d = collapse_dims<NT>(out->ndim, out->sizes, strides);
+  for (int t = 0; t < NT; ++t) strides[t] = pstrides[t];
+  Dims<NT> d = collapse_dims<NT>(out->ndim, psizes, strides);
 
   // Vectorise along the innermost collapsed dim when every operand is unit-stride (or
   // broadcast) there and every vector stays aligned.

@@ -203,6 +203,10 @@ def edge_cases() -> List[Case]:
     add(aten.add.Tensor, lambda d: (_to(d, normal((7, 599), f16, seed=1), normal((7, 599), f32, seed=2)), {}), tag="promote_odd")
     add(aten.mul.Tensor, lambda d: ([normal((9, 1001), f32, seed=1).to(d)[:, ::2], normal((501,), f32, seed=2).to(d)], {}), tag="strided_cols_odd")
     add(aten.clamp.Tensor, lambda d: (_to(d, normal((11, 401), f32, seed=1), normal((401,), f32, -0.5, 0.1, seed=2), normal((11, 1), f32, 0.5, 0.1, seed=3)), {}), tag="bounds_broadcast_odd")
+    # channels-last operand with a per-channel broadcast: the kernel walks the dims in the output's memory order
+    add(aten.mul.Tensor, lambda d: ([normal((6, 40, 9, 7), f16, seed=1).to(d).to(memory_format=torch.channels_last), normal((1, 40, 1, 1), f16, seed=2).to(d)], {}), tag="channels_last_scale")
+    add(aten.add.Tensor, lambda d: ([normal((4, 24, 5, 6), f32, seed=1).to(d).to(memory_format=torch.channels_last), normal((4, 24, 5, 6), f32, seed=2).to(d)], {}), tag="channels_last_plus_nchw")
+    add(aten.where.self, lambda d: ([(normal((3, 16, 4, 5), f32, seed=1) > 0).to(d).to(memory_format=torch.channels_last), normal((3, 16, 4, 5), f32, seed=2).to(d).to(memory_format=torch.channels_last), normal((16, 1, 1), f32, seed=3).to(d)], {}), exact=True, tag="channels_last_three_way")
 
     # ---- unary: relu / clamp
     for dt in (f32, f16, bf16):
