@@ -1769,8 +1769,9 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     const bool b_nt = b_rs == 1 && b_cs % 8 == 0 && aligned16(b);
     const bool b_nn = b_cs == 1 && b_rs % 8 == 0 && aligned16(b);
     const bool fits = M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
-    // Tiny problems are cheaper on the generic kernel than on a mostly empty 256x256 tile.
-    const bool worth = M * N >= 128 * 128 && K >= 32;
+    // Tiny problems are cheaper on the generic kernel than on mostly empty MFMA tiles; a single row
+    // against a large weight (decoding one token) is not tiny: it streams the whole weight.
+    const bool worth = K >= 32 && (M * N >= 128 * 128 || M * N * K >= (int64_t(1) << 22));
     // Row-major B needs N % 8 == 0 (its rows must start on 16-byte boundaries); transposed B takes
     // any N — a 50257-wide vocabulary projection stores its misaligned output rows element-wise.
     const bool b_nn_ok = b_nn && N % 8 == 0;
@@ -1885,7 +1886,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     const bool b_nn = b_cs == 1 && b_rs % 4 == 0 && aligned16(b);
     const bool fits = M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
     const bool b_nn_ok = b_nn && N % 4 == 0;
-    if (a_ok && (b_nt || b_nn_ok) && K % FBK == 0 && K > 0 && fits && M * N >= 64 * 64) {
+    if (a_ok && (b_nt || b_nn_ok) && K % FBK == 0 && K > 0 && fits && (M * N >= 64 * 64 || M * N * K >= (int64_t(1) << 22))) {
       GemmArgs g{};
       g.a = a; g.b = b; g.c = c; g.out = out;
       g.lda = a_rs;

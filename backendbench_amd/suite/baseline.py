@@ -425,6 +425,11 @@ def edge_cases() -> List[Case]:
     add(aten.addmm.default, lambda d: ([normal((200,), f32, seed=3).to(d), normal((64, 1024), f32, seed=1).to(d), normal((200, 1024), f32, 0, 0.05, seed=2).to(d).t()], {}), tag="splitk_linear_f32")
     add(aten.mm.default, lambda d: (_to(d, normal((64, 1040), f32, seed=1), normal((1040, 256), f32, 0, 0.05, seed=2)), {}), tag="splitk_f32")
     add(aten.mm.default, lambda d: ([normal((320, 512), bf16, seed=1).to(d).t(), normal((320, 768), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_transposed")
+    # one row against a large weight (decoding one token): MFMA tiles split along K, not the FMA fallback
+    add(aten.mm.default, lambda d: ([normal((1, 2048), bf16, seed=1).to(d), normal((1024, 2048), bf16, 0, 0.05, seed=2).to(d).t()], {}), tag="single_row_bf16")
+    add(aten.mm.default, lambda d: (_to(d, normal((1, 4096), f32, seed=1), normal((4096, 1000), f32, 0, 0.05, seed=2)), {}), tag="single_row_f32")
+    add(aten.addmm.default, lambda d: ([normal((1024,), f16, seed=3).to(d), normal((3, 2048), f16, seed=1).to(d), normal((1024, 2048), f16, 0, 0.05, seed=2).to(d).t()], {}), tag="three_rows_bias_f16")
+    add(aten.mm.default, lambda d: ([normal((2048, 512), bf16, seed=1).to(d).t(), normal((2048, 768), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_transposed_k2048")
     add(aten.mm.default, lambda d: (_to(d, torch.eye(256, dtype=bf16), normal((256, 256), bf16, seed=2)), {}), exact=True, tag="identity")
     add(aten.mm.default, lambda d: (_to(d, torch.empty(2, 0, dtype=f32), torch.empty(0, 3, dtype=f32)), {}), tag="k0")
     add(aten.mm.default, lambda d: (_to(d, torch.empty(0, 8, dtype=bf16), normal((8, 16), bf16, seed=1)), {}), tag="m0")
