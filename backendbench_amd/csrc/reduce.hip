@@ -6,8 +6,9 @@
 //   rows_block   inner == 1, long or few rows: one 256-thread block per (row, split),
 //                wave reduce then LDS combine across the four waves;
 //   rows_thread  inner == 1, red <= 32: one thread per row;
-//   rows_sub     inner == 1, 32 < red <= 128, many rows (pooling over a 7x7 map): sixteen lanes
-//                per row, four rows per wave, DPP reduce inside the 16-lane row;
+//   rows_sub     inner == 1, many rows of at most 64 vectors (pooling over a 7x7 map, a 197-wide
+//                attention row): sixteen lanes per row, four rows per wave, DPP reduce inside the
+//                16-lane row;
 //   cols         inner > 1: 64 lanes along inner (coalesced, one 128-bit load each when inner
 //                allows) x 4 along red, LDS combine;
 //   final        second pass over per-split partial states when a launch was split
@@ -260,15 +261,13 @@ __global__ __launch_bounds__(kRedBlock) void rows_block_kernel(const T* __restri
   }
 }
 
-// Sixteen lanes per row: the wave's four rows are one contiguous span of memory, every lane
-// reads elements j, j + 16, ... of its row.  All lanes of a wave stay in the loop (the DPP
-// reduce is wave-wide); rows past the end accumulate nothing and write nothing.
-// VEC: rows are whole 16-byte vectors on 16-byte boundaries; lane j takes vectors j, j + 16, ...
-template <typename T, typename O, typename R, int FIN, bool VEC>
+// Sixteen lanes per row, four rows per wave (one contiguous span of memory); MODE as in
+// accumulate_span: vectors for aligned rows, the aligned window around a misaligned row, or
+// single elements.  All lanes of a wave stay in the loop (the DPP reduce is wave-wide); rows past
+// the end accumulate nothing and write nothing.
+template <typename T, typename O, typename R, int FIN, int MODE>
 __global__ __launch_bounds__(kRedBlock) void rows_sub_kernel(const T* __restrict__ x, O* __restrict__ out,
                                                             int64_t outer, int64_t red, double divisor) {
-  using A = typename R::acc_t;
-  constexpr int V = Vec<T>::N;
   const int j = threadIdx.x & 15;
   const int64_t group0 = ((int64_t)blockIdx.x * kRedBlock + threadIdx.x) >> 4;
   const int64_t ngroups = (int64_t)gridDim.x * (kRedBlock / 16);
@@ -278,15 +277,8 @@ __global__ __launch_bounds__(kRedBlock) void rows_sub_kernel(const T* __restrict
     typename R::State st = R::init();
     if (row < outer) {
       const T* p = x + row * red;
-      if constexpr (VEC) {
-        for (int64_t i = (int64_t)j * V; i < red; i += 16 * V) {
-          const Vec<T> v = load_vec_nt(p + i);
-#pragma unroll
-          for (int e = 0; e < V; ++e) R::acc(st, (A)v.v[e], i + e);
-        }
-      } else {
-        for (int64_t i = j; i < red; i += 16) R::acc(st, (A)p[i], i);
-      }
+      const int a = MODE == 2 ? reduce_row_misalignment(p) : 0;
+      accumulate_span<T, R, MODE>(st, p, 0, red + a, j, 16, a, red);
     }
     st = row16_reduce(st, (R*)nullptr);
     if (j == 0 && row < outer) write_final<R, O, FIN>(out, row, st, divisor);
@@ -439,7 +431,7 @@ static Plan plan_reduce(int64_t outer, int64_t red, int64_t inner, int elem_size
   const int64_t want_blocks = kNumCU * 4;
   if (inner == 1) {
     if (red <= 8 && outer >= 4096) { p.kind = ROWS_THREAD; return p; }
-    if (red <= 16 * V && outer >= 8192) { p.kind = ROWS_SUB; return p; }  // up to one vector per lane (scalar rows: <= 128)
+    if (red <= 64 * V && outer >= 8192) { p.kind = ROWS_SUB; return p; }  // up to four vectors per lane: one batch
     if (red <= 32 && outer >= 4096) { p.kind = ROWS_THREAD; return p; }
     if (outer >= 2048 && red <= 16384) { p.kind = ROWS_WAVE; return p; }
     p.kind = ROWS_BLOCK;
@@ -497,9 +489,11 @@ static int run_reduce(const void* xv, int64_t outer, int64_t red, int64_t inner,
     case ROWS_SUB: {
       const int grid = grid_for(outer, kRedBlock / 16, kNumCU * 16);
       if (aligned16(x) && red % V == 0)
-        hipLaunchKernelGGL((rows_sub_kernel<T, O, R, FIN, true>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+        hipLaunchKernelGGL((rows_sub_kernel<T, O, R, FIN, 1>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+      else if (V > 1 && red > 128)  // shorter misaligned rows: single elements beat the masked window
+        hipLaunchKernelGGL((rows_sub_kernel<T, O, R, FIN, 2>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
       else
-        hipLaunchKernelGGL((rows_sub_kernel<T, O, R, FIN, false>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
+        hipLaunchKernelGGL((rows_sub_kernel<T, O, R, FIN, 0>), dim3(grid), dim3(kRedBlock), 0, st, x, out, outer, red, divisor);
       break;
     }
     case ROWS_WAVE: {

@@ -322,6 +322,12 @@ def edge_cases() -> List[Case]:
         add(aten.amax.default, lambda d, red=red, dt=dt, rows=rows: (_to(d, poison(normal((rows, red), dt, seed=3), 0.002, 5), [-1]), {}), tag=f"short_rows_{red}_{t}")
         add(aten.argmax.default, lambda d, red=red, dt=dt, rows=rows: (_to(d, poison((normal((rows, red), dt, seed=4) * 2).round(), 0.002, 6), -1), {}), exact=True, tag=f"short_rows_{red}_{t}")
     add(aten.mean.dim, lambda d: (_to(d, normal((16, 600, 7, 7), f16, 1.0, seed=1), [-1, -2], True), {}), tag="pool_7x7")
+    # many misaligned rows of 129 .. 512 elements (a 197-wide attention row): sixteen lanes per row over the aligned window
+    for red, dt in ((197, f16), (131, f32), (255, bf16), (509, f16)):
+        t = f"{dt}".split(".")[-1]
+        add(aten.sum.dim_IntList, lambda d, red=red, dt=dt: (_to(d, normal((8200, red), dt, seed=1), [-1], True), {}), tag=f"attn_rows_{red}_{t}")
+        add(aten.amax.default, lambda d, red=red, dt=dt: (_to(d, poison(normal((8200, red), dt, seed=3), 0.002, 5), [-1]), {}), tag=f"attn_rows_{red}_{t}")
+        add(aten.argmax.default, lambda d, red=red, dt=dt: (_to(d, poison((normal((8200, red), dt, seed=4) * 2).round(), 0.002, 6), -1), {}), exact=True, tag=f"attn_rows_{red}_{t}")
     add(aten.sum.dim_IntList, lambda d: (_to(d, randint((9000, 40), 100, 1, i32, low=-100), [-1]), {}), exact=True, tag="short_rows_int")
     add(aten.sum.dim_IntList, lambda d: ([normal((9000 * 64 + 1,), f32, seed=7).to(d)[1:].view(9000, 64), [-1]], {}), tag="short_rows_offset_view")
 
