@@ -23,6 +23,24 @@ template <typename T> struct MulF {
     return static_cast<T>(static_cast<M>(a) * static_cast<M>(b));
   }
 };
+// fp32 result from one fp32 and one half-precision operand (type promotion of a mixed-precision
+// residual add or scale): the narrow operand is widened in registers instead of by a separate
+// cast pass over memory.
+template <typename TA, typename TB> struct AddMixF {
+  using out_t = float; using in0_t = TA; using in1_t = TB; using in2_t = Unused;
+  static constexpr int NIN = 2;
+  float alpha;
+  __device__ __forceinline__ float operator()(TA a, TB b, Unused) const {
+    return static_cast<float>(a) + alpha * static_cast<float>(b);
+  }
+};
+template <typename TA, typename TB> struct MulMixF {
+  using out_t = float; using in0_t = TA; using in1_t = TB; using in2_t = Unused;
+  static constexpr int NIN = 2;
+  __device__ __forceinline__ float operator()(TA a, TB b, Unused) const {
+    return static_cast<float>(a) * static_cast<float>(b);
+  }
+};
 template <typename T> struct MaximumF {
   using out_t = T; using in0_t = T; using in1_t = T; using in2_t = Unused;
   static constexpr int NIN = 2;
@@ -191,11 +209,28 @@ extern "C" int mi355_binary(int op, const mi355_tensor* a, const mi355_tensor* b
   if ((rc = check_tensor(a, "mi355_binary", "a"))) return rc;
   if ((rc = check_tensor(b, "mi355_binary", "b"))) return rc;
   if ((rc = check_tensor(out, "mi355_binary", "out"))) return rc;
-  MI355_REQUIRE(a->dtype == out->dtype && b->dtype == out->dtype,
-                "mi355_binary: operands must already have the output dtype (%s, %s -> %s)",
-                dtype_name(a->dtype), dtype_name(b->dtype), dtype_name(out->dtype));
   const mi355_tensor* ins[2] = {a, b};
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (out->dtype == MI355_F32 && a->dtype != b->dtype && (op == MI355_ADD || op == MI355_MUL)) {
+    // add / mul of an fp32 and an f16 / bf16 operand into fp32
+    auto run = [&](auto ta, auto tb) -> int {
+      using TA = decltype(ta);
+      using TB = decltype(tb);
+      if (op == MI355_ADD) {
+        AddMixF<TA, TB> f;
+        f.alpha = static_cast<float>(alpha_f);
+        return launch_elementwise(f, ins, out, st, "mi355_binary(add, mixed)");
+      }
+      return launch_elementwise(MulMixF<TA, TB>{}, ins, out, st, "mi355_binary(mul, mixed)");
+    };
+    if (a->dtype == MI355_F32 && b->dtype == MI355_F16) return run(float{}, f16_t{});
+    if (a->dtype == MI355_F32 && b->dtype == MI355_BF16) return run(float{}, bf16_t{});
+    if (a->dtype == MI355_F16 && b->dtype == MI355_F32) return run(f16_t{}, float{});
+    if (a->dtype == MI355_BF16 && b->dtype == MI355_F32) return run(bf16_t{}, float{});
+  }
+  MI355_REQUIRE(a->dtype == out->dtype && b->dtype == out->dtype,
+                "mi355_binary: operands must already have the output dtype (%s, %s -> %s), except fp32 with f16 / bf16 for add and mul",
+                dtype_name(a->dtype), dtype_name(b->dtype), dtype_name(out->dtype));
   MI355_DISPATCH_NUMERIC(out->dtype, "mi355_binary", {
     using M = typename OpMath<T>::type;
     switch (op) {

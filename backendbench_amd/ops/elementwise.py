@@ -94,6 +94,14 @@ def _as_operand(self, other):
     return torch.full((), other, dtype=torch.result_type(self, other), device=self.device)
 
 
+_MIXED_OPS = (_lib.ADD, _lib.MUL)
+_HALF = (torch.float16, torch.bfloat16)
+
+
+def _one_fp32_one_half(da, db):
+    return (da == torch.float32 and db in _HALF) or (db == torch.float32 and da in _HALF)
+
+
 def _binary(op, a, b, alpha=1):
     b = _as_operand(a, b)
     dtype = a.dtype if a.dtype == b.dtype else torch.result_type(a, b)
@@ -102,8 +110,9 @@ def _binary(op, a, b, alpha=1):
     if dtype == torch.bool:  # or / and / or: compute in u8, any non-zero is True
         return cast(_binary(op, cast(a, torch.uint8), cast(b, torch.uint8), 1 if alpha else 0), torch.bool)
     shape = a.shape if a.shape == b.shape else _broadcast_shape(a.shape, b.shape)
-    a = cast(a, dtype)
-    b = cast(b, dtype)
+    if not (dtype == torch.float32 and op in _MIXED_OPS and _one_fp32_one_half(a.dtype, b.dtype)):
+        a = cast(a, dtype)   # fp32 (+|*) f16 / bf16 is widened inside the kernel, everything else here
+        b = cast(b, dtype)
     if a.stride() != b.stride():
         a, b = _align_layouts(shape, (a, b))
     out = _out_like_inputs(shape, dtype, (a, b))
@@ -131,7 +140,9 @@ def _binary_inplace(op, functional, self, other, **kw):
     if self.numel() == 0:
         return self
     alpha_f, alpha_i = _alpha_args(dtype, kw.get("alpha", 1))
-    b = cast(other if other.is_cuda else other.to(self.device), dtype)
+    b = other if other.is_cuda else other.to(self.device)
+    if not (op in _MIXED_OPS and _one_fp32_one_half(dtype, b.dtype)):
+        b = cast(b, dtype)
     mine = _lib.desc(self)
     launch("mi355_binary", op, mine, _desc_as(b, self.shape), alpha_f, alpha_i, mine)
     return self

@@ -203,6 +203,11 @@ def edge_cases() -> List[Case]:
     add(aten.add.Tensor, lambda d: (_to(d, normal((7, 599), f16, seed=1), normal((7, 599), f32, seed=2)), {}), tag="promote_odd")
     add(aten.mul.Tensor, lambda d: ([normal((9, 1001), f32, seed=1).to(d)[:, ::2], normal((501,), f32, seed=2).to(d)], {}), tag="strided_cols_odd")
     add(aten.clamp.Tensor, lambda d: (_to(d, normal((11, 401), f32, seed=1), normal((401,), f32, -0.5, 0.1, seed=2), normal((11, 1), f32, 0.5, 0.1, seed=3)), {}), tag="bounds_broadcast_odd")
+    # fp32 with f16 / bf16: the narrow operand is widened inside the kernel
+    add(aten.mul.Tensor, lambda d: (_to(d, normal((33, 64), f32, seed=1), normal((64,), bf16, seed=2)), {}), tag="f32_times_bf16_row")
+    add(aten.add.Tensor, lambda d: ([normal((40, 24), f16, seed=1).to(d).t(), normal((24, 40), f32, seed=2).to(d)], {"alpha": -1.5}), tag="f16_t_plus_f32_alpha")
+    add(aten.mul.Tensor, lambda d: (_to(d, poison(normal((5, 0, 3), bf16, seed=1), 0.0, 1), normal((5, 1, 3), f32, seed=2)), {}), tag="mixed_empty")
+    add(aten.add.Tensor, lambda d: (_to(d, poison(normal((4100,), f16, seed=1), 0.01, 3), normal((4100,), f32, seed=2)), {}), tag="mixed_flat_specials")
     # channels-last operand with a per-channel broadcast: the kernel walks the dims in the output's memory order
     add(aten.mul.Tensor, lambda d: ([normal((6, 40, 9, 7), f16, seed=1).to(d).to(memory_format=torch.channels_last), normal((1, 40, 1, 1), f16, seed=2).to(d)], {}), tag="channels_last_scale")
     add(aten.add.Tensor, lambda d: ([normal((4, 24, 5, 6), f32, seed=1).to(d).to(memory_format=torch.channels_last), normal((4, 24, 5, 6), f32, seed=2).to(d)], {}), tag="channels_last_plus_nchw")

@@ -77,7 +77,9 @@ typedef enum mi355_binary_op {
 } mi355_binary_op;
 
 /* out = a (op) b with a, b already broadcast to out's shape (stride 0 where expanded)
- * and already of out's dtype.  MI355_ADD computes a + alpha*b (alpha_f for floating
+ * and already of out's dtype (one exception, ATen's type promotion done in registers: for
+ * MI355_ADD / MI355_MUL into fp32, one of a, b may be f16 or bf16 while the other is fp32).
+ * MI355_ADD computes a + alpha*b (alpha_f for floating
  * dtypes, alpha_i for integer dtypes).  MI355_MAXIMUM / MI355_MINIMUM propagate NaN.
  * `out` may be `a` itself (in-place overloads).
  * Slots: add__Tensor (op_map.py:266), mul__Tensor (op_map.py:749),
