@@ -92,7 +92,7 @@ static int run_index_select(const void* src, const void* index, int idx_dtype, v
                             int64_t n_idx, int64_t row_units, int32_t* err, hipStream_t st) {
   const int64_t rows = outer * n_idx;
   const bool i64 = idx_dtype == MI355_I64;
-  if (row_units >= kWave) {
+  if (row_units >= 2 * kWave) {  // rows of 2 KB and more: a wave per row; shorter rows: a thread per 16-byte unit
     const int grid = grid_for(rows, kIxBlock / kWave, kNumCU * 32);
     if (i64) hipLaunchKernelGGL((index_rows_wave_kernel<U, int64_t>), dim3(grid), dim3(kIxBlock), 0, st, (const U*)src, index, (U*)out, outer, n_src, n_idx, row_units, err);
     else hipLaunchKernelGGL((index_rows_wave_kernel<U, int32_t>), dim3(grid), dim3(kIxBlock), 0, st, (const U*)src, index, (U*)out, outer, n_src, n_idx, row_units, err);
