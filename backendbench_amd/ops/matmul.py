@@ -3,7 +3,7 @@
 import torch
 
 from .. import _lib
-from ._common import cast, dense, device_managed, launch, new_dense
+from ._common import cast, copy_into, dense, device_managed, launch, new_dense
 
 _GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32, torch.float64)
 _SPLITK_MAX_OUT = 128 * 128 * 256  # the planner never splits problems with 256 or more 128x128 tiles
@@ -44,6 +44,21 @@ def _gemm(a, b, c, alpha, beta):
     # layout (a transposed left operand, sliced views) is densified once with the copy kernel: one
     # pass over the operand, instead of the whole product on the FMA fallback.
     if M * N >= 64 * 64 and K >= 16 and a.dtype != torch.float64:
+        V = 16 // a.element_size()
+        if K % V:
+            # rows of K elements would not start on 16-byte boundaries: both operands are copied
+            # once into K-contiguous buffers padded with zeros to a multiple of 64 (exact: the pad
+            # adds 0 * 0 terms), instead of running the whole product on the FMA fallback
+            Kp = (K + 63) // 64 * 64
+            ap = torch.zeros((M, Kp), dtype=a.dtype, device=a.device)
+            copy_into(ap[:, :K], a)
+            btp = torch.zeros((N, Kp), dtype=a.dtype, device=a.device)
+            copy_into(btp[:, :K], b.t())
+            a, b, K = ap, btp.t(), Kp
+        elif b.stride(1) == 1 and N > 1 and (N % V or b.stride(0) % V or b.data_ptr() % 16):
+            # a row-major right operand whose rows are misaligned (N = 1001): its transpose is
+            # K-contiguous, which the kernels take for any N
+            b = dense(b.t()).t()
         if a.stride(1) != 1 and M > 1 and K > 1:
             # a transposed left operand (x.t() @ dy) goes in as it is when the MFMA kernels take it
             direct = (a.stride(0) == 1 and a.element_size() == 2 and K % 64 == 0 and M % 8 == 0

@@ -436,6 +436,13 @@ def edge_cases() -> List[Case]:
     add(aten.addmm.default, lambda d: ([normal((200,), f32, seed=3).to(d), normal((64, 1024), f32, seed=1).to(d), normal((200, 1024), f32, 0, 0.05, seed=2).to(d).t()], {}), tag="splitk_linear_f32")
     add(aten.mm.default, lambda d: (_to(d, normal((64, 1040), f32, seed=1), normal((1040, 256), f32, 0, 0.05, seed=2)), {}), tag="splitk_f32")
     add(aten.mm.default, lambda d: ([normal((320, 512), bf16, seed=1).to(d).t(), normal((320, 768), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_transposed")
+    # layouts the MFMA kernels cannot address directly: K no multiple of the vector (operands copied into zero-padded
+    # K-contiguous buffers), a row-major right operand with misaligned rows (re-laid K-contiguous)
+    add(aten.mm.default, lambda d: (_to(d, normal((260, 100), bf16, seed=1), normal((100, 264), bf16, 0, 0.1, seed=2)), {}), tag="k_unaligned_bf16")
+    add(aten.addmm.default, lambda d: (_to(d, normal((264,), f32, seed=3), normal((130, 50), f32, seed=1), normal((50, 264), f32, 0, 0.1, seed=2)), {"beta": 0.5}), tag="k_unaligned_f32")
+    add(aten.mm.default, lambda d: ([poison(normal((300, 37), f16, seed=1), 0.01, 3).to(d), normal((261, 37), f16, 0, 0.1, seed=2).to(d).t()], {}), tag="k_unaligned_specials_f16")
+    add(aten.mm.default, lambda d: (_to(d, normal((300, 64), bf16, seed=1), normal((64, 263), bf16, 0, 0.1, seed=2)), {}), tag="nn_odd_n_bf16")
+    add(aten.addmm.default, lambda d: (_to(d, normal((1001,), f32, seed=3), normal((70, 128), f32, seed=1), normal((128, 1001), f32, 0, 0.1, seed=2)), {}), tag="nn_odd_n_f32")
     # one row against a large weight (decoding one token): MFMA tiles split along K, not the FMA fallback
     add(aten.mm.default, lambda d: ([normal((1, 2048), bf16, seed=1).to(d), normal((1024, 2048), bf16, 0, 0.05, seed=2).to(d).t()], {}), tag="single_row_bf16")
     add(aten.mm.default, lambda d: (_to(d, normal((1, 4096), f32, seed=1), normal((4096, 1000), f32, 0, 0.05, seed=2)), {}), tag="single_row_f32")
