@@ -185,16 +185,29 @@ __global__ __launch_bounds__(kSmBlock) void softmax_cols_kernel(const T* __restr
   }
 }
 
-// inner > 1 with 128-bit accesses along inner: block = (64, R).  Lane tx owns V consecutive
-// columns, the R row groups split the softmax axis; their online (max, sum) pairs meet in LDS,
-// then every thread normalises the rows it read (second read from L2).  inner % V == 0 and
-// 16-byte aligned operands.  grid = (ceil(inner / (64 V)), outer).
+// inner > 1: block = (64, R).  Lane tx owns V consecutive columns (one 128-bit access; V = 1:
+// single elements, for an inner extent or alignment that allows no vectors), the R row groups
+// split the softmax axis; their online (max, sum) pairs meet in LDS, then every thread
+// normalises the rows it read (second read from L2).  V > 1 needs inner % V == 0 and 16-byte
+// aligned operands.  grid = (ceil(inner / (64 V)), outer).
 constexpr int kSmColsR = 8;
-template <typename T, typename O, bool LOG>
+template <typename T, typename O, bool LOG, int V>
 __global__ __launch_bounds__(kWave * kSmColsR) void softmax_cols_vec_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                           int64_t n, int64_t inner) {
   using A = typename SmAcc<T>::type;
-  constexpr int V = Vec<T>::N, R = kSmColsR;
+  constexpr int R = kSmColsR;
+  struct Vals { T v[V]; };
+  auto load = [](const T* ptr) {
+    if constexpr (V == 1) {
+      return Vals{{*ptr}};
+    } else {
+      const Vec<T> t = load_vec(ptr);
+      Vals r;
+#pragma unroll
+      for (int j = 0; j < V; ++j) r.v[j] = t.v[j];
+      return r;
+    }
+  };
   __shared__ MS<A> smem[R][V][kWave];
   const int tx = threadIdx.x, ty = threadIdx.y;
   const int64_t col = ((int64_t)blockIdx.x * kWave + tx) * V;
@@ -206,7 +219,7 @@ __global__ __launch_bounds__(kWave * kSmColsR) void softmax_cols_vec_kernel(cons
   for (int j = 0; j < V; ++j) acc[j] = {-INFINITY, A(0)};
   if (live) {
     for (int64_t r = ty; r < n; r += R) {
-      const Vec<T> t = load_vec(p + r * inner);
+      const Vals t = load(p + r * inner);
 #pragma unroll
       for (int j = 0; j < V; ++j) ms_update(acc[j], static_cast<A>(t.v[j]));
     }
@@ -226,7 +239,7 @@ __global__ __launch_bounds__(kWave * kSmColsR) void softmax_cols_vec_kernel(cons
     ls[j] = sm_log(a.s);
   }
   for (int64_t r = ty; r < n; r += R) {
-    const Vec<T> t = load_vec(p + r * inner);
+    const Vals t = load(p + r * inner);
     VecN<O, V> o;
 #pragma unroll
     for (int j = 0; j < V; ++j) {
@@ -243,12 +256,21 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
   O* y = static_cast<O*>(yv);
   constexpr int V = Vec<T>::N;
   if (inner > 1) {
-    if (V > 1 && inner % V == 0 && n >= 4 * kSmColsR && aligned16(x) &&
+    // vectors along inner unless that leaves most of the chip without a block (a softmax over the
+    // first dim of a matrix): single columns per lane then give V times the blocks
+    const bool enough_blocks = ((inner + kWave * V - 1) / (kWave * V)) * outer >= kNumCU;
+    if (V > 1 && inner % V == 0 && n >= 4 * kSmColsR && aligned16(x) && enough_blocks &&
         reinterpret_cast<uintptr_t>(y) % (sizeof(O) * V) == 0 && outer < 65536) {
       const int64_t xb = (inner + kWave * V - 1) / (kWave * V);
       MI355_REQUIRE(xb < (int64_t(1) << 31), "mi355_softmax: inner extent too large");
-      hipLaunchKernelGGL((softmax_cols_vec_kernel<T, O, LOG>), dim3((unsigned)xb, (unsigned)outer), dim3(kWave, kSmColsR), 0, st, x, y, n, inner);
+      hipLaunchKernelGGL((softmax_cols_vec_kernel<T, O, LOG, V>), dim3((unsigned)xb, (unsigned)outer), dim3(kWave, kSmColsR), 0, st, x, y, n, inner);
       return check_launch("mi355_softmax(cols, vector)");
+    }
+    if (n >= 4 * kSmColsR && outer < 65536) {  // no vectors along inner (odd extent, misaligned): the same shape on single elements
+      const int64_t xb = (inner + kWave - 1) / kWave;
+      MI355_REQUIRE(xb < (int64_t(1) << 31), "mi355_softmax: inner extent too large");
+      hipLaunchKernelGGL((softmax_cols_vec_kernel<T, O, LOG, 1>), dim3((unsigned)xb, (unsigned)outer), dim3(kWave, kSmColsR), 0, st, x, y, n, inner);
+      return check_launch("mi355_softmax(cols, split rows)");
     }
     const int grid = grid_for(outer * inner, kSmBlock, kNumCU * 16);
     hipLaunchKernelGGL((softmax_cols_kernel<T, O, LOG>), dim3(grid), dim3(kSmBlock), 0, st, x, y, outer, n, inner);

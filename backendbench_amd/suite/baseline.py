@@ -346,6 +346,9 @@ def edge_cases() -> List[Case]:
     add(aten._softmax.default, lambda d: (_to(d, normal((3, 50000), f32, 0, 2, seed=1), -1, False), {}), tag="long_rows")
     add(aten._softmax.default, lambda d: (_to(d, normal((3, 20000), bf16, 0, 2, seed=1), -1, False), {}), tag="long_rows_bf16")
     add(aten._softmax.default, lambda d: (_to(d, normal((5, 300, 7), f32, seed=1), 1, False), {}), tag="mid")
+    add(aten._log_softmax.default, lambda d: (_to(d, poison(normal((3, 100, 33), f16, 0, 2, seed=1), 0.002, 4), 1, False), {}), tag="mid_odd_inner_f16")
+    add(aten._softmax.default, lambda d: (_to(d, normal((2, 40, 49), bf16, 0, 2, seed=1), 1, False), {}), tag="mid_7x7_bf16")
+    add(aten._softmax.default, lambda d: (_to(d, normal((64, 520), f32, 0, 2, seed=1), 0, False), {}), tag="first_dim_few_blocks")
     add(aten._softmax.default, lambda d: ([normal((40, 24), f32, seed=2).to(d).t(), -1, False], {}), tag="transposed")
     add(aten._softmax.default, lambda d: (_to(d, torch.tensor([[float("-inf"), float("-inf")], [float("inf"), 1.0], [float("nan"), 1.0],
                                                                  [float("-inf"), 0.0], [1.0, 2.0]], dtype=f32), -1, False), {}), tag="special")
