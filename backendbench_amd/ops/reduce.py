@@ -78,8 +78,32 @@ def _out_shape(x, dims, keepdim):
     return [s for d, s in enumerate(x.shape) if d not in dims]
 
 
+def _adjacent_runs(dims):
+    runs = [[dims[0]]]
+    for d in dims[1:]:
+        if d == runs[-1][-1] + 1:
+            runs[-1].append(d)
+        else:
+            runs.append([d])
+    return runs
+
+
 def _run_reduce(op, x, dims, keepdim, out_dtype):
     """x: tensor of a natively reducible dtype with numel > 0 and red > 0."""
+    if len(dims) > 1 and op in (_lib.SUM, _lib.MEAN, _lib.AMAX):
+        runs = _adjacent_runs(dims)
+        if len(runs) > 1 and (x.is_contiguous() or _memory_view3(x, dims) is None):
+            # Reduced dims that are not neighbours (a batch-norm style sum over N, H, W): the
+            # innermost run first, then the rest on the much smaller intermediate (kept in fp32 /
+            # int64 so that it is rounded once) - one pass over x instead of a permuting copy + a pass.
+            if out_dtype.is_floating_point:
+                inter = torch.float64 if x.dtype == torch.float64 else torch.float32
+            else:
+                inter = out_dtype
+            first = _run_reduce(op, x, runs[-1], True, inter)
+            rest = [d for run in runs[:-1] for d in run]
+            res = _run_reduce(op, first, rest, True, inter)
+            return cast(res, out_dtype).view(_out_shape(x, dims, keepdim))
     xd, outer, red, inner = _view3(x, dims)
     out = new_dense(_out_shape(x, dims, keepdim), out_dtype, x.device)
     lib = _lib.load()
