@@ -13,7 +13,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi355_aten.so"
-ABI_VERSION = 2
+ABI_VERSION = 3
 MAX_DIMS = 8
 
 # mi355_dtype
@@ -62,6 +62,7 @@ SIGNATURES = {
     "mi355_binary": (c_int, [c_int, _P, _P, c_double, c_int64, _P, c_void_p]),
     "mi355_unary": (c_int, [c_int, _P, c_int, c_double, c_double, c_int64, c_int64, _P, c_void_p]),
     "mi355_where": (c_int, [_P, _P, _P, _P, c_void_p]),
+    "mi355_clamp_tensor": (c_int, [_P, _P, _P, _P, c_void_p]),
     "mi355_copy": (c_int, [_P, _P, c_void_p]),
     "mi355_reduce_workspace_bytes": (c_int64, [c_int, c_int, c_int64, c_int64, c_int64]),
     "mi355_reduce": (

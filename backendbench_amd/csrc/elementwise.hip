@@ -298,6 +298,31 @@ extern "C" int mi355_where(const mi355_tensor* cond, const mi355_tensor* a, cons
   }
 }
 
+// min(max(x, lo), hi) with the NaN and signed-zero rules of the two binary ops, in one pass.
+template <typename T> struct ClampTensorF {
+  using out_t = T; using in0_t = T; using in1_t = T; using in2_t = T;
+  static constexpr int NIN = 3;
+  __device__ __forceinline__ T operator()(T x, T lo, T hi) const {
+    return MinimumF<T>{}(MaximumF<T>{}(x, lo, Unused{}), hi, Unused{});
+  }
+};
+
+extern "C" int mi355_clamp_tensor(const mi355_tensor* x, const mi355_tensor* lo, const mi355_tensor* hi,
+                                  const mi355_tensor* out, void* stream) {
+  int rc;
+  if ((rc = check_tensor(x, "mi355_clamp_tensor", "x"))) return rc;
+  if ((rc = check_tensor(lo, "mi355_clamp_tensor", "lo"))) return rc;
+  if ((rc = check_tensor(hi, "mi355_clamp_tensor", "hi"))) return rc;
+  if ((rc = check_tensor(out, "mi355_clamp_tensor", "out"))) return rc;
+  MI355_REQUIRE(x->dtype == out->dtype && lo->dtype == out->dtype && hi->dtype == out->dtype,
+                "mi355_clamp_tensor: x, lo and hi must already have the output dtype");
+  const mi355_tensor* ins[3] = {x, lo, hi};
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_NUMERIC(out->dtype, "mi355_clamp_tensor",
+                         { return launch_elementwise(ClampTensorF<T>{}, ins, out, st, "mi355_clamp_tensor"); });
+  return MI355_OK;
+}
+
 extern "C" int mi355_copy(const mi355_tensor* src, const mi355_tensor* dst, void* stream) {
   int rc;
   if ((rc = check_tensor(src, "mi355_copy", "src"))) return rc;

@@ -291,6 +291,20 @@ def clamp_tensor(self, min=None, max=None):
     """aten.clamp.Tensor: tensor bounds, min(max(self, lo), hi) with NaN propagation."""
     if min is None and max is None:
         raise RuntimeError("torch.clamp: At least one of 'min' or 'max' must not be None")
+    if min is not None and max is not None and self.dtype == min.dtype == max.dtype and self.is_cuda \
+            and not self.dtype.is_complex and self.dtype != torch.bool:
+        # both bounds, no promotion: one fused pass
+        if self.shape == min.shape == max.shape:
+            shape = self.shape
+        else:
+            shape = _broadcast_shape(self.shape, min.shape, max.shape)
+        x, lo, hi = self, min, max
+        if not (x.stride() == lo.stride() == hi.stride()):
+            x, lo, hi = _align_layouts(shape, (x, lo, hi))
+        out = _out_like_inputs(shape, self.dtype, (x, lo, hi))
+        if out.numel():
+            launch("mi355_clamp_tensor", _desc_as(x, shape), _desc_as(lo, shape), _desc_as(hi, shape), _lib.desc(out))
+        return out
     out = self
     if min is not None:
         out = _binary(_lib.MAXIMUM, out, min)

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define MI355_ABI_VERSION 2
+#define MI355_ABI_VERSION 3
 #define MI355_MAX_DIMS 8
 
 typedef enum mi355_dtype {
@@ -103,6 +103,13 @@ int mi355_unary(int op, const mi355_tensor* x, int bounds, double lo_f, double h
  * Slot: where__self (op_map.py:1132). */
 int mi355_where(const mi355_tensor* cond, const mi355_tensor* a, const mi355_tensor* b,
                 const mi355_tensor* out, void* stream);
+
+/* out = min(max(x, lo), hi) with tensor bounds, one pass; NaN in any operand propagates.  x, lo,
+ * hi already broadcast to out's shape and of out's dtype.  A call with one bound only is
+ * mi355_binary(MI355_MAXIMUM / MI355_MINIMUM).
+ * Slot: clamp__Tensor (op_map.py:372). */
+int mi355_clamp_tensor(const mi355_tensor* x, const mi355_tensor* lo, const mi355_tensor* hi,
+                       const mi355_tensor* out, void* stream);
 
 /* dst = (dst dtype) src, any strides on either side, same shape (src may broadcast).
  * Host-side helper for the slots above and below: type promotion and
