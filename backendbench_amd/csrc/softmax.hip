@@ -1,6 +1,7 @@
 // _softmax / _log_softmax over the middle axis of a dense [outer, dim, inner] view, fp32 math
 // (fp64 for f64 input, on the block and cols kernels only).
 //
+//   sub    inner == 1, rows of at most 32 vectors: 1 .. 32 lanes per row, several rows per wave;
 //   tile   inner == 1, row fits the registers of 1, 2 or 4 cooperating waves: one HBM read,
 //          max and sum by wave all-reduce (+ one LDS exchange between waves), one HBM write;
 //   block  inner == 1, longer rows: 256 threads keep an online (max, sum) pair in one
@@ -63,6 +64,72 @@ __global__ __launch_bounds__(sm_tile_block(W)) void softmax_tile_kernel(const T*
   auto fin = [ls, inv](float v, int64_t) { return LOG ? v - ls : v * inv; };
   if constexpr (SHIFT) tile.store_shifted(y + row * n, n, a, t, fin);
   else tile.store(y + row * n, n, t, fin);
+}
+
+// Rows of at most 32 vectors: G = 1 .. 32 lanes per row (the smallest power of two whose lanes,
+// at one 16-byte vector or V single elements each, cover the row), 64 / G rows per wave.  Max
+// and sum meet by DPP inside the 16-lane rows (G = 32: one more exchange across them), so a
+// [1M, 8] softmax runs 32 rows per wave instead of one.
+template <int G, typename Op> __device__ __forceinline__ float sub_allreduce(float v, Op op) {
+  if constexpr (G >= 2) v = op(v, dpp<0xB1>(v));    // quad_perm [1,0,3,2]
+  if constexpr (G >= 4) v = op(v, dpp<0x4E>(v));    // quad_perm [2,3,0,1]
+  if constexpr (G >= 8) v = op(v, dpp<0x141>(v));   // row_half_mirror: the other quad of 8 lanes
+  if constexpr (G >= 16) v = op(v, dpp<0x140>(v));  // row_mirror: the other half of 16 lanes
+  if constexpr (G >= 32) v = op(v, __shfl_xor(v, 16, kWave));
+  return v;
+}
+template <typename T, typename O, bool LOG, int G, bool VEC>
+__global__ __launch_bounds__(kSmBlock) void softmax_sub_kernel(const T* __restrict__ x, O* __restrict__ y,
+                                                              int64_t rows, int64_t n) {
+  constexpr int V = Vec<T>::N;
+  static_assert(kSmBlock % G == 0, "groups must not straddle blocks");
+  const int t = threadIdx.x % G;
+  int64_t row = ((int64_t)blockIdx.x * kSmBlock + threadIdx.x) / G;
+  const bool active = row < rows;  // the lanes of a group past the end still take part in the exchanges
+  if (!active) row = rows - 1;
+  const T* p = x + row * n;
+  float v[V];
+  if constexpr (VEC) {
+    if ((int64_t)t * V < n) {  // n % V == 0: a vector is inside the row or past it
+      const Vec<T> in = load_vec(p + t * V);
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] = static_cast<float>(in.v[j]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] = -INFINITY;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j) v[j] = t + G * j < n ? static_cast<float>(p[t + G * j]) : -INFINITY;
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < V; ++j) m = v[j] > m ? v[j] : m;
+  m = sub_allreduce<G>(m, MaxOp());
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const float d = v[j] - m;
+    const float e = __expf(d);
+    v[j] = LOG ? d : e;
+    s += e;
+  }
+  s = sub_allreduce<G>(s, SumOp());
+  if (!active) return;
+  const float ls = __logf(s), inv = 1.f / s;
+  O* q = y + row * n;
+  if constexpr (VEC) {
+    if ((int64_t)t * V < n) {
+      VecN<O, V> r;
+#pragma unroll
+      for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(LOG ? v[j] - ls : v[j] * inv);
+      st<O, V>(q + t * V, r);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      if (t + G * j < n) q[t + G * j] = static_cast<O>(LOG ? v[j] - ls : v[j] * inv);
+  }
 }
 
 // Online (max, sum) pair in the accumulation type A (float; double for f64 input); see the
@@ -291,8 +358,22 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
                               : (!tvec && (reinterpret_cast<uintptr_t>(x) / sizeof(T)) % TV ==
                                               (reinterpret_cast<uintptr_t>(y) / sizeof(O)) % TV);
   bool done = false;
+  if constexpr (!std::is_same<T, double>::value)
+  if (n <= 32 * V && outer < (int64_t(1) << 31)) {
+    // short rows: several per wave
+    const int64_t need = (n + V - 1) / V;
+#define MI355_SM_SUB(G_)                                                                                   \
+  if (!done && need <= G_) {                                                                               \
+    const unsigned nblk = (unsigned)((outer * G_ + kSmBlock - 1) / kSmBlock);                                \
+    if (vec) hipLaunchKernelGGL((softmax_sub_kernel<T, O, LOG, G_, true>), dim3(nblk), dim3(kSmBlock), 0, st, x, y, outer, n); \
+    else hipLaunchKernelGGL((softmax_sub_kernel<T, O, LOG, G_, false>), dim3(nblk), dim3(kSmBlock), 0, st, x, y, outer, n);    \
+    done = true;                                                                                           \
+  }
+    MI355_SM_SUB(1) MI355_SM_SUB(2) MI355_SM_SUB(4) MI355_SM_SUB(8) MI355_SM_SUB(16) MI355_SM_SUB(32)
+#undef MI355_SM_SUB
+  }
   if constexpr (!std::is_same<T, double>::value)  // f64 rows take the block kernel (double accumulation)
-  if (outer < (int64_t(1) << 31)) {
+  if (!done && outer < (int64_t(1) << 31)) {
     done = dispatch_row_tile<T>(tshift ? n + TV - 1 : n, tvec || tshift, [&](auto nv, auto w, auto v) {
       constexpr int NV = decltype(nv)::value, W = decltype(w)::value;
       constexpr bool VEC = decltype(v)::value;

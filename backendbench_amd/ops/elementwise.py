@@ -35,9 +35,14 @@ def _align_layouts(shape, tensors):
     """Full-shape operands that disagree on layout run on the strided kernel, where the odd one is
     read one scattered element per lane.  When some operand is row-major and another is its
     (batched) transpose, the transpose is made dense first with the tiled transposing copy: two
-    coalesced passes instead of one scattered pass."""
+    coalesced passes instead of one scattered pass.  Small problems keep the single pass: when the
+    whole operand is a couple of MB the second launch costs more than the scatter, and matrices of
+    up to 128 KB each (attention heads) stay in cache while their lines are picked apart."""
     full = [t for t in tensors if t.shape == shape]
     if len(full) < 2 or len(shape) < 2 or not any(t.is_contiguous() for t in full):
+        return tensors
+    esize = max(t.element_size() for t in full)
+    if shape[-1] * shape[-2] * esize <= (128 << 10) or shape.numel() * esize <= (2 << 20):
         return tensors
     out = []
     for t in tensors:

@@ -200,6 +200,10 @@ def edge_cases() -> List[Case]:
     add(aten.add.Tensor, lambda d: (_to(d, normal((3, 1367), bf16, seed=1), normal((1367,), bf16, seed=2)), {"alpha": 0.5}), tag="ragged_tail_bf16")
     add(aten.where.self, lambda d: (_to(d, normal((5, 1, 77), f32, seed=1) > 0, normal((5, 19, 77), f16, seed=2), normal((1, 19, 1), f16, seed=3)), {}), exact=True, tag="three_way_77")
     add(aten.maximum.default, lambda d: ([normal((67, 65), f32, seed=1).to(d), normal((65, 67), f32, seed=2).to(d).t()], {}), tag="transposed_odd")
+    # one operand the transpose of the other's layout: large matrices are re-laid first, small or batched ones read in place
+    add(aten.add.Tensor, lambda d: ([normal((1100, 1030), f32, seed=1).to(d), normal((1030, 1100), f32, seed=2).to(d).t()], {}), tag="mixed_layout_large")
+    add(aten.mul.Tensor, lambda d: ([normal((4, 6, 64, 197), f16, seed=1).to(d).transpose(-1, -2), normal((4, 6, 197, 64), f16, seed=2).to(d)], {}), tag="mixed_layout_heads")
+    add(aten.where.self, lambda d: ([cond((900, 1200), 1).to(d), normal((1200, 900), f16, seed=2).to(d).t(), normal((900, 1200), f16, seed=3).to(d)], {}), exact=True, tag="mixed_layout_large")
     add(aten.add.Tensor, lambda d: (_to(d, normal((7, 599), f16, seed=1), normal((7, 599), f32, seed=2)), {}), tag="promote_odd")
     add(aten.mul.Tensor, lambda d: ([normal((9, 1001), f32, seed=1).to(d)[:, ::2], normal((501,), f32, seed=2).to(d)], {}), tag="strided_cols_odd")
     add(aten.clamp.Tensor, lambda d: (_to(d, normal((11, 401), f32, seed=1), normal((401,), f32, -0.5, 0.1, seed=2), normal((11, 1), f32, 0.5, 0.1, seed=3)), {}), tag="bounds_broadcast_odd")
@@ -384,6 +388,15 @@ def edge_cases() -> List[Case]:
     add(aten._softmax.default, lambda d: (_to(d, normal((37, 129), f64, 0, 2, seed=1), -1, False), {}), tag="last_f64")
     add(aten._softmax.default, lambda d: (_to(d, normal((5, 30, 7), f64, seed=1), 1, False), {}), tag="mid_f64")
     add(aten._log_softmax.default, lambda d: (_to(d, normal((3, 5000), f64, 0, 2, seed=1), -1, False), {}), tag="long_rows_f64")
+    # short rows: 1, 2, 4, 8, 16 and 32 lanes per row, vector and single-element layouts
+    for rl, dt, t in ((2, f32, "f32"), (3, f16, "f16"), (8, f32, "f32"), (10, f32, "f32"), (16, bf16, "bf16"), (24, f16, "f16"),
+                     (49, f32, "f32"), (64, f16, "f16"), (100, bf16, "bf16"), (128, f32, "f32"), (255, f16, "f16"), (256, bf16, "bf16")):
+        add(aten._softmax.default, lambda d, rl=rl, dt=dt: (_to(d, normal((1037, rl), dt, 0, 2, seed=rl), -1, False), {}), tag=f"short_{rl}_{t}")
+    add(aten._log_softmax.default, lambda d: (_to(d, poison(normal((515, 8), f32, 0, 2, seed=1), 0.01, 4), -1, False), {}), tag="short_8_naninf")
+    add(aten._log_softmax.default, lambda d: (_to(d, poison(normal((130, 40), f16, 0, 2, seed=1), 0.005, 4), -1, False), {}), tag="short_40_naninf_f16")
+    add(aten._softmax.default, lambda d: (_to(d, normal((333, 64), f16, 0, 2, seed=1), -1, True), {}), tag="short_64_half_to_float")
+    add(aten._log_softmax.default, lambda d: (_to(d, normal((77, 10), bf16, 0, 2, seed=1), -1, True), {}), tag="short_10_half_to_float")
+    add(aten._softmax.default, lambda d: ([normal((64, 40), f32, 0, 2, seed=1).to(d)[:, 4:36], -1, False], {}), tag="short_row_slice")
     # long rows: 8- and 16-wave register tiles, then the two-pass block kernel
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((5, 12288), bf16, 1, 2, seed=1), [12288], normal((12288,), bf16, 1, 0.1, seed=2), normal((12288,), bf16, 0, 0.1, seed=3), 1e-5), {}), tag="row12288_bf16")
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((3, 40000), f32, -2, 3, seed=1), [40000], normal((40000,), f32, 1, 0.1, seed=2), None, 1e-5), {}), tag="row40000_f32")
