@@ -1,5 +1,6 @@
 // native_layer_norm over the last N elements of M dense rows: returns y, mean, rstd.
 //
+//   sub    rows of at most 32 vectors: 1 .. 32 lanes per row, several rows per wave;
 //   tile   row fits the registers of 1, 2 or 4 cooperating waves: one HBM read; mean by
 //          all-reduce, then the centred second moment from the same registers (exact
 //          two-step statistics at single-pass traffic); y written once;
@@ -128,6 +129,84 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
   }
 }
 
+// Rows of at most 32 vectors: G = 1 .. 32 lanes per row, 64 / G rows per wave (per-head q/k
+// norms over 64 or 128 elements).  A lane holds one 16-byte vector of its row, or V single
+// elements (column t + G j) when rows are not vector-aligned, and loads the gamma / beta of its
+// columns once; sums meet by DPP exchanges among the lanes of the row.
+template <typename T, typename Wt, typename S, int G, bool VEC>
+__global__ __launch_bounds__(kLnBlock) void layernorm_sub_kernel(const T* __restrict__ x, const Wt* __restrict__ w,
+                                                                const Wt* __restrict__ b, T* __restrict__ y,
+                                                                S* __restrict__ mean_out, S* __restrict__ rstd_out,
+                                                                int64_t rows, int64_t n, float eps) {
+  constexpr int V = Vec<T>::N;
+  static_assert(kLnBlock % G == 0, "groups must not straddle blocks");
+  const int t = threadIdx.x % G;
+  int64_t row = ((int64_t)blockIdx.x * kLnBlock + threadIdx.x) / G;
+  const bool active = row < rows;  // lanes past the last row still take part in the exchanges
+  if (!active) row = rows - 1;
+  const T* p = x + row * n;
+  float v[V], gw[V], gb[V];
+  bool in[V];
+  if constexpr (VEC) {
+    const bool inside = (int64_t)t * V < n;  // n % V == 0: a vector is inside the row or past it
+    VecN<T, V> xv;
+    VecN<Wt, V> wv, bv;
+    if (inside) {
+      xv = ld_nt<T, V>(p + t * V);
+      if (w) wv = ld<Wt, V>(w + t * V);
+      if (b) bv = ld<Wt, V>(b + t * V);
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      in[j] = inside;
+      v[j] = inside ? static_cast<float>(xv.v[j]) : 0.f;
+      gw[j] = inside && w ? static_cast<float>(wv.v[j]) : 1.f;
+      gb[j] = inside && b ? static_cast<float>(bv.v[j]) : 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const int c = t + G * j;
+      in[j] = c < n;
+      v[j] = in[j] ? static_cast<float>(p[c]) : 0.f;
+      gw[j] = in[j] && w ? static_cast<float>(w[c]) : 1.f;
+      gb[j] = in[j] && b ? static_cast<float>(b[c]) : 0.f;
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < V; ++j) s += v[j];
+  const float inv_n = 1.f / (float)n;
+  const float mean = sub_allreduce<G>(s, SumOp()) * inv_n;
+  float q = 0.f;
+#pragma unroll
+  for (int j = 0; j < V; ++j) {
+    const float d = in[j] ? v[j] - mean : 0.f;
+    v[j] = d;
+    q += d * d;
+  }
+  const float var = sub_allreduce<G>(q, SumOp()) * inv_n;
+  const float rstd = rsqrtf(var + eps);
+  if (!active) return;
+  if (t == 0) {
+    mean_out[row] = static_cast<S>(mean);
+    rstd_out[row] = static_cast<S>(rstd);
+  }
+  T* out = y + row * n;
+  if constexpr (VEC) {
+    if (in[0]) {
+      VecN<T, V> r;
+#pragma unroll
+      for (int j = 0; j < V; ++j) r.v[j] = static_cast<T>(v[j] * rstd * gw[j] + gb[j]);
+      st_nt<T, V>(out + t * V, r);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j)
+      if (in[j]) out[t + G * j] = static_cast<T>(v[j] * rstd * gw[j] + gb[j]);
+  }
+}
+
 // Welford state and Chan's merge, in the accumulation type A (float; double for f64 input).
 template <typename T> struct LnAcc { using type = float; };
 template <> struct LnAcc<double> { using type = double; };
@@ -215,7 +294,21 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
   MI355_REQUIRE(M < (int64_t(1) << 31), "mi355_layer_norm: too many rows (%lld)", (long long)M);
   const size_t param_bytes = 2 * (size_t)N * sizeof(W);
   bool done = false;
+  if constexpr (!std::is_same<T, double>::value)
+  if (N <= 32 * V) {  // short rows: several per wave
+    const int64_t need = (N + V - 1) / V;
+#define MI355_LN_SUB(G_)                                                                                  \
+  if (!done && need <= G_) {                                                                              \
+    const unsigned nblk = (unsigned)((M * G_ + kLnBlock - 1) / kLnBlock);                                   \
+    if (vec) hipLaunchKernelGGL((layernorm_sub_kernel<T, W, S, G_, true>), dim3(nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps); \
+    else hipLaunchKernelGGL((layernorm_sub_kernel<T, W, S, G_, false>), dim3(nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);    \
+    done = true;                                                                                          \
+  }
+    MI355_LN_SUB(1) MI355_LN_SUB(2) MI355_LN_SUB(4) MI355_LN_SUB(8) MI355_LN_SUB(16) MI355_LN_SUB(32)
+#undef MI355_LN_SUB
+  }
   if constexpr (!std::is_same<T, double>::value)  // f64 rows take the block kernel (double accumulation)
+  if (!done)
   done = dispatch_row_tile<T>(N, vec, [&](auto nv, auto wv, auto v) {
     constexpr int NV = decltype(nv)::value, WG = decltype(wv)::value;
     constexpr bool VEC = decltype(v)::value;

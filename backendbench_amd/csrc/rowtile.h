@@ -153,6 +153,15 @@ __device__ __forceinline__ T group_allreduce(T v, Op op, T* smem) {
   }
 }
 
+// All-reduce over the G = 1 .. 32 adjacent lanes that share a short row (G a power of two).
+template <int G, typename Op> __device__ __forceinline__ float sub_allreduce(float v, Op op) {
+  if constexpr (G >= 2) v = op(v, dpp<0xB1>(v));    // quad_perm [1,0,3,2]
+  if constexpr (G >= 4) v = op(v, dpp<0x4E>(v));    // quad_perm [2,3,0,1]
+  if constexpr (G >= 8) v = op(v, dpp<0x141>(v));   // row_half_mirror: the other quad of 8 lanes
+  if constexpr (G >= 16) v = op(v, dpp<0x140>(v));  // row_mirror: the other half of 16 lanes
+  if constexpr (G >= 32) v = op(v, __shfl_xor(v, 16, kWave));
+  return v;
+}
 // Picks (NV, W) for rows of n elements of T and calls body(NV, W, VEC) with integral
 // constants; false when the row does not fit (16 slabs over 4 waves, or 64 values per lane over
 // max_w waves).  Aligned rows get at most

@@ -70,14 +70,6 @@ __global__ __launch_bounds__(sm_tile_block(W)) void softmax_tile_kernel(const T*
 // at one 16-byte vector or V single elements each, cover the row), 64 / G rows per wave.  Max
 // and sum meet by DPP inside the 16-lane rows (G = 32: one more exchange across them), so a
 // [1M, 8] softmax runs 32 rows per wave instead of one.
-template <int G, typename Op> __device__ __forceinline__ float sub_allreduce(float v, Op op) {
-  if constexpr (G >= 2) v = op(v, dpp<0xB1>(v));    // quad_perm [1,0,3,2]
-  if constexpr (G >= 4) v = op(v, dpp<0x4E>(v));    // quad_perm [2,3,0,1]
-  if constexpr (G >= 8) v = op(v, dpp<0x141>(v));   // row_half_mirror: the other quad of 8 lanes
-  if constexpr (G >= 16) v = op(v, dpp<0x140>(v));  // row_mirror: the other half of 16 lanes
-  if constexpr (G >= 32) v = op(v, __shfl_xor(v, 16, kWave));
-  return v;
-}
 template <typename T, typename O, bool LOG, int G, bool VEC>
 __global__ __launch_bounds__(kSmBlock) void softmax_sub_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                               int64_t rows, int64_t n) {

@@ -397,6 +397,14 @@ def edge_cases() -> List[Case]:
     add(aten._softmax.default, lambda d: (_to(d, normal((333, 64), f16, 0, 2, seed=1), -1, True), {}), tag="short_64_half_to_float")
     add(aten._log_softmax.default, lambda d: (_to(d, normal((77, 10), bf16, 0, 2, seed=1), -1, True), {}), tag="short_10_half_to_float")
     add(aten._softmax.default, lambda d: ([normal((64, 40), f32, 0, 2, seed=1).to(d)[:, 4:36], -1, False], {}), tag="short_row_slice")
+    # short rows: 1 .. 32 lanes per row, vector and single-element layouts, every gamma / beta combination
+    for rl, dt, t, hw, hb in ((4, f32, "f32", True, True), (8, f16, "f16", True, False), (10, f32, "f32", True, True), (16, bf16, "bf16", False, True),
+                              (49, f32, "f32", True, True), (64, f16, "f16", True, True), (100, bf16, "bf16", False, False), (128, f32, "f32", True, True),
+                              (128, bf16, "bf16", True, True), (255, f16, "f16", True, True), (256, bf16, "bf16", True, False)):
+        add(aten.native_layer_norm.default,
+            lambda d, rl=rl, dt=dt, hw=hw, hb=hb: (_to(d, normal((1037, rl), dt, 1, 2, seed=rl), [rl], normal((rl,), dt, 1, 0.1, seed=2) if hw else None,
+                                                      normal((rl,), dt, 0, 0.1, seed=3) if hb else None, 1e-5), {}), tag=f"short_{rl}_{t}")
+    add(aten.native_layer_norm.default, lambda d: (_to(d, normal((300, 12, 64), f16, 0, 2, seed=1), [64], normal((64,), f32, 1, 0.1, seed=2), normal((64,), f32, 0, 0.1, seed=3), 1e-6), {}), tag="short_64_f32_params")
     # long rows: 8- and 16-wave register tiles, then the two-pass block kernel
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((5, 12288), bf16, 1, 2, seed=1), [12288], normal((12288,), bf16, 1, 0.1, seed=2), normal((12288,), bf16, 0, 0.1, seed=3), 1e-5), {}), tag="row12288_bf16")
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((3, 40000), f32, -2, 3, seed=1), [40000], normal((40000,), f32, 1, 0.1, seed=2), None, 1e-5), {}), tag="row40000_f32")
