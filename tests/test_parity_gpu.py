@@ -557,6 +557,47 @@ def test_tensors_beyond_2_to_31_elements(backend):
     assert torch.equal(out.cpu(), want) and torch.equal(emb.cpu().view(5, 16384), want)
 
 
+def test_row_kernels_beyond_2_to_31_elements(backend):
+    """Row-wise kernels and the GEMM on one 4 GiB f16 buffer viewed as rows: the first and the last rows
+    (element offsets past 2^31) are compared with the CPU on the same slices."""
+    announce("row kernels beyond 2^31 elements")
+    n = (1 << 31) + 2048
+    a = torch.empty(n, dtype=torch.float16, device="cuda")
+    a.normal_(generator=torch.Generator(device="cuda").manual_seed(5))
+    a[n - 7] = 100.0
+    assert int(backend[aten.argmax.default](a).item()) == n - 7
+
+    def ends(t, k):
+        return torch.cat([t[:k], t[-k:]]).cpu()
+
+    def close(got, want):
+        return torch.allclose(got.float(), want.float(), atol=1e-2, rtol=1e-2)
+
+    a8 = a.view(-1, 8)
+    got = backend[aten.amax.default](a8, [1])
+    assert torch.equal(ends(got, 4096), ends(a8, 4096).amax(1))
+    got = backend[aten._softmax.default](a8, -1, False)
+    assert close(ends(got, 4096), torch.softmax(ends(a8, 4096).float(), -1))
+    del got
+    a1k = a.view(-1, 1024)
+    y, mean, rstd = backend[aten.native_layer_norm.default](a1k, [1024], None, None, 1e-5)
+    wy, wm, wr = torch.native_layer_norm(ends(a1k, 512).float(), [1024], None, None, 1e-5)
+    assert close(ends(y, 512), wy) and close(ends(mean, 512), wm) and close(ends(rstd, 512), wr)
+    del y
+    w = torch.randn(1024, 64, generator=torch.Generator().manual_seed(6)).to(torch.float16)
+    got = backend[aten.mm.default](a1k, w.cuda())
+    want = ends(a1k, 512).float() @ w.float()
+    assert torch.allclose(ends(got, 512).float(), want, atol=0.25, rtol=1e-2)  # |sum of 1024 products| ~ 32, f16 output
+    del got
+    a512 = a.view(-1, 512)
+    idx = torch.randint(0, a512.shape[0], (3000, 512), generator=torch.Generator().manual_seed(7))
+    idx[-1] = a512.shape[0] - 1
+    got = backend[aten.gather.default](a512, 0, idx.cuda())
+    sample = torch.tensor([0, 1500, 2999])
+    want = torch.gather(a.cpu().view(-1, 512), 0, idx[sample])
+    assert torch.equal(got[sample.cuda()].cpu(), want)
+
+
 @pytest.mark.parametrize("n", [2049, 197, 50257, 8193])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_misaligned_rows_see_exactly_their_own_elements(backend, n, dtype):
