@@ -1658,7 +1658,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
 }
 
 // ---------------------------------------------------------------- generic fallback
-constexpr int GT = 64, GK = 16;
+// Any strides; fp64 accumulates in fp64, the other dtypes in fp32:
+// 64x64 tile per block, 32-k steps, 4x4 outputs per thread.  The loads of step t + 1 are issued
+// into registers before the FMAs of step t, so a step costs its arithmetic and not a round trip
+// to memory; the element-to-thread mapping of each operand follows its contiguous dim.
+constexpr int GT = 64, GK = 32;
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__ A, int64_t a_rs, int64_t a_cs,
                                                           const T* __restrict__ B, int64_t b_rs, int64_t b_cs,
@@ -1666,20 +1670,36 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
                                                           T* __restrict__ D, int64_t M, int64_t N, int64_t K,
                                                           float alpha, float beta) {
   using Acc = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+  constexpr int PER = GT * GK / 256;  // elements of each operand a thread moves per step
   __shared__ Acc As[GK][GT + 1], Bs[GK][GT + 1];
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
   const int64_t bm = (int64_t)blockIdx.y * GT, bn = (int64_t)blockIdx.x * GT;
-  Acc acc[4][4] = {};
-  for (int64_t k0 = 0; k0 < K; k0 += GK) {
-    for (int e = threadIdx.x; e < GT * GK; e += 256) {
-      const int r = e / GK, kk = e % GK;
+  const bool a_k_fast = a_cs == 1 || a_rs != 1;  // consecutive threads along k, unless A is M-contiguous
+  const bool b_n_fast = b_cs == 1 || b_rs != 1;  // consecutive threads along n, unless B is K-contiguous
+  Acc ra[PER], rb[PER];
+  auto fetch = [&](int64_t k0) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = threadIdx.x + 256 * u;
+      const int r = a_k_fast ? e / GK : e % GT, kk = a_k_fast ? e % GK : e / GT;
       const int64_t m = bm + r, k = k0 + kk;
-      As[kk][r] = (m < M && k < K) ? static_cast<Acc>(A[m * a_rs + k * a_cs]) : Acc(0);
-      const int kk2 = e / GT, c = e % GT;
+      ra[u] = (m < M && k < K) ? static_cast<Acc>(A[m * a_rs + k * a_cs]) : Acc(0);
+      const int c = b_n_fast ? e % GT : e / GK, kk2 = b_n_fast ? e / GT : e % GK;
       const int64_t n = bn + c, k2 = k0 + kk2;
-      Bs[kk2][c] = (n < N && k2 < K) ? static_cast<Acc>(B[k2 * b_rs + n * b_cs]) : Acc(0);
+      rb[u] = (n < N && k2 < K) ? static_cast<Acc>(B[k2 * b_rs + n * b_cs]) : Acc(0);
+    }
+  };
+  Acc acc[4][4] = {};
+  fetch(0);
+  for (int64_t k0 = 0; k0 < K; k0 += GK) {
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int e = threadIdx.x + 256 * u;
+      As[a_k_fast ? e % GK : e / GT][a_k_fast ? e / GK : e % GT] = ra[u];
+      Bs[b_n_fast ? e / GT : e % GK][b_n_fast ? e % GT : e / GK] = rb[u];
     }
     __syncthreads();
+    if (k0 + GK < K) fetch(k0 + GK);
 #pragma unroll
     for (int kk = 0; kk < GK; ++kk) {
       Acc av[4], bv[4];
@@ -1769,9 +1789,11 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     const bool b_nt = b_rs == 1 && b_cs % 8 == 0 && aligned16(b);
     const bool b_nn = b_cs == 1 && b_rs % 8 == 0 && aligned16(b);
     const bool fits = M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
-    // Tiny problems are cheaper on the generic kernel than on mostly empty MFMA tiles; a single row
-    // against a large weight (decoding one token) is not tiny: it streams the whole weight.
-    const bool worth = K >= 32 && (M * N >= 128 * 128 || M * N * K >= (int64_t(1) << 22));
+    // Tiny outputs with a short K are cheaper on the generic kernel than on a mostly empty MFMA
+    // tile.  Anything with a K loop worth pipelining is not: [64, 512] x [512, 64] takes 72 us there
+    // and 8 us here, and a single row against a large weight (decoding one token) streams the
+    // whole weight.
+    const bool worth = K >= 32 && (M * N >= 32 * 32 || K >= 256 || M * N * K >= (int64_t(1) << 22));
     // Row-major B needs N % 8 == 0 (its rows must start on 16-byte boundaries); transposed B takes
     // any N — a 50257-wide vocabulary projection stores its misaligned output rows element-wise.
     const bool b_nn_ok = b_nn && N % 8 == 0;
@@ -1886,7 +1908,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     const bool b_nn = b_cs == 1 && b_rs % 4 == 0 && aligned16(b);
     const bool fits = M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
     const bool b_nn_ok = b_nn && N % 4 == 0;
-    if (a_ok && (b_nt || b_nn_ok) && K % FBK == 0 && K > 0 && fits && (M * N >= 64 * 64 || M * N * K >= (int64_t(1) << 22))) {
+    if (a_ok && (b_nt || b_nn_ok) && K % FBK == 0 && K > 0 && fits && (M * N >= 32 * 32 || K >= 256 || M * N * K >= (int64_t(1) << 22))) {
       GemmArgs g{};
       g.a = a; g.b = b; g.c = c; g.out = out;
       g.lda = a_rs;

@@ -473,6 +473,16 @@ def edge_cases() -> List[Case]:
     add(aten.addmm.default, lambda d: ([normal((1024,), f16, seed=3).to(d), normal((3, 2048), f16, seed=1).to(d), normal((1024, 2048), f16, 0, 0.05, seed=2).to(d).t()], {}), tag="three_rows_bias_f16")
     add(aten.mm.default, lambda d: ([normal((2048, 512), bf16, seed=1).to(d).t(), normal((2048, 768), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_transposed_k2048")
     add(aten.mm.default, lambda d: (_to(d, torch.eye(256, dtype=bf16), normal((256, 256), bf16, seed=2)), {}), exact=True, tag="identity")
+    # tiny outputs: long K goes to the MFMA kernels (split along K), the rest to the pipelined generic kernel in every layout
+    add(aten.mm.default, lambda d: (_to(d, normal((8, 1024), f16, seed=1), normal((1024, 8), f16, 0, 0.05, seed=2)), {}), tag="tiny_8x8_k1024_f16")
+    add(aten.mm.default, lambda d: ([normal((32, 512), bf16, seed=1).to(d), normal((32, 512), bf16, 0, 0.05, seed=2).to(d).t()], {}), tag="tiny_32x32_k512_nt_bf16")
+    add(aten.mm.default, lambda d: (_to(d, normal((64, 64), f16, seed=1), normal((64, 64), f16, 0, 0.1, seed=2)), {}), tag="tiny_64_cubed_f16")
+    add(aten.mm.default, lambda d: (_to(d, normal((16, 256), f32, seed=1), normal((256, 16), f32, 0, 0.1, seed=2)), {}), tag="tiny_16x16_k256_f32")
+    add(aten.mm.default, lambda d: (_to(d, normal((5, 300), f32, seed=1), normal((300, 7), f32, 0, 0.1, seed=2)), {}), tag="tiny_ragged_k300_f32")
+    add(aten.mm.default, lambda d: (_to(d, normal((1, 4096), f16, seed=1), normal((4096, 1), f16, 0, 0.02, seed=2)), {}), tag="dot_product_f16")
+    add(aten.mm.default, lambda d: ([normal((130, 70), f64, seed=1).to(d).t(), normal((50, 130), f64, 0, 0.1, seed=2).to(d).t()], {}), tag="f64_both_transposed")
+    add(aten.mm.default, lambda d: ([normal((90, 97), f64, seed=1).to(d), normal((75, 97), f64, 0, 0.1, seed=2).to(d).t()], {}), tag="f64_b_transposed_k97")
+    add(aten.addmm.default, lambda d: (_to(d, normal((24,), f16, seed=3), normal((24, 512), f16, seed=1), normal((512, 24), f16, 0, 0.05, seed=2)), {"beta": 0.5, "alpha": 2.0}), tag="tiny_24x24_k512_f16")
     add(aten.mm.default, lambda d: (_to(d, torch.empty(2, 0, dtype=f32), torch.empty(0, 3, dtype=f32)), {}), tag="k0")
     add(aten.mm.default, lambda d: (_to(d, torch.empty(0, 8, dtype=bf16), normal((8, 16), bf16, seed=1)), {}), tag="m0")
     add(aten.addmm.default, lambda d: (_to(d, normal((256, 512), bf16, seed=3), normal((256, 128), bf16, seed=1), normal((128, 512), bf16, 0, 0.1, seed=2)), {"beta": 0.5, "alpha": 2.0}), tag="full_c_alpha_beta")
