@@ -8,8 +8,9 @@ same kernels.
 """
 
 from ._common import check_index_errors
-from .elementwise import (add, add_, clamp, clamp_, clamp_max, clamp_min, clamp_tensor, maximum, minimum, mul, mul_,
-                          out_variant, relu, relu_, where)
+from .elementwise import (_inplace_from, add, add_, clamp, clamp_, clamp_max, clamp_max_, clamp_max_tensor, clamp_min,
+                          clamp_min_, clamp_min_tensor, clamp_tensor, maximum, minimum, mul, mul_, out_variant, relu,
+                          relu_, where)
 from .index import embedding, gather, index_select
 from .matmul import addmm, mm
 from .reduce import (amax, argmax, log_softmax, mean_default, mean_dim, native_layer_norm, softmax, sum_default,
@@ -43,12 +44,22 @@ VARIANT_SLOTS = {
     "mul___Tensor": mul_,
     "relu___default": relu_,
     "clamp___default": clamp_,
+    "add___Scalar": add_,
+    "mul___Scalar": mul_,
+    "clamp_min___default": clamp_min_,
+    "clamp_max___default": clamp_max_,
+    "clamp___Tensor": _inplace_from(clamp_tensor, "clamp_tensor_"),
+    "addmm___default": _inplace_from(addmm, "addmm_"),
     # sibling overloads on the same kernels
     "minimum__default": minimum,
     "clamp_min__default": clamp_min,
     "clamp_max__default": clamp_max,
     "clamp__Tensor": clamp_tensor,
     "_log_softmax__default": log_softmax,
+    "add__Scalar": add,   # a Python scalar takes the same promotion as a 0-d wrapped number
+    "mul__Scalar": mul,
+    "clamp_min__Tensor": clamp_min_tensor,
+    "clamp_max__Tensor": clamp_max_tensor,
     # out= overloads
     "add__out": out_variant(add),
     "mul__out": out_variant(mul),
@@ -65,6 +76,16 @@ VARIANT_SLOTS = {
     "addmm__out": out_variant(addmm),
     "index_select__out": out_variant(index_select),
     "gather__out": out_variant(gather),
+    "add__Scalar_out": out_variant(add),
+    "mul__Scalar_out": out_variant(mul),
+    "minimum__out": out_variant(minimum),
+    "clamp__Tensor_out": out_variant(clamp_tensor),
+    "clamp_min__out": out_variant(clamp_min),
+    "clamp_max__out": out_variant(clamp_max),
+    "_log_softmax__out": out_variant(log_softmax),
+    "sum__out": out_variant(sum_default),
+    "mean__dtype_out": out_variant(mean_default),
+    "embedding__out": out_variant(embedding),
 }
 
 SLOTS = {**CORE_SLOTS, **VARIANT_SLOTS}

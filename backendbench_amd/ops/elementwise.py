@@ -339,6 +339,44 @@ def where(condition, self, other):
     return out
 
 
+def _inplace_from(functional, name):
+    """`self = functional(self, ...)` for the in-place overloads with no kernel form of their own:
+    the result must be castable to self's dtype and have self's shape, as ATen requires."""
+
+    def impl(self, *args, **kwargs):
+        res = functional(self, *args, **kwargs)
+        if res.shape != self.shape:
+            raise RuntimeError(f"output with shape {list(self.shape)} doesn't match the broadcast shape {list(res.shape)}")
+        if not torch.can_cast(res.dtype, self.dtype):
+            raise RuntimeError(f"result type {str(res.dtype).replace('torch.', '').capitalize()} can't be cast to the "
+                               f"desired output type {str(self.dtype).replace('torch.', '').capitalize()}")
+        return copy_into_any(self, res if res.device == self.device else res.to(self.device))
+
+    impl.__name__ = name
+    impl.__doc__ = f"in-place variant of {functional.__name__}"
+    return impl
+
+
+def clamp_min_(self, min):
+    """aten.clamp_min_.default"""
+    return clamp_(self, min, None)
+
+
+def clamp_max_(self, max):
+    """aten.clamp_max_.default"""
+    return clamp_(self, None, max)
+
+
+def clamp_min_tensor(self, min):
+    """aten.clamp_min.Tensor: max(self, min) with NaN propagation and maximum's type promotion."""
+    return maximum(self, min)
+
+
+def clamp_max_tensor(self, max):
+    """aten.clamp_max.Tensor: min(self, max) with NaN propagation and minimum's type promotion."""
+    return minimum(self, max)
+
+
 def out_variant(functional):
     """`<op>.out(..., out=Tensor)` from the functional wrapper: compute, resize `out` if its
     shape differs (as ATen does), then store with a cast into `out`'s dtype and return `out`."""

@@ -200,6 +200,13 @@ def edge_cases() -> List[Case]:
     add(aten.add.Tensor, lambda d: (_to(d, normal((3, 1367), bf16, seed=1), normal((1367,), bf16, seed=2)), {"alpha": 0.5}), tag="ragged_tail_bf16")
     add(aten.where.self, lambda d: (_to(d, normal((5, 1, 77), f32, seed=1) > 0, normal((5, 19, 77), f16, seed=2), normal((1, 19, 1), f16, seed=3)), {}), exact=True, tag="three_way_77")
     add(aten.maximum.default, lambda d: ([normal((67, 65), f32, seed=1).to(d), normal((65, 67), f32, seed=2).to(d).t()], {}), tag="transposed_odd")
+    # Scalar overloads and the tensor-bound one-sided clamps
+    add(aten.add.Scalar, lambda d: ([normal((33, 65), bf16, seed=1).to(d), 1.5], {"alpha": 2}), tag="bf16_alpha")
+    add(aten.add.Scalar, lambda d: ([randint((6, 10), 50, 1, i32).to(d), 2.5], {}), tag="int_plus_float")
+    add(aten.mul.Scalar, lambda d: ([normal((128, 130), f16, seed=1).to(d), 0.125], {}), tag="f16")
+    add(aten.mul.Scalar, lambda d: ([randint((6, 10), 50, 1, i64).to(d), 3], {}), exact=True, tag="int")
+    add(aten.clamp_min.Tensor, lambda d: ([poison(normal((40, 24), f32, seed=1), 0.05, 3).to(d), normal((24,), f32, seed=2).to(d)], {}), tag="bcast_naninf")
+    add(aten.clamp_max.Tensor, lambda d: ([normal((40, 24), bf16, seed=1).to(d), normal((40, 1), bf16, seed=2).to(d)], {}), tag="bcast_col_bf16")
     # one operand the transpose of the other's layout: large matrices are re-laid first, small or batched ones read in place
     add(aten.add.Tensor, lambda d: ([normal((1100, 1030), f32, seed=1).to(d), normal((1030, 1100), f32, seed=2).to(d).t()], {}), tag="mixed_layout_large")
     add(aten.mul.Tensor, lambda d: ([normal((4, 6, 64, 197), f16, seed=1).to(d).transpose(-1, -2), normal((4, 6, 197, 64), f16, seed=2).to(d)], {}), tag="mixed_layout_heads")

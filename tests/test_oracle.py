@@ -65,13 +65,13 @@ def np_of(t):
 def numpy_result(case, args, kwargs):
     n = case.op.__name__
     a = [np_of(x) for x in args]
-    if n == "add.Tensor":
+    if n in ("add.Tensor", "add.Scalar"):
         return numpy_ref.add(a[0], a[1], kwargs.get("alpha", 1))
-    if n == "mul.Tensor":
+    if n in ("mul.Tensor", "mul.Scalar"):
         return numpy_ref.mul(a[0], a[1])
-    if n == "maximum.default":
+    if n in ("maximum.default", "clamp_min.Tensor"):
         return numpy_ref.maximum(*np.broadcast_arrays(a[0], a[1]))
-    if n == "minimum.default":
+    if n in ("minimum.default", "clamp_max.Tensor"):
         return numpy_ref.minimum(*np.broadcast_arrays(a[0], a[1]))
     if n == "clamp_min.default":
         return numpy_ref.clamp(a[0], a[1], None)

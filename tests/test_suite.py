@@ -55,7 +55,7 @@ def test_baseline_suite_covers_every_slot():
         op for op in slot_ops
         if not op._overloadname.endswith("out") and not op._schema.name.endswith("_")
     }
-    assert len(functional) == 24 and ops == functional
+    assert len(functional) == 28 and ops == functional
     assert {c.key.split(".")[0] for c in perf_cases()} == {"C1", "C2", "C3", "C4", "C5"}
     assert len(edge_cases()) >= 250
     only = BaselineTestSuite("cpu", scale=0.01, filter=["_softmax"])

@@ -119,6 +119,18 @@ def _binary(op, with_alpha=False):
     return make
 
 
+def _scalar_binary(with_alpha=False):
+    def make(d):
+        dt = d.dtype()
+        x = d.tensor(d.shape(), dt, special=True)
+        other = d.r.choice([2, -3, 0, 0.5, -1.25])
+        kw = {}
+        if with_alpha and d.r.random() < 0.5:
+            kw["alpha"] = d.r.choice([2, -3]) if not dt.is_floating_point and isinstance(other, int) else d.r.choice([2, -0.5, 1.5])
+        return [x, other], kw
+    return make
+
+
 def _unary(d):
     return [d.tensor(d.shape(), d.dtype(), special=True)], {}
 
@@ -264,6 +276,10 @@ def _gather(d):
 SWEEP = {
     aten.add.Tensor: (_binary(aten.add.Tensor, with_alpha=True), False),
     aten.mul.Tensor: (_binary(aten.mul.Tensor), False),
+    aten.add.Scalar: (_scalar_binary(with_alpha=True), False),
+    aten.mul.Scalar: (_scalar_binary(), False),
+    aten.clamp_min.Tensor: (_binary(aten.clamp_min.Tensor), False),   # zero ties as for maximum
+    aten.clamp_max.Tensor: (_binary(aten.clamp_max.Tensor), False),
     # Not bit-exact: on a tie of -0.0 and +0.0 ATen's own CPU kernels return the second operand in
     # their vectorised loop and the first in their scalar loop; the HIP kernels follow IEEE 754-2019
     # (-0 < +0), as the GPU build of ATen does.  Values, NaN and infinities are still compared.
