@@ -178,6 +178,44 @@ __global__ __launch_bounds__(256) void transpose_copy_kernel(const U* __restrict
   }
 }
 
+// The same for 2- and 4-byte elements when both sides allow 16-byte accesses (M, N and both row
+// pitches multiples of the vector length VL = 8 or 4, aligned bases): a thread moves VL elements
+// per global access instead of one.  Source vectors (VL consecutive m of row n) land in an
+// unpadded 64 x 64 tile whose 16-byte chunk index is XORed with n / VL; a destination vector (VL
+// consecutive n of row m) is gathered with VL single-element LDS reads that, over a wave, touch
+// distinct banks.
+template <typename U>
+__global__ __launch_bounds__(256) void transpose_copy_vec_kernel(const U* __restrict__ src, U* __restrict__ dst,
+                                                                int64_t M, int64_t N, int64_t src_n_stride,
+                                                                int64_t dst_m_stride, int64_t src_b_stride,
+                                                                int64_t dst_b_stride) {
+  constexpr int VL = 16 / sizeof(U), CH = 64 / VL, ROWS = 256 / CH;  // chunks per tile row, tile rows per pass
+  __shared__ __attribute__((aligned(16))) U tile[64 * 64];
+  const int64_t n0 = (int64_t)blockIdx.x * 64, m0 = (int64_t)blockIdx.y * 64;
+  const U* s = src + (int64_t)blockIdx.z * src_b_stride;
+  U* d = dst + (int64_t)blockIdx.z * dst_b_stride;
+  const int ch = threadIdx.x % CH, r = threadIdx.x / CH;
+#pragma unroll
+  for (int p = 0; p < 64 / ROWS; ++p) {
+    const int n = p * ROWS + r;
+    if (n0 + n < N && m0 + ch * VL < M) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(s + (n0 + n) * src_n_stride + m0 + ch * VL);
+      *reinterpret_cast<u32x4*>(tile + n * 64 + ((ch ^ (n / VL)) * VL)) = v;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int p = 0; p < 64 / ROWS; ++p) {
+    const int m = p * ROWS + r;
+    if (m0 + m < M && n0 + ch * VL < N) {
+      Vec<U> v;
+#pragma unroll
+      for (int j = 0; j < VL; ++j) v.v[j] = tile[(ch * VL + j) * 64 + (((m / VL) ^ ch) * VL) + (m % VL)];
+      store_vec(d + (m0 + m) * dst_m_stride + n0 + ch * VL, v);
+    }
+  }
+}
+
 // True (and the copy enqueued) when src -> dst is such a transposition.
 template <typename U>
 static bool try_transpose_copy(const mi355_tensor* src, const mi355_tensor* dst, hipStream_t st, int* rc) {
@@ -192,9 +230,19 @@ static bool try_transpose_copy(const mi355_tensor* src, const mi355_tensor* dst,
   const int64_t batch = d.ndim == 3 ? d.sizes[0] : 1;
   if (batch > 65535 || (M + 63) / 64 > 65535) return false;
   const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), (unsigned)batch);
+  const int64_t sb = d.ndim == 3 ? d.strides[0][0] : 0, db = d.ndim == 3 ? d.strides[1][0] : 0;
+  if constexpr (sizeof(U) == 2 || sizeof(U) == 4) {
+    constexpr int VL = 16 / sizeof(U);
+    if (M % VL == 0 && N % VL == 0 && d.strides[0][in] % VL == 0 && d.strides[1][im] % VL == 0 && sb % VL == 0 &&
+        db % VL == 0 && aligned16(src->data) && aligned16(dst->data)) {
+      hipLaunchKernelGGL((transpose_copy_vec_kernel<U>), grid, dim3(256), 0, st, (const U*)src->data, (U*)dst->data, M, N,
+                         d.strides[0][in], d.strides[1][im], sb, db);
+      *rc = check_launch("mi355_copy(transpose, vectors)");
+      return true;
+    }
+  }
   hipLaunchKernelGGL((transpose_copy_kernel<U>), grid, dim3(256), 0, st, (const U*)src->data, (U*)dst->data, M, N,
-                     d.strides[0][in], d.strides[1][im], d.ndim == 3 ? d.strides[0][0] : 0,
-                     d.ndim == 3 ? d.strides[1][0] : 0);
+                     d.strides[0][in], d.strides[1][im], sb, db);
   *rc = check_launch("mi355_copy(transpose)");
   return true;
 }

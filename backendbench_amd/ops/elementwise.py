@@ -31,23 +31,38 @@ def _out_like_inputs(shape, dtype, inputs):
     return new_dense(shape, dtype, inputs[0].device)
 
 
+def _is_permuted_dense(t):
+    """True when `t` is a permutation of a dense tensor (no gaps, no overlap)."""
+    expect = 1
+    for size, stride in sorted(zip(t.shape, t.stride()), key=lambda p: p[1]):
+        if size == 1:
+            continue
+        if stride != expect:
+            return False
+        expect *= size
+    return True
+
+
 def _align_layouts(shape, tensors):
     """Full-shape operands that disagree on layout run on the strided kernel, where the odd one is
-    read one scattered element per lane.  When some operand is row-major and another is its
-    (batched) transpose, the transpose is made dense first with the tiled transposing copy: two
-    coalesced passes instead of one scattered pass.  Small problems keep the single pass: when the
-    whole operand is a couple of MB the second launch costs more than the scatter, and matrices of
-    up to 128 KB each (attention heads) stay in cache while their lines are picked apart."""
+    read one scattered element per lane.  When some operand is row-major and another is a permuted
+    dense tensor whose last dim is not its contiguous one (a batched transpose, a channels-last
+    view), the permuted one is made row-major first with the tiled transposing copy: two coalesced
+    passes instead of one scattered pass.  Small problems keep the single pass: when the whole
+    operand is a couple of MB the second launch costs more than the scatter, and transposed
+    matrices of up to 128 KB each (attention heads) stay in cache while their lines are picked apart."""
     full = [t for t in tensors if t.shape == shape]
-    if len(full) < 2 or len(shape) < 2 or not any(t.is_contiguous() for t in full):
+    if len(full) < 2 or len(shape) < 2 or shape[-1] == 1 or not any(t.is_contiguous() for t in full):
         return tensors
     esize = max(t.element_size() for t in full)
-    if shape[-1] * shape[-2] * esize <= (128 << 10) or shape.numel() * esize <= (2 << 20):
+    if shape.numel() * esize <= (2 << 20):
         return tensors
+    small_matrices = shape[-1] * shape[-2] * esize <= (128 << 10)
     out = []
     for t in tensors:
-        if t.shape == shape and not t.is_contiguous() and t.transpose(-1, -2).is_contiguous():
-            t = dense(t)
+        if t.shape == shape and t.stride(-1) != 1 and not t.is_contiguous() and _is_permuted_dense(t):
+            if not (small_matrices and t.transpose(-1, -2).is_contiguous()):
+                t = dense(t)
         out.append(t)
     return out
 

@@ -209,6 +209,8 @@ def edge_cases() -> List[Case]:
     add(aten.clamp_max.Tensor, lambda d: ([normal((40, 24), bf16, seed=1).to(d), normal((40, 1), bf16, seed=2).to(d)], {}), tag="bcast_col_bf16")
     # one operand the transpose of the other's layout: large matrices are re-laid first, small or batched ones read in place
     add(aten.add.Tensor, lambda d: ([normal((1100, 1030), f32, seed=1).to(d), normal((1030, 1100), f32, seed=2).to(d).t()], {}), tag="mixed_layout_large")
+    add(aten.add.Tensor, lambda d: ([normal((8, 48, 48, 96), f16, seed=1).to(d).permute(0, 3, 1, 2), normal((8, 96, 48, 48), f16, seed=2).to(d)], {}), tag="channels_last_view_plus_dense_large")
+    add(aten.maximum.default, lambda d: ([normal((6, 300, 520), f32, seed=1).to(d), normal((520, 6, 300), f32, seed=2).to(d).permute(1, 2, 0)], {}), tag="rotated_dims_large")
     add(aten.mul.Tensor, lambda d: ([normal((4, 6, 64, 197), f16, seed=1).to(d).transpose(-1, -2), normal((4, 6, 197, 64), f16, seed=2).to(d)], {}), tag="mixed_layout_heads")
     add(aten.where.self, lambda d: ([cond((900, 1200), 1).to(d), normal((1200, 900), f16, seed=2).to(d).t(), normal((900, 1200), f16, seed=3).to(d)], {}), exact=True, tag="mixed_layout_large")
     add(aten.add.Tensor, lambda d: (_to(d, normal((7, 599), f16, seed=1), normal((7, 599), f32, seed=2)), {}), tag="promote_odd")

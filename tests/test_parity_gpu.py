@@ -712,7 +712,8 @@ def test_transposing_copy_matches_contiguous(backend):
     announce("transposing copy")
     g = torch.Generator().manual_seed(5)
     for dtype in (torch.float16, torch.float32, torch.int8, torch.int64, torch.bool):
-        for shape in ((64, 64), (100, 37), (1000, 513), (17, 4096), (3, 130, 70), (2, 5, 65, 129)):
+        for shape in ((64, 64), (100, 37), (1000, 513), (17, 4096), (3, 130, 70), (2, 5, 65, 129),
+                      (200, 136), (3, 264, 72), (1024, 520), (2, 3, 8, 4096)):   # 2-byte elements: the 16-byte form
             base = torch.randint(-100, 100, shape, generator=g).to(dtype).cuda()
             view = base.transpose(-1, -2)
             assert not view.is_contiguous()
@@ -722,6 +723,9 @@ def test_transposing_copy_matches_contiguous(backend):
         assert torch.equal(dense(view), view.contiguous()), dtype
         dst = torch.zeros(193, 400, dtype=dtype, device="cuda")[:, :300]   # destination rows longer too
         assert torch.equal(copy_into(dst, view), view)
+        view = wide[:, 8:200].t()                       # the same with 16-byte aligned pieces on both sides
+        dst = torch.zeros(192, 400, dtype=dtype, device="cuda")[:, 40:340]
+        assert torch.equal(copy_into(dst, view), view) and torch.equal(dense(view), view.contiguous()), dtype
     # a permutation that is not a (batched) 2-D transposition keeps using the strided kernel
     x = torch.randn(6, 7, 40, 50, generator=g).cuda().permute(3, 0, 2, 1)
     assert torch.equal(dense(x), x.contiguous())
