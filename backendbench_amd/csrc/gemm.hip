@@ -1658,18 +1658,21 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
 }
 
 // ---------------------------------------------------------------- generic fallback
-// Any strides; fp64 accumulates in fp64, the other dtypes in fp32:
-// 64x64 tile per block, 32-k steps, 4x4 outputs per thread.  The loads of step t + 1 are issued
-// into registers before the FMAs of step t, so a step costs its arithmetic and not a round trip
-// to memory; the element-to-thread mapping of each operand follows its contiguous dim.
-constexpr int GT = 64, GK = 32;
-template <typename T>
+// Any strides; fp64 accumulates in fp64, the other dtypes in fp32.  A block of 256 threads owns
+// a (16 TT) x (16 TT) tile, TT x TT outputs per thread (rows ty TT + i, columns tx + 16 j: lanes
+// along n, so LDS reads of B and the stores are conflict-free and coalesced), GK-k steps.  TT = 4:
+// 64x64 tiles, 32-k steps; TT = 8: 128x128 tiles, 16-k steps, half the LDS reads per FMA (large
+// fp64 products).  The loads of step t + 1 are issued into registers before the FMAs of step t,
+// so a step costs its arithmetic and not a round trip to memory; the element-to-thread mapping
+// of each operand's loads follows its contiguous dim.
+template <typename T, int TT>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__ A, int64_t a_rs, int64_t a_cs,
                                                           const T* __restrict__ B, int64_t b_rs, int64_t b_cs,
                                                           const T* __restrict__ C, int64_t c_rs, int64_t c_cs,
                                                           T* __restrict__ D, int64_t M, int64_t N, int64_t K,
                                                           float alpha, float beta) {
   using Acc = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
+  constexpr int GT = 16 * TT, GK = 128 / TT;
   constexpr int PER = GT * GK / 256;  // elements of each operand a thread moves per step
   __shared__ Acc As[GK][GT + 1], Bs[GK][GT + 1];
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
@@ -1689,7 +1692,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
       rb[u] = (n < N && k2 < K) ? static_cast<Acc>(B[k2 * b_rs + n * b_cs]) : Acc(0);
     }
   };
-  Acc acc[4][4] = {};
+  Acc acc[TT][TT] = {};
   fetch(0);
   for (int64_t k0 = 0; k0 < K; k0 += GK) {
 #pragma unroll
@@ -1702,24 +1705,26 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
     if (k0 + GK < K) fetch(k0 + GK);
 #pragma unroll
     for (int kk = 0; kk < GK; ++kk) {
-      Acc av[4], bv[4];
+      Acc av[TT], bv[TT];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+      for (int i = 0; i < TT; ++i) av[i] = As[kk][ty * TT + i];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) bv[j] = Bs[kk][tx * 4 + j];
+      for (int j = 0; j < TT; ++j) bv[j] = Bs[kk][tx + 16 * j];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < TT; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * bv[j];
+        for (int j = 0; j < TT; ++j) acc[i][j] += av[i] * bv[j];
     }
     __syncthreads();
   }
   const bool use_c = C != nullptr && beta != 0.f;
-  for (int i = 0; i < 4; ++i) {
-    const int64_t m = bm + ty * 4 + i;
+#pragma unroll
+  for (int i = 0; i < TT; ++i) {
+    const int64_t m = bm + ty * TT + i;
     if (m >= M) continue;
-    for (int j = 0; j < 4; ++j) {
-      const int64_t n = bn + tx * 4 + j;
+#pragma unroll
+    for (int j = 0; j < TT; ++j) {
+      const int64_t n = bn + tx + 16 * j;
       if (n >= N) continue;
       Acc v = (Acc)alpha * acc[i][j];
       if (use_c) v += (Acc)beta * static_cast<Acc>(C[m * c_rs + n * c_cs]);
@@ -1950,11 +1955,19 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       return finish_splitk<float>(g, nsplit, st);
     }
   }
-  const int64_t gx = (N + GT - 1) / GT, gy = (M + GT - 1) / GT;
+  // 128x128 tiles once they still give every CU a block, else 64x64
+  const bool big = ((M + 127) / 128) * ((N + 127) / 128) >= kNumCU && K >= 64;
+  const int64_t gt = big ? 128 : 64;
+  const int64_t gx = (N + gt - 1) / gt, gy = (M + gt - 1) / gt;
   MI355_REQUIRE(gy < 65536 && gx < (int64_t(1) << 31), "mi355_gemm: generic path needs M < 4M rows");
-  hipLaunchKernelGGL((gemm_generic_kernel<T>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                     static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
-                     static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (float)alpha, (float)beta);
+  if (big)
+    hipLaunchKernelGGL((gemm_generic_kernel<T, 8>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+                       static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
+                       static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (float)alpha, (float)beta);
+  else
+    hipLaunchKernelGGL((gemm_generic_kernel<T, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+                       static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
+                       static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (float)alpha, (float)beta);
   return check_launch("mi355_gemm(generic)");
 }
 

@@ -489,6 +489,8 @@ def edge_cases() -> List[Case]:
     add(aten.mm.default, lambda d: (_to(d, normal((16, 256), f32, seed=1), normal((256, 16), f32, 0, 0.1, seed=2)), {}), tag="tiny_16x16_k256_f32")
     add(aten.mm.default, lambda d: (_to(d, normal((5, 300), f32, seed=1), normal((300, 7), f32, 0, 0.1, seed=2)), {}), tag="tiny_ragged_k300_f32")
     add(aten.mm.default, lambda d: (_to(d, normal((1, 4096), f16, seed=1), normal((4096, 1), f16, 0, 0.02, seed=2)), {}), tag="dot_product_f16")
+    add(aten.mm.default, lambda d: (_to(d, normal((2050, 70), f64, seed=1), normal((70, 2041), f64, 0, 0.1, seed=2)), {}), tag="f64_128x128_tiles")
+    add(aten.addmm.default, lambda d: ([normal((2041,), f64, seed=3).to(d), normal((70, 2050), f64, seed=1).to(d).t(), normal((2041, 70), f64, 0, 0.1, seed=2).to(d).t()], {"beta": 0.5}), tag="f64_128x128_tiles_both_transposed")
     add(aten.mm.default, lambda d: ([normal((130, 70), f64, seed=1).to(d).t(), normal((50, 130), f64, 0, 0.1, seed=2).to(d).t()], {}), tag="f64_both_transposed")
     add(aten.mm.default, lambda d: ([normal((90, 97), f64, seed=1).to(d), normal((75, 97), f64, 0, 0.1, seed=2).to(d).t()], {}), tag="f64_b_transposed_k97")
     add(aten.addmm.default, lambda d: (_to(d, normal((24,), f16, seed=3), normal((24, 512), f16, seed=1), normal((512, 24), f16, 0, 0.05, seed=2)), {"beta": 0.5, "alpha": 2.0}), tag="tiny_24x24_k512_f16")
