@@ -77,24 +77,26 @@ struct GemmArgs {
   int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
   int32_t out_vec;  // out rows start on 16-byte boundaries (N a multiple of the vector width): vector stores
   // Split-K (128x128 kernels only): blockIdx.y = split, which covers k in [split * ksplit,
-  // min(K, (split + 1) * ksplit)) and writes its raw fp32 tile to ws[split][M][N].
+  // min(K, (split + 1) * ksplit)) and writes its raw fp32 tile to ws[split][M][ws_ld], ws_ld = N
+  // rounded up to a multiple of 4 (rows of every plane start on 16-byte boundaries for any N).
   float* ws;
   int32_t ksplit;
+  int32_t ws_ld;
 };
 
 // fp32 partial tile of one split: register r of acc[i][j] in lane l is
 // C[m0 + 32 i + l%32][n0 + 32 j + 8 (r/4) + 4 (l/32) + r%4]; N % 4 == 0 on the MFMA paths.
-template <int MI>
-__device__ __forceinline__ void store_partial_tile(const GemmArgs& g, const f32x16 (&acc)[MI][2], int lane, int m0,
+template <int MI, int NJ = 2>
+__device__ __forceinline__ void store_partial_tile(const GemmArgs& g, const f32x16 (&acc)[MI][NJ], int lane, int m0,
                                                    int n0) {
   const int fr = lane & 31, fg = lane >> 5;
-  float* W = g.ws + (int64_t)blockIdx.y * g.M * g.N;
+  float* W = g.ws + (int64_t)blockIdx.y * g.M * g.ws_ld;
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
     const int m = m0 + i * 32 + fr;
     if (m >= g.M) continue;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + j * 32 + q * 8 + fg * 4;
@@ -102,32 +104,45 @@ __device__ __forceinline__ void store_partial_tile(const GemmArgs& g, const f32x
         f32x4 r;
 #pragma unroll
         for (int e = 0; e < 4; ++e) r[e] = acc[i][j][q * 4 + e];
-        *reinterpret_cast<f32x4*>(W + (int64_t)m * g.N + n) = r;
+        *reinterpret_cast<f32x4*>(W + (int64_t)m * g.ws_ld + n) = r;  // columns past N land in the row's padding
       }
   }
 }
 
-// out = alpha * sum over splits of ws + beta * c, four consecutive n per thread.
+// out = alpha * sum over splits of ws + beta * c, four consecutive n per thread.  A group of
+// four columns that starts inside a row may end in its padding (N % 4 != 0): those output rows
+// are misaligned and are stored element by element.
 template <typename T>
-__global__ __launch_bounds__(256) void gemm_splitk_finish_kernel(GemmArgs g, int nsplit) {
-  const int64_t quads = (int64_t)g.M * g.N / 4;
+__device__ __forceinline__ void finish_store(const GemmArgs& g, const f32x4& sum, int64_t m, int64_t n) {
   const T* C = static_cast<const T*>(g.c);
   const bool use_c = C != nullptr && g.beta != 0.f;
-  T* D = static_cast<T*>(g.out);
-  const int64_t plane = (int64_t)g.M * g.N;
+  T* D = static_cast<T*>(g.out) + m * g.N + n;
+  VecN4<T> r;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float v = g.alpha * sum[e];
+    if (use_c && n + e < g.N) v += g.beta * static_cast<float>(C[m * g.c_rs + (n + e) * g.c_cs]);
+    r.v[e] = static_cast<T>(v);
+  }
+  if (g.ws_ld == g.N) {
+    *reinterpret_cast<VecN4<T>*>(D) = r;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (n + e < g.N) D[e] = r.v[e];
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_splitk_finish_kernel(GemmArgs g, int nsplit) {
+  const int64_t plane = (int64_t)g.M * g.ws_ld, quads = plane / 4;
+  const int qpr = g.ws_ld / 4;  // quads per row
   for (int64_t qd = (int64_t)blockIdx.x * 256 + threadIdx.x; qd < quads; qd += (int64_t)gridDim.x * 256) {
     const int64_t e0 = qd * 4;
     f32x4 sum = *reinterpret_cast<const f32x4*>(g.ws + e0);
     for (int sp = 1; sp < nsplit; ++sp) sum += *reinterpret_cast<const f32x4*>(g.ws + sp * plane + e0);
-    const int64_t m = e0 / g.N, n = e0 - m * g.N;
-    VecN4<T> r;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float v = g.alpha * sum[e];
-      if (use_c) v += g.beta * static_cast<float>(C[m * g.c_rs + (n + e) * g.c_cs]);
-      r.v[e] = static_cast<T>(v);
-    }
-    *reinterpret_cast<VecN4<T>*>(D + e0) = r;
+    const int64_t m = qd / qpr;
+    finish_store<T>(g, sum, m, (qd - m * qpr) * 4);
   }
 }
 
@@ -136,11 +151,8 @@ __global__ __launch_bounds__(256) void gemm_splitk_finish_kernel(GemmArgs g, int
 // two DPP steps combine them.
 template <typename T>
 __global__ __launch_bounds__(256) void gemm_splitk_finish4_kernel(GemmArgs g, int nsplit) {
-  const int64_t quads = (int64_t)g.M * g.N / 4;
-  const T* C = static_cast<const T*>(g.c);
-  const bool use_c = C != nullptr && g.beta != 0.f;
-  T* D = static_cast<T*>(g.out);
-  const int64_t plane = (int64_t)g.M * g.N;
+  const int64_t plane = (int64_t)g.M * g.ws_ld, quads = plane / 4;
+  const int qpr = g.ws_ld / 4;
   const int part = threadIdx.x & 3;
   const int64_t stride = (int64_t)gridDim.x * 64;
   const int64_t rounds = (quads + stride - 1) / stride;  // every lane of a wave stays in the loop: the combine below is wave-wide
@@ -159,15 +171,8 @@ __global__ __launch_bounds__(256) void gemm_splitk_finish4_kernel(GemmArgs g, in
       sum[e] = v;
     }
     if (!live || part != 0) continue;
-    const int64_t m = e0 / g.N, n = e0 - m * g.N;
-    VecN4<T> out;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float v = g.alpha * sum[e];
-      if (use_c) v += g.beta * static_cast<float>(C[m * g.c_rs + (n + e) * g.c_cs]);
-      out.v[e] = static_cast<T>(v);
-    }
-    *reinterpret_cast<VecN4<T>*>(D + e0) = out;
+    const int64_t m = qd / qpr;
+    finish_store<T>(g, sum, m, (qd - m * qpr) * 4);
   }
 }
 
@@ -1488,39 +1493,44 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
 // ---------------------------------------------------------------- MFMA kernel, fp32
 // v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate; 157 TFLOP/s dense peak).  Same shape as the
 // 128x128 half-precision kernel in bytes: four waves (2x2) of 64x64, 16-k steps (64-byte rows),
-// a ring of four 16 KB stages (A 128x16 + B 16x128 fp32) filled by global_load_lds_dwordx4
-// three steps ahead.  A lane reads one 16-byte chunk (4 consecutive k) per operand block and
+// a ring of S 16 KB stages (A 128x16 + B 16x128 fp32) filled by global_load_lds_dwordx4
+// S - 1 steps ahead (S = 4: 64 KB, two workgroups per CU; S = 8: 128 KB for problems that leave
+// a CU one workgroup anyway, where the deeper ring is what hides the fill latency).  A lane reads one 16-byte chunk (4 consecutive k) per operand block and
 // feeds MFMA e (e = 0..3) with its element e: the two k slots of that MFMA are then k = e of
 // the lower chunk (lanes 0-31) and of the upper chunk (lanes 32-63) — any pairing works as long
 // as both operands use the same one.  Row-major B has no transposing LDS read at 32 bits: a
 // lane gathers its four k with four ds_read_b32, rows of the panel offset by 128 bytes every
 // four k so that the two lane halves use different banks.  K % 16 == 0, N % 4 == 0.
 constexpr int FBK = 16;
-// [k][n] fp32 panel, 512 B per k row; 16-byte unit u of row k sits at u ^ (8 * ((k / 4) % 2)).
-__device__ __forceinline__ int swz_nf(int k, int n) {
-  return k * (SBN * 4) + (((n >> 2) ^ (((k >> 2) & 1) << 3)) << 4) + ((n & 3) << 2);
+// [k][n] fp32 panel, 4 TILE bytes per k row; 16-byte unit u of row k sits at u ^ (8 * ((k / 4) % 2)).
+template <int TILE> __device__ __forceinline__ int swz_nf(int k, int n) {
+  return k * (TILE * 4) + (((n >> 2) ^ (((k >> 2) & 1) << 3)) << 4) + ((n & 3) << 2);
 }
 
-template <bool B_NN, bool SPLIT>
+template <bool B_NN, bool SPLIT, int S, int TILE>
 __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
-  constexpr int S = kStages3;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  static_assert(TILE == 128 || TILE == 64, "128x128 or 64x64 tiles");
+  constexpr int MI = TILE / 64;                 // 32x32 blocks per wave and dim; also 1 KB regions per wave and panel
+  constexpr int kPanel = TILE * FBK * 4;        // bytes per operand per stage
+  constexpr int kStage = 2 * kPanel;
+  constexpr int UPR = TILE / 4;                 // 16-byte units per k row of a row-major B panel
   const int wm = wave >> 1, wn = wave & 1;
   int tm, tn;
   tile_coords(g, tm, tn);
-  const int bm = tm * SBM, bn = tn * SBN;
+  const int bm = tm * TILE, bn = tn * TILE;
   const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
   const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
   const float* A = static_cast<const float*>(g.a) + kbeg;
   const float* B = static_cast<const float*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
-  const float* a_src[2];
-  const float* b_src[2];
+  const float* a_src[MI];
+  const float* b_src[MI];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < MI; ++i) {
     const int q = wave + 4 * i;
     {  // K-contiguous panel: region q = rows 16q .. 16q+15, 4 chunks of 4 floats per row
       const int r = 16 * q + (lane >> 2), slot = lane & 3;
@@ -1535,8 +1545,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
       int gn = bn + r;
       gn = gn < g.N ? gn : g.N - 1;
       b_src[i] = B + (int64_t)gn * g.ldb + c * 4;
-    } else {  // N-contiguous panel: region q = k rows 2q, 2q+1, 32 units of 4 floats per row
-      const int k = 2 * q + (lane >> 5), pos = lane & 31;
+    } else {  // N-contiguous panel: region q = 64 / UPR k rows of UPR units of 4 floats
+      const int k = (64 / UPR) * q + lane / UPR, pos = lane % UPR;
       const int u = pos ^ (((k >> 2) & 1) << 3);
       int gn = bn + u * 4;
       gn = gn < g.N ? gn : 0;
@@ -1544,61 +1554,63 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
     }
   }
   auto request_tile = [&](int t) {
-    const uint32_t stage = lds_base + (uint32_t)(t % S) * kSStage;
+    const uint32_t stage = lds_base + (uint32_t)(t % S) * kStage;
     const int64_t k0 = (int64_t)t * FBK;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < MI; ++i) {
       const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
       lds_dma16(stage + region, a_src[i] + k0);
-      if constexpr (!B_NN) lds_dma16(stage + kSPanel + region, b_src[i] + k0);
-      else lds_dma16(stage + kSPanel + region, b_src[i] + k0 * g.ldb);
+      if constexpr (!B_NN) lds_dma16(stage + kPanel + region, b_src[i] + k0);
+      else lds_dma16(stage + kPanel + region, b_src[i] + k0 * g.ldb);
     }
   };
 
   const int fr = lane & 31, fg = lane >> 5;
   // Operand blocks of 8-k sub-step ks (0, 1) of step t: 4 floats per lane and block.
-  auto read_frags = [&](int t, int ks, f32x4 (&fa)[2], f32x4 (&fb)[2]) {
-    const unsigned char* pa = lds + (t % S) * kSStage;
-    const unsigned char* pb = pa + kSPanel;
+  auto read_frags = [&](int t, int ks, f32x4 (&fa)[MI], f32x4 (&fb)[MI]) {
+    const unsigned char* pa = lds + (t % S) * kStage;
+    const unsigned char* pb = pa + kPanel;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      fa[i] = *reinterpret_cast<const f32x4*>(pa + swz_k32(wm * 64 + i * 32 + fr, ks * 2 + fg));
+    for (int i = 0; i < MI; ++i)
+      fa[i] = *reinterpret_cast<const f32x4*>(pa + swz_k32(wm * 32 * MI + i * 32 + fr, ks * 2 + fg));
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < MI; ++j) {
       if constexpr (!B_NN) {
-        fb[j] = *reinterpret_cast<const f32x4*>(pb + swz_k32(wn * 64 + j * 32 + fr, ks * 2 + fg));
+        fb[j] = *reinterpret_cast<const f32x4*>(pb + swz_k32(wn * 32 * MI + j * 32 + fr, ks * 2 + fg));
       } else {
-        const int n = wn * 64 + j * 32 + fr;
+        const int n = wn * 32 * MI + j * 32 + fr;
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          fb[j][e] = *reinterpret_cast<const float*>(pb + swz_nf(ks * 8 + fg * 4 + e, n));
+          fb[j][e] = *reinterpret_cast<const float*>(pb + swz_nf<TILE>(ks * 8 + fg * 4 + e, n));
       }
     }
   };
 
-  f32x16 acc[2][2];
+  f32x16 acc[MI][MI];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < MI; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  auto mma = [&](f32x4 (&fa)[2], f32x4 (&fb)[2]) {
+  auto mma = [&](f32x4 (&fa)[MI], f32x4 (&fb)[MI]) {
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < MI; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[j][e], fa[i][e], acc[i][j], 0, 0, 0);
   };
 
   const int nk = (kend - kbeg) / FBK;
   for (int t = 0; t < S - 1 && t < nk; ++t) request_tile(t);
-  if (nk >= S - 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  // Step t reads tile t and the first half of tile t + 1: all but the newest S - 3 tiles must
+  // have landed (2 MI requests per thread and tile).
+  if (nk >= S - 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * MI * (S - 3)) : "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  f32x4 fa0[2], fb0[2], fa1[2], fb1[2];
+  f32x4 fa0[MI], fb0[MI], fa1[MI], fb1[MI];
   read_frags(0, 0, fa0, fb0);
   int it = 0;
   for (; it + S - 1 < nk; ++it) {
@@ -1607,7 +1619,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
     mma(fa0, fb0);
     read_frags(it + 1, 0, fa0, fb0);
     mma(fa1, fb1);
-    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * MI * (S - 3)) : "memory");
     __syncthreads();
   }
   for (; it < nk; ++it) {
@@ -1620,7 +1632,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
   }
 
   if constexpr (SPLIT) {
-    store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
+    store_partial_tile<MI, MI>(g, acc, lane, bm + wm * 32 * MI, bn + wn * 32 * MI);
     return;
   }
   // Register r of acc[i][j] in lane l is C[m0 + 32 i + l%32][n0 + 32 j + 8 (r/4) + 4 (l/32) + r%4]:
@@ -1629,14 +1641,14 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
   const bool use_c = C != nullptr && g.beta != 0.f;
   float* D = static_cast<float*>(g.out);
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int m = bm + wm * 64 + i * 32 + fr;
+  for (int i = 0; i < MI; ++i) {
+    const int m = bm + wm * 32 * MI + i * 32 + fr;
     if (m >= g.M) continue;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < MI; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int n = bn + wn * 64 + j * 32 + q * 8 + fg * 4;
+        const int n = bn + wn * 32 * MI + j * 32 + q * 8 + fg * 4;
         if (n >= g.N) continue;
         f32x4 r;
 #pragma unroll
@@ -1741,12 +1753,17 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 struct SplitPlan {
   int nsplit, ksplit;
 };
+// fp32 products that leave most CUs without a 128x128 tile run on 64x64 tiles.
+static int f32_tile(int64_t M, int64_t N) {
+  return ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN) < kNumCU * 3 / 4 ? 64 : 128;
+}
 static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   const int bk = elem_size == 4 ? FBK : BK3;
-  const int64_t tiles = ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN);
+  const int tile = elem_size == 4 ? f32_tile(M, N) : SBM;
+  const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
   SplitPlan p{1, (int)K};
   if (tiles >= kNumCU || K % bk != 0) return p;
-  const double ns_per_k = elem_size == 4 ? 70.0 : 12.8;
+  const double ns_per_k = elem_size == 4 ? (tile == 64 ? 20.0 : 70.0) : 12.8;
   const int64_t max_ns = K / (8 * bk) < 64 ? K / (8 * bk) : 64;
   double best = 0;
   int64_t best_ns = 1;
@@ -1773,7 +1790,7 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
 
 template <typename T>
 static int finish_splitk(const GemmArgs& g, int nsplit, hipStream_t st) {
-  const int64_t quads = (int64_t)g.M * g.N / 4;
+  const int64_t quads = (int64_t)g.M * g.ws_ld / 4;
   if (quads < (int64_t)kNumCU * 256 * 2 && nsplit >= 4) {  // under two blocks per CU: four lanes per group of columns
     const int grid = grid_for(quads, 64, kNumCU * 8);
     hipLaunchKernelGGL((gemm_splitk_finish4_kernel<T>), dim3(grid), dim3(256), 0, st, g, nsplit);
@@ -1858,12 +1875,14 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
         nblocks = (int64_t)g.tiles_m * g.tiles_n;
         const SplitPlan sp = plan_splitk(M, N, K, sizeof(T));
-        const bool split = sp.nsplit > 1 && N % 4 == 0 && workspace != nullptr &&
-                           workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+        const int64_t ws_ld = (N + 3) / 4 * 4;
+        const bool split = sp.nsplit > 1 && workspace != nullptr &&
+                           workspace_bytes >= (int64_t)sp.nsplit * M * ws_ld * 4 && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
         if (split) {
           nsplit = sp.nsplit;
           g.ws = static_cast<float*>(workspace);
           g.ksplit = sp.ksplit;
+          g.ws_ld = (int32_t)ws_ld;
         }
         // At most one workgroup per CU and whole 64-k pairs per split: the deep-ring kernel.
         const bool pairs = nblocks * nsplit <= kNumCU && K % 64 == 0 && (!split || sp.ksplit % 64 == 0);
@@ -1922,33 +1941,45 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       g.out_vec = N % 4 == 0 && aligned16(out);
       g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
       g.alpha = (float)alpha; g.beta = (float)beta;
-      g.tiles_m = (int32_t)((M + SBM - 1) / SBM);
-      g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
+      const int tile = f32_tile(M, N);
+      g.tiles_m = (int32_t)((M + tile - 1) / tile);
+      g.tiles_n = (int32_t)((N + tile - 1) / tile);
       const int64_t nblocks = (int64_t)g.tiles_m * g.tiles_n;
       MI355_REQUIRE(nblocks < (int64_t(1) << 31), "mi355_gemm: too many tiles");
       int nsplit = 1;
       const SplitPlan sp = plan_splitk(M, N, K, 4);
-      if (sp.nsplit > 1 && N % 4 == 0 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * N * 4 &&
+      const int64_t ws_ld = (N + 3) / 4 * 4;
+      if (sp.nsplit > 1 && workspace != nullptr && workspace_bytes >= (int64_t)sp.nsplit * M * ws_ld * 4 &&
           reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
         nsplit = sp.nsplit;
         g.ws = static_cast<float*>(workspace);
         g.ksplit = sp.ksplit;
+        g.ws_ld = (int32_t)ws_ld;
       }
+      // 64x64 tiles: eight 8 KB stages (64 KB, two workgroups per CU).  128x128 tiles: four 16 KB
+      // stages, or eight when a CU gets one workgroup anyway and the deeper ring hides the fills.
       const void* kern;
-      if (nsplit > 1) kern = b_nt ? (const void*)gemm_mfma_f32_kernel<false, true> : (const void*)gemm_mfma_f32_kernel<true, true>;
-      else kern = b_nt ? (const void*)gemm_mfma_f32_kernel<false, false> : (const void*)gemm_mfma_f32_kernel<true, false>;
-      static thread_local const void* attr_done[4] = {};
+      const bool deep = nblocks * nsplit <= kNumCU;
+      const int lds_bytes = tile == 64 ? 8 * 8192 : deep ? 8 * kSStage : kSmallLds;
+#define MI355_F32_KERNEL(S_, TILE_)                                                                              \
+  (nsplit > 1 ? (b_nt ? (const void*)gemm_mfma_f32_kernel<false, true, S_, TILE_> : (const void*)gemm_mfma_f32_kernel<true, true, S_, TILE_>) \
+              : (b_nt ? (const void*)gemm_mfma_f32_kernel<false, false, S_, TILE_> : (const void*)gemm_mfma_f32_kernel<true, false, S_, TILE_>))
+      if (tile == 64) kern = MI355_F32_KERNEL(8, 64);
+      else if (deep) kern = MI355_F32_KERNEL(8, 128);
+      else kern = MI355_F32_KERNEL(kStages3, 128);
+#undef MI355_F32_KERNEL
+      static thread_local const void* attr_done[12] = {};
       bool seen = false;
       for (const void* k : attr_done) seen = seen || k == kern;
       if (!seen) {
-        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kSmallLds);
+        hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess)
-          return set_error(MI355_ERR_LAUNCH, "mi355_gemm: cannot reserve %d bytes of LDS: %s", kSmallLds, hipGetErrorString(e));
+          return set_error(MI355_ERR_LAUNCH, "mi355_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
         for (const void*& k : attr_done)
           if (k == nullptr) { k = kern; break; }
       }
       void* params[] = {&g};
-      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks, (unsigned)nsplit), dim3(256), params, kSmallLds, st);
+      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks, (unsigned)nsplit), dim3(256), params, lds_bytes, st);
       if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma f32): launch failed: %s", hipGetErrorString(e));
       const int rc = check_launch("mi355_gemm(mfma f32)");
       if (rc || nsplit == 1) return rc;
@@ -1980,7 +2011,7 @@ extern "C" int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
   if (M <= 0 || N <= 0 || K <= 0 || (es != 2 && es != 4)) return 0;
   if (dtype != MI355_BF16 && dtype != MI355_F16 && dtype != MI355_F32) return 0;
   const SplitPlan p = plan_splitk(M, N, K, es);
-  return p.nsplit > 1 ? (int64_t)p.nsplit * M * N * 4 : 0;
+  return p.nsplit > 1 ? (int64_t)p.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
 }
 
 extern "C" int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs,

@@ -450,6 +450,12 @@ def edge_cases() -> List[Case]:
     for k in (16, 32, 48, 64, 80, 272):   # fp32 MFMA path: every prologue / steady-state / drain length
         add(aten.mm.default, lambda d, k=k: (_to(d, normal((132, k), f32, seed=1), normal((k, 140), f32, 0, 0.1, seed=2)), {}), tag=f"f32_ksteps_{k}")
     add(aten.mm.default, lambda d: ([normal((300, 96), f32, seed=1).to(d), normal((260, 96), f32, 0, 0.1, seed=2).to(d).t()], {}), tag="f32_b_transposed")
+    # more 128x128 tiles than CUs: the four-stage fp32 ring, two workgroups per CU (fewer tiles take the eight-stage ring)
+    # 196 tiles of 128x128: one workgroup per CU, the eight-stage ring on the large tiles
+    add(aten.mm.default, lambda d: (_to(d, normal((1700, 176), f32, seed=1), normal((176, 1752), f32, 0, 0.1, seed=2)), {}), tag="f32_196_tiles_k176")
+    add(aten.addmm.default, lambda d: ([normal((1700, 1), f32, seed=3).to(d), normal((1700, 80), f32, seed=1).to(d), normal((1750, 80), f32, 0, 0.1, seed=2).to(d).t()], {}), tag="f32_196_tiles_k80_nt_col_bias")
+    add(aten.mm.default, lambda d: (_to(d, normal((2100, 48), f32, seed=1), normal((48, 2064), f32, 0, 0.1, seed=2)), {}), tag="f32_many_tiles_k48")
+    add(aten.mm.default, lambda d: ([normal((2100, 208), f32, seed=1).to(d), normal((2064, 208), f32, 0, 0.1, seed=2).to(d).t()], {}), tag="f32_many_tiles_k208_nt")
     add(aten.addmm.default, lambda d: ([normal((260,), f32, seed=3).to(d), normal((300, 96), f32, seed=1).to(d), normal((260, 96), f32, 0, 0.1, seed=2).to(d).t()], {"beta": 0.5, "alpha": 2.0}), tag="f32_linear")
     add(aten.mm.default, lambda d: (_to(d, torch.eye(128, dtype=f32), normal((128, 128), f32, seed=2)), {}), exact=True, tag="f32_identity")
     add(aten.mm.default, lambda d: (_to(d, normal((70, 90), torch.float64, seed=1), normal((90, 50), torch.float64, 0, 0.1, seed=2)), {}), tag="f64")
@@ -468,6 +474,10 @@ def edge_cases() -> List[Case]:
     add(aten.addmm.default, lambda d: ([normal((1024,), bf16, seed=3).to(d), normal((24, 4096), bf16, seed=1).to(d), normal((1024, 4096), bf16, 0, 0.02, seed=2).to(d).t()], {"beta": 0.5, "alpha": 2.0}), tag="splitk_linear_bf16")
     add(aten.addmm.default, lambda d: ([normal((200,), f32, seed=3).to(d), normal((64, 1024), f32, seed=1).to(d), normal((200, 1024), f32, 0, 0.05, seed=2).to(d).t()], {}), tag="splitk_linear_f32")
     add(aten.mm.default, lambda d: (_to(d, normal((64, 1040), f32, seed=1), normal((1040, 256), f32, 0, 0.05, seed=2)), {}), tag="splitk_f32")
+    # split-K with an N that is no multiple of 4: partial planes keep padded rows, output rows are stored element-wise
+    add(aten.mm.default, lambda d: ([normal((24, 2048), bf16, seed=1).to(d), normal((1001, 2048), bf16, 0, 0.05, seed=2).to(d).t()], {}), tag="splitk_odd_n_bf16")
+    add(aten.mm.default, lambda d: (_to(d, normal((64, 1040), f32, seed=1), normal((1040, 250), f32, 0, 0.05, seed=2)), {}), tag="splitk_n250_f32")
+    add(aten.addmm.default, lambda d: ([normal((1001,), f16, seed=3).to(d), normal((40, 4096), f16, seed=1).to(d), normal((1001, 4096), f16, 0, 0.02, seed=2).to(d).t()], {"beta": 0.5, "alpha": 2.0}), tag="splitk_odd_n_bias_f16")
     add(aten.mm.default, lambda d: ([normal((320, 512), bf16, seed=1).to(d).t(), normal((320, 768), bf16, 0, 0.05, seed=2).to(d)], {}), tag="a_transposed")
     # layouts the MFMA kernels cannot address directly: K no multiple of the vector (operands copied into zero-padded
     # K-contiguous buffers), a row-major right operand with misaligned rows (re-laid K-contiguous)
