@@ -19,14 +19,16 @@ constexpr int kLnBlock = kRowBlock;
 // L2 for every row makes every wave of the launch hammer the same 16 KB — the few L2 channels
 // that hold them — and cost ~15 % of the kernel's time.  BLOCK = 256 (few rows) reads them
 // straight from L2 and keeps more blocks in flight.
-template <typename T, typename Wt, typename S, int NV, bool VEC, int W, int BLOCK>
+// SHIFT: rows do not start on 16-byte boundaries (odd row length); see RowTile::load_shifted.
+// gamma / beta are then indexed element by element (their vectors do not line up with the row's).
+template <typename T, typename Wt, typename S, int NV, bool VEC, int W, int BLOCK, bool SHIFT = false>
 __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restrict__ x, const Wt* __restrict__ w,
                                                               const Wt* __restrict__ b, T* __restrict__ y,
                                                               S* __restrict__ mean_out, S* __restrict__ rstd_out,
                                                               int64_t rows, int64_t n, float eps) {
   using Tile = RowTile<T, NV, VEC, W, BLOCK>;
   constexpr int V = Tile::V;
-  constexpr bool STAGE = VEC && BLOCK > kLnBlock && W <= 4;  // rows over 8 / 16 waves: one row per block, nothing to share
+  constexpr bool STAGE = VEC && !SHIFT && BLOCK > kLnBlock && W <= 4;  // rows over 8 / 16 waves: one row per block, nothing to share
   extern __shared__ __attribute__((aligned(32))) unsigned char ln_smem[];
   __shared__ float red_a[BLOCK / kWave], red_b[BLOCK / kWave];
   const Wt* gs = w;
@@ -36,7 +38,13 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
   const bool active = row < rows;  // inactive groups still walk through the barriers
   if (!active) row = rows - 1;
   Tile tile;
-  tile.load(x + row * n, n, t, 0.f);
+  int a = 0;
+  if constexpr (SHIFT) {
+    a = row_misalignment<T, V>(x + row * n);
+    tile.load_shifted(x + row * n, n, a, t, 0.f);
+  } else {
+    tile.load(x + row * n, n, t, 0.f);
+  }
   if constexpr (STAGE) {
     Wt* gl = reinterpret_cast<Wt*>(ln_smem);
     Wt* bl = gl + n;
@@ -62,7 +70,15 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
   float q = 0.f;
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
-    if constexpr (VEC) {
+    if constexpr (SHIFT) {
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const int64_t c = Tile::col(k, j, t) - a;  // window position -> column of the row
+        const float d = (c >= 0 && c < n) ? tile.v[k][j] - mean : 0.f;
+        tile.v[k][j] = d;
+        q += d * d;
+      }
+    } else if constexpr (VEC) {
       if (Tile::col(k, 0, t) < n) {
 #pragma unroll
         for (int j = 0; j < V; ++j) {
@@ -88,7 +104,14 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
     rstd_out[row] = static_cast<S>(rstd);
   }
   T* out = y + row * n;
-  if constexpr (VEC) {
+  if constexpr (SHIFT) {
+    tile.store_shifted(out, n, a, t, [=](float d, int64_t c) {
+      float r = d * rstd;
+      if (w) r *= static_cast<float>(w[c]);
+      if (b) r += static_cast<float>(b[c]);
+      return r;
+    });
+  } else if constexpr (VEC) {
     // The weight / bias null tests are made once, outside the unrolled loops: inside, the
     // compiler turns them into a branch per element.
     auto emit = [&](auto has_w, auto has_b) {
@@ -307,18 +330,37 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
     MI355_LN_SUB(1) MI355_LN_SUB(2) MI355_LN_SUB(4) MI355_LN_SUB(8) MI355_LN_SUB(16) MI355_LN_SUB(32)
 #undef MI355_LN_SUB
   }
+  // Rows that start off a 16-byte boundary (odd N) still take the vector layout, shifted per
+  // row, when input and output rows are misaligned by the same number of elements.  Rows under
+  // 4000 bytes stay on the single-element layout: there the element-wise gamma / beta indexing of the
+  // shifted form costs more than its vector accesses save.
+  const bool shift = !vec && V > 1 && N * sizeof(T) >= 4000 &&
+                     (reinterpret_cast<uintptr_t>(x) / sizeof(T)) % V == (reinterpret_cast<uintptr_t>(y) / sizeof(T)) % V;
   if constexpr (!std::is_same<T, double>::value)  // f64 rows take the block kernel (double accumulation)
   if (!done)
-  done = dispatch_row_tile<T>(N, vec, [&](auto nv, auto wv, auto v) {
+  done = dispatch_row_tile<T>(shift ? N + V - 1 : N, vec || shift, [&](auto nv, auto wv, auto v) {
     constexpr int NV = decltype(nv)::value, WG = decltype(wv)::value;
     constexpr bool VEC = decltype(v)::value;
     if constexpr (WG >= 8) {  // rows of 8 K - 64 K elements: a 512- or 1024-thread block per row
       constexpr int BLK = kWave * WG;
+      if constexpr (VEC) {
+        if (shift) {
+          hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, true, WG, BLK, true>), dim3((unsigned)M), dim3(BLK), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+          return;
+        }
+      }
       hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, VEC, WG, BLK>), dim3((unsigned)M), dim3(BLK), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
       return;
     }
     constexpr int BIG = 1024;
     constexpr int rpb_big = WG >= 8 ? 1 : BIG / (kWave * WG), rpb = WG >= 8 ? 1 : kLnBlock / (kWave * WG);
+    if constexpr (VEC) {
+      if (shift) {
+        const unsigned nblk = (unsigned)((M + rpb - 1) / rpb);
+        hipLaunchKernelGGL((layernorm_tile_kernel<T, W, S, NV, true, WG, kLnBlock, true>), dim3(nblk), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, M, N, (float)eps);
+        return;
+      }
+    }
     // Enough rows to fill the chip with 1024-thread blocks: share gamma/beta through LDS.
     if (VEC && has_params && param_bytes <= 48 * 1024 && M >= (int64_t)rpb_big * 2 * kNumCU) {
       const unsigned nblk = (unsigned)((M + rpb_big - 1) / rpb_big);

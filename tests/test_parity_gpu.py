@@ -640,12 +640,19 @@ def test_misaligned_rows_see_exactly_their_own_elements(backend, n, dtype):
     got = backend[aten.native_layer_norm.default](xg, [n], w.cuda(), None, 1e-5)
     ref = aten_cpu.reference(aten.native_layer_norm.default, [x, [n], w, None, 1e-5])
     assert ev.allclose(ref, tuple(t.cpu() for t in got)), f"layer_norm n={n}"
+    bias = torch.rand(n, generator=g).to(dtype)
+    got = backend[aten.native_layer_norm.default](xg, [n], w.cuda(), bias.cuda(), 1e-5)
+    ref = aten_cpu.reference(aten.native_layer_norm.default, [x, [n], w, bias, 1e-5])
+    assert ev.allclose(ref, tuple(t.cpu() for t in got)), f"layer_norm with bias n={n}"
     # the same through a view that starts one element into its storage
     flat = torch.cat([torch.zeros(1, dtype=dtype), x.reshape(-1)]).cuda()
     view = flat[1:].view(rows, n)
     assert view.data_ptr() % 16 != 0
     assert ev.allclose(aten_cpu.reference(aten.amax.default, [x, [-1]]), backend[aten.amax.default](view, [-1]).cpu())
     assert ev.allclose(aten_cpu.reference(aten._softmax.default, [x, -1, False]), backend[aten._softmax.default](view, -1, False).cpu())
+    got = backend[aten.native_layer_norm.default](view, [n], None, None, 1e-5)
+    ref = aten_cpu.reference(aten.native_layer_norm.default, [x, [n], None, None, 1e-5])
+    assert ev.allclose(ref, tuple(t.cpu() for t in got)), f"layer_norm on an offset view n={n}"
 
 
 @pytest.mark.parametrize("family", ["gpt2", "bert"])
