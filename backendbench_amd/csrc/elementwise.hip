@@ -41,6 +41,15 @@ template <typename TA, typename TB> struct MulMixF {
     return static_cast<float>(a) * static_cast<float>(b);
   }
 };
+// Floating point: the hardware maximum / minimum (v_max / v_min order -0 below +0 and return the
+// other operand for a NaN), then one unordered compare puts the NaN back, as ATen propagates it.
+// Three VALU instructions per element instead of a chain of compares and selects, which at two
+// bytes per element is what keeps these kernels on the memory side of the roofline.
+__device__ __forceinline__ float hw_max(float x, float y) { return __builtin_fmaxf(x, y); }
+__device__ __forceinline__ double hw_max(double x, double y) { return __builtin_fmax(x, y); }
+__device__ __forceinline__ float hw_min(float x, float y) { return __builtin_fminf(x, y); }
+__device__ __forceinline__ double hw_min(double x, double y) { return __builtin_fmin(x, y); }
+
 template <typename T> struct MaximumF {
   using out_t = T; using in0_t = T; using in1_t = T; using in2_t = Unused;
   static constexpr int NIN = 2;
@@ -48,11 +57,11 @@ template <typename T> struct MaximumF {
   __device__ __forceinline__ T operator()(T a, T b, Unused) const {
     const M x = static_cast<M>(a), y = static_cast<M>(b);
     if constexpr (IsFloat<T>::value) {
-      if (x != x) return a;
-      if (y != y) return b;
-      if (x == y) return __builtin_signbit(x) ? b : a;  // IEEE 754-2019 maximum: +0 above -0
+      const M r = hw_max(x, y);
+      return static_cast<T>(__builtin_isunordered(x, y) ? x + y : r);
+    } else {
+      return x > y ? a : b;
     }
-    return x > y ? a : b;
   }
 };
 
@@ -63,11 +72,11 @@ template <typename T> struct MinimumF {
   __device__ __forceinline__ T operator()(T a, T b, Unused) const {
     const M x = static_cast<M>(a), y = static_cast<M>(b);
     if constexpr (IsFloat<T>::value) {
-      if (x != x) return a;
-      if (y != y) return b;
-      if (x == y) return __builtin_signbit(x) ? a : b;  // IEEE 754-2019 minimum: -0 below +0
+      const M r = hw_min(x, y);
+      return static_cast<T>(__builtin_isunordered(x, y) ? x + y : r);
+    } else {
+      return x < y ? a : b;
     }
-    return x < y ? a : b;
   }
 };
 
@@ -86,18 +95,18 @@ template <typename T> struct ClampF {
   using out_t = T; using in0_t = T; using in1_t = Unused; using in2_t = Unused;
   static constexpr int NIN = 1;
   using M = typename OpMath<T>::type;
-  M lo, hi;
+  M lo, hi;  // floating point: a missing bound is -inf / +inf, a NaN bound is kept (it makes everything NaN)
   bool has_lo, has_hi;
   __device__ __forceinline__ T operator()(T a, Unused, Unused) const {
     M x = static_cast<M>(a);
     if constexpr (IsFloat<T>::value) {
-      if (x != x) return a;
-      if (has_lo && lo != lo) return static_cast<T>(lo);  // a NaN bound makes everything NaN
-      if (has_hi && hi != hi) return static_cast<T>(hi);
+      const M r = hw_min(hw_max(x, lo), hi);  // hi applied last: lo > hi gives hi
+      return static_cast<T>(x != x ? x : (lo != lo ? lo : (hi != hi ? hi : r)));
+    } else {
+      if (has_lo && x < lo) x = lo;
+      if (has_hi && x > hi) x = hi;
+      return static_cast<T>(x);
     }
-    if (has_lo && x < lo) x = lo;
-    if (has_hi && x > hi) x = hi;  // applied last: lo > hi gives hi
-    return static_cast<T>(x);
   }
 };
 
@@ -314,8 +323,8 @@ extern "C" int mi355_unary(int op, const mi355_tensor* x, int bounds, double lo_
         ClampF<T> f;
         f.has_lo = bounds & 1;
         f.has_hi = bounds & 2;
-        f.lo = IsFloat<T>::value ? static_cast<M>(lo_f) : static_cast<M>(lo_i);
-        f.hi = IsFloat<T>::value ? static_cast<M>(hi_f) : static_cast<M>(hi_i);
+        f.lo = IsFloat<T>::value ? (f.has_lo ? static_cast<M>(lo_f) : static_cast<M>(-INFINITY)) : static_cast<M>(lo_i);
+        f.hi = IsFloat<T>::value ? (f.has_hi ? static_cast<M>(hi_f) : static_cast<M>(INFINITY)) : static_cast<M>(hi_i);
         return launch_elementwise(f, ins, out, st, "mi355_unary(clamp)");
       }
       default: return set_error(MI355_ERR_INVALID, "mi355_unary: unknown op %d", op);
@@ -351,7 +360,14 @@ template <typename T> struct ClampTensorF {
   using out_t = T; using in0_t = T; using in1_t = T; using in2_t = T;
   static constexpr int NIN = 3;
   __device__ __forceinline__ T operator()(T x, T lo, T hi) const {
-    return MinimumF<T>{}(MaximumF<T>{}(x, lo, Unused{}), hi, Unused{});
+    if constexpr (IsFloat<T>::value) {
+      using M = typename OpMath<T>::type;
+      const M v = static_cast<M>(x), l = static_cast<M>(lo), h = static_cast<M>(hi);
+      const M r = hw_min(hw_max(v, l), h);
+      return static_cast<T>((__builtin_isunordered(v, l) || h != h) ? v + l + h : r);
+    } else {
+      return MinimumF<T>{}(MaximumF<T>{}(x, lo, Unused{}), hi, Unused{});
+    }
   }
 };
 
