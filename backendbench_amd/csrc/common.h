@@ -2,6 +2,7 @@
 // access, wave64 reductions (DPP inside 16-lane rows, bpermute across rows), dimension
 // collapsing and the thread-local error string behind mi355_last_error().
 #pragma once
+#include <type_traits>
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -152,7 +153,9 @@ struct SumOp {
 // NaN-propagating max (either operand NaN -> NaN), the ATen amax/maximum rule.
 struct MaxNanOp {
   template <typename T> __device__ __forceinline__ T operator()(T a, T b) const {
-    if constexpr (IsFloat<T>::value) {
+    if constexpr (std::is_same<T, float>::value) {
+      return __builtin_elementwise_maximum(a, b);  // v_maximum3_f32: IEEE 754-2019 maximum, one instruction
+    } else if constexpr (IsFloat<T>::value) {
       return (is_nan(a) || a > b) ? a : b;  // b NaN: a > b false -> b
     } else {
       return a > b ? a : b;
