@@ -102,7 +102,12 @@ template <typename T> struct ClampF {
   __device__ __forceinline__ T operator()(T a, Unused, Unused) const {
     M x = static_cast<M>(a);
     if constexpr (IsFloat<T>::value) {
-      return static_cast<T>(nan_min(nan_max(x, lo), hi));  // hi applied last: lo > hi gives hi; any NaN gives NaN
+      // the NaN-ignoring v_max / v_min and one select for a NaN input measured faster here than the
+      // NaN-propagating pair (uniform bounds: their NaN tests are scalar)
+      M r;
+      if constexpr (sizeof(M) == 8) r = __builtin_fmin(__builtin_fmax(x, lo), hi);
+      else r = __builtin_fminf(__builtin_fmaxf(x, lo), hi);  // hi applied last: lo > hi gives hi
+      return static_cast<T>(x != x ? x : (lo != lo ? lo : (hi != hi ? hi : r)));
     } else {
       if (has_lo && x < lo) x = lo;
       if (has_hi && x > hi) x = hi;

@@ -45,7 +45,7 @@ __global__ __launch_bounds__(sm_tile_block(W)) void softmax_tile_kernel(const T*
 #pragma unroll
   for (int k = 0; k < NV; ++k)
 #pragma unroll
-    for (int j = 0; j < V; ++j) m = __builtin_elementwise_maximum(m, tile.v[k][j]);  // two elements per v_maximum3_f32; a NaN poisons the row either way
+    for (int j = 0; j < V; ++j) m = __builtin_fmaxf(m, tile.v[k][j]);  // v_max3_f32 takes two elements; a NaN is skipped here and poisons the sum below
   m = group_allreduce<W>(m, MaxOp(), red_max);
   float s = 0.f;
 #pragma unroll
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kSmBlock) void softmax_sub_kernel(const T* __restri
   }
   float m = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < V; ++j) m = __builtin_elementwise_maximum(m, v[j]);
+  for (int j = 0; j < V; ++j) m = __builtin_fmaxf(m, v[j]);
   m = sub_allreduce<G>(m, MaxOp());
   float s = 0.f;
 #pragma unroll
