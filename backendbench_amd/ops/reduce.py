@@ -225,8 +225,20 @@ def _softmax_impl(self, dim, half_to_float, log):
         return out
     x = dense(self)
     shape = x.shape if x.dim() else (1,)
+    outer, n, inner = prod(shape[:d]), shape[d], prod(shape[d + 1 :])
+    if (inner > 1 and n >= 256 and outer * ((inner + 63) // 64) < 256 and x.numel() >= 131072
+            and x.dtype != torch.float64):
+        # A long softmax axis over few columns gives the column kernels a handful of blocks that each
+        # walk the axis serially.  Two tiled transposing copies around the row kernel are far
+        # cheaper: [32, 1000, 49] fp32 takes 81 us on the column kernel and 26 us this way.
+        rows = dense(x.view(outer, n, inner).transpose(1, 2))
+        res = new_dense(rows.shape, out_dtype, self.device)
+        launch("mi355_softmax", rows.data_ptr(), _lib.dtype_code(x.dtype), res.data_ptr(), _lib.dtype_code(out_dtype),
+               outer * inner, n, 1, 1 if log else 0)
+        copy_into(out.view(outer, n, inner), res.transpose(1, 2))
+        return out
     launch("mi355_softmax", x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(out_dtype),
-           prod(shape[:d]), shape[d], prod(shape[d + 1 :]), 1 if log else 0)
+           outer, n, inner, 1 if log else 0)
     return out
 
 

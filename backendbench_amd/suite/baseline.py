@@ -397,6 +397,11 @@ def edge_cases() -> List[Case]:
     add(aten._softmax.default, lambda d: (_to(d, normal((37, 129), f64, 0, 2, seed=1), -1, False), {}), tag="last_f64")
     add(aten._softmax.default, lambda d: (_to(d, normal((5, 30, 7), f64, seed=1), 1, False), {}), tag="mid_f64")
     add(aten._log_softmax.default, lambda d: (_to(d, normal((3, 5000), f64, 0, 2, seed=1), -1, False), {}), tag="long_rows_f64")
+    # softmax axis in the middle with a short inner extent: transposed to rows and back
+    add(aten._softmax.default, lambda d: (_to(d, normal((8, 400, 49), f32, 0, 2, seed=1), 1, False), {}), tag="mid_short_inner_f32")
+    add(aten._log_softmax.default, lambda d: (_to(d, poison(normal((4, 300, 60), bf16, 0, 2, seed=1), 0.002, 4), 1, False), {}), tag="mid_short_inner_naninf_bf16")
+    add(aten._softmax.default, lambda d: (_to(d, normal((12, 256, 48), f16, 0, 2, seed=1), 1, True), {}), tag="mid_short_inner_half_to_float")
+    add(aten._softmax.default, lambda d: (_to(d, normal((2100, 8, 8), f32, 0, 2, seed=1), 0, False), {}), tag="first_dim_8x8_inner")
     # short rows: 1, 2, 4, 8, 16 and 32 lanes per row, vector and single-element layouts
     for rl, dt, t in ((2, f32, "f32"), (3, f16, "f16"), (8, f32, "f32"), (10, f32, "f32"), (16, bf16, "bf16"), (24, f16, "f16"),
                      (49, f32, "f32"), (64, f16, "f16"), (100, bf16, "bf16"), (128, f32, "f32"), (255, f16, "f16"), (256, bf16, "bf16")):
