@@ -349,6 +349,13 @@ def edge_cases() -> List[Case]:
     add(aten.sum.dim_IntList, lambda d: (_to(d, randint((9000, 40), 100, 1, i32, low=-100), [-1]), {}), exact=True, tag="short_rows_int")
     add(aten.sum.dim_IntList, lambda d: ([normal((9000 * 64 + 1,), f32, seed=7).to(d)[1:].view(9000, 64), [-1]], {}), tag="short_rows_offset_view")
 
+    # a long reduced axis over few columns: transposed to rows first
+    add(aten.sum.dim_IntList, lambda d: (_to(d, normal((70000, 8), f16, 0, 1, seed=1), [0]), {}), tag="few_columns_f16")
+    add(aten.amax.default, lambda d: (_to(d, poison(normal((3000, 50), f32, seed=1), 0.0001, 4), [0]), {}), tag="few_columns_naninf")
+    add(aten.argmax.default, lambda d: (_to(d, torch.round(normal((4, 9000, 5), f32, 0, 3, seed=1)), 1), {}), exact=True, tag="few_columns_ties")
+    add(aten.mean.dim, lambda d: (_to(d, normal((2, 5000, 16), bf16, 1, 2, seed=1), [1], True), {}), tag="few_columns_keepdim_bf16")
+    add(aten.sum.dim_IntList, lambda d: ([normal((70000, 8), f32, 0, 1, seed=1).to(d).t(), [1]], {}), tag="few_columns_transposed_view")
+    add(aten.sum.dim_IntList, lambda d: (_to(d, randint((40000, 6), 100, 1, i32), [0]), {}), exact=True, tag="few_columns_int")
     # ---- _softmax
     for dt in (f32, f16, bf16):
         t = f"{dt}".split(".")[-1]
