@@ -50,9 +50,9 @@ def _gemm(a, b, c, alpha, beta):
             # once into K-contiguous buffers padded with zeros to a multiple of 64 (exact: the pad
             # adds 0 * 0 terms), instead of running the whole product on the FMA fallback
             Kp = (K + 63) // 64 * 64
-            ap = torch.zeros((M, Kp), dtype=a.dtype, device=a.device)
+            both = torch.zeros((M + N, Kp), dtype=a.dtype, device=a.device)  # one fill for both operands
+            ap, btp = both[:M], both[M:]
             copy_into(ap[:, :K], a)
-            btp = torch.zeros((N, Kp), dtype=a.dtype, device=a.device)
             copy_into(btp[:, :K], b.t())
             a, b, K = ap, btp.t(), Kp
         elif b.stride(1) == 1 and N > 1 and (N % V or b.stride(0) % V or b.data_ptr() % 16):
