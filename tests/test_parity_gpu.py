@@ -549,6 +549,29 @@ def test_trace_replay_scores_every_op_correct(backend):
     assert seen == 20
 
 
+def test_evaluator_scores_the_whole_gpu_suite(backend):
+    """The evaluator's own flow (reference from the stock operator on the same device, then the
+    directory backend) over every operator of the GPU-built suite: all correct, a finite speed-up
+    for every operator.  Cases that ATen's GPU kernels refuse stay out of a suite built for the GPU."""
+    import math
+
+    from backendbench_amd.suite import BaselineTestSuite
+
+    announce("evaluator over the GPU baseline suite")
+    suite = BaselineTestSuite("cuda", scale=0.05)
+    n_ops = 0
+    for test in suite:
+        assert test.op in backend, test.op
+        c_score, p_score, c_res, p_res = ev.eval_one_op(test.op, backend[test.op], test.correctness_tests,
+                                                        test.performance_tests)
+        wrong = [r.args[:120] for r in c_res if not r.is_correct]
+        assert c_score == 1.0 and not wrong, (test.op, wrong[:3])
+        assert math.isfinite(float(p_score)) and float(p_score) > 0, test.op
+        n_ops += 1
+    assert n_ops == 28
+    assert not any(c.extra.get("cpu_reference_only") for t in suite for c in [x.case for x in t.correctness_tests])
+
+
 def test_tensors_beyond_2_to_31_elements(backend):
     """Element counts and byte offsets past 2^31 / 2^32: the kernels index with 64 bits."""
     announce("tensors beyond 2^31 elements")
