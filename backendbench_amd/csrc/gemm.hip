@@ -1856,14 +1856,16 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
           return b_nt ? (const void*)gemm_mfma_small_kernel<T, false, SP, false> : (const void*)gemm_mfma_small_kernel<T, true, SP, false>;
         }
       };
-      // Too few 256x256 tiles for the chip but between half a round and one round of 256x128
-      // tiles, and a K loop long enough to amortise the one-workgroup-per-CU pipeline: the
-      // four-wave kernel on 256x128 tiles.  MI355_GEMM_TILE=256x128 forces it (a test knob).
+      // Too few 256x256 tiles for the chip but close to one full round of 256x128 tiles, and a K loop
+      // long enough to amortise the one-workgroup-per-CU pipeline: the four-wave kernel on 256x128
+      // tiles.  Its time does not depend on the tile count up to 256, while the 128x128 kernel's grows
+      // with it; measured crossover at about 230 tiles for K = 3072 and 250 for K = 1024.
+      // MI355_GEMM_TILE=256x128 forces it (a test knob).
       const int64_t tiles_mid = (int64_t)g.tiles_m * ((N + 127) / 128);
       const char* forced_tile = getenv("MI355_GEMM_TILE");
       const bool mid = !ktail && K % 64 == 0 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "256x128") == 0
-                                               : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > kNumCU / 2 && tiles_mid <= kNumCU);
+                                               : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > (K >= 2048 ? 228 : 248) && tiles_mid <= kNumCU);
       if (mid) {
         g.tiles_n = (int32_t)((N + 127) / 128);
         nblocks = tiles_mid;
