@@ -197,6 +197,29 @@ def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
         assert ev.bit_equal(ref, out[rows.cuda()].cpu()), (layout, shape, K)
 
 
+@pytest.mark.parametrize("layout", ["nn", "nt"])
+@pytest.mark.parametrize("shape", [(200, 330), (1700, 1752), (2100, 2064)])
+def test_fp32_gemm_every_k_loop_length(backend, layout, shape):
+    """The fp32 MFMA kernel in its three forms: [200, K] x [K, 330] runs on 64x64 tiles (eight-stage
+    ring, split along K once K is long enough), [1700, K] x [K, 1752] has 196 tiles of 128x128 (one
+    workgroup per CU, eight stages), [2100, K] x [K, 2064] has 289 (four stages, two per CU).  K walks
+    through every prologue / steady / drain length of both ring depths; small-integer operands make the
+    fp32 accumulation exact in any order, so the sampled rows must be bit-equal to the oracle's."""
+    M, N = shape
+    announce(f"fp32 GEMM K loop lengths, {layout}, {M}x{N}")
+    g = torch.Generator().manual_seed(8)
+    rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 31, 32, 63, 64, 127, 128, M - 65, M - 64, M - 1])]))
+    for K in list(range(16, 16 * 21, 16)) + [400, 1040, 2064]:
+        a = torch.randint(-2, 3, (M, K), generator=g).float().cuda()
+        if layout[1] == "t":
+            b = torch.randint(-2, 3, (N, K), generator=g).float().cuda().t()
+        else:
+            b = torch.randint(-2, 3, (K, N), generator=g).float().cuda()
+        out = backend[aten.mm.default](a, b)
+        ref = aten_cpu.reference(aten.mm.default, [a[rows.cuda()], b])
+        assert ev.bit_equal(ref, out[rows.cuda()].cpu()), (layout, shape, K)
+
+
 def test_cpu_tensors_round_trip_through_the_gpu(backend):
     """The smoke suite hands CPU tensors (BackendBench/suite/smoke.py:25,30): the result must
     come back on the CPU and match ATen."""
