@@ -98,3 +98,7 @@ def test_workspace_planners_run_on_the_host():
     assert skinny > 0 and skinny % (16 * 4096 * 4) == 0 and skinny // (16 * 4096 * 4) <= 64
     assert lib.mi355_gemm_workspace_bytes(16, 4096, 4096, _lib.I32) == 0     # no integer GEMM
     assert lib.mi355_gemm_workspace_bytes(16, 4096, 32, _lib.BF16) == 0      # K too short to split
+    odd = lib.mi355_gemm_workspace_bytes(24, 1001, 2048, _lib.BF16)          # rows of a plane are padded to 4 columns
+    assert odd > 0 and odd % (24 * 1004 * 4) == 0
+    tiny = lib.mi355_gemm_workspace_bytes(64, 250, 1040, _lib.F32)           # fp32, 64x64 tiles
+    assert tiny > 0 and tiny % (64 * 252 * 4) == 0
