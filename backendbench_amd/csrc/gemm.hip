@@ -1749,7 +1749,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 // and the k extent of each (a multiple of the kernel's k step).  The split count minimises a
 // small cost model fitted to this chip: a 128x128 workgroup alone on a CU spends ~12.8 ns per k
 // (fp32: ~70 ns), two on a CU ~0.7 of that each, and a split adds a finishing launch (~3 us)
-// plus the fp32 partial planes written and read once at ~4 TB/s.  Each split keeps >= 8 k steps.
+// plus the fp32 partial planes written and read once at ~4 TB/s.  Each split keeps >= 8 k steps
+// (>= 4 when the output is one or two tiles).
 struct SplitPlan {
   int nsplit, ksplit;
 };
@@ -1764,7 +1765,8 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   SplitPlan p{1, (int)K};
   if (tiles >= kNumCU || K % bk != 0) return p;
   const double ns_per_k = elem_size == 4 ? (tile == 64 ? 20.0 : 70.0) : 12.8;
-  const int64_t max_ns = K / (8 * bk) < 64 ? K / (8 * bk) : 64;
+  const int min_steps = tiles <= 2 ? 4 : 8;  // one or two tiles: the launch is all latency, shorter splits still pay
+  const int64_t max_ns = K / (min_steps * bk) < 64 ? K / (min_steps * bk) : 64;
   double best = 0;
   int64_t best_ns = 1;
   for (int64_t ns = 1; ns <= max_ns; ++ns) {
