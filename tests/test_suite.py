@@ -119,3 +119,24 @@ def test_committed_trace_fixture_parses():
             assert any(isinstance(a, torch.Tensor) for a in args)
             n_inputs += 1
     assert n_inputs == 44
+
+
+def test_short_rows_trace_fixture_parses():
+    """tests/golden/short_rows_and_layouts_trace.txt (the inputs of the committed kernel-trace profile of the
+    short-row, transposing and fp32-tile kernels): five operators, nine inputs, one of them a strided view."""
+    import os
+
+    from backendbench_amd.ops import SLOTS
+    from backendbench_amd.utils import deserialize_args, op_name_to_folder_name
+
+    path = os.path.join(os.path.dirname(__file__), "golden", "short_rows_and_layouts_trace.txt")
+    ops = list(TraceTestSuite("trace", path))
+    assert len(ops) == 5 and sum(len(t.inputs) for t in ops) == 9
+    strided = 0
+    for t in ops:
+        assert op_name_to_folder_name(t.op.__name__) in SLOTS, t.op
+        for text in t.inputs:
+            small = re.sub(r"\d{3,}", "4", text)
+            args, _ = deserialize_args(small)
+            strided += sum(isinstance(a, torch.Tensor) and not a.is_contiguous() for a in args)
+    assert strided == 1
