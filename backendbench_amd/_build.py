@@ -40,8 +40,18 @@ FLAGS = [
 ]
 
 
-def _compile(src: str) -> Path:
+def _fresh(src: str, obj: Path) -> bool:
+    """True when `obj` is newer than its source and every header beside it."""
+    if not obj.exists():
+        return False
+    deps = [CSRC / src, *CSRC.glob("*.h"), PKG_DIR.parent / "include" / "mi355_aten.h", Path(__file__)]
+    return obj.stat().st_mtime > max(d.stat().st_mtime for d in deps)
+
+
+def _compile(src: str, incremental: bool = False) -> Path:
     obj = OBJ_DIR / (Path(src).stem + ".o")
+    if incremental and _fresh(src, obj):
+        return obj
     cmd = [HIPCC, *FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
@@ -49,11 +59,13 @@ def _compile(src: str) -> Path:
     return obj
 
 
-def build(verbose: bool = True, jobs: int = 7) -> Path:
-    """Compile every kernel source for gfx950 and link the shared library."""
+def build(verbose: bool = True, jobs: int = 7, incremental: bool = False) -> Path:
+    """Compile every kernel source for gfx950 and link the shared library.  `incremental`
+    (developer convenience, `--incremental` on the command line) keeps objects that are newer
+    than their source and the headers; the default recompiles everything."""
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(_compile, SOURCES))
+        objs = list(pool.map(lambda s: _compile(s, incremental), SOURCES))
     tmp = LIB_PATH.with_suffix(".so.tmp")
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -66,5 +78,5 @@ def build(verbose: bool = True, jobs: int = 7) -> Path:
 
 
 if __name__ == "__main__":
-    build()
+    build(incremental="--incremental" in sys.argv[1:])
     sys.exit(0)
