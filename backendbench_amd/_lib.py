@@ -13,7 +13,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi355_aten.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 MAX_DIMS = 8
 
 # mi355_dtype
@@ -68,6 +68,11 @@ SIGNATURES = {
     "mi355_reduce": (
         c_int,
         [c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_void_p],
+    ),
+    "mi355_reduce_static_max_bytes": (c_int64, []),
+    "mi355_reduce_static": (
+        c_int,
+        [c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p],
     ),
     "mi355_softmax": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "mi355_layer_norm": (

@@ -15,6 +15,8 @@
 //                to fill the chip (few rows, long reduction).
 #include "common.h"
 
+#include <mutex>
+
 #include <type_traits>
 
 namespace mi355 {
@@ -641,4 +643,52 @@ extern "C" int mi355_reduce(int op, const void* x, int in_dtype, int64_t outer, 
   }
   return set_error(MI355_ERR_UNSUPPORTED, "mi355_reduce: no kernel for op %d, %s -> %s", op,
                    dtype_name(in_dtype), dtype_name(out_dtype));
+}
+
+// ---------------------------------------------------------------- allocation-free form
+// Scratch for callers that cannot allocate (HIP graph capture, serving loops): one array per
+// GPU, held from library load until the process ends.  Host code never uses the array's name
+// as an address: the per-device address comes from hipGetSymbolAddress once per device.
+constexpr int64_t kStaticScratchBytes = 4 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch`, per device; nullptr = not asked yet
+static std::mutex g_scratch_mutex;
+
+static int scratch_address(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return set_error(MI355_ERR_LAUNCH, "mi355_reduce_static: hipGetDevice failed or device %d out of range: %s", dev,
+                     hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return set_error(MI355_ERR_LAUNCH, "mi355_reduce_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                       hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return MI355_OK;
+}
+
+extern "C" int64_t mi355_reduce_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int mi355_reduce_static(int op, const void* x, int in_dtype, int64_t outer, int64_t red, int64_t inner,
+                                   void* out, int out_dtype, void* stream) {
+  const int64_t need = mi355_reduce_workspace_bytes(op, in_dtype, outer, red, inner);
+  if (need == 0) return mi355_reduce(op, x, in_dtype, outer, red, inner, out, out_dtype, nullptr, 0, stream);
+  MI355_REQUIRE(need <= kStaticScratchBytes,
+                "mi355_reduce_static: this reduction needs %lld bytes of scratch, the built-in buffer holds %lld; "
+                "call mi355_reduce with a workspace of the caller's",
+                (long long)need, (long long)kStaticScratchBytes);
+  void* ptr = nullptr;
+  const int rc = scratch_address(&ptr);
+  if (rc) return rc;
+  // Every partial result the second pass reads is written by the first pass of the same call:
+  // nothing in the buffer has to start at zero.
+  return mi355_reduce(op, x, in_dtype, outer, red, inner, out, out_dtype, ptr, need, stream);
 }

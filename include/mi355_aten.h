@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define MI355_ABI_VERSION 3
+#define MI355_ABI_VERSION 4
 #define MI355_MAX_DIMS 8
 
 typedef enum mi355_dtype {
@@ -140,6 +140,18 @@ int64_t mi355_reduce_workspace_bytes(int op, int in_dtype, int64_t outer, int64_
 int mi355_reduce(int op, const void* x, int in_dtype, int64_t outer, int64_t red,
                  int64_t inner, void* out, int out_dtype, void* workspace,
                  int64_t workspace_bytes, void* stream);
+
+/* mi355_reduce for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * Same arguments and results as mi355_reduce minus the workspace: the partial results of a
+ * split reduction go to a buffer built into the library (one per GPU, mi355_reduce_static_max_bytes()
+ * = 4 MiB, held until the process ends).  Calls no allocator.  A reduction whose
+ * mi355_reduce_workspace_bytes() exceeds the buffer is refused with MI355_ERR_INVALID.
+ * All calls on one GPU share that GPU's buffer: calls that may overlap in time on one GPU
+ * (different streams, different threads) race; calls ordered on one stream do not. */
+int64_t mi355_reduce_static_max_bytes(void);
+int mi355_reduce_static(int op, const void* x, int in_dtype, int64_t outer, int64_t red,
+                        int64_t inner, void* out, int out_dtype, void* stream);
 
 /* y = softmax (log_softmax != 0: log-softmax) over the middle axis of dense x viewed as
  * [outer, dim, inner]; fp32 math.  out_dtype = in_dtype, or MI355_F32 for half_to_float.
