@@ -25,6 +25,7 @@ SOURCES = [
     "layernorm.hip",
     "index.hip",
     "gemm.hip",
+    "calib.hip",
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -59,7 +60,35 @@ def _compile(src: str, incremental: bool = False) -> Path:
     return obj
 
 
-def build(verbose: bool = True, jobs: int = 7, incremental: bool = False) -> Path:
+TRACE_LIB_PATH = LIB_DIR / "libmi355_gemm_trace.so"
+
+
+def build_trace(verbose: bool = True) -> Path:
+    """The GEMM source once more with -DMI355_GEMM_TRACE: the four-wave kernels then stamp the
+    shader clock (s_memtime) around the phases of every tile and of every step of the K loop and
+    leave the sums in the caller's workspace (layout beside the stamps in csrc/gemm.hip).  A
+    diagnostic build of its own, read by `bench.py --only-op C3.mm_down --trace`; the product
+    library carries no stamps."""
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    objs = []
+    for src, extra in (("gemm.hip", ["-DMI355_GEMM_TRACE"]), ("common.hip", [])):
+        obj = OBJ_DIR / (Path(src).stem + ".trace.o")
+        proc = subprocess.run([HIPCC, *FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)], capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {src} (trace build):\n{proc.stdout}\n{proc.stderr}")
+        objs.append(obj)
+    tmp = TRACE_LIB_PATH.with_suffix(".so.tmp")
+    proc = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed (trace build):\n{proc.stdout}\n{proc.stderr}")
+    os.replace(tmp, TRACE_LIB_PATH)
+    if verbose:
+        print(f"built {TRACE_LIB_PATH} ({TRACE_LIB_PATH.stat().st_size // 1024} KiB)")
+    return TRACE_LIB_PATH
+
+
+def build(verbose: bool = True, jobs: int = 8, incremental: bool = False) -> Path:
     """Compile every kernel source for gfx950 and link the shared library.  `incremental`
     (developer convenience, `--incremental` on the command line) keeps objects that are newer
     than their source and the headers; the default recompiles everything."""
@@ -78,5 +107,8 @@ def build(verbose: bool = True, jobs: int = 7, incremental: bool = False) -> Pat
 
 
 if __name__ == "__main__":
-    build(incremental="--incremental" in sys.argv[1:])
+    if "--trace" in sys.argv[1:]:
+        build_trace()
+    else:
+        build(incremental="--incremental" in sys.argv[1:])
     sys.exit(0)

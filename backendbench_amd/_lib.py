@@ -13,7 +13,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi355_aten.so"
-ABI_VERSION = 4
+ABI_VERSION = 6
 MAX_DIMS = 8
 
 # mi355_dtype
@@ -86,6 +86,8 @@ SIGNATURES = {
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
          c_int64, c_int64, c_double, c_double, c_int, c_void_p, c_int64, c_void_p],
     ),
+    "mi355_gemm_tile_columns": (c_int, [c_int64, c_int64, c_int64, ctypes.POINTER(c_int32), ctypes.POINTER(c_int32)]),
+    "mi355_calib_mfma": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mi355_index_select": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p],

@@ -1,0 +1,144 @@
+// Calibration kernel: the matrix-core instruction stream of the four-wave GEMM kernel with no
+// memory traffic at all.  One wave per SIMD holds the register tile of gemm_mfma_w4_kernel (two
+// sets of 2 x 4 A fragments and 2 x 4 B fragments, 256 fp32 accumulators) and issues the same 32
+// v_mfma_f32_32x32x16 per 32-k step in the same order, alternating between the two fragment
+// sets, for `steps` steps.  The fragments are loaded once from the caller's buffers, so the
+// operand DATA is the caller's choice: the sustained rate of this loop on a given data
+// distribution is what the chip's power / clock envelope leaves to any GEMM on that data, before
+// a byte is moved.  mi355_calib_mfma only serves measurement (bench.py --only-op calib.mfma).
+#include "common.h"
+
+namespace mi355 {
+
+typedef __bf16 cbf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 cf16x8 __attribute__((ext_vector_type(8)));
+typedef float cf32x16 __attribute__((ext_vector_type(16)));
+typedef float cf32x4 __attribute__((ext_vector_type(4)));
+
+template <typename F> struct CalibMfma;
+template <> struct CalibMfma<cbf16x8> {
+  static __device__ __forceinline__ cf32x16 run32(cbf16x8 a, cbf16x8 b, cf32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ cf32x4 run16(cbf16x8 a, cbf16x8 b, cf32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct CalibMfma<cf16x8> {
+  static __device__ __forceinline__ cf32x16 run32(cf16x8 a, cf16x8 b, cf32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ cf32x4 run16(cf16x8 a, cf16x8 b, cf32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+};
+
+// ORDER 0: the GEMM kernel's order (B fragment first operand, held over four MFMAs; A fragment
+//          second, changing every MFMA).
+// ORDER 1: operands swapped between the two ports.
+// ORDER 2: second operand held over four MFMAs, first changing.
+template <typename F, int ORDER>
+__global__ __launch_bounds__(256) void calib_mfma32_kernel(const F* __restrict__ a, const F* __restrict__ b, float* __restrict__ out, int steps) {
+  const int64_t lane_slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  F xa[2][2][4], xb[2][2][4];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        xa[s][ks][i] = a[lane_slot * 16 + (s * 2 + ks) * 4 + i];
+        xb[s][ks][i] = b[lane_slot * 16 + (s * 2 + ks) * 4 + i];
+      }
+  cf32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  for (int t = 0; t < steps; t += 2) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if constexpr (ORDER == 0) acc[q][p] = CalibMfma<F>::run32(xb[s][ks][p], xa[s][ks][q], acc[q][p]);
+            else if constexpr (ORDER == 1) acc[q][p] = CalibMfma<F>::run32(xa[s][ks][q], xb[s][ks][p], acc[q][p]);
+            else acc[p][q] = CalibMfma<F>::run32(xb[s][ks][q], xa[s][ks][p], acc[p][q]);
+          }
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) sum += acc[i][j][e];
+  out[lane_slot] = sum;
+}
+
+// The same register tile on v_mfma_f32_16x16x32: 8 x 8 blocks of 16 x 16 (64 accumulators of four
+// registers), eight A and eight B fragments per 32-k step, 64 MFMAs of half the work each.
+template <typename F>
+__global__ __launch_bounds__(256) void calib_mfma16_kernel(const F* __restrict__ a, const F* __restrict__ b, float* __restrict__ out, int steps) {
+  const int64_t lane_slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  F xa[2][8], xb[2][8];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      xa[s][i] = a[lane_slot * 16 + s * 8 + i];
+      xb[s][i] = b[lane_slot * 16 + s * 8 + i];
+    }
+  cf32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+  for (int t = 0; t < steps; t += 2) {
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int p = 0; p < 8; ++p)
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc[q][p] = CalibMfma<F>::run16(xb[s][p], xa[s][q], acc[q][p]);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum += acc[i][j][e];
+  out[lane_slot] = sum;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+// blocks x 256 threads, each wave issuing `steps` (even) 32-k steps of a 128 x 128 register tile:
+// 2 * 128 * 128 * 32 flop per wave and step.  a, b: 16 fragments of 16 bytes per thread
+// (blocks * 256 * 256 bytes each); out: blocks * 256 floats.  variant 0..2: 32x32x16 in the three
+// operand orders, 3: 16x16x32.
+extern "C" int mi355_calib_mfma(const void* a, const void* b, void* out, int dtype, int blocks, int steps, int variant,
+                                void* stream) {
+  MI355_REQUIRE(a != nullptr && b != nullptr && out != nullptr, "mi355_calib_mfma: NULL buffer");
+  MI355_REQUIRE(blocks > 0 && steps > 0 && steps % 2 == 0, "mi355_calib_mfma: blocks > 0 and an even number of steps");
+  MI355_REQUIRE(dtype == MI355_BF16 || dtype == MI355_F16, "mi355_calib_mfma: bf16 or f16");
+  MI355_REQUIRE(variant >= 0 && variant <= 3, "mi355_calib_mfma: variant 0..3");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* o = static_cast<float*>(out);
+#define MI355_CALIB(F_)                                                                                                        \
+  {                                                                                                                            \
+    const F_* pa = static_cast<const F_*>(a);                                                                                  \
+    const F_* pb = static_cast<const F_*>(b);                                                                                  \
+    switch (variant) {                                                                                                         \
+      case 0: hipLaunchKernelGGL((calib_mfma32_kernel<F_, 0>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;       \
+      case 1: hipLaunchKernelGGL((calib_mfma32_kernel<F_, 1>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;       \
+      case 2: hipLaunchKernelGGL((calib_mfma32_kernel<F_, 2>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;       \
+      default: hipLaunchKernelGGL((calib_mfma16_kernel<F_>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;         \
+    }                                                                                                                          \
+  }
+  if (dtype == MI355_BF16) MI355_CALIB(cbf16x8) else MI355_CALIB(cf16x8)
+#undef MI355_CALIB
+  return check_launch("mi355_calib_mfma");
+}

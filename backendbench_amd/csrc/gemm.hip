@@ -74,6 +74,7 @@ struct GemmArgs {
   int32_t M, N, K;
   float alpha, beta;
   int32_t tiles_m, tiles_n;
+  int32_t tail_n;  // gemm_mfma_w4_mixed_kernel: 192-wide tile columns behind the tiles_n 256-wide ones
   int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
   int32_t out_vec;  // out rows start on 16-byte boundaries (N a multiple of the vector width): vector stores
   // Split-K (128x128 kernels only): blockIdx.y = split, which covers k in [split * ksplit,
@@ -179,21 +180,23 @@ __global__ __launch_bounds__(256) void gemm_splitk_finish4_kernel(GemmArgs g, in
 // Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous
 // band of tile ids, then walk the band in groups of 8 tile-rows so A and B panels repeat
 // in that XCD's L2.
-__device__ __forceinline__ void tile_coords(const GemmArgs& g, int& tm, int& tn) {
-  const int nblocks = g.tiles_m * g.tiles_n;
-  int pid = blockIdx.x;
+__device__ __forceinline__ void tile_coords(const int tiles_m, const int tiles_n, int pid, int& tm, int& tn) {
+  const int nblocks = tiles_m * tiles_n;
   const int per_xcd = (nblocks + kNumXCD - 1) / kNumXCD;
   const int full = nblocks % kNumXCD;  // XCDs that own `per_xcd` tiles when not divisible
   const int xcd = pid % kNumXCD, local = pid / kNumXCD;
   if (full == 0) pid = xcd * per_xcd + local;
   else pid = (xcd < full ? xcd * per_xcd : full * per_xcd + (xcd - full) * (per_xcd - 1)) + local;
   constexpr int GROUP = 8;
-  const int in_group = GROUP * g.tiles_n;
+  const int in_group = GROUP * tiles_n;
   const int group = pid / in_group;
   const int first_m = group * GROUP;
-  const int rows = g.tiles_m - first_m < GROUP ? g.tiles_m - first_m : GROUP;
+  const int rows = tiles_m - first_m < GROUP ? tiles_m - first_m : GROUP;
   tm = first_m + (pid % in_group) % rows;
   tn = (pid % in_group) / rows;
+}
+__device__ __forceinline__ void tile_coords(const GemmArgs& g, int& tm, int& tn) {
+  tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
 }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -217,8 +220,9 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
 // 16 KB slice of the (now idle) LDS ring, and reads it back row-major: every global store
 // instruction then writes 8 complete 128-byte rows.  Must be called by all waves after the
 // last barrier of the main loop (the ring is no longer read).
-// A wave with more than two 32-column blocks (NJ > 2) calls this once per pair of blocks, J0 = 0, 2, ...
-template <typename T, int MI, int J0 = 0, int NJ>
+// A wave with more than two 32-column blocks (NJ > 2) calls this once per pair of blocks, J0 = 0, 2, ...;
+// NB = 1 stores the single block J0 (the last one of an odd count): the left 64 bytes of every slab row.
+template <typename T, int MI, int J0 = 0, int NB = 2, int NJ>
 __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x16 (&acc)[MI][NJ], unsigned char* lds,
                                                   int wave, int lane, int m0, int n0) {
   const int fr = lane & 31, fg = lane >> 5;
@@ -228,10 +232,10 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
   // A bias row (c broadcast along m: the Linear-layer addmm) is the same for every row of the
   // tile: its 8 groups of four columns are loaded once, scaled by beta, and reused for all rows.
   const bool row_bias = use_c && g.c_vec && g.c_rs == 0;
-  float bias[2][4][4];
+  float bias[NB][4][4];
   if (row_bias) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + j * 32 + q * 8 + fg * 4;
@@ -248,7 +252,7 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
       const int m = m0 + row;
       const int mc = m < g.M ? m : g.M - 1;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < NB; ++j) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int nl = j * 32 + q * 8 + fg * 4;
@@ -297,7 +301,7 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
       const int row = chunk >> 3, s = chunk & 7;
       const u32x4 v = *reinterpret_cast<const u32x4*>(slab + row * 128 + ((s ^ ((row >> 1) & 7)) << 4));
       const int m = m0 + row, n = n0 + s * 8;
-      if (m >= g.M || n >= g.N) continue;
+      if (m >= g.M || n >= g.N || s >= NB * 4) continue;
       *reinterpret_cast<u32x4*>(D + (int64_t)m * g.N + n) = v;
     }
   } else {
@@ -309,7 +313,7 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
 #pragma unroll 8
     for (int row = 0; row < rows; ++row) {
       const T v = *reinterpret_cast<const T*>(slab + row * 128 + (((lane >> 3) ^ ((row >> 1) & 7)) << 4) + ((lane & 7) << 1));
-      if (n < g.N) D[(int64_t)(m0 + row) * g.N + n] = v;
+      if (n < g.N && lane < NB * 32) D[(int64_t)(m0 + row) * g.N + n] = v;
     }
   }
 }
@@ -469,6 +473,16 @@ __device__ __forceinline__ void lds_dma16(uint32_t lds_byte_offset, const void* 
   asm volatile("s_mov_b32 m0, %0\n\t"
                "s_nop 0\n\t"
                "global_load_lds_dwordx4 %1, off" ::"s"(lds_byte_offset), "v"(gptr)
+               : "memory");
+}
+
+// The same fill with the address split into a uniform 64-bit base (SGPR pair) and a 32-bit byte
+// offset per lane: the offsets of a wave's requests are loop invariants (one VGPR each instead of
+// a pointer pair) and a k step only moves the scalar base.
+__device__ __forceinline__ void lds_dma16s(uint32_t lds_byte_offset, uint32_t lane_byte_offset, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\t"
+               "s_nop 0\n\t"
+               "global_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_byte_offset), "s"(base)
                : "memory");
 }
 
@@ -815,24 +829,31 @@ __device__ __forceinline__ int swz_n128(int k, int u) {
 // problems that do not fill the chip with 256x256 tiles.
 // A_T: the left operand is M-contiguous (a transposed view, e.g. x.t() @ dy): its panel stays k-major
 // in LDS like a row-major B and is transposed by the LDS read.
-template <typename T, bool B_NN, int NJ, bool A_T>
-__global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
+// NJA < NJ (3 of 4): the tile is 32 NJA x 2 columns wide (256 x 192) on the LDS layout and fills of the
+// NJ form; the panel columns past the tile are fetched (clamped at the matrix edge) and not used.
+// Such tiles cost about three quarters of a 256 x 256 one and let a last, partly filled round
+// of tiles be cut to fit the chip (see gemm_mfma_w4_mixed_kernel).
+template <typename T, bool B_NN, int NJ, bool A_T, int NJA = NJ>
+__device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, const int bm, const int bn) {
   static_assert(NJ == 2 || NJ == 4, "wave tile is 128 x 32 NJ");
-  constexpr int BNT = NJ * 64;  // tile width
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  static_assert(NJA == NJ || (NJ == 4 && NJA == 3), "narrow form: three of four column blocks");
   using frag_t = typename Mfma<T>::frag;
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave >> 1, wn = wave & 1;
-  int tm, tn;
-  tile_coords(g, tm, tn);
-  const int bm = tm * BM, bn = tn * BNT;
   const T* A = static_cast<const T*>(g.a);
   const T* B = static_cast<const T*>(g.b);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+#ifdef MI355_GEMM_TRACE
+  const uint64_t tr_entry = __builtin_readcyclecounter();
+#endif
 
-  const T* a_src[8];
-  const T* b_src[NJ];
+  // Fill addresses: a uniform base per operand (moved along k by the requests) plus one 32-bit byte
+  // offset per lane and request (the host checks that they fit: leading dimensions below 4 M elements).
+  const T* a_base = A_T ? A : A + (int64_t)bm * g.lda;   // K-contiguous A: offsets are relative to the tile's first row
+  const T* b_base = B_NN ? B : B + (int64_t)bn * g.ldb;  // K-contiguous B: relative to the tile's first column
+  uint32_t a_off[8];
+  uint32_t b_off[NJ];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     if constexpr (A_T) {  // M-contiguous A: the pair slot holds 64 k-rows of 512 B (swz_n), region = two k-rows
@@ -840,13 +861,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
       const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
       int gm = bm + u * 8;
       gm = gm < g.M ? gm : 0;
-      a_src[i] = A + (int64_t)k * g.lda + gm;
+      a_off[i] = ((uint32_t)k * (uint32_t)g.lda + (uint32_t)gm) * 2u;
     } else {
       const int r = 8 * (wave + 4 * i) + (lane >> 3), slot = lane & 7;
       const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
-      int gr = bm + r;
-      gr = gr < g.M ? gr : g.M - 1;
-      a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+      const int lr = bm + r < g.M ? r : g.M - 1 - bm;  // rows past M re-read the last row
+      a_off[i] = ((uint32_t)lr * (uint32_t)g.lda + (uint32_t)c * 8u) * 2u;
     }
   }
 #pragma unroll
@@ -856,30 +876,29 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
       const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
       int gn = bn + u * 8;
       gn = gn < g.N ? gn : 0;
-      b_src[i] = B + (int64_t)k * g.ldb + gn;
+      b_off[i] = ((uint32_t)k * (uint32_t)g.ldb + (uint32_t)gn) * 2u;
     } else if constexpr (B_NN) {  // 256-byte k-rows (swz_n128): region = four k-rows
       const int k = 4 * (wave + 4 * i) + (lane >> 4), pos = lane & 15;
       const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
       int gn = bn + u * 8;
       gn = gn < g.N ? gn : 0;
-      b_src[i] = B + (int64_t)k * g.ldb + gn;
+      b_off[i] = ((uint32_t)k * (uint32_t)g.ldb + (uint32_t)gn) * 2u;
     } else {
       const int r = 16 * (wave + 4 * i) + (lane >> 2), slot = lane & 3;
       const int c = slot ^ ((r >> 2) & 3);
-      int gn = bn + r;
-      gn = gn < g.N ? gn : g.N - 1;
-      b_src[i] = B + (int64_t)gn * g.ldb + c * 8;
+      const int ln = bn + r < g.N ? r : g.N - 1 - bn;
+      b_off[i] = ((uint32_t)ln * (uint32_t)g.ldb + (uint32_t)c * 8u) * 2u;
     }
   }
   // Fill requests: A request i (0..7) of the slot at byte offset a_slot, holding steps t, t+1;
   // B request i (0..NJ-1) of step t.
   auto request_a = [&](int i, int t, uint32_t a_slot) {
-    lds_dma16(lds_base + a_slot + (uint32_t)(wave + 4 * i) * 1024u,
-              a_src[i] + (A_T ? (int64_t)t * BK3 * g.lda : (int64_t)t * BK3));
+    lds_dma16s(lds_base + a_slot + (uint32_t)(wave + 4 * i) * 1024u, a_off[i],
+               a_base + (A_T ? (int64_t)t * BK3 * g.lda : (int64_t)t * BK3));
   };
   auto request_b = [&](int i, int t) {
-    lds_dma16(lds_base + kBRing64 + (uint32_t)(t & 3) * kPanel3 + (uint32_t)(wave + 4 * i) * 1024u,
-              b_src[i] + (B_NN ? (int64_t)t * BK3 * g.ldb : (int64_t)t * BK3));
+    lds_dma16s(lds_base + kBRing64 + (uint32_t)(t & 3) * kPanel3 + (uint32_t)(wave + 4 * i) * 1024u, b_off[i],
+               b_base + (B_NN ? (int64_t)t * BK3 * g.ldb : (int64_t)t * BK3));
   };
 
   const int fr = lane & 31, fg = lane >> 5;
@@ -890,7 +909,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   // request a_first .. a_first+3 of the slot fill_slot (steps ta, ta+1), then the four B requests
   // of step tb — so that the fills leave the wave one at a time over the second half of the step
   // instead of as a burst behind the barrier (the burst form ran the all-zero GEMM 20 % slower).
-  auto io_step = [&](int t, uint32_t a_slot, int half, frag_t (&xa)[2][4], frag_t (&xb)[2][NJ], bool fill_a, int ta,
+  auto io_step = [&](int t, uint32_t a_slot, int half, frag_t (&xa)[2][4], frag_t (&xb)[2][NJA], bool fill_a, int ta,
                      uint32_t fill_slot, int a_first, bool fill_b, int tb) __attribute__((always_inline)) {
     const unsigned char* pa = lds + a_slot;
     const unsigned char* pb = lds + kBRing64 + (t & 3) * kPanel3;
@@ -917,35 +936,37 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
         if (ks == 1) fill(i);
       }
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
+      for (int j = 0; j < NJA; ++j) {
         if constexpr (B_NN) {
           const int k = ks * 16 + tr_k;
-          const int n = wn * (NJ * 32) + j * 32 + tr_n;
+          const int n = wn * (NJA * 32) + j * 32 + tr_n;
           const int off_lo = NJ == 4 ? swz_n(k, n >> 3) : swz_n128(k, n >> 3);
           const int off_hi = NJ == 4 ? swz_n(k + 4, n >> 3) : swz_n128(k + 4, n >> 3);
           const s16x4 lo = lds_read_tr(pb + off_lo + ((n & 7) << 1));
           const s16x4 hi = lds_read_tr(pb + off_hi + ((n & 7) << 1));
           xb[ks][j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
         } else {
-          xb[ks][j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * (NJ * 32) + j * 32 + fr, ks * 2 + fg));
+          xb[ks][j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * (NJA * 32) + j * 32 + fr, ks * 2 + fg));
         }
         if (ks == 1) fill(4 + j);
       }
+      if constexpr (NJA < NJ)
+        if (ks == 1) fill(4 + NJA);  // the fills keep the NJ form: one more B request than column blocks
     }
   };
 
-  f32x16 acc[4][NJ];
+  f32x16 acc[4][NJA];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
+    for (int j = 0; j < NJA; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  auto mma_step = [&](frag_t (&xa)[2][4], frag_t (&xb)[2][NJ]) __attribute__((always_inline)) {
+  auto mma_step = [&](frag_t (&xa)[2][4], frag_t (&xb)[2][NJA]) __attribute__((always_inline)) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-      for (int j = 0; j < NJ; ++j)
+      for (int j = 0; j < NJA; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[i][j] = Mfma<T>::run(xb[ks][j], xa[ks][i], acc[i][j]);
   };
@@ -961,7 +982,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
 #define MI355_X4(X) X X X X
 #define MI355_MDD MI355_MD __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
 #define MI355_W4_SCHEDULE                                                     \
-  if constexpr (NJ == 4 && A_T && B_NN) {      /* 32 reads, 32 MFMAs */       \
+  if constexpr (NJA == 3 && A_T && B_NN) {     /* 28 reads, 24 MFMAs */       \
+    MI355_X4(MI355_MDD) MI355_X4(MI355_X4(MI355_MD)) MI355_X4(MI355_MD)       \
+  } else if constexpr (NJA == 3 && (A_T || B_NN)) { /* 22 / 20 reads */       \
+    MI355_X4(MI355_X4(MI355_MD)) MI355_X4(MI355_MD) MI355_MD MI355_MD         \
+  } else if constexpr (NJA == 3) {             /* 14 reads */                 \
+    MI355_X4(MI355_MDM) MI355_X4(MI355_MDM) MI355_X4(MI355_MD) MI355_MD MI355_MD \
+  } else if constexpr (NJ == 4 && A_T && B_NN) { /* 32 reads, 32 MFMAs */     \
     MI355_X4(MI355_MDD) MI355_X4(MI355_MDD) MI355_X4(MI355_X4(MI355_MD))      \
   } else if constexpr (NJ == 4 && A_T) {       /* 24 reads */                 \
     MI355_X4(MI355_X4(MI355_MD)) MI355_X4(MI355_MD) MI355_X4(MI355_MDM)       \
@@ -1013,29 +1040,75 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   else if (nk > 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  frag_t fa[2][2][4], fb[2][2][NJ];
+  frag_t fa[2][2][4], fb[2][2][NJA];
   uint32_t cur = 0;  // A slot of steps t, t+1 (t even)
   io_step(0, cur, 0, fa[0], fb[0], false, 0, 0u, 0, false, 0);
   __syncthreads();  // every wave has its fragments of step 0: the B slot of step 0 may be refilled
   int t = 0;
+#ifdef MI355_GEMM_TRACE
+  // Diagnostic build only (-DMI355_GEMM_TRACE, libmi355_gemm_trace.so): shader-clock stamps
+  // (s_memtime, read one step after they are issued, so no wait is added).  Lane 0 of every wave
+  // leaves 16 uint64 in the caller's workspace at ((block * 4 + wave) * 16):
+  //   [0..5]  sums over the steady-state loop of, for the even and the odd step of an iteration:
+  //           ticks issuing the step's MFMAs / reads / fills, ticks in s_waitcnt for the fills,
+  //           ticks from there to behind the barrier (the odd one includes the loop's back edge
+  //           and ~170 ticks of this bookkeeping);
+  //   [6] ticks in the loop   [7] loop iterations   [8], [9] longest single fill wait / barrier wait
+  //   [10] stamp at loop entry   [11] HW_ID   [12] stamp at tile entry   [13] at loop exit
+  //   [14] behind the remainder and drain steps   [15] when the tile's stores have completed.
+  const uint64_t tr_begin = __builtin_readcyclecounter();
+  uint64_t tp0 = tr_begin, tp1 = tr_begin, tp2 = tr_begin, tp3 = tr_begin, tp4 = tr_begin, tp5 = tr_begin;
+  uint64_t tr_sum[6] = {0, 0, 0, 0, 0, 0};
+  uint64_t tr_max[2] = {0, 0};
+#define MI355_TR_STAMP(v) asm volatile("s_memtime %0" : "=s"(v)::"memory");
+#define MI355_TR_C0 { tr_sum[0] += tp1 - tp0; tr_sum[1] += tp2 - tp1; tr_sum[2] += tp3 - tp2; \
+    if (tp2 - tp1 > tr_max[0]) tr_max[0] = tp2 - tp1; if (tp3 - tp2 > tr_max[1]) tr_max[1] = tp3 - tp2; }
+#define MI355_TR_C1 { tr_sum[3] += tp4 - tp3; tr_sum[4] += tp5 - tp4; tr_sum[5] += tp0 - tp5; }
+#else
+#define MI355_TR_STAMP(v)
+#define MI355_TR_C0
+#define MI355_TR_C1
+#endif
   for (; t + 7 < nk; t += 2) {
     const uint32_t nxt = next_slot(cur);
+    MI355_TR_C0 MI355_TR_STAMP(tp0)
     // even step t
     io_step(t + 1, cur, 1, fa[1], fb[1], true, t + 4, next_slot(nxt), 4, true, t + 4);
     mma_step(fa[0], fb[0]);
     MI355_W4_SCHEDULE
+    MI355_TR_STAMP(tp1)
     if constexpr (NJ == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    MI355_TR_STAMP(tp2)
     __syncthreads();
+    MI355_TR_C1 MI355_TR_STAMP(tp3)
     // odd step t+1
     io_step(t + 2, nxt, 0, fa[0], fb[0], true, t + 6, cur, 0, true, t + 5);
     mma_step(fa[1], fb[1]);
     MI355_W4_SCHEDULE
+    MI355_TR_STAMP(tp4)
     if constexpr (NJ == 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    MI355_TR_STAMP(tp5)
     __syncthreads();
     cur = nxt;
   }
+#ifdef MI355_GEMM_TRACE
+  {
+    const uint64_t tr_end = __builtin_readcyclecounter();
+    if (lane == 0 && g.ws != nullptr) {
+      uint64_t* o = reinterpret_cast<uint64_t*>(g.ws) + ((int64_t)blockIdx.x * 4 + wave) * 16;
+      for (int q = 0; q < 6; ++q) o[q] = tr_sum[q];
+      o[6] = tr_end - tr_begin; o[7] = (uint64_t)(t / 2); o[8] = tr_max[0]; o[9] = tr_max[1]; o[10] = tr_begin;
+      o[11] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));  // HW_REG_HW_ID (XCC / SE / CU of this wave)
+      o[12] = tr_entry;
+      o[13] = tr_end;
+    }
+  }
+#endif
+#undef MI355_TR_STAMP
+#undef MI355_TR_C0
+#undef MI355_TR_C1
 #undef MI355_W4_SCHEDULE
 #undef MI355_X4
 #undef MI355_MDD
@@ -1070,10 +1143,53 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
     cur = nxt;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing is in flight: the last two steps issue no fills)
+#ifdef MI355_GEMM_TRACE
+  const uint64_t tr_drained = __builtin_readcyclecounter();
+#endif
 
-  store_tile_result<T, 4, 0>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * (NJ * 32));
-  if constexpr (NJ == 4) store_tile_result<T, 4, 2>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 128 + 64);
+  store_tile_result<T, 4, 0>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * (NJA * 32));
+  if constexpr (NJA == 4) store_tile_result<T, 4, 2>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 128 + 64);
+  if constexpr (NJA == 3) store_tile_result<T, 4, 2, 1>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 96 + 64);
+#ifdef MI355_GEMM_TRACE
+  {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const uint64_t tr_stored = __builtin_readcyclecounter();
+    if (lane == 0 && g.ws != nullptr) {
+      uint64_t* o = reinterpret_cast<uint64_t*>(g.ws) + ((int64_t)blockIdx.x * 4 + wave) * 16;
+      o[14] = tr_drained;
+      o[15] = tr_stored;
+    }
+  }
+#endif
 }
+
+template <typename T, bool B_NN, int NJ, bool A_T>
+__global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  w4_tile<T, B_NN, NJ, A_T>(g, lds, tm * BM, tn * (NJ * 64));
+}
+
+// The same tiles in two widths in one launch: blocks [0, tiles_m * tiles_n) are 256 x 256 tiles of the
+// columns [0, 256 tiles_n); the blocks behind them are 256 x 192 tiles of the columns from there on
+// (tiles_m * tail_n of them).  Workgroups are dispatched in block order, so the narrow tiles form
+// the last round: a tile count that leaves the last round of 256-wide tiles partly empty (688 tiles
+// on 256 CUs: 2.69 rounds, paid as 3) becomes two full rounds plus one round of cheaper tiles.
+template <typename T, bool B_NN, bool A_T>
+__global__ __launch_bounds__(256) void gemm_mfma_w4_mixed_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int wide = g.tiles_m * g.tiles_n;
+  int tm, tn;
+  if ((int)blockIdx.x < wide) {
+    tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
+    w4_tile<T, B_NN, 4, A_T, 4>(g, lds, tm * BM, tn * 256);
+  } else {
+    tile_coords(g.tiles_m, g.tail_n, blockIdx.x - wide, tm, tn);
+    w4_tile<T, B_NN, 4, A_T, 3>(g, lds, tm * BM, g.tiles_n * 256 + tn * 192);
+  }
+}
+
 
 // ---------------------------------------------------------------- MFMA kernel, 128x128 tiles
 // For problems that do not fill the chip with 256x256 tiles.  Four waves (2x2), each a 64x64
@@ -1790,6 +1906,57 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   return p;
 }
 
+// Widths for the four-wave kernel's tile columns: `wide` columns of 256 followed by `narrow` columns
+// of 192 (gemm_mfma_w4_mixed_kernel), chosen to minimise the time of the launch when workgroups
+// go to the CUs in block order, one per CU; narrow == 0 is the plain 256-wide grid.  A 192-wide
+// tile is priced at kNarrowCost of a 256-wide one (three quarters of the MFMAs on the same fills).
+struct MixedPlan {
+  int wide, narrow;
+};
+constexpr double kNarrowCost = 0.85;  // measured: 0.78 of the K loop's ticks, the per-tile prologue and epilogue in full
+constexpr int64_t kMixedMinK = 4096;  // shorter K loops: the per-tile overhead of the extra tiles eats the gain
+static double mixed_makespan(int64_t n_wide, int64_t n_narrow) {
+  // wide tiles first: after them `late` CUs are free at time rounds + 1, the others at `rounds`
+  const int64_t rounds = n_wide / kNumCU, late = n_wide % kNumCU;
+  double t[2] = {(double)rounds, (double)rounds + 1.0};
+  int64_t cnt[2] = {kNumCU - late, late};
+  double end = late ? t[1] : t[0];
+  if (n_wide == 0) end = 0.0;
+  while (n_narrow > 0) {
+    const int e = (cnt[1] > 0 && t[1] < t[0]) || cnt[0] == 0 ? 1 : 0;
+    const int64_t take = n_narrow < cnt[e] ? n_narrow : cnt[e];
+    n_narrow -= take;
+    const double fin = t[e] + kNarrowCost;
+    if (fin > end) end = fin;
+    if (take == cnt[e]) {
+      t[e] = fin;
+    } else {  // last, partial batch: nothing is scheduled behind it
+      break;
+    }
+  }
+  return end;
+}
+static MixedPlan plan_mixed(int64_t tiles_m, int64_t N) {
+  static thread_local int64_t key_m = -1, key_n = -1;
+  static thread_local MixedPlan cached{0, 0};
+  if (key_m == tiles_m && key_n == N) return cached;
+  const int64_t all_wide = (N + 255) / 256;
+  MixedPlan best{(int)all_wide, 0};
+  double best_t = mixed_makespan(tiles_m * all_wide, 0);
+  for (int64_t narrow = 1; narrow * 192 < N + 192; ++narrow) {
+    const int64_t rest = N - narrow * 192;
+    const int64_t wide = rest > 0 ? (rest + 255) / 256 : 0;
+    if (wide * 256 + (narrow - 1) * 192 >= N) continue;  // the last narrow column would start past the matrix
+    const double t = mixed_makespan(tiles_m * wide, tiles_m * narrow);
+    if (t < best_t - 0.1) {  // a mixed grid has to pay for itself
+      best_t = t;
+      best = MixedPlan{(int)wide, (int)narrow};
+    }
+  }
+  key_m = tiles_m; key_n = N; cached = best;
+  return best;
+}
+
 template <typename T>
 static int finish_splitk(const GemmArgs& g, int nsplit, hipStream_t st) {
   const int64_t quads = (int64_t)g.M * g.ws_ld / 4;
@@ -1823,7 +1990,10 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
     const bool b_nn_ok = b_nn && N % 8 == 0;
     // An M-contiguous left operand (a transposed view) is taken as it is by the four-wave and the
     // 128x128 kernels when its k-rows start on 16-byte boundaries and K is a multiple of 64.
-    const bool a_t = !a_ok && a_rs == 1 && a_cs % 8 == 0 && aligned16(a) && M % 8 == 0 && K % 64 == 0;
+    // The four-wave kernels address their fills with 32-bit byte offsets from a per-tile base:
+    // up to 256 rows of either operand must span less than 4 GB.
+    const bool ld32 = (a_ok ? a_rs : a_cs) < (1 << 22) && (b_nt ? b_cs : b_rs) < (1 << 22);
+    const bool a_t = !a_ok && a_rs == 1 && a_cs % 8 == 0 && aligned16(a) && M % 8 == 0 && K % 64 == 0 && ld32;
     if ((a_ok || a_t) && (b_nt || b_nn_ok) && K % 8 == 0 && fits && worth && K > 0) {
       GemmArgs g{};
       g.a = a; g.b = b; g.c = c; g.out = out;
@@ -1865,7 +2035,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // MI355_GEMM_TILE=256x128 forces it (a test knob).
       const int64_t tiles_mid = (int64_t)g.tiles_m * ((N + 127) / 128);
       const char* forced_tile = getenv("MI355_GEMM_TILE");
-      const bool mid = !ktail && K % 64 == 0 &&
+      const bool mid = !ktail && K % 64 == 0 && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "256x128") == 0
                                                : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > (K >= 2048 ? 228 : 248) && tiles_mid <= kNumCU);
       if (mid) {
@@ -1900,10 +2070,23 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         // Four waves of 128x128 run the steady state 3-5 % faster and pay ~2 us more per tile
         // (two-pass epilogue), which evens out near K = 2048.  MI355_GEMM_WAVES=4|8 forces one form.
         const char* forced = getenv("MI355_GEMM_WAVES");
-        const bool w4 = a_t || (forced != nullptr ? forced[0] == '4' : K >= 2048);  // the eight-wave kernels have no M-contiguous-A form
+        const bool w4 = a_t || (ld32 && (forced != nullptr ? forced[0] == '4' : K >= 2048));  // the eight-wave kernels have no M-contiguous-A form
         if (w4) {
           kern = pick_w4(std::integral_constant<int, 4>{});
           threads = 256;
+          // More than one round of tiles with a ragged last round: cut the last columns into 192-wide tiles.
+          const bool plain = forced_tile != nullptr && strcmp(forced_tile, "256x256") == 0;
+          const bool force_mixed = forced_tile != nullptr && strcmp(forced_tile, "mixed") == 0;  // any K (a test knob)
+          if (nblocks > kNumCU && !plain && (K >= kMixedMinK || force_mixed)) {
+            const MixedPlan mp = plan_mixed(g.tiles_m, N);
+            if (mp.narrow > 0) {
+              g.tiles_n = mp.wide;
+              g.tail_n = mp.narrow;
+              nblocks = (int64_t)g.tiles_m * (mp.wide + mp.narrow);
+              if (a_t) kern = b_nt ? (const void*)gemm_mfma_w4_mixed_kernel<T, false, true> : (const void*)gemm_mfma_w4_mixed_kernel<T, true, true>;
+              else kern = b_nt ? (const void*)gemm_mfma_w4_mixed_kernel<T, false, false> : (const void*)gemm_mfma_w4_mixed_kernel<T, true, false>;
+            }
+          }
         } else {
           kern = b_nt ? (const void*)gemm_mfma_dma64_kernel<T, false> : (const void*)gemm_mfma_dma64_kernel<T, true>;
         }
@@ -1922,6 +2105,9 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         for (const void*& k : attr_done)
           if (k == nullptr) { k = kern; break; }
       }
+#ifdef MI355_GEMM_TRACE
+      if (nsplit == 1) g.ws = workspace_bytes >= nblocks * 4 * 16 * 8 ? static_cast<float*>(workspace) : nullptr;
+#endif
       void* params[] = {&g};
       hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks, (unsigned)nsplit), dim3(threads), params, lds_bytes, st);
       if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma): launch failed: %s", hipGetErrorString(e));
@@ -2016,6 +2202,16 @@ extern "C" int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
   if (dtype != MI355_BF16 && dtype != MI355_F16 && dtype != MI355_F32) return 0;
   const SplitPlan p = plan_splitk(M, N, K, es);
   return p.nsplit > 1 ? (int64_t)p.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
+}
+
+extern "C" int mi355_gemm_tile_columns(int64_t M, int64_t N, int64_t K, int32_t* wide, int32_t* narrow) {
+  MI355_REQUIRE(M > 0 && N > 0 && wide != nullptr && narrow != nullptr, "mi355_gemm_tile_columns: bad argument");
+  const int64_t tiles_m = (M + BM - 1) / BM;
+  MixedPlan mp{(int)((N + BN - 1) / BN), 0};
+  if (tiles_m * mp.wide > kNumCU && K >= kMixedMinK) mp = plan_mixed(tiles_m, N);
+  *wide = mp.wide;
+  *narrow = mp.narrow;
+  return MI355_OK;
 }
 
 extern "C" int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs,

@@ -49,6 +49,12 @@ def parse():
     ap.add_argument("--ops", default="all", help="comma-separated substrings of per-op rows to time, or 'none'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy")
+    ap.add_argument("--variant", type=int, default=0,
+                    help="with --only-op calib.mfma: 0 = the mm kernel's MFMA order, 1 = operands swapped between the "
+                         "ports, 2 = the other operand held across MFMAs, 3 = v_mfma_f32_16x16x32")
+    ap.add_argument("--trace", action="store_true",
+                    help="with --only-op C3.mm_up|C3.mm_down: run the cycle-stamped diagnostic build of the GEMM "
+                         "(libmi355_gemm_trace.so) and print where a tile's shader-clock ticks go")
     ap.add_argument("--fill", default=None, choices=["zeros", "ones", "sign"],
                     help="with --only-op: overwrite the floating-point inputs with zeros, ones or values from "
                          "{-1, 0, 1} (shows how far a kernel's time depends on the data through the power/clock envelope)")
@@ -85,6 +91,12 @@ def main():
     # One op only, timed exactly like its per_op row, so that a profiler's per-kernel average
     # covers the same launches.  "calib.copy" is a plain 128 MiB -> 128 MiB copy with the
     # library's copy kernel (known traffic, for scaling hardware byte counters).
+    if args.only_op == "calib.mfma":
+        print(json.dumps(calib_mfma(dev, args.fill, args.variant)))
+        return
+    if args.only_op and args.trace:
+        print(json.dumps(gemm_trace(by_key[args.only_op], dev, args.fill)))
+        return
     if args.only_op:
         if args.only_op == "calib.copy":
             from backendbench_amd.ops._common import copy_into
@@ -224,6 +236,113 @@ def main():
         "geomean_speedup_vs_cpu": geomean, "per_op": per_op,
     }
     print(json.dumps(line))
+
+
+def calib_mfma(dev, fill=None, variant=0, blocks=256, steps=2752, launches=20):
+    """Sustained rate of the mm kernel's MFMA stream with no memory traffic (mi355_calib_mfma): one
+    workgroup of four waves per CU, each wave a 128 x 128 register tile, `steps` 32-k steps per
+    launch (eight times the K loop of the [4096,11008] x [11008,4096] product).  Operand data as
+    the GEMM configuration prescribes (left N(0,1), right N(0,0.02), bf16) unless `fill` overrides
+    it: what this loop sustains is the ceiling the power / clock envelope leaves a GEMM on that data."""
+    import torch
+
+    from backendbench_amd import _lib
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(0)
+    n = blocks * 256 * 16 * 8  # bf16 elements per operand buffer
+    a = torch.randn(n, generator=g).bfloat16()
+    b = (torch.randn(n, generator=g) * 0.02).bfloat16()
+    if fill == "zeros":
+        a.zero_(), b.zero_()
+    elif fill == "ones":
+        a.fill_(1.0), b.fill_(1.0)
+    elif fill == "sign":
+        a = torch.randint(-1, 2, (n,), generator=g).bfloat16()
+        b = torch.randint(-1, 2, (n,), generator=g).bfloat16()
+    a, b = a.to(dev), b.to(dev)
+    out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    stream = _lib.current_stream_handle()
+
+    def run():
+        _lib.check(lib.mi355_calib_mfma(a.data_ptr(), b.data_ptr(), out.data_ptr(), _lib.BF16, blocks, steps, variant, stream))
+
+    for _ in range(3):
+        run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(launches):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / launches
+    flops = blocks * 4 * steps * 2 * 128 * 128 * 32
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"only_op": "calib.mfma", "variant": variant, "fill": fill or "N(0,1) x N(0,0.02)", "ms": round(ms, 4),
+            "flops": flops, "tflops": round(tf, 1), "frac_of_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+            "timing": f"{launches} launches of {blocks} x 4 waves x {steps} steps, events around the loop"}
+
+
+def gemm_trace(case, dev, fill=None):
+    """One mm of this row through the stamped diagnostic build (see the MI355_GEMM_TRACE block in
+    csrc/gemm.hip for the record layout): mean shader-clock ticks per phase of a tile and per step
+    of the K loop, the gap between two tiles on one CU, and ticks per microsecond of kernel time
+    (the average shader clock, which is what moves with the operand data)."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from backendbench_amd import _build, _lib
+
+    if not _build.TRACE_LIB_PATH.exists():
+        raise RuntimeError(f"{_build.TRACE_LIB_PATH} is missing: python -m backendbench_amd._build --trace")
+    lib = ctypes.CDLL(str(_build.TRACE_LIB_PATH))
+    fn = lib.mi355_gemm
+    fn.restype, fn.argtypes = _lib.SIGNATURES["mi355_gemm"]
+    (a, b), _ = case.make(dev)
+    if fill:
+        for t in (a, b):
+            t.copy_(torch.randint(-1, 2, t.shape, device=dev).to(t.dtype)) if fill == "sign" else t.fill_(0.0 if fill == "zeros" else 1.0)
+    M, K = a.shape
+    N = b.shape[1]
+    out = torch.empty(M, N, dtype=a.dtype, device=dev)
+    ws = torch.zeros(1 << 20, dtype=torch.int64, device=dev)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(3):
+        ws.zero_()
+        e0.record()
+        _lib.check(fn(a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), None, 0, 0,
+                      out.data_ptr(), M, N, K, 1.0, 0.0, _lib.dtype_code(a.dtype), ws.data_ptr(), ws.numel() * 8,
+                      _lib.current_stream_handle()))
+        e1.record()
+        torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3
+    rec = ws.cpu().numpy().reshape(-1, 4, 16)
+    rec = rec[rec[:, 0, 7] > 0]
+    w0 = rec[:, 0, :].astype(np.float64)
+    iters = w0[:, 7]
+    entry, begin, end, drained, stored = w0[:, 12], w0[:, 10], w0[:, 13], w0[:, 14], w0[:, 15]
+    hw = rec[:, 0, 11]
+    cu_key = (np.arange(len(rec)) % 8) * 4096 + (hw & 0xFF00)  # XCD (block % 8), SE / SH / CU bits of HW_ID
+    gaps = []
+    for k in np.unique(cu_key):
+        idx = np.where(cu_key == k)[0]
+        idx = idx[np.argsort(entry[idx])]
+        gaps += list(entry[idx[1:]] - stored[idx[:-1]])
+    per_step = (w0[:, :6] / iters[:, None]).mean(axis=0)
+    names = ["even_issue", "even_fill_wait", "even_barrier", "odd_issue", "odd_fill_wait", "odd_barrier_and_back_edge"]
+    whole = float(np.mean(stored - entry))
+    return {"only_op": case.key, "trace": True, "fill": fill or "as configured", "kernel_us": round(us, 1), "tiles": int(len(rec)),
+            "ticks_per_step_pair": {n: round(float(v), 1) for n, v in zip(names, per_step)},
+            "mfma_ticks_per_step_pair_at_full_rate": 2048,
+            "ticks_per_tile": {"prologue": round(float(np.mean(begin - entry))), "steady_loop": round(float(np.mean(end - begin))),
+                               "remainder_and_drain": round(float(np.mean(drained - end))),
+                               "epilogue_until_stored": round(float(np.mean(stored - drained))), "whole_tile": round(whole)},
+            "ticks_between_tiles_on_a_cu": round(float(np.median(gaps))) if gaps and len(rec) > 256 else None,
+            "rounds_of_tiles": round(len(rec) / 256, 3),
+            "approx_ticks_per_us": round(whole * max(1.0, np.ceil(len(rec) / 256)) / us) if us > 0 else None}
 
 
 def graph_bench(fn, args, kwargs, pool_bytes=768 * 2**20, target_ms=60.0):

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define MI355_ABI_VERSION 4
+#define MI355_ABI_VERSION 6
 #define MI355_MAX_DIMS 8
 
 typedef enum mi355_dtype {
@@ -189,6 +189,25 @@ int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t
                int64_t b_cs, const void* c, int64_t c_rs, int64_t c_cs, void* out,
                int64_t M, int64_t N, int64_t K, double alpha, double beta, int dtype,
                void* workspace, int64_t workspace_bytes, void* stream);
+
+/* How the large-tile bf16 / f16 kernel cuts the N columns of an [M, N] output (K a multiple of 64):
+ * `wide` tile columns of 256 followed by `narrow` tile columns of 192.  narrow > 0 when K >= 4096,
+ * the 256 x 256 tiles make more than one round over the 256 CUs, and cutting the last columns
+ * narrower shortens the ragged last round.  Host-only planning query for tests and documentation;
+ * no counterpart in the reference. */
+int mi355_gemm_tile_columns(int64_t M, int64_t N, int64_t K, int32_t* wide, int32_t* narrow);
+
+/* Measurement only, no counterpart in the reference: the matrix-core instruction stream of the
+ * large-tile mm kernel (per wave a 128 x 128 fp32 register tile, 32 v_mfma_f32_32x32x16 per 32-k
+ * step) with no memory traffic in the loop.  `blocks` workgroups of four waves run `steps` (even)
+ * steps on operand fragments loaded once from a and b (16 fragments of 16 bytes per thread each:
+ * blocks * 65536 bytes; the caller chooses the data), out receives blocks * 256 floats.  Work:
+ * blocks * 4 * steps * 2 * 128 * 128 * 32 flop.  variant 0: the mm kernel's operand order; 1: operands
+ * swapped between the two ports; 2: the other operand held across MFMAs; 3: v_mfma_f32_16x16x32.
+ * Its sustained rate on a given data distribution is the ceiling the power / clock envelope leaves to
+ * mi355_gemm on that data. */
+int mi355_calib_mfma(const void* a, const void* b, void* out, int dtype, int blocks, int steps,
+                     int variant, void* stream);
 
 /* ---- indexing --------------------------------------------------------------------- */
 

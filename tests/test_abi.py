@@ -28,7 +28,7 @@ def header_enum(name):
 def test_header_declares_the_expected_entry_points():
     fns = declared_functions()
     assert "mi355_gemm" in fns and "mi355_softmax" in fns and "mi355_index_select" in fns
-    assert len(fns) == 17
+    assert len(fns) == 19
 
 
 def test_every_declared_symbol_is_exported_and_bound():
@@ -102,3 +102,27 @@ def test_workspace_planners_run_on_the_host():
     assert odd > 0 and odd % (24 * 1004 * 4) == 0
     tiny = lib.mi355_gemm_workspace_bytes(64, 250, 1040, _lib.F32)           # fp32, 64x64 tiles
     assert tiny > 0 and tiny % (64 * 252 * 4) == 0
+
+
+def _tile_columns(M, N, K=4096):
+    import ctypes
+
+    lib = _lib.load()
+    wide, narrow = ctypes.c_int32(), ctypes.c_int32()
+    assert lib.mi355_gemm_tile_columns(M, N, K, ctypes.byref(wide), ctypes.byref(narrow)) == 0
+    return wide.value, narrow.value
+
+
+def test_gemm_tile_column_plan():
+    """256-wide tile columns followed by 192-wide ones when a ragged last round of tiles would idle CUs."""
+    assert _tile_columns(4096, 4096) == (16, 0)            # 256 tiles: exactly one round
+    assert _tile_columns(2048, 2048) == (8, 0)             # fewer tiles than CUs: nothing to balance
+    assert _tile_columns(4096, 11008, 2048) == (43, 0)     # short K loop: the plain grid
+    wide, narrow = _tile_columns(4096, 11008)              # 688 tiles = 2.69 rounds of 256-wide tiles
+    assert narrow > 0 and 16 * wide % 256 == 0             # two full rounds, then one round of narrow tiles
+    assert 16 * narrow <= 256
+    for M, N in [(4096, 11008), (4104, 4500), (8192, 8192), (3000, 50257), (16384, 1000)]:
+        wide, narrow = _tile_columns(M, N)
+        assert wide * 256 + narrow * 192 >= N                                   # the columns cover the output
+        assert narrow == 0 or wide * 256 + (narrow - 1) * 192 < N               # every narrow column starts inside it
+        assert narrow > 0 or (wide - 1) * 256 < N

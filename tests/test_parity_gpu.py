@@ -110,24 +110,18 @@ def test_headline_argmax_full_size(backend):
 
 @pytest.mark.parametrize("key", ["C3.mm_up", "C3.addmm_up", "C3.mm_down", "C3.addmm_down"])
 def test_headline_gemm_full_size(backend, key):
-    """7B-MLP GEMMs at full size.  Row i of the product depends on row i of the left operand
-    only, so the oracle is run on 96 sampled rows (and the first/last rows of every 256-row
-    tile band) instead of all 4096; linearity in alpha is checked on the whole output."""
+    """7B-MLP GEMMs at full size: the whole [4096, N] product against the oracle (ATen on the
+    host CPU runs one of these in about a tenth of a second), then linearity in alpha."""
     announce(key)
     case = next(c for c in PERF if c.key == key)
     args, kwargs = case.make("cuda")
     out = backend[case.op](*args, **kwargs)
     torch.cuda.synchronize()
-    a_pos = 1 if "addmm" in key else 0
-    M = args[a_pos].shape[0]
-    rows = torch.randint(0, M, (96,), generator=torch.Generator().manual_seed(1))
-    rows = torch.unique(torch.cat([rows, torch.arange(0, M, 256), torch.arange(255, M, 256)]))
-    sub = list(args)
-    sub[a_pos] = args[a_pos][rows.cuda()]
-    ref = aten_cpu.reference(case.op, sub, kwargs)
-    got = out[rows.cuda()].cpu()
-    assert got.dtype == ref.dtype and ev.allclose(ref, got), ev.compute_errors(ref, got)
-    assert torch.isfinite(out.float()).all()
+    ref = aten_cpu.reference(case.op, args, kwargs)
+    got = out.cpu()
+    assert got.shape == ref.shape and got.dtype == ref.dtype
+    assert ev.allclose(ref, got), ev.compute_errors(ref, got)
+    assert torch.isfinite(got.float()).all()
     if "addmm" in key:
         doubled = backend[case.op](*args, alpha=2.0, beta=0.0)
         plain = backend[aten.mm.default](args[1], args[2])
@@ -168,6 +162,46 @@ def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch
         bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
         out2 = backend[aten.addmm.default](bias, a, b)
         assert ev.bit_equal((out.float() + bias.float()).to(torch.bfloat16), out2), (layout, K, "bias")
+
+
+@pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
+def test_mixed_width_tile_grid(backend, layout, monkeypatch):
+    """More than one round of 256x256 tiles with a ragged last round: the four-wave kernel cuts the last
+    columns into 192-wide tiles (one launch, two tile widths).  [4104, K] x [K, 4500] has 17 x 18 tiles of
+    256x256; the planner must choose a mixed grid for it, the result must be bit-equal to the plain grid's
+    (same k order per element) and, on small-integer operands, to the oracle's on sampled rows.  Covers the
+    ragged last tile row, the ragged last (narrow) tile column and every K-loop length of the kernel."""
+    import ctypes
+
+    from backendbench_amd import _lib
+    announce(f"mixed-width tile grid, {layout}")
+    M, N = 4104, 4500
+    wide, narrow = ctypes.c_int32(), ctypes.c_int32()
+    assert _lib.load().mi355_gemm_tile_columns(M, N, 4096, ctypes.byref(wide), ctypes.byref(narrow)) == 0
+    assert narrow.value > 0, "this shape is meant to take the mixed grid"
+    monkeypatch.setenv("MI355_GEMM_WAVES", "4")
+    g = torch.Generator().manual_seed(11)
+    edge = wide.value * 256
+    rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 255, 256, 4095, 4096, 4103])]))
+    for K in (64, 128, 192, 256, 320, 384, 448, 512, 576, 1024, 2112, 4096):
+        if layout[0] == "t":
+            a = torch.randint(-1, 2, (K, M), generator=g).to(torch.bfloat16).cuda().t()
+        else:
+            a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+        if layout[1] == "t":
+            b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
+        else:
+            b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
+        bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
+        monkeypatch.setenv("MI355_GEMM_TILE", "mixed")      # the mixed grid whatever K is (by itself: K >= 4096)
+        mixed = backend[aten.addmm.default](bias, a, b)
+        monkeypatch.setenv("MI355_GEMM_TILE", "256x256")
+        plain = backend[aten.addmm.default](bias, a, b)
+        monkeypatch.delenv("MI355_GEMM_TILE")
+        assert ev.bit_equal(plain, mixed), (layout, K)
+        ref = aten_cpu.reference(aten.addmm.default, [bias, a[rows.cuda()], b])
+        assert ev.bit_equal(ref, mixed[rows.cuda()].cpu()), (layout, K)
+        assert ev.bit_equal(ref[:, edge - 8:edge + 200], mixed[rows.cuda()][:, edge - 8:edge + 200].cpu())  # across the seam
 
 
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
