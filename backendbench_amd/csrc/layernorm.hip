@@ -152,6 +152,97 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
   }
 }
 
+// Many rows that each fit one wave's registers (NV slabs of 64 lanes x one 128-bit vector:
+// up to 4096 two-byte or 2048 four-byte elements): every wave walks rows wave, wave + waves, ...
+// with the NEXT row's loads issued before the current row is reduced, so the memory system
+// always holds a row per wave in flight while the reductions and the normalisation run.  One wave
+// per row: both all-reduces stay inside the wave (DPP + bpermute), no barrier in the loop.
+// gamma / beta are staged once per block in LDS (2 n elements of dynamic shared memory).  Same
+// statistics as the tile kernel (mean, then the centred second moment from the registers).
+template <typename T, typename S, int NV, bool HW, bool HB>
+__global__ __launch_bounds__(kLnBlock) __attribute__((amdgpu_waves_per_eu(4, 8))) void layernorm_stream_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                                   const T* __restrict__ b, T* __restrict__ y,
+                                                                   S* __restrict__ mean_out, S* __restrict__ rstd_out,
+                                                                   int64_t rows, int64_t n, float eps) {
+  constexpr int V = Vec<T>::N;
+  extern __shared__ __attribute__((aligned(32))) unsigned char ln_smem[];  // gamma, then beta: 2 n elements
+  T* gl = reinterpret_cast<T*>(ln_smem);
+  T* bl = gl + n;
+  const int lane = threadIdx.x % kWave;
+  const int64_t waves = (int64_t)gridDim.x * (kLnBlock / kWave);
+  int64_t row = (int64_t)blockIdx.x * (kLnBlock / kWave) + threadIdx.x / kWave;
+  bool in[NV];
+  VecN<T, V> nxt[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int64_t c = ((int64_t)k * kWave + lane) * V;
+    in[k] = c < n;  // n % V == 0: a vector is inside the row or past it
+    if (in[k] && row < rows) nxt[k] = ld_nt<T, V>(x + row * n + c);
+  }
+  // gamma / beta once per block into LDS, behind the first row's loads
+  if constexpr (HW || HB) {
+    for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kLnBlock * V) {
+      if constexpr (HW) st<T, V>(gl + c, ld<T, V>(w + c));
+      if constexpr (HB) st<T, V>(bl + c, ld<T, V>(b + c));
+    }
+    __syncthreads();
+  }
+  const float inv_n = 1.f / (float)n;
+  for (; row < rows; row += waves) {
+    float v[NV][V];
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[k][j] = in[k] ? static_cast<float>(nxt[k].v[j]) : 0.f;
+    const int64_t ahead = row + waves;
+    if (ahead < rows) {
+#pragma unroll
+      for (int k = 0; k < NV; ++k)
+        if (in[k]) nxt[k] = ld_nt<T, V>(x + ahead * n + ((int64_t)k * kWave + lane) * V);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int j = 0; j < V; ++j) s += v[k][j];
+    const float mean = wave_allreduce(s, SumOp()) * inv_n;
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+      if (in[k]) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          const float d = v[k][j] - mean;
+          v[k][j] = d;
+          q += d * d;
+        }
+      }
+    const float rstd = rsqrtf(wave_allreduce(q, SumOp()) * inv_n + eps);
+    if (lane == 0) {
+      mean_out[row] = static_cast<S>(mean);
+      rstd_out[row] = static_cast<S>(rstd);
+    }
+    T* out = y + row * n;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+      if (in[k]) {
+        const int64_t c = ((int64_t)k * kWave + lane) * V;
+        VecN<T, V> g, be, r;
+        if constexpr (HW) g = ld<T, V>(gl + c);
+        if constexpr (HB) be = ld<T, V>(bl + c);
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+          float f = v[k][j] * rstd;
+          if constexpr (HW && HB) f = f * static_cast<float>(g.v[j]) + static_cast<float>(be.v[j]);
+          else if constexpr (HW) f *= static_cast<float>(g.v[j]);
+          else if constexpr (HB) f += static_cast<float>(be.v[j]);
+          r.v[j] = static_cast<T>(f);
+        }
+        st_nt<T, V>(out + c, r);
+      }
+  }
+}
+
 // Rows of at most 32 vectors: G = 1 .. 32 lanes per row, 64 / G rows per wave (per-head q/k
 // norms over 64 or 128 elements).  A lane holds one 16-byte vector of its row, or V single
 // elements (column t + G j) when rows are not vector-aligned, and loads the gamma / beta of its
@@ -329,6 +420,41 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
   }
     MI355_LN_SUB(1) MI355_LN_SUB(2) MI355_LN_SUB(4) MI355_LN_SUB(8) MI355_LN_SUB(16) MI355_LN_SUB(32)
 #undef MI355_LN_SUB
+  }
+  // Thousands of aligned rows of one wave's worth of registers each, gamma / beta of the input's
+  // dtype: the streaming kernel (rows prefetched one ahead, no LDS, no barrier).
+  if constexpr (std::is_same<T, W>::value && !std::is_same<T, double>::value)
+  if (!done && vec && N > 32 * V && N <= 8 * kWave * V && M >= 4 * kNumCU) {
+    // Grid: the blocks that are resident at once (the register tile decides how many), cut so
+    // that every wave gets the same number of rows when M allows it.
+    auto launch = [&](auto nv) {
+      constexpr int NV = decltype(nv)::value;
+      auto go = [&](auto hw, auto hb) {
+        constexpr bool HW_ = decltype(hw)::value, HB_ = decltype(hb)::value;
+        const void* kern = (const void*)layernorm_stream_kernel<T, S, NV, HW_, HB_>;
+        static thread_local int resident = 0;  // blocks per CU, per instantiation
+        if (resident == 0) {
+          int nb = 0;
+          if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, kLnBlock, has_params ? param_bytes : 0) != hipSuccess || nb < 1) nb = 2;
+          resident = nb;
+        }
+        const int64_t max_waves = (int64_t)kNumCU * resident * (kLnBlock / kWave);
+        const int64_t per_wave = (M + max_waves - 1) / max_waves;
+        const int64_t nwaves = (M + per_wave - 1) / per_wave;
+        const unsigned nblk = (unsigned)((nwaves + kLnBlock / kWave - 1) / (kLnBlock / kWave));
+        hipLaunchKernelGGL((layernorm_stream_kernel<T, S, NV, HW_, HB_>), dim3(nblk), dim3(kLnBlock), has_params ? param_bytes : 0, st, x,
+                           reinterpret_cast<const T*>(w), reinterpret_cast<const T*>(b), y, mean, rstd, M, N, (float)eps);
+      };
+      using std::true_type;
+      using std::false_type;
+      if (w && b) go(true_type(), true_type());
+      else if (w) go(true_type(), false_type());
+      else if (b) go(false_type(), true_type());
+      else go(false_type(), false_type());
+    };
+    if (N <= 4 * kWave * V) launch(std::integral_constant<int, 4>());
+    else launch(std::integral_constant<int, 8>());
+    done = true;
   }
   // Rows that start off a 16-byte boundary (odd N) still take the vector layout, shifted per
   // row, when input and output rows are misaligned by the same number of elements.  Rows under

@@ -66,6 +66,67 @@ __global__ __launch_bounds__(sm_tile_block(W)) void softmax_tile_kernel(const T*
   else tile.store(y + row * n, n, t, fin);
 }
 
+// Many aligned rows that each fit one wave's registers (NV slabs of 64 lanes x one 128-bit
+// vector: up to 4096 two-byte or 2048 four-byte elements), output of the input's dtype: a wave
+// walks rows wave, wave + waves, ... and issues the next row's loads before it reduces the
+// current one.  One wave per row: max and sum stay inside the wave, no LDS, no barrier.
+template <typename T, int NV, bool LOG>
+__global__ __launch_bounds__(kSmBlock) __attribute__((amdgpu_waves_per_eu(4, 8))) void softmax_stream_kernel(
+    const T* __restrict__ x, T* __restrict__ y, int64_t rows, int64_t n) {
+  constexpr int V = Vec<T>::N;
+  const int lane = threadIdx.x % kWave;
+  const int64_t waves = (int64_t)gridDim.x * (kSmBlock / kWave);
+  int64_t row = (int64_t)blockIdx.x * (kSmBlock / kWave) + threadIdx.x / kWave;
+  bool in[NV];
+  VecN<T, V> nxt[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int64_t c = ((int64_t)k * kWave + lane) * V;
+    in[k] = c < n;  // n % V == 0: a vector is inside the row or past it
+    if (in[k] && row < rows) nxt[k] = ld_nt<T, V>(x + row * n + c);
+  }
+  for (; row < rows; row += waves) {
+    float v[NV][V];
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[k][j] = in[k] ? static_cast<float>(nxt[k].v[j]) : -INFINITY;
+    const int64_t ahead = row + waves;
+    if (ahead < rows) {
+#pragma unroll
+      for (int k = 0; k < NV; ++k)
+        if (in[k]) nxt[k] = ld_nt<T, V>(x + ahead * n + ((int64_t)k * kWave + lane) * V);
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int j = 0; j < V; ++j) m = __builtin_fmaxf(m, v[k][j]);  // a NaN is skipped here and poisons the sum below
+    m = wave_allreduce(m, MaxOp());
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        const float d = v[k][j] - m;
+        const float e = __expf(d);
+        v[k][j] = LOG ? d : e;
+        s += e;
+      }
+    s = wave_allreduce(s, SumOp());
+    const float ls = __logf(s), inv = 1.f / s;
+    T* out = y + row * n;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+      if (in[k]) {
+        VecN<T, V> r;
+#pragma unroll
+        for (int j = 0; j < V; ++j) r.v[j] = static_cast<T>(LOG ? v[k][j] - ls : v[k][j] * inv);
+        st_nt<T, V>(out + ((int64_t)k * kWave + lane) * V, r);
+      }
+  }
+}
+
 // Rows of at most 32 vectors: G = 1 .. 32 lanes per row (the smallest power of two whose lanes,
 // at one 16-byte vector or V single elements each, cover the row), 64 / G rows per wave.  Max
 // and sum meet by DPP inside the 16-lane rows (G = 32: one more exchange across them), so a
@@ -363,6 +424,28 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
   }
     MI355_SM_SUB(1) MI355_SM_SUB(2) MI355_SM_SUB(4) MI355_SM_SUB(8) MI355_SM_SUB(16) MI355_SM_SUB(32)
 #undef MI355_SM_SUB
+  }
+  // Thousands of aligned rows of one wave's worth of registers each, same dtype out: the streaming kernel
+  if constexpr (std::is_same<T, O>::value && !std::is_same<T, double>::value)
+  if (!done && vec && n > 32 * V && n <= 8 * kWave * V && outer >= 4 * kNumCU) {
+    auto go = [&](auto nv) {
+      constexpr int NV = decltype(nv)::value;
+      const void* kern = (const void*)softmax_stream_kernel<T, NV, LOG>;
+      static thread_local int resident = 0;  // blocks per CU, per instantiation
+      if (resident == 0) {
+        int nb = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, kSmBlock, 0) != hipSuccess || nb < 1) nb = 2;
+        resident = nb;
+      }
+      const int64_t max_waves = (int64_t)kNumCU * resident * (kSmBlock / kWave);
+      const int64_t per_wave = (outer + max_waves - 1) / max_waves;
+      const int64_t nwaves = (outer + per_wave - 1) / per_wave;
+      const unsigned nblk = (unsigned)((nwaves + kSmBlock / kWave - 1) / (kSmBlock / kWave));
+      hipLaunchKernelGGL((softmax_stream_kernel<T, NV, LOG>), dim3(nblk), dim3(kSmBlock), 0, st, x, reinterpret_cast<T*>(y), outer, n);
+    };
+    if (n <= 4 * kWave * V) go(std::integral_constant<int, 4>());
+    else go(std::integral_constant<int, 8>());
+    done = true;
   }
   if constexpr (!std::is_same<T, double>::value)  // f64 rows take the block kernel (double accumulation)
   if (!done && outer < (int64_t(1) << 31)) {

@@ -212,6 +212,7 @@ def main():
     want = None if args.ops == "all" else ([] if args.ops == "none" else args.ops.split(","))
     per_op = []
     cpu_times = {}
+    copy_cache = {}
     for case in cases:
         if want is not None and not any(w in case.key for w in want):
             continue
@@ -223,6 +224,9 @@ def main():
         if case.bound == "hbm":
             gbs = case.work / (ms * 1e-3) / 1e9
             row.update(bound="hbm", bytes=int(case.work), gbs=round(gbs, 1), frac=round(gbs / HBM_PEAK_GBS, 4))
+            # what a plain copy of the same number of bytes (half read, half written) reaches, timed the same way
+            copy_ms = copy_ms_for(int(case.work), dev, copy_cache)
+            row.update(copy_ms_same_bytes=round(copy_ms, 5), vs_copy=round(copy_ms / ms, 3))
         else:
             tf = case.work / (ms * 1e-3) / 1e12
             row.update(bound="mfma", flops=int(case.work), tflops=round(tf, 1), frac=round(tf / MFMA_BF16_PEAK_TFLOPS, 4))
@@ -272,6 +276,22 @@ def main():
         "geomean_speedup_vs_cpu": geomean, "per_op": per_op,
     }
     print(json.dumps(line))
+
+
+def copy_ms_for(nbytes, dev, cache):
+    """Mean ms per launch of the library's flat copy kernel moving `nbytes` in total (half read,
+    half written), with graph_bench's recipe: the size-matched ceiling of a memory-bound row
+    (launch ramp and tail included, which dominate rows of a few tens of megabytes)."""
+    import torch
+
+    from backendbench_amd.ops._common import copy_into
+
+    n = max(1024, (nbytes // 2) // 4096 * 1024)  # fp32 elements of the source
+    if n not in cache:
+        src = torch.empty(n, dtype=torch.float32, device=dev).normal_()
+        cache[n] = graph_bench(lambda s: copy_into(torch.empty_like(s), s), [src], {})[0]
+        del src
+    return cache[n]
 
 
 def calib_mfma(dev, fill=None, variant=0, blocks=256, steps=2752, launches=20):
