@@ -1798,7 +1798,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
                                                           const T* __restrict__ B, int64_t b_rs, int64_t b_cs,
                                                           const T* __restrict__ C, int64_t c_rs, int64_t c_cs,
                                                           T* __restrict__ D, int64_t M, int64_t N, int64_t K,
-                                                          float alpha, float beta) {
+                                                          typename std::conditional<std::is_same<T, double>::value, double, float>::type alpha,
+                                                          typename std::conditional<std::is_same<T, double>::value, double, float>::type beta) {
   using Acc = typename std::conditional<std::is_same<T, double>::value, double, float>::type;
   constexpr int GT = 16 * TT, GK = 128 / TT;
   constexpr int PER = GT * GK / 256;  // elements of each operand a thread moves per step
@@ -1845,7 +1846,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
     }
     __syncthreads();
   }
-  const bool use_c = C != nullptr && beta != 0.f;
+  const bool use_c = C != nullptr && beta != Acc(0);  // tested in the accumulation type: a tiny f64 beta still counts
 #pragma unroll
   for (int i = 0; i < TT; ++i) {
     const int64_t m = bm + ty * TT + i;
@@ -1854,8 +1855,8 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
     for (int j = 0; j < TT; ++j) {
       const int64_t n = bn + tx + 16 * j;
       if (n >= N) continue;
-      Acc v = (Acc)alpha * acc[i][j];
-      if (use_c) v += (Acc)beta * static_cast<Acc>(C[m * c_rs + n * c_cs]);
+      Acc v = alpha * acc[i][j];
+      if (use_c) v += beta * static_cast<Acc>(C[m * c_rs + n * c_cs]);
       D[m * N + n] = static_cast<T>(v);
     }
   }
@@ -1890,6 +1891,7 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
     ks = (ks + bk - 1) / bk * bk;
     const int64_t real_ns = (K + ks - 1) / ks;
     if (real_ns != ns) continue;  // this count rounds to one already tried
+    if (K - (ns - 1) * ks < (int64_t)min_steps * bk) continue;  // the last split would fall under the minimum
     const int64_t per_cu = (tiles * ns + kNumCU - 1) / kNumCU;
     double t = (double)per_cu * (per_cu >= 2 ? 0.7 : 1.0) * (double)ks * ns_per_k;
     if (ns > 1) t += 3000.0 + (double)ns * (double)M * (double)N * 8.0 / 4000.0;  // ns; 4 TB/s = 4000 B/ns
@@ -2181,14 +2183,15 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
   const int64_t gt = big ? 128 : 64;
   const int64_t gx = (N + gt - 1) / gt, gy = (M + gt - 1) / gt;
   MI355_REQUIRE(gy < 65536 && gx < (int64_t(1) << 31), "mi355_gemm: generic path needs M < 4M rows");
+  using GA = typename std::conditional<std::is_same<T, double>::value, double, float>::type;  // f64 keeps alpha / beta in f64
   if (big)
     hipLaunchKernelGGL((gemm_generic_kernel<T, 8>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
                        static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
-                       static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (float)alpha, (float)beta);
+                       static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (GA)alpha, (GA)beta);
   else
     hipLaunchKernelGGL((gemm_generic_kernel<T, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
                        static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
-                       static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (float)alpha, (float)beta);
+                       static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (GA)alpha, (GA)beta);
   return check_launch("mi355_gemm(generic)");
 }
 

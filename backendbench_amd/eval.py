@@ -19,7 +19,7 @@ import math
 import time
 import traceback
 from dataclasses import dataclass
-from typing import List, Tuple
+from typing import Optional, List, Tuple
 
 import torch
 
@@ -56,6 +56,13 @@ class PerformanceTestResult:
     error_msg: str = ""
     successfully_ran: bool = False
     test_type: str = "performance"
+    # Roofline columns (not in the reference's record, BackendBench/eval.py:36-46): filled when the
+    # suite's test says how much algorithmic work one call is (the `baseline` suite's headline rows).
+    algorithmic_work: Optional[float] = None   # bytes (bound "hbm") or flop (bound "mfma") per call
+    bound: Optional[str] = None
+    achieved: Optional[float] = None           # GB/s or TFLOP/s at benchmark_time_ms
+    achieved_unit: Optional[str] = None
+    roofline_frac: Optional[float] = None      # achieved / MI355X peak (8 TB/s HBM, 2.5 PFLOP/s dense bf16 MFMA)
 
 
 _EXC_TEMPLATE = """
@@ -226,6 +233,25 @@ def _bench_fn():
     return gpu_bench if torch.cuda.is_available() else cpu_bench
 
 
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def roofline_columns(test, time_ms, on_gpu):
+    """Roofline fields of a performance record from the work the suite's test declares
+    (`test.case.work` / `.bound`); empty when it declares none or the time is not a GPU time."""
+    case = getattr(test, "case", None)
+    work, bound = getattr(case, "work", 0), getattr(case, "bound", None)
+    if not on_gpu or not work or not time_ms or bound not in ("hbm", "mfma"):
+        return {}
+    if bound == "hbm":
+        achieved, unit, peak = work / (time_ms * 1e-3) / 1e9, "GB/s", HBM_PEAK_GBS
+    else:
+        achieved, unit, peak = work / (time_ms * 1e-3) / 1e12, "TFLOP/s", MFMA_BF16_PEAK_TFLOPS
+    return {"algorithmic_work": float(work), "bound": bound, "achieved": achieved, "achieved_unit": unit,
+            "roofline_frac": achieved / peak}
+
+
 def eval_performance(op, impl, tests) -> Tuple[float, List[PerformanceTestResult]]:
     bench = _bench_fn()
     base_times, test_times, results = [], [], []
@@ -246,7 +272,8 @@ def eval_performance(op, impl, tests) -> Tuple[float, List[PerformanceTestResult
             mine = bench(lambda: impl(*args, **kwargs))
             results.append(PerformanceTestResult(op_name=op.__name__, args=args_str, speedup=base / mine,
                                                  benchmark_time_ms=mine, reference_time_ms=base,
-                                                 successfully_ran=True))
+                                                 successfully_ran=True,
+                                                 **roofline_columns(test, mine, bench is gpu_bench)))
         except Exception as exc:
             msg = format_exception(exc, op, args, kwargs, traceback.format_exc())
             results.append(PerformanceTestResult(op_name=op.__name__, args=args_str, speedup=None,

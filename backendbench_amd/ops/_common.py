@@ -74,6 +74,8 @@ _entry = {}
 
 def launch(name, *args):
     """Call one C entry point with the current stream appended; raise on failure."""
+    if _pending:
+        poll_index_errors()
     fn = _entry.get(name)
     if fn is None:
         fn = _entry[name] = getattr(_lib.load(), name)
@@ -136,10 +138,18 @@ def norm_dim(dim, ndim):
 
 # ---- out-of-range indices ----------------------------------------------------------
 # The indexing kernels never dereference a bad index; they zero the output there and set a
-# device flag.  Reading the flag needs a device sync, so by default it is read only when
-# check_index_errors() is called (the evaluator does after every test); set
-# MI355_SYNC_INDEX_CHECK=1 to check after every indexing call, like the CPU kernels do.
+# sticky device flag.  The error then surfaces the way a device-side assert of the stock
+# kernels does, asynchronously and without a device sync:
+#   * after an indexing launch the flag is copied to pinned host memory on the same stream
+#     (one copy in flight at a time) and an event is recorded;
+#   * every later call of any operator of this backend looks at that event; once it has completed
+#     and the flag is set, the call raises IndexError naming the earlier indexing call;
+#   * check_index_errors() synchronises and raises at once (this repository's evaluator calls it
+#     after every test; MI355_SYNC_INDEX_CHECK=1 makes every indexing call do so, which is the
+#     CPU kernels' behaviour at the cost of a device sync per call).
+# Nothing is enqueued while the stream is being captured into a graph.
 _flags = {}
+_pending = []  # [(device key, pinned host int32, event)]: at most one entry per device
 
 
 def index_error_flag(device):
@@ -155,9 +165,45 @@ def sync_index_check():
     return os.environ.get("MI355_SYNC_INDEX_CHECK", "0") == "1"
 
 
-def check_index_errors():
-    """Raise IndexError if any indexing kernel saw an out-of-range index since the last call."""
+def note_index_launch(device):
+    """Called behind every indexing launch: start the asynchronous read-back of the device flag
+    unless one is already in flight for this device or the stream is being captured."""
+    key = device.index if device.index is not None else torch.cuda.current_device()
+    for k, _, _ in _pending:
+        if k == key:
+            return
+    if torch.cuda.is_current_stream_capturing():
+        return
+    host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+    host.copy_(_flags[key], non_blocking=True)
+    done = torch.cuda.Event()
+    done.record()
+    _pending.append((key, host, done))
+
+
+def poll_index_errors():
+    """Non-blocking: raise IndexError if a finished read-back shows that an earlier indexing call of
+    this backend met an out-of-range index.  Called at the start of every operator launch."""
+    if torch.cuda.is_current_stream_capturing():
+        return  # no event queries inside a graph capture; the read-back stays pending
     bad = False
+    for entry in list(_pending):
+        key, host, done = entry
+        if not done.query():
+            continue
+        _pending.remove(entry)
+        if int(host[0]) != 0:
+            bad = True
+            _flags[key].zero_()
+    if bad:
+        raise IndexError("index out of range in self (met by an earlier index_select / embedding / gather call of "
+                         "this backend, whose output was zero-filled at that index)")
+
+
+def check_index_errors():
+    """Synchronise and raise IndexError if any indexing kernel saw an out-of-range index since the last check."""
+    bad = False
+    _pending.clear()
     for f in _flags.values():
         if int(f.item()) != 0:
             bad = True

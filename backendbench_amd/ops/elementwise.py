@@ -143,10 +143,44 @@ def _binary(op, a, b, alpha=1):
     return out
 
 
+def _dense_no_overlap(t):
+    """Every element at its own address and no gaps: strides sorted ascending equal the running product of sizes."""
+    expect = 1
+    for size, stride in sorted(((sz, st) for sz, st in zip(t.shape, t.stride()) if sz != 1), key=lambda p: p[1]):
+        if stride != expect:
+            return False
+        expect *= size
+    return True
+
+
+def _check_inplace_overlap(self, other=None):
+    """ATen's refusals for a written-to tensor (TensorIterator's memory-overlap checks): `self` expanded
+    over a stride-0 dim has several elements at one address; `other` sharing part of self's memory under
+    another layout (x.add_(x.t()), x.add_(x[0])) would be read after it was overwritten."""
+    if self.numel() == 0:
+        return
+    if any(sz > 1 and st == 0 for sz, st in zip(self.shape, self.stride())):
+        raise RuntimeError("unsupported operation: more than one element of the written-to tensor refers to a single "
+                           "memory location. Please clone() the tensor before performing the operation.")
+    if not isinstance(other, torch.Tensor) or other.numel() == 0 or other.device != self.device:
+        return
+    if other.untyped_storage().data_ptr() != self.untyped_storage().data_ptr():
+        return
+    if not (_dense_no_overlap(self) and _dense_no_overlap(other)):
+        return  # ATen calls these "too hard" and lets them through
+    a0, b0 = self.data_ptr(), other.data_ptr()
+    a1, b1 = a0 + self.numel() * self.element_size(), b0 + other.numel() * other.element_size()
+    same_range = a0 == b0 and a1 == b1
+    if (same_range and self.stride() != other.stride()) or (not same_range and a0 < b1 and b0 < a1):
+        raise RuntimeError("unsupported operation: some elements of the input tensor and the written-to tensor refer to "
+                           "a single memory location. Please clone() the tensor before performing the operation.")
+
+
 def _binary_inplace(op, functional, self, other, **kw):
     """self (op)= other: the result type must be castable to self's dtype and broadcasting must
     not change self's shape, as for every ATen in-place overload.  `functional` is the
     out-of-place wrapper, used when the arithmetic dtype differs from self's or self is on the CPU."""
+    _check_inplace_overlap(self, other)
     other = _as_operand(self, other)
     dtype = self.dtype if self.dtype == other.dtype else torch.result_type(self, other)
     full = self.shape if self.shape == other.shape else _broadcast_shape(self.shape, other.shape)
@@ -216,6 +250,9 @@ def minimum(self, other):
     return _binary(_lib.MINIMUM, self, other)
 
 
+_C_NAMES = {torch.uint8: "uint8_t", torch.int8: "int8_t", torch.int16: "int16_t", torch.int32: "int", torch.int64: "int64_t"}
+
+
 def _unary(op, x, out_dtype, bounds=0, lo=None, hi=None, inplace=False):
     x = cast(x, out_dtype)
     out = x if inplace else torch.empty_like(x)  # preserve_format: dense permutations keep their layout
@@ -229,6 +266,13 @@ def _unary(op, x, out_dtype, bounds=0, lo=None, hi=None, inplace=False):
         lo_f = hi_f = 0.0
         lo_i = int(lo) if lo is not None else 0
         hi_i = int(hi) if hi is not None else 0
+        # ATen refuses a bound the tensor's dtype cannot hold (c10::overflows: a negative bound on an
+        # unsigned dtype wraps, down to -max); past that the kernel's narrowing would wrap it silently.
+        info = torch.iinfo(out_dtype)
+        floor = -info.max if info.min == 0 else info.min
+        for bound in (lo_i, hi_i):
+            if not floor <= bound <= info.max:
+                raise RuntimeError(f"value cannot be converted to type {_C_NAMES.get(out_dtype, str(out_dtype))} without overflow")
     launch("mi355_unary", op, _lib.desc(x), bounds, lo_f, hi_f, lo_i, hi_i, _lib.desc(out))
     return out
 
@@ -248,6 +292,7 @@ def relu(self):
 def relu_(self):
     """aten.relu_.default"""
     _check_relu_dtype(self)
+    _check_inplace_overlap(self)
     if not _is_gpu_tensor(self):
         return copy_into_any(self, relu(self))
     _unary(_lib.RELU, self, self.dtype, inplace=True)
@@ -283,6 +328,7 @@ def clamp_(self, min=None, max=None):
     """aten.clamp_.default"""
     if min is None and max is None:
         raise RuntimeError("torch.clamp: At least one of 'min' or 'max' must not be None")
+    _check_inplace_overlap(self)
     dtype = _clamp_dtype(self, (min, max))
     if not torch.can_cast(dtype, self.dtype):
         raise RuntimeError(f"result type {str(dtype).replace('torch.', '').capitalize()} can't be cast to the "

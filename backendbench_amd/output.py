@@ -2,7 +2,9 @@
 
 Writes the same four files, with the same fields, as BackendBench/output.py:116-288:
 full_results.json (every test result, sorted by op then args), operator_summary.csv (one
-row per operator), failed_tests.json and OVERALL_SUMMARY.md.
+row per operator), failed_tests.json and OVERALL_SUMMARY.md.  Beyond the reference's fields,
+performance records and operator rows carry roofline columns (algorithmic_work, bound,
+achieved, achieved_unit, roofline_frac) when the suite declares the work of a timed case.
 """
 
 import csv
@@ -53,6 +55,18 @@ def prepare_results(correctness_results, performance_results):
             "max_absolute_error": max((e[0] for e in errs), default=0.0),
             "max_relative_error": max((e[1] for e in errs), default=0.0),
         }
+        # Roofline columns, beyond the reference's (BackendBench/output.py:151-176): present when the
+        # suite declared the algorithmic work of its timed cases.  With several timed cases the row
+        # carries the one with the most work (the headline shape).
+        roof = [r for r in ps if r.successfully_ran and getattr(r, "roofline_frac", None) is not None]
+        top = max(roof, key=lambda r: r.algorithmic_work) if roof else None
+        summaries[op_name].update({
+            "algorithmic_work": top.algorithmic_work if top else "",
+            "bound": top.bound if top else "",
+            "achieved": top.achieved if top else "",
+            "achieved_unit": top.achieved_unit if top else "",
+            "roofline_frac": top.roofline_frac if top else "",
+        })
     failed = sorted([asdict(r) for r in correctness_results if not r.is_correct]
                     + [asdict(r) for r in performance_results if not r.successfully_ran], key=order)
     return all_results, failed, summaries

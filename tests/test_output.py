@@ -30,7 +30,35 @@ def test_prepare_results():
     assert summary["relu.default"]["passed_performance_tests"] == 0 and summary["relu.default"]["geomean_speedup"] == 0.0
     assert list(s) == ["operator", "total_tests", "correctness_tests", "performance_tests", "passed_correctness_tests",
                        "passed_performance_tests", "failed_correctness_tests", "failed_performance_tests",
-                       "correctness_rate", "avg_speedup", "geomean_speedup", "max_absolute_error", "max_relative_error"]
+                       "correctness_rate", "avg_speedup", "geomean_speedup", "max_absolute_error", "max_relative_error",
+                       "algorithmic_work", "bound", "achieved", "achieved_unit", "roofline_frac"]
+    assert s["roofline_frac"] == "" and s["bound"] == ""       # no declared work: the columns stay empty
+
+
+def test_roofline_columns():
+    """Records of timed cases whose suite declares their algorithmic work carry GB/s or TFLOP/s and the
+    fraction of the MI355X peak; the operator row takes the case with the most work."""
+    from types import SimpleNamespace
+
+    from backendbench_amd.eval import roofline_columns
+
+    hbm = SimpleNamespace(case=SimpleNamespace(work=134217728.0, bound="hbm"))
+    cols = roofline_columns(hbm, 0.024, True)
+    assert cols["achieved_unit"] == "GB/s" and abs(cols["achieved"] - 134217728 / 0.024e-3 / 1e9) < 1e-6
+    assert abs(cols["roofline_frac"] - cols["achieved"] / 8000.0) < 1e-12
+    mfma = SimpleNamespace(case=SimpleNamespace(work=369367187456.0, bound="mfma"))
+    cols = roofline_columns(mfma, 0.25, True)
+    assert cols["achieved_unit"] == "TFLOP/s" and abs(cols["achieved"] - 1477.468749824) < 1e-6
+    assert abs(cols["roofline_frac"] - 1477.468749824 / 2500.0) < 1e-9
+    assert roofline_columns(hbm, 0.024, False) == {}           # CPU timings (seconds, not a GPU rate)
+    assert roofline_columns(SimpleNamespace(), 0.024, True) == {}
+    p = [PerformanceTestResult("mm.default", "small", 1.5, 0.01, 0.015, successfully_ran=True,
+                               **roofline_columns(SimpleNamespace(case=SimpleNamespace(work=1e9, bound="mfma")), 0.01, True)),
+         PerformanceTestResult("mm.default", "big", 1.2, 0.25, 0.3, successfully_ran=True, **cols)]
+    _, _, summary = prepare_results([], p)
+    row = summary["mm.default"]
+    assert row["algorithmic_work"] == 369367187456.0 and row["bound"] == "mfma" and row["achieved_unit"] == "TFLOP/s"
+    assert abs(row["roofline_frac"] - 0.5909874999296) < 1e-9
 
 
 def test_summary_rows_and_text():

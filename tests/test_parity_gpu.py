@@ -231,6 +231,40 @@ def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
         assert ev.bit_equal(ref, out[rows.cuda()].cpu()), (layout, shape, K)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_split_k_with_ragged_k(backend, dtype):
+    """One-tile outputs split along K where K is not a multiple of the split length (K = 672, 544, 416
+    at M = N = 64, plus a 100 x 70 output): every split, the last one included, must cover its own k
+    range exactly.  Small-integer operands: bit-equal to the oracle whatever the order of the partial sums."""
+    from backendbench_amd import _lib
+    announce(f"split-K with ragged K, {dtype}")
+    assert _lib.load().mi355_gemm_workspace_bytes(64, 64, 672, _lib.dtype_code(dtype)) > 0   # the planner does split these
+    g = torch.Generator().manual_seed(9)
+    for M, N, K in [(64, 64, 672), (64, 64, 544), (64, 64, 416), (64, 64, 1184), (100, 70, 928), (64, 64, 4000)]:
+        for nt in (False, True):
+            a = torch.randint(-1, 2, (M, K), generator=g).to(dtype).cuda()
+            b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t() if nt else torch.randint(-1, 2, (K, N + (-N) % 8), generator=g).to(dtype).cuda()
+            out = backend[aten.mm.default](a, b)
+            ref = aten_cpu.reference(aten.mm.default, [a, b])
+            assert ev.bit_equal(ref, out.cpu()), (M, N, K, nt)
+
+
+def test_f64_addmm_keeps_alpha_and_beta_in_f64(backend):
+    """alpha = 0.1 and beta = 0.3 are not fp32 numbers: an f64 addmm must apply them in f64 (1e-12
+    against the oracle, where an fp32 round trip of the scalars leaves 1e-8), and a beta too small for
+    fp32 must still count."""
+    announce("f64 addmm scalars")
+    g = torch.Generator().manual_seed(10)
+    c = torch.randn(37, 29, generator=g, dtype=torch.float64)
+    a = torch.randn(37, 53, generator=g, dtype=torch.float64)
+    b = torch.randn(53, 29, generator=g, dtype=torch.float64)
+    got = backend[aten.addmm.default](c.cuda(), a.cuda(), b.cuda(), beta=0.3, alpha=0.1).cpu()
+    ref = aten_cpu.reference(aten.addmm.default, [c, a, b], {"beta": 0.3, "alpha": 0.1})
+    assert torch.allclose(got, ref, rtol=1e-12, atol=1e-12), (got - ref).abs().max()
+    tiny = backend[aten.addmm.default](c.cuda() * 1e60, a.cuda(), b.cuda(), beta=1e-60, alpha=0.0).cpu()
+    assert torch.allclose(tiny, c, rtol=1e-12, atol=1e-12)
+
+
 @pytest.mark.parametrize("layout", ["nn", "nt"])
 @pytest.mark.parametrize("shape", [(200, 330), (1700, 1752), (2100, 2064)])
 def test_fp32_gemm_every_k_loop_length(backend, layout, shape):
@@ -266,6 +300,36 @@ def test_cpu_tensors_round_trip_through_the_gpu(backend):
     assert y.device.type == "cpu"
     outs = backend[aten.native_layer_norm.default](x, [7], None, None, 1e-5)
     assert all(o.device.type == "cpu" for o in outs)
+
+
+def test_out_of_range_index_surfaces_without_an_evaluator(backend, monkeypatch):
+    """A caller that never polls (the reference's evaluator, a live model under enable()): the call with
+    the bad index returns (its row zero-filled, nothing dereferenced), and once the device has run it the
+    next call of any operator of this backend raises IndexError, as a device-side assert of the stock
+    kernels would surface at a later call.  After the raise the backend is clean again."""
+    from backendbench_amd.ops import check_index_errors
+
+    announce("deferred out-of-range index error")
+    monkeypatch.delenv("MI355_SYNC_INDEX_CHECK", raising=False)
+    check_index_errors()
+    table = torch.randn(11, 6, device="cuda")
+    idx = torch.tensor([2, 11, 4], device="cuda")
+    got = backend[aten.index_select.default](table, 0, idx)          # does not raise
+    torch.cuda.synchronize()
+    assert ev.bit_equal(got[0], table[2]) and ev.bit_equal(got[2], table[4])
+    assert torch.count_nonzero(got[1]).item() == 0                       # the bad row is zero-filled
+    with pytest.raises(IndexError, match="earlier index_select / embedding / gather"):
+        backend[aten.relu.default](table)                                # any later call reports it
+    assert ev.bit_equal(backend[aten.relu.default](table).cpu(), torch.relu(table).cpu())   # clean again
+    got = backend[aten.gather.default](table, 1, torch.tensor([[7]], device="cuda"))
+    torch.cuda.synchronize()
+    with pytest.raises(IndexError):
+        backend[aten.embedding.default](table, torch.tensor([1], device="cuda"))
+    good = backend[aten.embedding.default](table, torch.tensor([1], device="cuda"))
+    torch.cuda.synchronize()
+    backend[aten.relu.default](table)                                    # nothing pending: no raise
+    assert ev.bit_equal(good, table[1:2])
+    check_index_errors()
 
 
 def test_error_behaviour_matches_the_oracle(backend, monkeypatch):
@@ -461,6 +525,34 @@ def test_inplace_overloads_reject_what_aten_rejects(backend):
         with pytest.raises(expected):
             backend[op](*args)
     assert torch.equal(ints.cpu(), torch.arange(6))   # nothing was written
+    # memory overlap between the written-to tensor and an operand, or inside the written-to tensor
+    def overlap_cases(dev):
+        sq = torch.arange(9.0, device=dev).reshape(3, 3)
+        return [(aten.add_.Tensor, lambda: [sq.clone(), None], "t"), (aten.add_.Tensor, lambda: [sq.clone(), None], "row"),
+                (aten.mul_.Tensor, lambda: [torch.ones(3, device=dev).expand(2, 3), torch.ones(2, 3, device=dev)], None),
+                (aten.relu_.default, lambda: [torch.ones(3, device=dev).expand(2, 3)], None),
+                (aten.clamp_.default, lambda: [torch.ones(3, device=dev).expand(2, 3), 0.0, 0.5], None)]
+    for (op, mk, view), (_, mk_cpu, _v) in zip(overlap_cases("cuda"), overlap_cases("cpu")):
+        def fill(args):
+            if view == "t": args[1] = args[0].t()
+            if view == "row": args[1] = args[0][0]
+            return args
+        expected = aten_cpu.raises(op, fill(mk_cpu()))
+        assert expected is RuntimeError, (op, view)
+        with pytest.raises(RuntimeError, match="single memory location"):
+            backend[op](*fill(mk()))
+    x = torch.arange(9.0, device="cuda").reshape(3, 3)
+    assert ev.bit_equal(backend[aten.add_.Tensor](x, x).cpu(), torch.arange(9.0).reshape(3, 3) * 2)   # full overlap is fine
+    # integer clamp bounds the dtype cannot hold (a negative bound on uint8 wraps, as in ATen)
+    for dtype, kw in ((torch.int8, {"max": 300}), (torch.uint8, {"min": -5}), (torch.uint8, {"min": -300}), (torch.int16, {"min": -40000}),
+                      (torch.uint8, {"max": 256})):
+        t = torch.arange(0, 100, 7).to(dtype)
+        expected = aten_cpu.raises(aten.clamp.default, [t], kw)
+        if expected is None:
+            assert ev.bit_equal(aten.clamp.default(t, **kw), backend[aten.clamp.default](t.cuda(), **kw).cpu()), (dtype, kw)
+        else:
+            with pytest.raises(expected, match="without overflow"):
+                backend[aten.clamp.default](t.cuda(), **kw)
 
 
 def _out_cases():
