@@ -13,7 +13,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi355_aten.so"
-ABI_VERSION = 6
+ABI_VERSION = 7
 MAX_DIMS = 8
 
 # mi355_dtype
@@ -74,11 +74,13 @@ SIGNATURES = {
         c_int,
         [c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p],
     ),
-    "mi355_softmax": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "mi355_row_workspace_bytes": (c_int64, [c_int64, c_int64, c_int]),
+    "mi355_softmax": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p, c_int64,
+                              c_void_p]),
     "mi355_layer_norm": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
-         c_double, c_void_p],
+         c_double, c_void_p, c_int64, c_void_p],
     ),
     "mi355_gemm_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int]),
     "mi355_gemm": (

@@ -183,6 +183,33 @@ __device__ __forceinline__ T block_allreduce(T v, Op op, T* smem, T identity) {
   return r;
 }
 
+// ---------------------------------------------------------------- few, very long rows
+// Softmax and layer norm over a handful of rows of tens of thousands of elements and more leave
+// the chip idle at one block per row.  Such rows are cut into `nsplit` chunks of `chunk` elements
+// (a multiple of 256 vectors): a first launch leaves one partial state per (row, chunk) in the
+// caller's workspace (kRowPartialBytes each), a second combines a row's partials and writes its
+// chunk of the output.  nsplit == 1: not worth splitting.
+constexpr int kRowPartialBytes = 24;
+struct RowSplit {
+  int64_t nsplit, chunk;
+};
+inline RowSplit plan_row_split(int64_t rows, int64_t n, int elem_size) {
+  RowSplit p{1, n};
+  const int64_t unit = 256 * (16 / elem_size);  // one vector per thread of a 256-thread block
+  if (rows <= 0 || rows >= 64 || n < 32768 || n < 8 * unit) return p;
+  int64_t ns = (2 * kNumCU + rows - 1) / rows;
+  const int64_t max_ns = n / (4 * unit);  // at least four vectors per thread and chunk
+  if (ns > max_ns) ns = max_ns;
+  if (ns > 256) ns = 256;
+  if (ns <= 1) return p;
+  int64_t chunk = (n + ns - 1) / ns;
+  chunk = (chunk + unit - 1) / unit * unit;
+  p.chunk = chunk;
+  p.nsplit = (n + chunk - 1) / chunk;
+  if (p.nsplit <= 1) p = RowSplit{1, n};
+  return p;
+}
+
 // ---------------------------------------------------------------- strided views
 // Up to MI355_MAX_DIMS collapsed dims shared by `NT` tensors; passed to kernels by value.
 template <int NT> struct Dims {

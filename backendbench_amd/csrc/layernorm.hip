@@ -391,9 +391,90 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_block_kernel(const T* __re
   }
 }
 
+// Few, very long rows (plan_row_split): blockIdx.x = chunk, blockIdx.y = row.  Pass 1 leaves the
+// Welford state of every chunk in the workspace; pass 2 merges the states of its row (Chan),
+// writes mean / rstd (chunk 0) and normalises its chunk.  VEC: x and y rows 16-byte aligned and
+// N a multiple of the vector width; gamma / beta are indexed by element (they stay in cache).
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kLnBlock) void layernorm_split_partial_kernel(const T* __restrict__ x, unsigned char* __restrict__ ws,
+                                                                          int64_t n, int64_t chunk) {
+  using A = typename LnAcc<T>::type;
+  constexpr int V = Vec<T>::N;
+  __shared__ WF<A> smem[kLnBlock / kWave];
+  const T* row = x + (int64_t)blockIdx.y * n;
+  const int64_t c0 = (int64_t)blockIdx.x * chunk, c1 = c0 + chunk < n ? c0 + chunk : n;
+  WF<A> a{A(0), A(0), A(0)};
+  if constexpr (VEC) {
+    for (int64_t c = c0 + (int64_t)threadIdx.x * V; c < c1; c += (int64_t)kLnBlock * V) {
+      const Vec<T> t = load_vec(row + c);
+#pragma unroll
+      for (int j = 0; j < V; ++j) wf_update(a, static_cast<A>(t.v[j]));
+    }
+  } else {
+    for (int64_t c = c0 + threadIdx.x; c < c1; c += kLnBlock) wf_update(a, static_cast<A>(row[c]));
+  }
+  a = wf_wave_reduce(a);
+  if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = a;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    a = smem[0];
+#pragma unroll
+    for (int k = 1; k < kLnBlock / kWave; ++k) a = wf_merge(a, smem[k]);
+    *reinterpret_cast<WF<A>*>(ws + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * kRowPartialBytes) = a;
+  }
+}
+
+template <typename T, typename W, typename S, bool VEC>
+__global__ __launch_bounds__(kLnBlock) void layernorm_split_finish_kernel(const T* __restrict__ x, const W* __restrict__ w,
+                                                                         const W* __restrict__ b, T* __restrict__ y,
+                                                                         S* __restrict__ mean_out, S* __restrict__ rstd_out,
+                                                                         const unsigned char* __restrict__ ws, int64_t n,
+                                                                         int64_t chunk, float eps) {
+  using A = typename LnAcc<T>::type;
+  constexpr int V = Vec<T>::N;
+  __shared__ WF<A> smem[kLnBlock / kWave];
+  WF<A> a{A(0), A(0), A(0)};
+  for (int sp = threadIdx.x; sp < (int)gridDim.x; sp += kLnBlock)
+    a = wf_merge(a, *reinterpret_cast<const WF<A>*>(ws + ((int64_t)blockIdx.y * gridDim.x + sp) * kRowPartialBytes));
+  a = wf_wave_reduce(a);
+  if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = a;
+  __syncthreads();
+  a = smem[0];
+#pragma unroll
+  for (int k = 1; k < kLnBlock / kWave; ++k) a = wf_merge(a, smem[k]);
+  const A mean = a.mean;
+  A rstd;
+  if constexpr (std::is_same<A, double>::value) rstd = 1.0 / sqrt(a.m2 / (double)n + (double)eps);
+  else rstd = rsqrtf(a.m2 / (float)n + eps);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    mean_out[blockIdx.y] = static_cast<S>(mean);
+    rstd_out[blockIdx.y] = static_cast<S>(rstd);
+  }
+  const T* row = x + (int64_t)blockIdx.y * n;
+  T* out = y + (int64_t)blockIdx.y * n;
+  const int64_t c0 = (int64_t)blockIdx.x * chunk, c1 = c0 + chunk < n ? c0 + chunk : n;
+  auto norm = [&](A v, int64_t c) {
+    A r = (v - mean) * rstd;
+    if (w) r *= static_cast<A>(w[c]);
+    if (b) r += static_cast<A>(b[c]);
+    return r;
+  };
+  if constexpr (VEC) {
+    for (int64_t c = c0 + (int64_t)threadIdx.x * V; c < c1; c += (int64_t)kLnBlock * V) {
+      const Vec<T> t = load_vec(row + c);
+      VecN<T, V> r;
+#pragma unroll
+      for (int j = 0; j < V; ++j) r.v[j] = static_cast<T>(norm(static_cast<A>(t.v[j]), c + j));
+      st<T, V>(out + c, r);
+    }
+  } else {
+    for (int64_t c = c0 + threadIdx.x; c < c1; c += kLnBlock) out[c] = static_cast<T>(norm(static_cast<A>(row[c]), c));
+  }
+}
+
 template <typename T, typename W, typename S>
 static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void* mv, void* rv, int64_t M,
-                  int64_t N, double eps, hipStream_t st) {
+                  int64_t N, double eps, void* ws, int64_t ws_bytes, hipStream_t st) {
   const T* x = static_cast<const T*>(xv);
   const W* w = static_cast<const W*>(wv);
   const W* b = static_cast<const W*>(bv);
@@ -408,6 +489,23 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
   MI355_REQUIRE(M < (int64_t(1) << 31), "mi355_layer_norm: too many rows (%lld)", (long long)M);
   const size_t param_bytes = 2 * (size_t)N * sizeof(W);
   bool done = false;
+  // few, very long rows: two launches over (row, chunk) when the caller brought the scratch for it
+  {
+    const RowSplit sp = plan_row_split(M, N, sizeof(T));
+    if (sp.nsplit > 1 && ws != nullptr && ws_bytes >= M * sp.nsplit * kRowPartialBytes && reinterpret_cast<uintptr_t>(ws) % 8 == 0) {
+      unsigned char* wsp = static_cast<unsigned char*>(ws);
+      const dim3 grid((unsigned)sp.nsplit, (unsigned)M);
+      const bool xv16 = N % V == 0 && aligned16(x) && aligned16(y);
+      if (xv16) {
+        hipLaunchKernelGGL((layernorm_split_partial_kernel<T, true>), grid, dim3(kLnBlock), 0, st, x, wsp, N, sp.chunk);
+        hipLaunchKernelGGL((layernorm_split_finish_kernel<T, W, S, true>), grid, dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, wsp, N, sp.chunk, (float)eps);
+      } else {
+        hipLaunchKernelGGL((layernorm_split_partial_kernel<T, false>), grid, dim3(kLnBlock), 0, st, x, wsp, N, sp.chunk);
+        hipLaunchKernelGGL((layernorm_split_finish_kernel<T, W, S, false>), grid, dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, wsp, N, sp.chunk, (float)eps);
+      }
+      return check_launch("mi355_layer_norm(split rows)");
+    }
+  }
   if constexpr (!std::is_same<T, double>::value)
   if (N <= 32 * V) {  // short rows: several per wave
     const int64_t need = (N + V - 1) / V;
@@ -503,11 +601,14 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
   return check_launch("mi355_layer_norm");
 }
 
+static thread_local void* g_ln_ws = nullptr;
+static thread_local int64_t g_ln_ws_bytes = 0;
+
 template <typename T, typename W>
 static int run_ln_stat(int stat_dtype, int dtype, const void* x, const void* w, const void* b, void* y, void* m,
                        void* r, int64_t M, int64_t N, double eps, hipStream_t st) {
-  if (stat_dtype == MI355_F32) return run_ln<T, W, float>(x, w, b, y, m, r, M, N, eps, st);
-  if (stat_dtype == dtype) return run_ln<T, W, T>(x, w, b, y, m, r, M, N, eps, st);
+  if (stat_dtype == MI355_F32) return run_ln<T, W, float>(x, w, b, y, m, r, M, N, eps, g_ln_ws, g_ln_ws_bytes, st);
+  if (stat_dtype == dtype) return run_ln<T, W, T>(x, w, b, y, m, r, M, N, eps, g_ln_ws, g_ln_ws_bytes, st);
   return set_error(MI355_ERR_UNSUPPORTED, "mi355_layer_norm: stat dtype must be f32 or the input dtype");
 }
 
@@ -517,7 +618,9 @@ using namespace mi355;
 
 extern "C" int mi355_layer_norm(const void* x, int dtype, const void* weight, const void* bias, int w_dtype,
                                 void* y, void* mean, void* rstd, int stat_dtype, int64_t M, int64_t N, double eps,
-                                void* stream) {
+                                void* workspace, int64_t workspace_bytes, void* stream) {
+  g_ln_ws = workspace;
+  g_ln_ws_bytes = workspace_bytes;
   MI355_REQUIRE(M >= 0 && N > 0, "mi355_layer_norm: bad extents M=%lld N=%lld", (long long)M, (long long)N);
   if (M == 0) return MI355_OK;
   MI355_REQUIRE(x && y && mean && rstd, "mi355_layer_norm: NULL data pointer");

@@ -285,6 +285,72 @@ __global__ __launch_bounds__(BLOCK) void softmax_block_kernel(const T* __restric
   }
 }
 
+// Few, very long rows (plan_row_split): blockIdx.x = chunk, blockIdx.y = row.  Pass 1 leaves the
+// (max, sum) pair of every chunk in the workspace; pass 2 combines the pairs of its row and writes
+// its chunk.  VEC: rows 16-byte aligned and n a multiple of the vector width.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kSmBlock) void softmax_split_partial_kernel(const T* __restrict__ x, unsigned char* __restrict__ ws,
+                                                                        int64_t n, int64_t chunk) {
+  using A = typename SmAcc<T>::type;
+  constexpr int V = Vec<T>::N;
+  __shared__ MS<A> smem[kSmBlock / kWave];
+  const T* row = x + (int64_t)blockIdx.y * n;
+  const int64_t c0 = (int64_t)blockIdx.x * chunk, c1 = c0 + chunk < n ? c0 + chunk : n;
+  MS<A> acc{-INFINITY, A(0)};
+  if constexpr (VEC) {
+    for (int64_t c = c0 + (int64_t)threadIdx.x * V; c < c1; c += (int64_t)kSmBlock * V) {
+      const Vec<T> t = load_vec(row + c);
+#pragma unroll
+      for (int j = 0; j < V; ++j) ms_update(acc, static_cast<A>(t.v[j]));
+    }
+  } else {
+    for (int64_t c = c0 + threadIdx.x; c < c1; c += kSmBlock) ms_update(acc, static_cast<A>(row[c]));
+  }
+  acc = ms_wave_reduce(acc);
+  if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    acc = smem[0];
+#pragma unroll
+    for (int w = 1; w < kSmBlock / kWave; ++w) acc = ms_combine(acc, smem[w]);
+    *reinterpret_cast<MS<A>*>(ws + ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * kRowPartialBytes) = acc;
+  }
+}
+
+template <typename T, typename O, bool VEC, bool LOG>
+__global__ __launch_bounds__(kSmBlock) void softmax_split_finish_kernel(const T* __restrict__ x, O* __restrict__ y,
+                                                                       const unsigned char* __restrict__ ws, int64_t n,
+                                                                       int64_t chunk) {
+  using A = typename SmAcc<T>::type;
+  constexpr int V = Vec<T>::N;
+  __shared__ MS<A> smem[kSmBlock / kWave];
+  MS<A> acc{-INFINITY, A(0)};
+  for (int sp = threadIdx.x; sp < (int)gridDim.x; sp += kSmBlock)
+    acc = ms_combine(acc, *reinterpret_cast<const MS<A>*>(ws + ((int64_t)blockIdx.y * gridDim.x + sp) * kRowPartialBytes));
+  acc = ms_wave_reduce(acc);
+  if (threadIdx.x % kWave == 0) smem[threadIdx.x / kWave] = acc;
+  __syncthreads();
+  acc = smem[0];
+#pragma unroll
+  for (int w = 1; w < kSmBlock / kWave; ++w) acc = ms_combine(acc, smem[w]);
+  const A m = acc.m, inv = A(1) / acc.s, ls = sm_log(acc.s);
+  auto fin = [=](A v) { return LOG ? (v - m) - ls : sm_exp(v - m) * inv; };
+  const T* row = x + (int64_t)blockIdx.y * n;
+  O* out = y + (int64_t)blockIdx.y * n;
+  const int64_t c0 = (int64_t)blockIdx.x * chunk, c1 = c0 + chunk < n ? c0 + chunk : n;
+  if constexpr (VEC) {
+    for (int64_t c = c0 + (int64_t)threadIdx.x * V; c < c1; c += (int64_t)kSmBlock * V) {
+      const Vec<T> t = load_vec(row + c);
+      VecN<O, V> r;
+#pragma unroll
+      for (int j = 0; j < V; ++j) r.v[j] = static_cast<O>(fin(static_cast<A>(t.v[j])));
+      st<O, V>(out + c, r);
+    }
+  } else {
+    for (int64_t c = c0 + threadIdx.x; c < c1; c += kSmBlock) out[c] = static_cast<O>(fin(static_cast<A>(row[c])));
+  }
+}
+
 template <typename T, typename O, bool LOG>
 __global__ __launch_bounds__(kSmBlock) void softmax_cols_kernel(const T* __restrict__ x, O* __restrict__ y,
                                                                int64_t outer, int64_t n, int64_t inner) {
@@ -371,7 +437,8 @@ __global__ __launch_bounds__(kWave * kSmColsR) void softmax_cols_vec_kernel(cons
 }
 
 template <typename T, typename O, bool LOG>
-static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64_t inner, hipStream_t st) {
+static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64_t inner, void* ws, int64_t ws_bytes,
+                       hipStream_t st) {
   const T* x = static_cast<const T*>(xv);
   O* y = static_cast<O*>(yv);
   constexpr int V = Vec<T>::N;
@@ -411,6 +478,22 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
                               : (!tvec && (reinterpret_cast<uintptr_t>(x) / sizeof(T)) % TV ==
                                               (reinterpret_cast<uintptr_t>(y) / sizeof(O)) % TV);
   bool done = false;
+  // few, very long rows: two launches over (row, chunk) when the caller brought the scratch for it
+  {
+    const RowSplit sp = plan_row_split(outer, n, sizeof(T));
+    if (sp.nsplit > 1 && ws != nullptr && ws_bytes >= outer * sp.nsplit * kRowPartialBytes && reinterpret_cast<uintptr_t>(ws) % 8 == 0) {
+      unsigned char* w = static_cast<unsigned char*>(ws);
+      const dim3 grid((unsigned)sp.nsplit, (unsigned)outer);
+      if (vec) {
+        hipLaunchKernelGGL((softmax_split_partial_kernel<T, true>), grid, dim3(kSmBlock), 0, st, x, w, n, sp.chunk);
+        hipLaunchKernelGGL((softmax_split_finish_kernel<T, O, true, LOG>), grid, dim3(kSmBlock), 0, st, x, y, w, n, sp.chunk);
+      } else {
+        hipLaunchKernelGGL((softmax_split_partial_kernel<T, false>), grid, dim3(kSmBlock), 0, st, x, w, n, sp.chunk);
+        hipLaunchKernelGGL((softmax_split_finish_kernel<T, O, false, LOG>), grid, dim3(kSmBlock), 0, st, x, y, w, n, sp.chunk);
+      }
+      return check_launch("mi355_softmax(split rows)");
+    }
+  }
   if constexpr (!std::is_same<T, double>::value)
   if (n <= 32 * V && outer < (int64_t(1) << 31)) {
     // short rows: several per wave
@@ -483,13 +566,27 @@ static int run_softmax(const void* xv, void* yv, int64_t outer, int64_t n, int64
 
 using namespace mi355;
 
+// File-scope so that the dispatch below stays one line per dtype pair.
+static thread_local void* g_sm_ws = nullptr;
+static thread_local int64_t g_sm_ws_bytes = 0;
+
 template <typename T, typename O>
 static int run_softmax_any(int log_softmax, const void* x, void* y, int64_t outer, int64_t dim, int64_t inner, hipStream_t st) {
-  return log_softmax ? run_softmax<T, O, true>(x, y, outer, dim, inner, st) : run_softmax<T, O, false>(x, y, outer, dim, inner, st);
+  return log_softmax ? run_softmax<T, O, true>(x, y, outer, dim, inner, g_sm_ws, g_sm_ws_bytes, st)
+                     : run_softmax<T, O, false>(x, y, outer, dim, inner, g_sm_ws, g_sm_ws_bytes, st);
+}
+
+extern "C" int64_t mi355_row_workspace_bytes(int64_t rows, int64_t n, int dtype) {
+  const int es = dtype_size(dtype);
+  if (es == 0 || rows <= 0 || n <= 0) return 0;
+  const RowSplit sp = plan_row_split(rows, n, es);
+  return sp.nsplit > 1 ? rows * sp.nsplit * kRowPartialBytes : 0;
 }
 
 extern "C" int mi355_softmax(const void* x, int in_dtype, void* y, int out_dtype, int64_t outer, int64_t dim,
-                             int64_t inner, int log_softmax, void* stream) {
+                             int64_t inner, int log_softmax, void* workspace, int64_t workspace_bytes, void* stream) {
+  g_sm_ws = inner == 1 ? workspace : nullptr;
+  g_sm_ws_bytes = workspace_bytes;
   MI355_REQUIRE(outer >= 0 && dim >= 0 && inner >= 0, "mi355_softmax: negative extent");
   if (outer == 0 || dim == 0 || inner == 0) return MI355_OK;
   MI355_REQUIRE(x != nullptr && y != nullptr, "mi355_softmax: NULL data pointer");

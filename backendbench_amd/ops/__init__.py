@@ -10,7 +10,7 @@ same kernels.
 from ._common import check_index_errors
 from .elementwise import (_inplace_from, add, add_, clamp, clamp_, clamp_max, clamp_max_, clamp_max_tensor, clamp_min,
                           clamp_min_, clamp_min_tensor, clamp_tensor, maximum, minimum, mul, mul_, out_variant, relu,
-                          relu_, where)
+                          relu_, tuple_out_variant, where)
 from .index import embedding, gather, index_select
 from .matmul import addmm, mm
 from .reduce import (amax, argmax, log_softmax, mean_default, mean_dim, native_layer_norm, softmax, sum_default,
@@ -86,6 +86,7 @@ VARIANT_SLOTS = {
     "sum__out": out_variant(sum_default),
     "mean__dtype_out": out_variant(mean_default),
     "embedding__out": out_variant(embedding),
+    "native_layer_norm__out": tuple_out_variant(native_layer_norm, 3),
 }
 
 SLOTS = {**CORE_SLOTS, **VARIANT_SLOTS}

@@ -438,6 +438,31 @@ def clamp_max_tensor(self, max):
     return minimum(self, max)
 
 
+def tuple_out_variant(functional, n):
+    """`<op>.out(..., out0=, out1=, ...)` of an operator with `n` results (native_layer_norm.out):
+    each result goes into its own out tensor, resized and cast as in out_variant; returns them."""
+
+    def impl(*args, **kwargs):
+        outs = [kwargs.pop(f"out{i}") for i in range(n)]
+        results = functional(*args, **kwargs)
+        for res, out in zip(results, outs):
+            if not torch.can_cast(res.dtype, out.dtype):
+                raise RuntimeError(f"result type {str(res.dtype).replace('torch.', '').capitalize()} can't be cast to "
+                                   f"the desired output type {str(out.dtype).replace('torch.', '').capitalize()}")
+        done = []
+        for res, out in zip(results, outs):
+            if tuple(out.shape) != tuple(res.shape):
+                out.resize_(res.shape)
+            if res.device != out.device:
+                res = res.to(out.device)
+            done.append(copy_into_any(out, res))
+        return tuple(done)
+
+    impl.__name__ = functional.__name__ + "_out"
+    impl.__doc__ = f"out= variant of {functional.__name__} ({n} results)"
+    return impl
+
+
 def out_variant(functional):
     """`<op>.out(..., out=Tensor)` from the functional wrapper: compute, resize `out` if its
     shape differs (as ATen does), then store with a cast into `out`'s dtype and return `out`."""

@@ -88,6 +88,17 @@ def _adjacent_runs(dims):
     return runs
 
 
+def _row_workspace(rows, n, x):
+    """Scratch for the split form of softmax / layer norm over few, very long rows (None when the
+    library does not split this shape).  The planning call is skipped for shapes it never splits."""
+    if rows >= 64 or n < 32768:
+        return None, 0
+    nbytes = _lib.load().mi355_row_workspace_bytes(rows, n, _lib.dtype_code(x.dtype))
+    if nbytes <= 0:
+        return None, 0
+    return torch.empty(nbytes, dtype=torch.uint8, device=x.device), nbytes
+
+
 def _run_reduce(op, x, dims, keepdim, out_dtype):
     """x: tensor of a natively reducible dtype with numel > 0 and red > 0."""
     if len(dims) > 1 and op in (_lib.SUM, _lib.MEAN, _lib.AMAX):
@@ -241,11 +252,12 @@ def _softmax_impl(self, dim, half_to_float, log):
         rows = dense(x.view(outer, n, inner).transpose(1, 2))
         res = new_dense(rows.shape, out_dtype, self.device)
         launch("mi355_softmax", rows.data_ptr(), _lib.dtype_code(x.dtype), res.data_ptr(), _lib.dtype_code(out_dtype),
-               outer * inner, n, 1, 1 if log else 0)
+               outer * inner, n, 1, 1 if log else 0, None, 0)
         copy_into(out.view(outer, n, inner), res.transpose(1, 2))
         return out
+    ws, ws_bytes = _row_workspace(outer, n, x) if inner == 1 else (None, 0)
     launch("mi355_softmax", x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), _lib.dtype_code(out_dtype),
-           outer, n, inner, 1 if log else 0)
+           outer, n, inner, 1 if log else 0, ws.data_ptr() if ws is not None else None, ws_bytes)
     return out
 
 
@@ -303,7 +315,9 @@ def native_layer_norm(input, normalized_shape, weight, bias, eps):
     x = dense(input)
     w = dense(weight) if weight is not None else None
     b = dense(bias) if bias is not None else None
+    ws, ws_bytes = _row_workspace(M, N, x)
     launch("mi355_layer_norm", x.data_ptr(), _lib.dtype_code(x.dtype), w.data_ptr() if w is not None else None,
            b.data_ptr() if b is not None else None, _lib.dtype_code(w_dtype or x.dtype), y.data_ptr(),
-           mean.data_ptr(), rstd.data_ptr(), _lib.dtype_code(stat_dtype), M, N, float(eps))
+           mean.data_ptr(), rstd.data_ptr(), _lib.dtype_code(stat_dtype), M, N, float(eps),
+           ws.data_ptr() if ws is not None else None, ws_bytes)
     return y, mean, rstd

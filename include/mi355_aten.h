@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define MI355_ABI_VERSION 6
+#define MI355_ABI_VERSION 7
 #define MI355_MAX_DIMS 8
 
 typedef enum mi355_dtype {
@@ -153,19 +153,30 @@ int64_t mi355_reduce_static_max_bytes(void);
 int mi355_reduce_static(int op, const void* x, int in_dtype, int64_t outer, int64_t red,
                         int64_t inner, void* out, int out_dtype, void* stream);
 
+/* Bytes of scratch mi355_softmax (over the last dim) and mi355_layer_norm can use for `rows` rows of
+ * `n` elements of `dtype` (0 = none): a handful of very long rows (fewer than 64 rows of 32768
+ * elements and more) are cut into chunks over the whole chip, with one partial state per (row,
+ * chunk) in the scratch between the two launches of the call. */
+int64_t mi355_row_workspace_bytes(int64_t rows, int64_t n, int dtype);
+
 /* y = softmax (log_softmax != 0: log-softmax) over the middle axis of dense x viewed as
  * [outer, dim, inner]; fp32 math.  out_dtype = in_dtype, or MI355_F32 for half_to_float.
+ * workspace: device memory, 8-byte aligned, of mi355_row_workspace_bytes(outer, dim, in_dtype)
+ * bytes (only used when inner == 1), or NULL / smaller: then long rows take one block each.
  * Slots: _softmax__default (op_map.py:193), _log_softmax__default (op_map.py:151). */
 int mi355_softmax(const void* x, int in_dtype, void* y, int out_dtype, int64_t outer,
-                  int64_t dim, int64_t inner, int log_softmax, void* stream);
+                  int64_t dim, int64_t inner, int log_softmax, void* workspace,
+                  int64_t workspace_bytes, void* stream);
 
 /* Layer norm over the last N elements of each of M dense rows.  weight/bias may be NULL
  * and may differ in dtype from x (w_dtype).  mean/rstd are dense [M] in stat_dtype
  * (MI355_F32 or x's dtype).  Biased variance, rstd = 1/sqrt(var + eps).
- * Slot: native_layer_norm__default (op_map.py:776). */
+ * workspace: as for mi355_softmax, mi355_row_workspace_bytes(M, N, dtype) bytes or NULL.
+ * Slots: native_layer_norm__default (op_map.py:776), native_layer_norm__out. */
 int mi355_layer_norm(const void* x, int dtype, const void* weight, const void* bias,
                      int w_dtype, void* y, void* mean, void* rstd, int stat_dtype,
-                     int64_t M, int64_t N, double eps, void* stream);
+                     int64_t M, int64_t N, double eps, void* workspace,
+                     int64_t workspace_bytes, void* stream);
 
 /* ---- matrix multiply -------------------------------------------------------------- */
 

@@ -28,7 +28,7 @@ def header_enum(name):
 def test_header_declares_the_expected_entry_points():
     fns = declared_functions()
     assert "mi355_gemm" in fns and "mi355_softmax" in fns and "mi355_index_select" in fns
-    assert len(fns) == 19
+    assert len(fns) == 20
 
 
 def test_every_declared_symbol_is_exported_and_bound():
@@ -63,7 +63,7 @@ def test_enum_values_match_header(name, value):
 def test_argument_errors_are_reported_without_a_gpu():
     """Validation happens before any launch, so the error path is testable on the host."""
     lib = _lib.load()
-    rc = lib.mi355_softmax(None, _lib.F32, None, _lib.F32, 4, 4, 1, 0, None)
+    rc = lib.mi355_softmax(None, _lib.F32, None, _lib.F32, 4, 4, 1, 0, None, 0, None)
     assert rc == -1 and b"NULL" in lib.mi355_last_error()
     rc = lib.mi355_reduce(_lib.SUM, None, _lib.F32, 4, 0, 1, None, _lib.F32, None, 0, None)
     assert rc == -1 and b"bad extents" in lib.mi355_last_error()

@@ -30,7 +30,7 @@ PERF = perf_cases()
 def backend():
     assert torch.cuda.is_available(), "these tests need the MI355X"
     b = DirectoryBackend(os.path.join(ROOT, "generated_kernels"))
-    assert len(b.compiled_kernels) == 63
+    assert len(b.compiled_kernels) == 64
     return b
 
 
@@ -614,6 +614,60 @@ def test_out_overloads_fill_the_given_tensor(backend, case):
     assert ev.allclose(ref, res.cpu(), exact=not ref.dtype.is_floating_point or key in ("where.self_out", "index_select.out", "gather.out", "embedding.out")), key
 
 
+@pytest.mark.parametrize("shape,dtype", [((2, 786432), torch.float32), ((3, 100001), torch.float32), ((1, 1 << 20), torch.bfloat16),
+                                         ((5, 65536), torch.float16), ((2, 70000), torch.float64), ((63, 32768), torch.bfloat16)])
+def test_few_very_long_rows_split_over_the_chip(backend, shape, dtype):
+    """A handful of rows of tens of thousands of elements: softmax, log-softmax and layer norm cut every row
+    into chunks (two launches, partial states in a scratch buffer).  Aligned and odd row lengths, every
+    float dtype, a +inf and a NaN planted in different rows; compared with the oracle to the usual bar."""
+    from backendbench_amd import _lib
+    announce(f"few long rows {shape} {dtype}")
+    rows, n = shape
+    assert _lib.load().mi355_row_workspace_bytes(rows, n, _lib.dtype_code(dtype)) > 0, "meant to take the split form"
+    g = torch.Generator().manual_seed(rows * 7 + n)
+    x = (torch.randn(shape, generator=g) * 3).to(dtype)
+    x[0, n // 3] = 40.0                                   # one dominant element
+    if rows > 2:
+        x[1, 5] = float("inf")
+        x[2, n - 1] = float("nan")
+    xg = x.cuda()
+    for op, args in ((aten._softmax.default, [xg, -1, False]), (aten._log_softmax.default, [xg, 1, False])):
+        got = backend[op](*args)
+        ref = aten_cpu.reference(op, args)
+        assert ev.allclose(ref, got.cpu()), (op, ev.compute_errors(ref, got.cpu()))
+    if dtype in (torch.float16, torch.bfloat16):
+        got = backend[aten._softmax.default](xg, -1, True)
+        assert got.dtype == torch.float32 and ev.allclose(aten_cpu.reference(aten._softmax.default, [xg, -1, True]), got.cpu())
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(dtype).cuda()
+    b = (0.1 * torch.randn(n, generator=g)).to(dtype).cuda()
+    finite = torch.nan_to_num(x, nan=0.5, posinf=2.0).cuda()
+    for params in ((w, b), (None, None), (w, None)):
+        args = [finite, [n], params[0], params[1], 1e-5]
+        got = backend[aten.native_layer_norm.default](*args)
+        ref = aten_cpu.reference(aten.native_layer_norm.default, args)
+        for r, o in zip(ref, got):
+            assert r.shape == o.shape and r.dtype == o.dtype and ev.allclose(r, o.cpu()), ev.compute_errors(r, o.cpu())
+    if dtype == torch.bfloat16:   # fp32 gamma / beta on a half input
+        args = [finite, [n], w.float(), b.float(), 1e-5]
+        got = backend[aten.native_layer_norm.default](*args)
+        ref = aten_cpu.reference(aten.native_layer_norm.default, args)
+        assert all(ev.allclose(r, o.cpu()) for r, o in zip(ref, got))
+
+
+def test_native_layer_norm_out_fills_three_tensors(backend):
+    """native_layer_norm.out (BackendBench/scripts/op_map.py:776): y, mean and rstd go into out0 / out1 / out2,
+    which are resized when their shapes differ, and the same three objects come back."""
+    announce("native_layer_norm.out")
+    x, w, b = _t((6, 5, 40), seed=3), _t((40,), seed=4), _t((40,), seed=5)
+    outs = [torch.full((1,), 7.0).cuda(), torch.full((6, 5, 1), 7.0).cuda(), torch.empty(0).cuda()]
+    res = backend[aten.native_layer_norm.out](x.cuda(), [40], w.cuda(), b.cuda(), 1e-5, out0=outs[0], out1=outs[1], out2=outs[2])
+    torch.cuda.synchronize()
+    ref = aten.native_layer_norm.out(x, [40], w, b, 1e-5, out0=torch.empty(0), out1=torch.empty(0), out2=torch.empty(0))
+    assert len(res) == 3 and all(r is o for r, o in zip(res, outs))
+    for r, want in zip(res, ref):
+        assert r.shape == want.shape and ev.allclose(want, r.cpu())
+
+
 def test_out_overload_rejects_a_narrowing_cast(backend):
     announce("out= error behaviour")
     a = torch.ones(4, device="cuda")
@@ -830,7 +884,7 @@ def test_misaligned_rows_see_exactly_their_own_elements(backend, n, dtype):
 @pytest.mark.parametrize("family", ["gpt2", "bert"])
 def test_transformers_model_under_the_dispatcher_override(backend, family):
     """A randomly initialised Hugging Face model (built from a config, nothing downloaded) gives
-    the same hidden states with the 63 slots overriding ATen's HIP kernels as without, in fp32
+    the same hidden states with the 64 slots overriding ATen's HIP kernels as without, in fp32
     and in bf16; the spy shows the model really runs through the C ABI."""
     transformers = pytest.importorskip("transformers")
     import backendbench_amd
