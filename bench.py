@@ -34,8 +34,8 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, TFLOP/s
 # HBM bytes per launch from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
 # same counter reads for a plain 128 MiB copy); measured once per kernel with rocprofv3 --pmc,
-# summary in profiles/layernorm_tile_kernel__C2_layer_norm.md.  Not re-measured by this script.
-MEASURED_TRAFFIC_BYTES = {"C2.layer_norm": 134_520_000}
+# summary in profiles/C2_row_kernels__softmax_layer_norm.md.  Not re-measured by this script.
+MEASURED_TRAFFIC_BYTES = {"C2.layer_norm": 138_790_000, "C2.softmax": 134_300_000}
 
 
 def parse():
