@@ -1606,6 +1606,127 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   else store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
 }
 
+// ---------------------------------------------------------------- MFMA kernel, 64x64 tiles
+// bf16 / f16 products whose 128x128 tiles would leave most CUs without work (a 197-token ViT
+// layer against a 768-wide weight: 12 tiles; 1024^3: 64) and whose K loop is too short to split:
+// 64x64 tiles, four waves (2x2) of one 32x32 MFMA block each, 64-k stages (A 64x64 + B 64x64 =
+// 16 KB, whole 128-byte lines for both operands) in a ring of S stages filled S-1 stages ahead by
+// global_load_lds_dwordx4 (four requests per wave and stage, scalar base + 32-bit lane offset).
+// One barrier per stage; the per-stage work is four MFMAs per wave, so the kernel lives on how
+// many stages it keeps in flight: S = 8 (128 KB) when a CU gets one workgroup, else S = 4 (two
+// per CU).  K % 64 == 0.  A K-contiguous; B K-contiguous (swz_k64 rows) or N-contiguous (128-byte
+// k-rows, transposed by the LDS read).
+constexpr int TBM = 64, TBN = 64;
+constexpr int kTPanel = TBM * 64 * 2;  // 8 KB per operand per stage
+constexpr int kTStage = 2 * kTPanel;   // 16 KB
+// N-contiguous 64-wide panel: 128 B per k row, the two 64-byte halves swapped on k rows 2, 3 mod 4
+// so that the four k rows of a transposing read fall into four different 64-byte bank groups.
+__device__ __forceinline__ int swz_n64(int k, int u) {
+  return k * 128 + ((((u >> 2) ^ ((k >> 1) & 1))) << 6) + ((u & 3) << 4);
+}
+
+template <typename T, bool B_NN, int S>
+__global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  using frag_t = typename Mfma<T>::frag;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  const int bm = tm * TBM, bn = tn * TBN;
+  const T* a_base = static_cast<const T*>(g.a) + (int64_t)bm * g.lda;
+  const T* b_base = static_cast<const T*>(g.b) + (B_NN ? 0 : (int64_t)bn * g.ldb);
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  // Region q = wave + 4 i (i < 2) of a panel is LDS bytes [q * 1024, q * 1024 + 1024): eight rows of 128 B.
+  uint32_t a_off[2], b_off[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int q = wave + 4 * i;
+    const int r = 8 * q + (lane >> 3), slot = lane & 7;
+    {
+      const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
+      const int lr = bm + r < g.M ? r : g.M - 1 - bm;  // rows past M re-read the last row
+      a_off[i] = ((uint32_t)lr * (uint32_t)g.lda + (uint32_t)c * 8u) * 2u;
+    }
+    if constexpr (!B_NN) {
+      const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
+      const int ln = bn + r < g.N ? r : g.N - 1 - bn;
+      b_off[i] = ((uint32_t)ln * (uint32_t)g.ldb + (uint32_t)c * 8u) * 2u;
+    } else {  // k row r of the stage, LDS position `slot` holds unit u
+      const int u = (((slot >> 2) ^ ((r >> 1) & 1)) << 2) | (slot & 3);
+      int gn = bn + u * 8;
+      gn = gn < g.N ? gn : 0;
+      b_off[i] = ((uint32_t)r * (uint32_t)g.ldb + (uint32_t)gn) * 2u;
+    }
+  }
+  auto request_stage = [&](int t) {
+    const uint32_t stage = lds_base + (uint32_t)(t % S) * kTStage;
+    const T* pa = a_base + (int64_t)t * 64;
+    const T* pb = b_base + (B_NN ? (int64_t)t * 64 * g.ldb : (int64_t)t * 64);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t region = (uint32_t)(wave + 4 * i) * 1024u;
+      lds_dma16s(stage + region, a_off[i], pa);
+      lds_dma16s(stage + kTPanel + region, b_off[i], pb);
+    }
+  };
+  auto wait_younger = [](int stages) {  // stages requested behind the one about to be read: 4 loads each
+    switch (stages) {
+      case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+      case 1: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+      case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+      case 3: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+      case 4: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+      case 5: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
+    }
+  };
+
+  const int fr = lane & 31, fg = lane >> 5;
+  const int tr_k = fg * 8 + ((lane & 15) >> 2);
+  const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  // Two accumulators (even / odd 16-k sub-steps) halve the chain of dependent MFMAs, the only
+  // arithmetic of a stage; they are added once at the end.
+  f32x16 acc[1][1], acc_odd;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[0][0][e] = acc_odd[e] = 0.f;
+
+  const int nk = g.K / 64;
+  for (int t = 0; t < S - 1 && t < nk; ++t) request_stage(t);
+  for (int t = 0; t < nk; ++t) {
+    const int last_requested = t + S - 2 < nk - 1 ? t + S - 2 : nk - 1;
+    wait_younger(last_requested - t);
+    __syncthreads();  // stage t has landed for every wave, and every wave is done with stage t-1
+    const unsigned char* pa = lds + (t % S) * kTStage;
+    const unsigned char* pb = pa + kTPanel;
+    frag_t fa[4], fb[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      fa[ks] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 32 + fr, ks * 2 + fg));
+      if constexpr (!B_NN) {
+        fb[ks] = *reinterpret_cast<const frag_t*>(pb + swz_k64(wn * 32 + fr, ks * 2 + fg));
+      } else {
+        const int k = ks * 16 + tr_k;
+        const int n = wn * 32 + tr_n;
+        const s16x4 lo = lds_read_tr(pb + swz_n64(k, n >> 3) + ((n & 7) << 1));
+        const s16x4 hi = lds_read_tr(pb + swz_n64(k + 4, n >> 3) + ((n & 7) << 1));
+        fb[ks] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    }
+    if (t + S - 1 < nk) request_stage(t + S - 1);  // into the slot of stage t-1, behind this stage's LDS reads
+    acc[0][0] = Mfma<T>::run(fb[0], fa[0], acc[0][0]);
+    acc_odd = Mfma<T>::run(fb[1], fa[1], acc_odd);
+    acc[0][0] = Mfma<T>::run(fb[2], fa[2], acc[0][0]);
+    acc_odd = Mfma<T>::run(fb[3], fa[3], acc_odd);
+  }
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[0][0][e] += acc_odd[e];
+  __syncthreads();  // the ring becomes the epilogue's staging area
+  store_tile_result<T, 1, 0, 1>(g, acc, lds, wave, lane, bm + wm * 32, bn + wn * 32);
+}
+
 // ---------------------------------------------------------------- MFMA kernel, fp32
 // v_mfma_f32_32x32x2_f32 (fp32 in, fp32 accumulate; 157 TFLOP/s dense peak).  Same shape as the
 // 128x128 half-precision kernel in bytes: four waves (2x2) of 64x64, 16-k steps (64-byte rows),
@@ -2040,7 +2161,27 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool mid = !ktail && K % 64 == 0 && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "256x128") == 0
                                                : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > (K >= 2048 ? 228 : 248) && tiles_mid <= kNumCU);
-      if (mid) {
+      // Fewer 128x128 tiles than half the CUs: 64x64 tiles reach four times as many (measured on this
+      // chip: [197,768]x[768,768] 11.6 -> 7.5 us, 1024^3 14.6 -> 9.4 us).  A 64x64 workgroup walks K at
+      // about 0.3 us per 64 k, so a few tiles with a long K stay on the 128x128 kernels, which split K
+      // over the chip.  A single row of tiles (M <= 64) also takes them at larger N: half of a 128-row
+      // tile would be padding ([32,768]x[768,32000]: 17.5 -> 13.3 us).  MI355_GEMM_TILE=64x64 forces them, =128x128 keeps them off: test knobs.
+      const int64_t nb128 = ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN);
+      const int64_t nb64 = ((M + TBM - 1) / TBM) * ((N + TBN - 1) / TBN);
+      const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
+                       (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
+                                               : (nb128 < kNumCU / 2 || (M <= 64 && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
+                                                     (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2)));
+      if (t64) {
+        g.tiles_m = (int32_t)((M + TBM - 1) / TBM);
+        g.tiles_n = (int32_t)((N + TBN - 1) / TBN);
+        nblocks = nb64;
+        threads = 256;
+        const bool deep = nblocks <= kNumCU;
+        lds_bytes = (deep ? 8 : 4) * kTStage;
+        if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8> : (const void*)gemm_mfma_t64_kernel<T, true, 8>;
+        else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4> : (const void*)gemm_mfma_t64_kernel<T, true, 4>;
+      } else if (mid) {
         g.tiles_n = (int32_t)((N + 127) / 128);
         nblocks = tiles_mid;
         kern = pick_w4(std::integral_constant<int, 2>{});
@@ -2097,7 +2238,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
       }
       // More than 64 KB of dynamic LDS needs the attribute once per kernel and process.
-      static thread_local const void* attr_done[48] = {};
+      static thread_local const void* attr_done[64] = {};
       bool seen = false;
       for (const void* k : attr_done) seen = seen || k == kern;
       if (!seen) {

@@ -231,6 +231,35 @@ def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
         assert ev.bit_equal(ref, out[rows.cuda()].cpu()), (layout, shape, K)
 
 
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+@pytest.mark.parametrize("shape", [(197, 776), (1000, 1080), (64, 64), (33, 4104)])
+def test_tile64_gemm_every_k_loop_length(backend, layout, shape, monkeypatch):
+    """The 64x64-tile kernel (products whose 128x128 tiles would leave most CUs idle): [197, K] x [K, 776] has
+    4 x 13 tiles with ragged last row and column (one workgroup per CU: the eight-stage ring), [1000, K] x
+    [K, 1080] has 16 x 17 = 272 (more than one per CU: the four-stage ring).  K walks from one stage to more
+    than twice the ring depth.  Small-integer operands: bit-equal to the oracle; a bias row through the
+    epilogue; the kernel is forced so that every K takes it, and once left to the planner."""
+    M, N = shape
+    announce(f"64x64-tile GEMM K loop lengths, {layout}, {M}x{N}")
+    g = torch.Generator().manual_seed(12)
+    for K in (64, 128, 192, 256, 384, 448, 512, 576, 640, 1024, 1088, 2048):
+        a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+        if layout[1] == "t":
+            b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
+        else:
+            b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
+        bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
+        monkeypatch.setenv("MI355_GEMM_TILE", "64x64")
+        out = backend[aten.addmm.default](bias, a, b, beta=2.0)
+        half = backend[aten.mm.default](a.half(), b.half())
+        monkeypatch.delenv("MI355_GEMM_TILE")
+        ref = aten_cpu.reference(aten.addmm.default, [bias, a, b], {"beta": 2.0})
+        assert ev.bit_equal(ref, out.cpu()), (layout, shape, K)
+        assert ev.bit_equal(aten_cpu.reference(aten.mm.default, [a.half(), b.half()]), half.cpu()), (layout, shape, K, "f16")
+        auto = backend[aten.addmm.default](bias, a, b, beta=2.0)
+        assert ev.bit_equal(ref, auto.cpu()), (layout, shape, K, "planner's choice")
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_split_k_with_ragged_k(backend, dtype):
     """One-tile outputs split along K where K is not a multiple of the split length (K = 672, 544, 416
