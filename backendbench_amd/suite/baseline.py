@@ -430,6 +430,15 @@ def edge_cases() -> List[Case]:
             lambda d, rl=rl, dt=dt, hw=hw, hb=hb: (_to(d, normal((1037, rl), dt, 1, 2, seed=rl), [rl], normal((rl,), dt, 1, 0.1, seed=2) if hw else None,
                                                       normal((rl,), dt, 0, 0.1, seed=3) if hb else None, 1e-5), {}), tag=f"short_{rl}_{t}")
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((300, 12, 64), f16, 0, 2, seed=1), [64], normal((64,), f32, 1, 0.1, seed=2), normal((64,), f32, 0, 0.1, seed=3), 1e-6), {}), tag="short_64_f32_params", stock_gpu=False)
+    # a thousand and more mid-length rows: the streaming kernels (one wave per row, next row prefetched), four- and
+    # eight-slab register tiles, rows that do not fill the last slab, row counts that do not divide by the waves
+    for rows, rl, dt, t, hw, hb in ((1100, 1000, f32, "f32", True, True), (1030, 1800, f32, "f32", True, False), (1500, 2056, bf16, "bf16", False, False),
+                                    (1024, 4096, f16, "f16", True, True), (2050, 520, bf16, "bf16", False, True), (1027, 2048, f32, "f32", True, True)):
+        add(aten.native_layer_norm.default,
+            lambda d, rows=rows, rl=rl, dt=dt, hw=hw, hb=hb: (_to(d, normal((rows, rl), dt, 1, 2, seed=rl), [rl], normal((rl,), dt, 1, 0.1, seed=2) if hw else None,
+                                                                 normal((rl,), dt, 0, 0.1, seed=3) if hb else None, 1e-5), {}), tag=f"stream_{rows}x{rl}_{t}")
+        add(aten._softmax.default if hw else aten._log_softmax.default,
+            lambda d, rows=rows, rl=rl, dt=dt: (_to(d, poison(normal((rows, rl), dt, 0, 2, seed=rl + 1), 0.0002, 5), -1, False), {}), tag=f"stream_{rows}x{rl}_{t}")
     # long rows: 8- and 16-wave register tiles, then the two-pass block kernel
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((5, 12288), bf16, 1, 2, seed=1), [12288], normal((12288,), bf16, 1, 0.1, seed=2), normal((12288,), bf16, 0, 0.1, seed=3), 1e-5), {}), tag="row12288_bf16")
     add(aten.native_layer_norm.default, lambda d: (_to(d, normal((3, 40000), f32, -2, 3, seed=1), [40000], normal((40000,), f32, 1, 0.1, seed=2), None, 1e-5), {}), tag="row40000_f32")
