@@ -229,6 +229,20 @@ __global__ __launch_bounds__(kIxBlock) void gather_rows_lds_kernel(const U* __re
   const int64_t r = blockIdx.y;
   const U* s = src + r * len;
   constexpr int UV = 16 / sizeof(U);
+  const int64_t j0 = (int64_t)blockIdx.x * per_split;
+  const int64_t j1 = j0 + per_split < n_idx ? j0 + per_split : n_idx;
+  const int64_t* ix = index + r * idx_row_stride;  // 0: every row uses the same indices (index_select)
+  U* o = out + r * n_idx;
+  const bool vec = n_idx % 4 == 0 && per_split % 4 == 0 && (reinterpret_cast<uintptr_t>(ix) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(o) % (4 * sizeof(U))) == 0;
+  // The first indices of every thread are requested before the row is staged, and every later batch
+  // one step ahead: the index stream (two thirds of the bytes) never waits behind the barrier.
+  VecN<int64_t, 2> na{}, nb{};
+  const int64_t jf = j0 + (int64_t)threadIdx.x * 4;
+  if (vec && jf < j1) {
+    na = ld_nt<int64_t, 2>(ix + jf);
+    nb = ld_nt<int64_t, 2>(ix + jf + 2);
+  }
   if (len % UV == 0 && (reinterpret_cast<uintptr_t>(s) & 15) == 0) {
     for (int64_t i = (int64_t)threadIdx.x * UV; i < len; i += (int64_t)kIxBlock * UV)
       st<U, UV>(row + i, ld_nt<U, UV>(s + i));
@@ -236,15 +250,14 @@ __global__ __launch_bounds__(kIxBlock) void gather_rows_lds_kernel(const U* __re
     for (int64_t i = threadIdx.x; i < len; i += kIxBlock) row[i] = s[i];
   }
   __syncthreads();
-  const int64_t j0 = (int64_t)blockIdx.x * per_split;
-  const int64_t j1 = j0 + per_split < n_idx ? j0 + per_split : n_idx;
-  const int64_t* ix = index + r * idx_row_stride;  // 0: every row uses the same indices (index_select)
-  U* o = out + r * n_idx;
-  const bool vec = n_idx % 4 == 0 && per_split % 4 == 0 && (reinterpret_cast<uintptr_t>(ix) & 15) == 0 &&
-                   (reinterpret_cast<uintptr_t>(o) % (4 * sizeof(U))) == 0;
   if (vec) {
-    for (int64_t j = j0 + (int64_t)threadIdx.x * 4; j < j1; j += (int64_t)kIxBlock * 4) {
-      const VecN<int64_t, 2> a = ld_nt<int64_t, 2>(ix + j), b = ld_nt<int64_t, 2>(ix + j + 2);
+    for (int64_t j = jf; j < j1; j += (int64_t)kIxBlock * 4) {
+      const VecN<int64_t, 2> a = na, b = nb;
+      const int64_t jn = j + (int64_t)kIxBlock * 4;
+      if (jn < j1) {
+        na = ld_nt<int64_t, 2>(ix + jn);
+        nb = ld_nt<int64_t, 2>(ix + jn + 2);
+      }
       const int64_t id[4] = {a.v[0], a.v[1], b.v[0], b.v[1]};
       VecN<U, 4> v;
 #pragma unroll
