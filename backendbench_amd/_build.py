@@ -25,6 +25,7 @@ SOURCES = [
     "layernorm.hip",
     "index.hip",
     "gemm.hip",
+    "gemm_x16.hip",
     "calib.hip",
 ]
 

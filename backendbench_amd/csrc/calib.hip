@@ -29,6 +29,9 @@ template <> struct CalibMfma<cf16x8> {
 //          second, changing every MFMA).
 // ORDER 1: operands swapped between the two ports.
 // ORDER 2: second operand held over four MFMAs, first changing.
+// ORDER 3: the four MFMAs of a pair of steps that feed one accumulator block issued back to back
+//          (k innermost): every MFMA takes its addend from the one before it.
+// ORDER 4: the same in chains of two (the two 16-k halves of one step).
 template <typename F, int ORDER>
 __global__ __launch_bounds__(256) void calib_mfma32_kernel(const F* __restrict__ a, const F* __restrict__ b, float* __restrict__ out, int steps) {
   const int64_t lane_slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -50,6 +53,28 @@ __global__ __launch_bounds__(256) void calib_mfma32_kernel(const F* __restrict__
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
   for (int t = 0; t < steps; t += 2) {
+    if constexpr (ORDER == 3) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) acc[q][p] = CalibMfma<F>::run32(xb[s][ks][p], xa[s][ks][q], acc[q][p]);
+      continue;
+    }
+    if constexpr (ORDER == 4) {
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) acc[q][p] = CalibMfma<F>::run32(xb[s][ks][p], xa[s][ks][q], acc[q][p]);
+      continue;
+    }
 #pragma unroll
     for (int s = 0; s < 2; ++s)
 #pragma unroll
@@ -75,7 +100,7 @@ __global__ __launch_bounds__(256) void calib_mfma32_kernel(const F* __restrict__
 
 // The same register tile on v_mfma_f32_16x16x32: 8 x 8 blocks of 16 x 16 (64 accumulators of four
 // registers), eight A and eight B fragments per 32-k step, 64 MFMAs of half the work each.
-template <typename F>
+template <typename F, bool CHAIN = false>
 __global__ __launch_bounds__(256) void calib_mfma16_kernel(const F* __restrict__ a, const F* __restrict__ b, float* __restrict__ out, int steps) {
   const int64_t lane_slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
   F xa[2][8], xb[2][8];
@@ -94,12 +119,68 @@ __global__ __launch_bounds__(256) void calib_mfma16_kernel(const F* __restrict__
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
   for (int t = 0; t < steps; t += 2) {
+    if constexpr (CHAIN) {  // the two MFMAs of a pair of steps on one accumulator block back to back
+#pragma unroll
+      for (int p = 0; p < 8; ++p)
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+#pragma unroll
+          for (int s = 0; s < 2; ++s) acc[q][p] = CalibMfma<F>::run16(xb[s][p], xa[s][q], acc[q][p]);
+      continue;
+    }
 #pragma unroll
     for (int s = 0; s < 2; ++s)
 #pragma unroll
       for (int p = 0; p < 8; ++p)
 #pragma unroll
         for (int q = 0; q < 8; ++q) acc[q][p] = CalibMfma<F>::run16(xb[s][p], xa[s][q], acc[q][p]);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum += acc[i][j][e];
+  out[lane_slot] = sum;
+}
+
+// 16x16x32 with chains of L MFMAs per accumulator block (L = 1, 2, 4): four k-sets of 4 + 4 fragments
+// (two for L < 4), reused by all four 4 x 4 quadrants of the 8 x 8 block grid; the quadrants are
+// walked one after the other (what a kernel that keeps one quadrant's fragments live would issue).
+template <typename F, int L>
+__global__ __launch_bounds__(256) void calib_mfma16q_kernel(const F* __restrict__ a, const F* __restrict__ b, float* __restrict__ out, int steps) {
+  constexpr int NS = L == 4 ? 4 : 2;
+  const int64_t lane_slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  F xa[NS][4], xb[NS][4];
+#pragma unroll
+  for (int s = 0; s < NS; ++s)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      xa[s][i] = a[lane_slot * 16 + s * 4 + i];
+      xb[s][i] = b[lane_slot * 16 + s * 4 + i];
+    }
+  cf32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+  for (int t = 0; t < steps; t += NS) {
+#pragma unroll
+    for (int g = 0; g < NS; g += L)
+#pragma unroll
+      for (int quad = 0; quad < 4; ++quad)
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int s = g; s < g + L; ++s)
+              acc[(quad >> 1) * 4 + q][(quad & 1) * 4 + p] =
+                  CalibMfma<F>::run16(xb[s][p], xa[s][q], acc[(quad >> 1) * 4 + q][(quad & 1) * 4 + p]);
+    __builtin_amdgcn_sched_barrier(0);
   }
   float sum = 0.f;
 #pragma unroll
@@ -118,13 +199,15 @@ using namespace mi355;
 // blocks x 256 threads, each wave issuing `steps` (even) 32-k steps of a 128 x 128 register tile:
 // 2 * 128 * 128 * 32 flop per wave and step.  a, b: 16 fragments of 16 bytes per thread
 // (blocks * 256 * 256 bytes each); out: blocks * 256 floats.  variant 0..2: 32x32x16 in the three
-// operand orders, 3: 16x16x32.
+// operand orders, 3: 16x16x32, 4 / 5: 32x32x16 with the MFMAs on one accumulator block chained in
+// fours / twos, 6: 16x16x32 chained in twos, 7 / 8 / 9: 16x16x32 walked quadrant by quadrant in chains
+// of 1 / 2 / 4 (steps % 4 == 0).
 extern "C" int mi355_calib_mfma(const void* a, const void* b, void* out, int dtype, int blocks, int steps, int variant,
                                 void* stream) {
   MI355_REQUIRE(a != nullptr && b != nullptr && out != nullptr, "mi355_calib_mfma: NULL buffer");
-  MI355_REQUIRE(blocks > 0 && steps > 0 && steps % 2 == 0, "mi355_calib_mfma: blocks > 0 and an even number of steps");
+  MI355_REQUIRE(blocks > 0 && steps > 0 && steps % 4 == 0, "mi355_calib_mfma: blocks > 0 and a number of steps divisible by four");
   MI355_REQUIRE(dtype == MI355_BF16 || dtype == MI355_F16, "mi355_calib_mfma: bf16 or f16");
-  MI355_REQUIRE(variant >= 0 && variant <= 3, "mi355_calib_mfma: variant 0..3");
+  MI355_REQUIRE(variant >= 0 && variant <= 9, "mi355_calib_mfma: variant 0..9");
   hipStream_t st = static_cast<hipStream_t>(stream);
   float* o = static_cast<float*>(out);
 #define MI355_CALIB(F_)                                                                                                        \
@@ -135,7 +218,13 @@ extern "C" int mi355_calib_mfma(const void* a, const void* b, void* out, int dty
       case 0: hipLaunchKernelGGL((calib_mfma32_kernel<F_, 0>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;       \
       case 1: hipLaunchKernelGGL((calib_mfma32_kernel<F_, 1>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;       \
       case 2: hipLaunchKernelGGL((calib_mfma32_kernel<F_, 2>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;       \
-      default: hipLaunchKernelGGL((calib_mfma16_kernel<F_>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;         \
+      case 3: hipLaunchKernelGGL((calib_mfma16_kernel<F_>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;          \
+      case 4: hipLaunchKernelGGL((calib_mfma32_kernel<F_, 3>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;       \
+      case 5: hipLaunchKernelGGL((calib_mfma32_kernel<F_, 4>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;       \
+      case 6: hipLaunchKernelGGL((calib_mfma16_kernel<F_, true>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;    \
+      case 7: hipLaunchKernelGGL((calib_mfma16q_kernel<F_, 1>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;      \
+      case 8: hipLaunchKernelGGL((calib_mfma16q_kernel<F_, 2>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;      \
+      default: hipLaunchKernelGGL((calib_mfma16q_kernel<F_, 4>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;     \
     }                                                                                                                          \
   }
   if (dtype == MI355_BF16) MI355_CALIB(cbf16x8) else MI355_CALIB(cf16x8)

@@ -23,18 +23,10 @@
 #include <type_traits>
 
 #include "common.h"
+#include "gemm_shared.h"
 
 namespace mi355 {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-template <typename T> struct alignas(sizeof(T) * 4) VecN4 {
-  T v[4];
-};
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 // v_mfma_f32_32x32x16: measured at ~96 % of the 2.5 PFLOP/s bf16 peak on MI355X when issued
 // back to back; the 16x16x32 form tops out near 60 %, so the 32x32 form is the only one used.
@@ -54,7 +46,6 @@ template <> struct Mfma<f16_t> {
   }
 };
 
-constexpr int BM = 256, BN = 256;
 // N-contiguous panel ([k][n], the row-major "NN" B, 512 B per k): byte offset of 16-byte unit u
 // (0..31) of row k.  64-byte segments are rotated by k%4 (XOR on the segment index) so that a
 // transposing 64-bit read by 32 lanes — 4 consecutive k-rows x 64 B, see lds_read_tr — covers
@@ -63,27 +54,6 @@ __device__ __forceinline__ int swz_n(int k, int u) {
   return k * (BN * 2) + ((((u >> 2) ^ (k & 3))) << 6) + ((u & 3) << 4);
 }
 
-struct GemmArgs {
-  const void* a;
-  const void* b;
-  const void* c;
-  void* out;
-  int64_t lda, ldb;  // element stride between rows of a ([M][K]) and between the K-contiguous
-                     // rows of b ([N][K], NT) or the N-contiguous rows of b ([K][N], NN)
-  int64_t c_rs, c_cs;
-  int32_t M, N, K;
-  float alpha, beta;
-  int32_t tiles_m, tiles_n;
-  int32_t tail_n;  // gemm_mfma_w4_mixed_kernel: 192-wide tile columns behind the tiles_n 256-wide ones
-  int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
-  int32_t out_vec;  // out rows start on 16-byte boundaries (N a multiple of the vector width): vector stores
-  // Split-K (128x128 kernels only): blockIdx.y = split, which covers k in [split * ksplit,
-  // min(K, (split + 1) * ksplit)) and writes its raw fp32 tile to ws[split][M][ws_ld], ws_ld = N
-  // rounded up to a multiple of 4 (rows of every plane start on 16-byte boundaries for any N).
-  float* ws;
-  int32_t ksplit;
-  int32_t ws_ld;
-};
 
 // fp32 partial tile of one split: register r of acc[i][j] in lane l is
 // C[m0 + 32 i + l%32][n0 + 32 j + 8 (r/4) + 4 (l/32) + r%4]; N % 4 == 0 on the MFMA paths.
@@ -177,39 +147,7 @@ __global__ __launch_bounds__(256) void gemm_splitk_finish4_kernel(GemmArgs g, in
   }
 }
 
-// Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous
-// band of tile ids, then walk the band in groups of 8 tile-rows so A and B panels repeat
-// in that XCD's L2.
-__device__ __forceinline__ void tile_coords(const int tiles_m, const int tiles_n, int pid, int& tm, int& tn) {
-  const int nblocks = tiles_m * tiles_n;
-  const int per_xcd = (nblocks + kNumXCD - 1) / kNumXCD;
-  const int full = nblocks % kNumXCD;  // XCDs that own `per_xcd` tiles when not divisible
-  const int xcd = pid % kNumXCD, local = pid / kNumXCD;
-  if (full == 0) pid = xcd * per_xcd + local;
-  else pid = (xcd < full ? xcd * per_xcd : full * per_xcd + (xcd - full) * (per_xcd - 1)) + local;
-  constexpr int GROUP = 8;
-  const int in_group = GROUP * tiles_n;
-  const int group = pid / in_group;
-  const int first_m = group * GROUP;
-  const int rows = tiles_m - first_m < GROUP ? tiles_m - first_m : GROUP;
-  tm = first_m + (pid % in_group) % rows;
-  tn = (pid % in_group) / rows;
-}
-__device__ __forceinline__ void tile_coords(const GemmArgs& g, int& tm, int& tn) {
-  tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
-}
 
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-
-// ds_read_b64_tr_b16: within each block of 16 lanes, lane s supplies the address of 4
-// consecutive 16-bit elements ("row s/4, columns 4*(s%4)..+3" of a 4 x 16 block) and lane i
-// receives column i of the 4 rows.  With rows = k and columns = n this turns an N-contiguous
-// LDS panel into the K-contiguous MFMA operand.
-__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (__attribute__((address_space(3))) s16x4*)(uintptr_t)(const_cast<unsigned char*>(p)));
-}
 
 // ---------------------------------------------------------------- epilogue
 // A wave's (32 MI)x64 result: register r of acc[i][j] in lane l is C[m0 + 32 i + l%32][n0 + 32 j +
@@ -469,22 +407,6 @@ __global__ __launch_bounds__(512) void gemm_mfma_kernel(GemmArgs g) {
 // the newest tile may still be in flight), so every tile has two iterations to arrive.  The
 // loads are issued from inline asm, so the compiler's own wait-count bookkeeping does not see
 // them and adds no waits of its own.  Needs K % 32 == 0 (no zero fill on this path).
-__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_offset, const void* gptr) {
-  asm volatile("s_mov_b32 m0, %0\n\t"
-               "s_nop 0\n\t"
-               "global_load_lds_dwordx4 %1, off" ::"s"(lds_byte_offset), "v"(gptr)
-               : "memory");
-}
-
-// The same fill with the address split into a uniform 64-bit base (SGPR pair) and a 32-bit byte
-// offset per lane: the offsets of a wave's requests are loop invariants (one VGPR each instead of
-// a pointer pair) and a k step only moves the scalar base.
-__device__ __forceinline__ void lds_dma16s(uint32_t lds_byte_offset, uint32_t lane_byte_offset, const void* base) {
-  asm volatile("s_mov_b32 m0, %0\n\t"
-               "s_nop 0\n\t"
-               "global_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_byte_offset), "s"(base)
-               : "memory");
-}
 
 template <typename T, bool B_NN>
 __global__ __launch_bounds__(512) void gemm_mfma_dma_kernel(GemmArgs g) {
@@ -2172,7 +2094,13 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
                                                : (nb128 < kNumCU / 2 || (M <= 64 && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
                                                      (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2)));
-      if (t64) {
+      // The 16x16x32 form of the four-wave kernel (gemm_x16.hip).  MI355_GEMM_TILE=x16 forces it for any tile count.
+      const bool x16 = K % 128 == 0 && K >= 256 && !a_t && ld32 && forced_tile != nullptr && strcmp(forced_tile, "x16") == 0;
+      if (x16) {
+        kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
+        threads = 256;
+        lds_bytes = kX16Lds;
+      } else if (t64) {
         g.tiles_m = (int32_t)((M + TBM - 1) / TBM);
         g.tiles_n = (int32_t)((N + TBN - 1) / TBN);
         nblocks = nb64;
@@ -2214,6 +2142,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         // (two-pass epilogue), which evens out near K = 2048.  MI355_GEMM_WAVES=4|8 forces one form.
         const char* forced = getenv("MI355_GEMM_WAVES");
         const bool w4 = a_t || (ld32 && (forced != nullptr ? forced[0] == '4' : K >= 2048));  // the eight-wave kernels have no M-contiguous-A form
+        lds_bytes = kGemmLds64;
         if (w4) {
           kern = pick_w4(std::integral_constant<int, 4>{});
           threads = 256;
@@ -2233,7 +2162,6 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         } else {
           kern = b_nt ? (const void*)gemm_mfma_dma64_kernel<T, false> : (const void*)gemm_mfma_dma64_kernel<T, true>;
         }
-        lds_bytes = kGemmLds64;
       } else {
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
       }

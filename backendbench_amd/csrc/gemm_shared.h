@@ -1,0 +1,101 @@
+// Types and helpers shared by the GEMM kernel sources (gemm.hip, gemm_x16.hip): the argument
+// block, the block -> tile map, the transposing LDS read and the global -> LDS fill requests.
+#pragma once
+#include "common.h"
+
+namespace mi355 {
+
+constexpr int BM = 256, BN = 256;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct alignas(sizeof(T) * 4) VecN4 {
+  T v[4];
+};
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct GemmArgs {
+  const void* a;
+  const void* b;
+  const void* c;
+  void* out;
+  int64_t lda, ldb;  // element stride between rows of a ([M][K]) and between the K-contiguous
+                     // rows of b ([N][K], NT) or the N-contiguous rows of b ([K][N], NN)
+  int64_t c_rs, c_cs;
+  int32_t M, N, K;
+  float alpha, beta;
+  int32_t tiles_m, tiles_n;
+  int32_t tail_n;  // gemm_mfma_w4_mixed_kernel: 192-wide tile columns behind the tiles_n 256-wide ones
+  int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
+  int32_t out_vec;  // out rows start on 16-byte boundaries (N a multiple of the vector width): vector stores
+  // Split-K (128x128 kernels only): blockIdx.y = split, which covers k in [split * ksplit,
+  // min(K, (split + 1) * ksplit)) and writes its raw fp32 tile to ws[split][M][ws_ld], ws_ld = N
+  // rounded up to a multiple of 4 (rows of every plane start on 16-byte boundaries for any N).
+  float* ws;
+  int32_t ksplit;
+  int32_t ws_ld;
+};
+
+// Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous
+// band of tile ids, then walk the band in groups of 8 tile-rows so A and B panels repeat
+// in that XCD's L2.
+__device__ __forceinline__ void tile_coords(const int tiles_m, const int tiles_n, int pid, int& tm, int& tn) {
+  const int nblocks = tiles_m * tiles_n;
+  const int per_xcd = (nblocks + kNumXCD - 1) / kNumXCD;
+  const int full = nblocks % kNumXCD;  // XCDs that own `per_xcd` tiles when not divisible
+  const int xcd = pid % kNumXCD, local = pid / kNumXCD;
+  if (full == 0) pid = xcd * per_xcd + local;
+  else pid = (xcd < full ? xcd * per_xcd : full * per_xcd + (xcd - full) * (per_xcd - 1)) + local;
+  constexpr int GROUP = 8;
+  const int in_group = GROUP * tiles_n;
+  const int group = pid / in_group;
+  const int first_m = group * GROUP;
+  const int rows = tiles_m - first_m < GROUP ? tiles_m - first_m : GROUP;
+  tm = first_m + (pid % in_group) % rows;
+  tn = (pid % in_group) / rows;
+}
+__device__ __forceinline__ void tile_coords(const GemmArgs& g, int& tm, int& tn) {
+  tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
+}
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+// ds_read_b64_tr_b16: within each block of 16 lanes, lane s supplies the address of 4
+// consecutive 16-bit elements ("row s/4, columns 4*(s%4)..+3" of a 4 x 16 block) and lane i
+// receives column i of the 4 rows.  With rows = k and columns = n this turns an N-contiguous
+// LDS panel into the K-contiguous MFMA operand.
+__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) s16x4*)(uintptr_t)(const_cast<unsigned char*>(p)));
+}
+
+// global_load_lds_dwordx4: one wave-level load moves 64 x 16 bytes from global memory straight into
+// 1 KB of LDS (lane l lands at M0 + 16 l) without passing through VGPRs.  Issued from inline asm: the
+// compiler's wait-count bookkeeping does not see these loads, the kernels count them (s_waitcnt vmcnt).
+__device__ __forceinline__ void lds_dma16(uint32_t lds_byte_offset, const void* gptr) {
+  asm volatile("s_mov_b32 m0, %0\n\t"
+               "s_nop 0\n\t"
+               "global_load_lds_dwordx4 %1, off" ::"s"(lds_byte_offset), "v"(gptr)
+               : "memory");
+}
+
+// The same fill with the address split into a uniform 64-bit base (SGPR pair) and a 32-bit byte
+// offset per lane: the offsets of a wave's requests are loop invariants (one VGPR each instead of
+// a pointer pair) and a k step only moves the scalar base.
+__device__ __forceinline__ void lds_dma16s(uint32_t lds_byte_offset, uint32_t lane_byte_offset, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\t"
+               "s_nop 0\n\t"
+               "global_load_lds_dwordx4 %1, %2" ::"s"(lds_byte_offset), "v"(lane_byte_offset), "s"(base)
+               : "memory");
+}
+
+// gemm_x16.hip: the 256x256-tile kernel on v_mfma_f32_16x16x32 (bf16 / f16, K % 128 == 0, K >= 256, K-contiguous
+// a; b K-contiguous or row-major), its dynamic LDS size, and the host-side kernel handle.
+constexpr int kX16Lds = 5 * 32768;
+const void* gemm_x16_kernel(bool is_bf16, bool b_nn);
+
+}  // namespace mi355
