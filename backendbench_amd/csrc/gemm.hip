@@ -2094,12 +2094,33 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
                                                : (nb128 < kNumCU / 2 || (M <= 64 && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
                                                      (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2)));
-      // The 16x16x32 form of the four-wave kernel (gemm_x16.hip).  MI355_GEMM_TILE=x16 forces it for any tile count.
-      const bool x16 = K % 128 == 0 && K >= 256 && !a_t && ld32 && forced_tile != nullptr && strcmp(forced_tile, "x16") == 0;
+      // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
+      // with 256x256 tiles when K is a multiple of 128: measured against the 32x32x16 form on
+      // [4096,K]x[K,16384], it is level at K = 512 and 4 - 15 % faster from K = 768 on (C3: [4096,4096]x
+      // [4096,11008] 306 -> 279 us, [4096,11008]x[11008,4096] 270 -> 249 us).  MI355_GEMM_TILE=x16
+      // forces it for any tile count (=x16mixed: with the mixed-width grid at any K), =256x256 / =mixed keep
+      // the 32x32x16 form (test knobs).
+      const bool x16_ok = K % 128 == 0 && K >= 256 && !a_t && ld32;
+      const bool x16_mixed_forced = forced_tile != nullptr && strcmp(forced_tile, "x16mixed") == 0;  // mixed widths at any K
+      const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced
+                                                         : K >= 512 && nblocks >= kNumCU * 3 / 4 && !mid && !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
       if (x16) {
         kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
         threads = 256;
         lds_bytes = kX16Lds;
+        // The mixed-width grid (192-wide tiles in the last round) is built for this form too, but it does not
+        // pay here: [4096,4096]x[4096,11008] takes 284.6 us with it and 285.6 us without - a last round
+        // that leaves CUs idle runs at a higher clock under the power limit, and a 192-wide tile issues the
+        // same fills as a 256-wide one.  Only MI355_GEMM_TILE=x16mixed selects it.
+        if (nblocks > kNumCU && x16_mixed_forced) {
+          const MixedPlan mp = plan_mixed(g.tiles_m, N);
+          if (mp.narrow > 0) {
+            g.tiles_n = mp.wide;
+            g.tail_n = mp.narrow;
+            nblocks = (int64_t)g.tiles_m * (mp.wide + mp.narrow);
+            kern = gemm_x16_mixed_kernel(std::is_same<T, bf16_t>::value, !b_nt);
+          }
+        }
       } else if (t64) {
         g.tiles_m = (int32_t)((M + TBM - 1) / TBM);
         g.tiles_n = (int32_t)((N + TBN - 1) / TBN);

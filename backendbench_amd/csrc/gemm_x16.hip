@@ -24,6 +24,10 @@
 
 #include "gemm_shared.h"
 
+#ifndef MI355_X16_ABLATE
+#define MI355_X16_ABLATE 0
+#endif
+
 namespace mi355 {
 
 template <typename T> struct Mfma16;
@@ -50,11 +54,11 @@ __device__ __forceinline__ int xswz_k(int r, int c) { return r * 128 + ((c ^ ((r
 // land in eight distinct segments.
 __device__ __forceinline__ int xswz_seg(int k) { return (k & 3) | (((k >> 3) & 1) << 2); }
 
-// Epilogue: the wave's 128 x 128 result, 64 columns at a time, through a 16 KB slab of the idle ring
+// Epilogue: the wave's 128 x 32 NPQ result, 16 NPQ columns at a time, through a 16 KB slab of the idle ring
 // (rows of 128 B, 16-byte slot s of row r at s ^ ((r / 2) % 8)) and out in whole 128-byte rows.
 // Register e of acc[i][j] in lane l is C[m0 + 16 i + l % 16][n0 + 16 j + 4 (l / 16) + e] (operands swapped).
-template <typename T>
-__device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32x4 (&acc)[8][8], unsigned char* lds,
+template <typename T, int NPQ>
+__device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32x4 (&acc)[8][2 * NPQ], unsigned char* lds,
                                                     int wave, int lane, int m0, int n0) {
   const int lr = lane & 15, lg = lane >> 4;
   const T* C = static_cast<const T*>(g.c);
@@ -64,11 +68,11 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
   T* D = static_cast<T*>(g.out);
 #pragma unroll
   for (int y = 0; y < 2; ++y) {
-    const int nh = n0 + y * 64;
-    float bias[4][4];
+    const int nh = n0 + y * (16 * NPQ);
+    float bias[NPQ][4];
     if (row_bias) {
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
+      for (int p = 0; p < NPQ; ++p) {
         const int n = nh + p * 16 + lg * 4;
         const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (n + 4 <= g.N ? n : 0));
 #pragma unroll
@@ -81,10 +85,10 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
       const int m = m0 + row;
       const int mc = m < g.M ? m : g.M - 1;
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
+      for (int p = 0; p < NPQ; ++p) {
         const int nl = p * 16 + lg * 4;
         const int n = nh + nl;
-        const f32x4 v = acc[i][y * 4 + p];
+        const f32x4 v = acc[i][y * NPQ + p];
         VecN4<T> r;
         if (row_bias) {
 #pragma unroll
@@ -123,7 +127,7 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
         const int row = chunk >> 3, s = chunk & 7;
         const u32x4 v = *reinterpret_cast<const u32x4*>(slab + row * 128 + ((s ^ ((row >> 1) & 7)) << 4));
         const int m = m0 + row, n = nh + s * 8;
-        if (m >= g.M || n >= g.N) continue;
+        if (m >= g.M || n >= g.N || s >= 2 * NPQ) continue;
         *reinterpret_cast<u32x4*>(D + (int64_t)m * g.N + n) = v;
       }
     } else {
@@ -133,64 +137,77 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
 #pragma unroll 8
       for (int row = 0; row < rows; ++row) {
         const T v = *reinterpret_cast<const T*>(slab + row * 128 + (((lane >> 3) ^ ((row >> 1) & 7)) << 4) + ((lane & 7) << 1));
-        if (n < g.N) D[(int64_t)(m0 + row) * g.N + n] = v;
+        if (n < g.N && lane < 16 * NPQ) D[(int64_t)(m0 + row) * g.N + n] = v;
       }
     }
   }
 }
 
-template <typename T, bool B_NN>
-__global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+// Fill requests.  x16_set_m0 sets the LDS base of the requests behind it; request i of a group of four
+// lands 1024 i bytes further (the instruction offset, which also moves the global address: the lane
+// offsets take it back out).
+__device__ __forceinline__ void x16_set_m0(uint32_t lds_byte_offset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" ::"s"(lds_byte_offset) : "memory");
+}
+template <int I>
+__device__ __forceinline__ void x16_fill(uint32_t lane_byte_offset, const void* base) {
+  asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" ::"v"(lane_byte_offset), "s"(base), "n"(1024 * I) : "memory");
+}
+constexpr int kXBias = 3072;  // the bases point this many bytes low, so that lane offset - 1024 i stays non-negative
+
+// NPQ = 4: a 256 x 256 tile.  NPQ = 3: a 256 x 192 tile on the same LDS layout and fill requests - a wave
+// owns 96 columns, 48 per half, its quadrants are 4 x 3 blocks (24 MFMAs), and the 16 columns per
+// half-wave that the B sub-panels hold beyond that are fetched (the next columns, clamped at the matrix
+// edge) and not used.  Such tiles let a last, partly filled round of tiles be cut to fit the chip.
+template <typename T, bool B_NN, int NPQ>
+__device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, const int bm, const int bn) {
+  static_assert(NPQ == 3 || NPQ == 4, "wave tile is 128 x 32 NPQ");
   using frag_t = typename Mfma16<T>::frag;
-  int tm, tn;
-  tile_coords(g, tm, tn);
-  const int bm = tm * BM, bn = tn * BN;
+  constexpr int WCOLS = 32 * NPQ, HCOLS = 16 * NPQ;  // columns per wave and per half
   const int tid = threadIdx.x, lane = tid % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave >> 1, wn = wave & 1;
-  const T* A = static_cast<const T*>(g.a);
-  const T* B = static_cast<const T*>(g.b);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
-  // Fill addresses: a uniform base per operand (moved along k by the requests) plus one 32-bit byte
-  // offset per lane, request and half (the host checks that they fit: leading dimensions below 4 M
-  // elements).  Request i of a sub-panel is its 1 KB region wave + 4 i: eight rows of a K-contiguous
-  // sub-panel (lane = row % 8 * 8 + chunk position) or four k-rows of a row-major one.
-  const T* a_base = A + (int64_t)bm * g.lda;
-  const T* b_base = B_NN ? B : B + (int64_t)bn * g.ldb;
+  // Fill addresses: a uniform base per operand (moved along k) plus one 32-bit byte offset per lane,
+  // request and half (the host checks that they fit: leading dimensions below 4 M elements).  A wave
+  // fills the four consecutive 1 KB regions 4 wave .. 4 wave + 3 of a sub-panel: eight rows each of a
+  // K-contiguous sub-panel (lane = row % 8 * 8 + chunk position), four k-rows of a row-major one.
+  const unsigned char* a_base = reinterpret_cast<const unsigned char*>(static_cast<const T*>(g.a) + (int64_t)bm * g.lda) - kXBias;
+  const unsigned char* b_base =
+      reinterpret_cast<const unsigned char*>(B_NN ? static_cast<const T*>(g.b) : static_cast<const T*>(g.b) + (int64_t)bn * g.ldb) - kXBias;
+  const int64_t a_step = 128;                                   // bytes per 64-k stage
+  const int64_t b_step = B_NN ? (int64_t)128 * g.ldb : 128;
   uint32_t a_off[2][4], b_off[2][4];
 #pragma unroll
   for (int x = 0; x < 2; ++x)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int r = 8 * (wave + 4 * i) + (lane >> 3);
+      const int r = 8 * (4 * wave + i) + (lane >> 3);
       const int c = (lane & 7) ^ ((r >> 1) & 7);
       int lr = (r >> 6) * 128 + x * 64 + (r & 63);  // rows of wave row r / 64, half x
       lr = bm + lr < g.M ? lr : g.M - 1 - bm;         // rows past M re-read the last row
-      a_off[x][i] = ((uint32_t)lr * (uint32_t)g.lda + (uint32_t)c * 8u) * 2u;
+      a_off[x][i] = ((uint32_t)lr * (uint32_t)g.lda + (uint32_t)c * 8u) * 2u + (uint32_t)(kXBias - 1024 * i);
       if constexpr (B_NN) {
-        const int k = 4 * (wave + 4 * i) + (lane >> 4), pos = lane & 15;
+        const int k = 4 * (4 * wave + i) + (lane >> 4), pos = lane & 15;
         const int cc = ((((pos >> 1) ^ xswz_seg(k)) << 1) | (pos & 1)) * 8;  // first of the 8 columns this lane fetches
-        int gn = bn + (cc >> 6) * 128 + x * 64 + (cc & 63);
+        int gn = bn + (cc >> 6) * WCOLS + x * HCOLS + (cc & 63);
         gn = gn < g.N ? gn : 0;
-        b_off[x][i] = ((uint32_t)k * (uint32_t)g.ldb + (uint32_t)gn) * 2u;
+        b_off[x][i] = ((uint32_t)k * (uint32_t)g.ldb + (uint32_t)gn) * 2u + (uint32_t)(kXBias - 1024 * i);
       } else {
-        int ln = (r >> 6) * 128 + x * 64 + (r & 63);
+        int ln = (r >> 6) * WCOLS + x * HCOLS + (r & 63);
         ln = bn + ln < g.N ? ln : g.N - 1 - bn;
-        b_off[x][i] = ((uint32_t)ln * (uint32_t)g.ldb + (uint32_t)c * 8u) * 2u;
+        b_off[x][i] = ((uint32_t)ln * (uint32_t)g.ldb + (uint32_t)c * 8u) * 2u + (uint32_t)(kXBias - 1024 * i);
       }
     }
-  // Request q (0..3: A, 4..7: B) of the pair that holds halves (x, y) of stage s, into the slot at slot_off.
-  auto request = [&](int q, int x, int y, int s, uint32_t slot_off) __attribute__((always_inline)) {
-    if (q < 4) {
-      lds_dma16s(lds_base + slot_off + (uint32_t)(wave + 4 * q) * 1024u, x ? a_off[1][q] : a_off[0][q], a_base + (int64_t)s * 64);
-    } else {
-      const int i = q - 4;
-      lds_dma16s(lds_base + slot_off + (uint32_t)kXSub + (uint32_t)(wave + 4 * i) * 1024u, y ? b_off[1][i] : b_off[0][i],
-                 b_base + (B_NN ? (int64_t)s * 64 * g.ldb : (int64_t)s * 64));
-    }
+  auto fill_i = [&](auto I_, const uint32_t (&vo)[4], const unsigned char* base) __attribute__((always_inline)) {
+    constexpr int I = decltype(I_)::value;
+    x16_fill<I>(vo[I], base);
   };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
 
   const int l16 = lane & 15, lg = lane >> 4;
   // Fragment (blk, s) of a set: 16 rows x 32 k, lane = (k group lg, row l16).
@@ -206,12 +223,12 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
     return __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   };
 
-  frag_t ra[2][2][4], rb[2][2][4];  // [half][32-k half of the stage][block]
-  f32x4 acc[8][8];
+  frag_t ra[2][2][4], rb[2][2][NPQ];  // [half][32-k half of the stage][block]
+  f32x4 acc[8][2 * NPQ];
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int j = 0; j < 2 * NPQ; ++j)
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
   // the zeros are written here, far ahead of the first MFMA that reads them (the compiler would
@@ -219,92 +236,126 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
 #pragma unroll
   for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) asm volatile("" : "+a"(acc[i][j]));
+    for (int j = 0; j < 2 * NPQ; ++j) asm volatile("" : "+a"(acc[i][j]));
 
-  // The MFMA as an asm statement: the accumulator block is tied to its AGPRs (with the builtin the
-  // register allocator rotates the 256 accumulators through copies and spills), and the "memory"
+  // The two MFMAs of a couple as one asm statement: the accumulator block is tied to its AGPRs (with the
+  // builtin the register allocator rotates the 256 accumulators through copies and spills), nothing
+  // comes between the two (the second takes its addend straight from the first), and the "memory"
   // clobber keeps the LDS reads and fill requests of a quadrant where they are written, between the
-  // MFMAs.  Back-to-back MFMAs on one accumulator block need no wait states; nothing else reads the
+  // couples.  Back-to-back MFMAs on one accumulator block need no wait states; nothing else reads the
   // accumulators before the epilogue.
-  auto mfma = [&](f32x4& c, const frag_t& b, const frag_t& a) __attribute__((always_inline)) {
+  auto mfma2 = [&](f32x4& c, const frag_t& b0, const frag_t& a0, const frag_t& b1, const frag_t& a1) __attribute__((always_inline)) {
     if constexpr (std::is_same<T, bf16_t>::value)
-      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(__builtin_bit_cast(u32x4, b)), "v"(__builtin_bit_cast(u32x4, a)) : "memory");
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %3, %4, %0"
+                   : "+a"(c)
+                   : "v"(__builtin_bit_cast(u32x4, b0)), "v"(__builtin_bit_cast(u32x4, a0)), "v"(__builtin_bit_cast(u32x4, b1)),
+                     "v"(__builtin_bit_cast(u32x4, a1))
+                   : "memory");
     else
-      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(__builtin_bit_cast(u32x4, b)), "v"(__builtin_bit_cast(u32x4, a)) : "memory");
+      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\tv_mfma_f32_16x16x32_f16 %0, %3, %4, %0"
+                   : "+a"(c)
+                   : "v"(__builtin_bit_cast(u32x4, b0)), "v"(__builtin_bit_cast(u32x4, a0)), "v"(__builtin_bit_cast(u32x4, b1)),
+                     "v"(__builtin_bit_cast(u32x4, a1))
+                   : "memory");
   };
 
   // One quadrant: 32 MFMAs on blocks (4 X + q, 4 Y + p), the two halves of the stage chained; the
   // operand whose set is the newer one runs in the outer loop, so its fragments are needed one by one.
   // LOAD: 0 nothing, 1 the A set into ra[LSET], 2 the B set into rb[LSET], read from the pair at `pair`
-  // in the order in which a later quadrant consumes them: one fragment behind every third MFMA of the
-  // first 24, and a fill request (first request FQ) behind every second fragment.
-  auto quadrant = [&](auto X_, auto Y_, auto AOUTER_, auto LOAD_, auto LSET_, const unsigned char* pair, bool fill, auto FQ_,
-                      int fx, int fy, int fs, uint32_t fslot) __attribute__((always_inline)) {
+  // in the order in which a later quadrant consumes them.  Memory instructions only go behind the
+  // second MFMA of a chained couple: the fragment reads behind the first couples, one each, and (FILL)
+  // the four requests of one sub-panel, base m0v, behind every second one of the last seven couples.
+  auto quadrant = [&](auto X_, auto Y_, auto AOUTER_, auto LOAD_, auto LSET_, auto FILL_, const unsigned char* pair, uint32_t m0v,
+                      const uint32_t (&vo)[4], const unsigned char* fbase) __attribute__((always_inline)) {
     constexpr int X = decltype(X_)::value, Y = decltype(Y_)::value, LOAD = decltype(LOAD_)::value, LSET = decltype(LSET_)::value;
-    constexpr int fq = decltype(FQ_)::value;
-    constexpr bool AOUTER = decltype(AOUTER_)::value;
+    constexpr bool AOUTER = decltype(AOUTER_)::value, FILL = decltype(FILL_)::value && !(MI355_X16_ABLATE & 1);
+    constexpr int NC = 4 * NPQ;  // couples
 #pragma unroll
-    for (int m = 0; m < 32; ++m) {
-      const int o = m >> 3, n = (m >> 1) & 3, s = m & 1;
-      const int q = AOUTER ? o : n, p = AOUTER ? n : o;
-      mfma(acc[4 * X + q][4 * Y + p], rb[Y][s][p], ra[X][s][q]);
-      if (m < 24 && m % 3 == 2) {
-        const int r = m / 3;  // fragment r of the set: block r / 2, half r % 2
-        if constexpr (LOAD == 1) {
+    for (int c = 0; c < NC; ++c) {
+      const int q = AOUTER ? c / NPQ : c % 4, p = AOUTER ? c % NPQ : c / 4;
+      mfma2(acc[4 * X + q][NPQ * Y + p], rb[Y][0][p], ra[X][0][q], rb[Y][1][p], ra[X][1][q]);
+      if (c < (LOAD == 2 ? 2 * NPQ : 8)) {
+        const int r = c;  // fragment r of the set: block r / 2, half r % 2
+        if constexpr ((MI355_X16_ABLATE & 4) != 0) {
+        } else if constexpr (LOAD == 1) {
           ra[LSET][r & 1][r >> 1] = read_k(pair, wm, r >> 1, r & 1);
         } else if constexpr (LOAD == 2) {
           if constexpr (B_NN) rb[LSET][r & 1][r >> 1] = read_n(pair + kXSub, r >> 1, r & 1);
           else rb[LSET][r & 1][r >> 1] = read_k(pair + kXSub, wn, r >> 1, r & 1);
         }
-        if ((r & 1) && fill) request(fq + (r >> 1), fx, fy, fs, fslot);
+      }
+      if constexpr (FILL) {
+        if (c == NC - 7) { x16_set_m0(m0v); fill_i(I0{}, vo, fbase); }
+        if (c == NC - 5) fill_i(I1{}, vo, fbase);
+        if (c == NC - 3) fill_i(I2{}, vo, fbase);
+        if (c == NC - 1) fill_i(I3{}, vo, fbase);
       }
     }
   };
 
   auto bump = [](uint32_t v) { return v + (uint32_t)kXPair == (uint32_t)(kXSlots * kXPair) ? 0u : v + (uint32_t)kXPair; };
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
-  using I4 = std::integral_constant<int, 4>;
 
   // Half-stage t = 4 u + HH (HH static: the register sets alternate with a period of two stages).
-  // Computes two quadrants of stage t / 2, reads pair t + 1 and requests pair t + 5 into the slot at
-  // `fl`.  The steps have no conditional parts: past the end of K the reads fetch a stale slot into
-  // registers nobody uses again and the requests fetch the last stage once more into slots nobody reads
-  // (four pairs per tile), so the accumulators never cross a branch between two MFMA statements - the
-  // compiler would be free to copy them there, and it does not know the wait states such a copy needs.
-  const int ns = g.K / 64;
+  // Computes two quadrants of stage t / 2, reads pair t + 1 (READ) and requests pair t + 5 (FILL; fa, fb:
+  // where its stage starts in a and b) into the slot at `fl`, then waits until at most WAIT requests
+  // are in flight (pair t + 2 is in) and meets the other waves (SYNC).  No branches between the MFMA
+  // statements: the compiler would be free to copy the accumulators there, and it does not know the
+  // wait states such a copy needs.
   uint32_t rd = kXPair, fl = 0;
-  auto half_stage = [&](auto HH_, int t) __attribute__((always_inline)) {
-    constexpr int HH = decltype(HH_)::value;
+  auto half_stage = [&](auto HH_, auto FILL_, auto READ_, auto WAIT_, auto SYNC_, const unsigned char* fa, const unsigned char* fb)
+                        __attribute__((always_inline)) {
+    constexpr int HH = decltype(HH_)::value, WAIT = decltype(WAIT_)::value;
+    constexpr bool READ = decltype(READ_)::value;
     constexpr int H = (HH >> 1) & 1;                      // parity of the stage being computed
     constexpr int XR = ((HH + 1) & 1) ? 1 - (((HH + 1) >> 1) & 1) : (((HH + 1) >> 1) & 1);  // A half held by pair t + 1
     constexpr int XF = ((HH + 5) & 1) ? 1 - (((HH + 5) >> 1) & 1) : (((HH + 5) >> 1) & 1);  // and by pair t + 5
     constexpr int YF = (HH + 5) & 1;
     using XRc = std::integral_constant<int, XR>;
-    const int fs = (t + 5) >> 1 < ns ? (t + 5) >> 1 : ns - 1;
+    using LA = std::integral_constant<int, READ ? 1 : 0>;
+    using LB = std::integral_constant<int, READ ? 2 : 0>;
     const unsigned char* pair = lds + rd;
+    const uint32_t m0a = lds_base + fl + (uint32_t)wave * 4096u, m0b = m0a + (uint32_t)kXSub;
     if constexpr ((HH & 1) == 0) {
       // first half of the stage: (B0, A_H) then (B0, A_(1-H)); pair t + 1 = {A_(1-H)(S), B1(S)}
-      quadrant(std::integral_constant<int, H>{}, I0{}, std::true_type{}, I1{}, XRc{}, pair, true, I0{}, XF, YF, fs, fl);
-      quadrant(std::integral_constant<int, 1 - H>{}, I0{}, std::true_type{}, I2{}, I1{}, pair, true, I4{}, XF, YF, fs, fl);
+      quadrant(std::integral_constant<int, H>{}, I0{}, std::true_type{}, LA{}, XRc{}, FILL_, pair, m0a, a_off[XF], fa);
+      quadrant(std::integral_constant<int, 1 - H>{}, I0{}, std::true_type{}, LB{}, I1{}, FILL_, pair, m0b, b_off[YF], fb);
     } else {
       // second half: (B1, A_(1-H)) then (B1, A_H); pair t + 1 = {A_h'(S+1), B0(S+1)}, h' = 1 - H
-      quadrant(std::integral_constant<int, 1 - H>{}, I1{}, std::false_type{}, I2{}, I0{}, pair, true, I4{}, XF, YF, fs, fl);
-      quadrant(std::integral_constant<int, H>{}, I1{}, std::false_type{}, I1{}, XRc{}, pair, true, I0{}, XF, YF, fs, fl);
+      quadrant(std::integral_constant<int, 1 - H>{}, I1{}, std::false_type{}, LB{}, I0{}, FILL_, pair, m0b, b_off[YF], fb);
+      quadrant(std::integral_constant<int, H>{}, I1{}, std::false_type{}, LA{}, XRc{}, FILL_, pair, m0a, a_off[XF], fa);
     }
-    asm volatile("s_waitcnt vmcnt(24)" ::: "memory");  // pair t + 2 is in: only the requests of pairs t + 3 .. t + 5 fly
-    __syncthreads();
+    if constexpr (WAIT == 24 && !(MI355_X16_ABLATE & 8)) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    if constexpr (WAIT == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    if constexpr (WAIT == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    if constexpr (WAIT == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if constexpr (decltype(SYNC_)::value && !(MI355_X16_ABLATE & 2)) __syncthreads();
     rd = bump(rd);
     fl = bump(fl);
   };
+  using W24 = std::integral_constant<int, 24>;
+  using W16 = std::integral_constant<int, 16>;
+  using W8 = std::integral_constant<int, 8>;
+  using W0 = std::integral_constant<int, 0>;
+  using WN = std::integral_constant<int, -1>;
+  using Yes = std::true_type;
+  using No = std::false_type;
 
   // Prologue: pairs 0..4 (K >= 256: they all exist); pairs 0 and 1 must be in before anything is read.
 #pragma unroll
   for (int gi = 0; gi < kXSlots; ++gi) {
     const int s = gi >> 1, second = gi & 1, h = s & 1;
-#pragma unroll
-    for (int q = 0; q < 8; ++q) request(q, second ? 1 - h : h, second, s, (uint32_t)gi * kXPair);
+    const int x = second ? 1 - h : h;
+    const uint32_t m0a = lds_base + (uint32_t)gi * kXPair + (uint32_t)wave * 4096u;
+    x16_set_m0(m0a);
+    fill_i(I0{}, a_off[x], a_base + s * a_step);
+    fill_i(I1{}, a_off[x], a_base + s * a_step);
+    fill_i(I2{}, a_off[x], a_base + s * a_step);
+    fill_i(I3{}, a_off[x], a_base + s * a_step);
+    x16_set_m0(m0a + (uint32_t)kXSub);
+    fill_i(I0{}, b_off[second], b_base + s * b_step);
+    fill_i(I1{}, b_off[second], b_base + s * b_step);
+    fill_i(I2{}, b_off[second], b_base + s * b_step);
+    fill_i(I3{}, b_off[second], b_base + s * b_step);
   }
   asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
   __syncthreads();
@@ -312,6 +363,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
   for (int q = 0; q < 4; ++q) {
     ra[0][0][q] = read_k(lds, wm, q, 0);
     ra[0][1][q] = read_k(lds, wm, q, 1);
+    if (q >= NPQ) continue;
     if constexpr (B_NN) {
       rb[0][0][q] = read_n(lds + kXSub, q, 0);
       rb[0][1][q] = read_n(lds + kXSub, q, 1);
@@ -322,23 +374,67 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
   }
   __syncthreads();  // every wave holds pair 0: its slot may be refilled
 
-  const int np = 2 * ns;  // ns is even (K % 128 == 0): whole pairs of stages
-  for (int t = 0; t < np; t += 4) {
-    half_stage(I0{}, t);
-    half_stage(I1{}, t + 1);
-    half_stage(I2{}, t + 2);
-    half_stage(std::integral_constant<int, 3>{}, t + 3);
+  // Half-stages t .. t + 3 request pairs t + 5 .. t + 8 = stages t / 2 + 2, + 3, + 3, + 4.
+  const int np = g.K / 32;  // pairs = half-stages; a multiple of 4 (K % 128 == 0), at least 8
+  const unsigned char* fa = a_base + 2 * a_step;
+  const unsigned char* fb = b_base + 2 * b_step;
+  int t = 0;
+  for (; t + 8 < np; t += 4) {
+    half_stage(I0{}, Yes{}, Yes{}, W24{}, Yes{}, fa, fb);
+    half_stage(I1{}, Yes{}, Yes{}, W24{}, Yes{}, fa + a_step, fb + b_step);
+    half_stage(I2{}, Yes{}, Yes{}, W24{}, Yes{}, fa + a_step, fb + b_step);
+    half_stage(I3{}, Yes{}, Yes{}, W24{}, Yes{}, fa + 2 * a_step, fb + 2 * b_step);
+    fa += 2 * a_step;
+    fb += 2 * b_step;
   }
-  // the surplus requests still land in the ring, which the epilogue reuses; the last MFMA's result is
-  // read by VALU moves next
-  asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-  __syncthreads();
-  store_tile_result16<T>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * 128);
+  // The last two pairs of stages: the requests run out (pairs np - 3 .. np - 1 are the last), then the reads.
+  half_stage(I0{}, Yes{}, Yes{}, W24{}, Yes{}, fa, fb);
+  half_stage(I1{}, Yes{}, Yes{}, W24{}, Yes{}, fa + a_step, fb + b_step);
+  half_stage(I2{}, Yes{}, Yes{}, W24{}, Yes{}, fa + a_step, fb + b_step);
+  half_stage(I3{}, No{}, Yes{}, W16{}, Yes{}, fa, fb);
+  half_stage(I0{}, No{}, Yes{}, W8{}, Yes{}, fa, fb);
+  half_stage(I1{}, No{}, Yes{}, W0{}, Yes{}, fa, fb);
+  half_stage(I2{}, No{}, Yes{}, WN{}, Yes{}, fa, fb);
+  half_stage(I3{}, No{}, No{}, WN{}, No{}, fa, fb);
+  // the last MFMA's result is read by VALU moves next; every wave is past its last LDS read (the barrier
+  // that ended the half-stage before the last) and no request is in flight, so the ring is free
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  store_tile_result16<T, NPQ>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS);
+}
+
+template <typename T, bool B_NN>
+__global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  x16_tile<T, B_NN, 4>(g, lds, tm * BM, tn * BN);
+}
+
+// Two tile widths in one launch: blocks [0, tiles_m * tiles_n) are 256 x 256 tiles of the columns
+// [0, 256 tiles_n); the blocks behind them are 256 x 192 tiles of the columns from there on (tiles_m *
+// tail_n of them).  Workgroups are dispatched in block order, so the narrow tiles form the last round.
+template <typename T, bool B_NN>
+__global__ __launch_bounds__(256) void gemm_mfma_x16_mixed_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int wide = g.tiles_m * g.tiles_n;
+  int tm, tn;
+  if ((int)blockIdx.x < wide) {
+    tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
+    x16_tile<T, B_NN, 4>(g, lds, tm * BM, tn * BN);
+  } else {
+    tile_coords(g.tiles_m, g.tail_n, blockIdx.x - wide, tm, tn);
+    x16_tile<T, B_NN, 3>(g, lds, tm * BM, g.tiles_n * BN + tn * 192);
+  }
 }
 
 const void* gemm_x16_kernel(bool is_bf16, bool b_nn) {
   if (is_bf16) return b_nn ? (const void*)gemm_mfma_x16_kernel<bf16_t, true> : (const void*)gemm_mfma_x16_kernel<bf16_t, false>;
   return b_nn ? (const void*)gemm_mfma_x16_kernel<f16_t, true> : (const void*)gemm_mfma_x16_kernel<f16_t, false>;
+}
+
+const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn) {
+  if (is_bf16) return b_nn ? (const void*)gemm_mfma_x16_mixed_kernel<bf16_t, true> : (const void*)gemm_mfma_x16_mixed_kernel<bf16_t, false>;
+  return b_nn ? (const void*)gemm_mfma_x16_mixed_kernel<f16_t, true> : (const void*)gemm_mfma_x16_mixed_kernel<f16_t, false>;
 }
 
 }  // namespace mi355

@@ -204,6 +204,48 @@ def test_mixed_width_tile_grid(backend, layout, monkeypatch):
         assert ev.bit_equal(ref[:, edge - 8:edge + 200], mixed[rows.cuda()][:, edge - 8:edge + 200].cpu())  # across the seam
 
 
+@pytest.mark.parametrize("tile", ["x16", "x16mixed", "planner"])
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+def test_x16_gemm_every_k_loop_length(backend, layout, tile, monkeypatch):
+    """The 256x256-tile kernel on v_mfma_f32_16x16x32 (the planner's choice for products that fill the chip
+    when K is a multiple of 128 from 512 on): [4104, K] x [K, 4500] has 17 x 18 tiles with a ragged last tile
+    row and column; K walks from the shortest loop the kernel takes (two pairs of stages: only the peeled
+    end of the pipeline) through every count of steady-state iterations up to 4096.  MI355_GEMM_TILE=x16
+    forces the kernel for every K, =x16mixed its two-width grid (192-wide tiles behind the 256-wide ones:
+    the seam is checked), and "planner" leaves the choice to the library.  Small-integer operands make the
+    fp32 accumulation exact, so sampled rows must be bit-equal to the oracle's; a bias row and an f16 run go
+    through the same epilogue."""
+    import ctypes
+
+    from backendbench_amd import _lib
+    announce(f"16x16x32 GEMM K loop lengths, {layout}, {tile}")
+    M, N = 4104, 4500
+    wide, narrow = ctypes.c_int32(), ctypes.c_int32()
+    assert _lib.load().mi355_gemm_tile_columns(M, N, 4096, ctypes.byref(wide), ctypes.byref(narrow)) == 0
+    assert narrow.value > 0
+    edge = wide.value * 256
+    g = torch.Generator().manual_seed(13)
+    rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 63, 64, 127, 128, 255, 256, 4095, 4096, 4103])]))
+    for K in (256, 384, 512, 640, 768, 896, 1024, 1152, 1280, 2048, 4096):
+        a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+        if layout[1] == "t":
+            b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
+        else:
+            b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
+        bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
+        if tile != "planner":
+            monkeypatch.setenv("MI355_GEMM_TILE", tile)
+        out = backend[aten.addmm.default](bias, a, b)
+        half = backend[aten.mm.default](a.half(), b.half())
+        if tile != "planner":
+            monkeypatch.delenv("MI355_GEMM_TILE")
+        ref = aten_cpu.reference(aten.addmm.default, [bias, a[rows.cuda()], b])
+        assert ev.bit_equal(ref, out[rows.cuda()].cpu()), (layout, tile, K)
+        assert ev.bit_equal(ref[:, edge - 8:edge + 200], out[rows.cuda()][:, edge - 8:edge + 200].cpu()), (layout, tile, K, "seam")
+        ref16 = aten_cpu.reference(aten.mm.default, [a.half()[rows.cuda()], b.half()])
+        assert ev.bit_equal(ref16, half[rows.cuda()].cpu()), (layout, tile, K, "f16")
+
+
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
 @pytest.mark.parametrize("shape", [(704, 900), (2000, 2500)])
 def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
