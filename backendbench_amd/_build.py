@@ -65,14 +65,14 @@ TRACE_LIB_PATH = LIB_DIR / "libmi355_gemm_trace.so"
 
 
 def build_trace(verbose: bool = True) -> Path:
-    """The GEMM source once more with -DMI355_GEMM_TRACE: the four-wave kernels then stamp the
+    """The GEMM sources once more with -DMI355_GEMM_TRACE: the four-wave kernels then stamp the
     shader clock (s_memtime) around the phases of every tile and of every step of the K loop and
     leave the sums in the caller's workspace (layout beside the stamps in csrc/gemm.hip).  A
     diagnostic build of its own, read by `bench.py --only-op C3.mm_down --trace`; the product
     library carries no stamps."""
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     objs = []
-    for src, extra in (("gemm.hip", ["-DMI355_GEMM_TRACE"]), ("common.hip", [])):
+    for src, extra in (("gemm.hip", ["-DMI355_GEMM_TRACE"]), ("gemm_x16.hip", ["-DMI355_GEMM_TRACE"]), ("common.hip", [])):
         obj = OBJ_DIR / (Path(src).stem + ".trace.o")
         proc = subprocess.run([HIPCC, *FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)], capture_output=True, text=True)
         if proc.returncode != 0:

@@ -192,6 +192,75 @@ __global__ __launch_bounds__(256) void calib_mfma16q_kernel(const F* __restrict_
   out[lane_slot] = sum;
 }
 
+// The same quadrant walk with the MFMAs as asm statements, so that their order is exactly the written one:
+// MODE 0: the two MFMAs on an accumulator block back to back; 1: an s_nop between the two; 2: two blocks
+// interleaved (a0 b0 a1 b1: the addend comes from the MFMA before the last); 3: all first halves of a
+// quadrant, then all second halves (the addend is 16 MFMAs old); 4: as 1 with three s_nop.
+template <typename F, int MODE>
+__global__ __launch_bounds__(256) void calib_mfma16a_kernel(const F* __restrict__ a, const F* __restrict__ b, float* __restrict__ out, int steps) {
+  typedef uint32_t cu32x4 __attribute__((ext_vector_type(4)));
+  const int64_t lane_slot = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  cu32x4 xa[2][4], xb[2][4];
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      xa[s][i] = __builtin_bit_cast(cu32x4, a[lane_slot * 16 + s * 4 + i]);
+      xb[s][i] = __builtin_bit_cast(cu32x4, b[lane_slot * 16 + s * 4 + i]);
+    }
+  cf32x4 acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+      asm volatile("" : "+a"(acc[i][j]));
+    }
+  constexpr bool BF = sizeof(a[0][0]) == 2 && !__is_same(F, cf16x8);
+#define MI355_CALIB_M(C, B_, A_)                                                                                    \
+  if constexpr (BF) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(C) : "v"(B_), "v"(A_));        \
+  else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(C) : "v"(B_), "v"(A_));
+  for (int t = 0; t < steps; t += 2) {
+#pragma unroll
+    for (int quad = 0; quad < 4; ++quad) {
+      const int i0 = (quad >> 1) * 4, j0 = (quad & 1) * 4;
+      if constexpr (MODE == 3) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int c = 0; c < 16; ++c) { MI355_CALIB_M(acc[i0 + (c & 3)][j0 + (c >> 2)], xb[s][c >> 2], xa[s][c & 3]) }
+      } else if constexpr (MODE == 2) {
+#pragma unroll
+        for (int c = 0; c < 16; c += 2) {
+          MI355_CALIB_M(acc[i0 + (c & 3)][j0 + (c >> 2)], xb[0][c >> 2], xa[0][c & 3])
+          MI355_CALIB_M(acc[i0 + ((c + 1) & 3)][j0 + (c >> 2)], xb[0][c >> 2], xa[0][(c + 1) & 3])
+          MI355_CALIB_M(acc[i0 + (c & 3)][j0 + (c >> 2)], xb[1][c >> 2], xa[1][c & 3])
+          MI355_CALIB_M(acc[i0 + ((c + 1) & 3)][j0 + (c >> 2)], xb[1][c >> 2], xa[1][(c + 1) & 3])
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < 16; ++c) {
+          MI355_CALIB_M(acc[i0 + (c & 3)][j0 + (c >> 2)], xb[0][c >> 2], xa[0][c & 3])
+          if constexpr (MODE == 1) asm volatile("s_nop 0");
+          if constexpr (MODE == 4) asm volatile("s_nop 0\n\ts_nop 0\n\ts_nop 0");
+          MI355_CALIB_M(acc[i0 + (c & 3)][j0 + (c >> 2)], xb[1][c >> 2], xa[1][c & 3])
+        }
+      }
+    }
+  }
+#undef MI355_CALIB_M
+  asm volatile("s_nop 15\n\ts_nop 15");
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sum += acc[i][j][e];
+  out[lane_slot] = sum;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -201,13 +270,15 @@ using namespace mi355;
 // (blocks * 256 * 256 bytes each); out: blocks * 256 floats.  variant 0..2: 32x32x16 in the three
 // operand orders, 3: 16x16x32, 4 / 5: 32x32x16 with the MFMAs on one accumulator block chained in
 // fours / twos, 6: 16x16x32 chained in twos, 7 / 8 / 9: 16x16x32 walked quadrant by quadrant in chains
-// of 1 / 2 / 4 (steps % 4 == 0).
+// of 1 / 2 / 4 (steps % 4 == 0), 10 .. 14: the quadrant walk in chains of two as asm statements in exactly
+// the written order: back to back / an s_nop between the two / two blocks interleaved / all first halves
+// then all second halves / three s_nop between the two.
 extern "C" int mi355_calib_mfma(const void* a, const void* b, void* out, int dtype, int blocks, int steps, int variant,
                                 void* stream) {
   MI355_REQUIRE(a != nullptr && b != nullptr && out != nullptr, "mi355_calib_mfma: NULL buffer");
   MI355_REQUIRE(blocks > 0 && steps > 0 && steps % 4 == 0, "mi355_calib_mfma: blocks > 0 and a number of steps divisible by four");
   MI355_REQUIRE(dtype == MI355_BF16 || dtype == MI355_F16, "mi355_calib_mfma: bf16 or f16");
-  MI355_REQUIRE(variant >= 0 && variant <= 9, "mi355_calib_mfma: variant 0..9");
+  MI355_REQUIRE(variant >= 0 && variant <= 14, "mi355_calib_mfma: variant 0..14");
   hipStream_t st = static_cast<hipStream_t>(stream);
   float* o = static_cast<float*>(out);
 #define MI355_CALIB(F_)                                                                                                        \
@@ -224,7 +295,12 @@ extern "C" int mi355_calib_mfma(const void* a, const void* b, void* out, int dty
       case 6: hipLaunchKernelGGL((calib_mfma16_kernel<F_, true>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;    \
       case 7: hipLaunchKernelGGL((calib_mfma16q_kernel<F_, 1>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;      \
       case 8: hipLaunchKernelGGL((calib_mfma16q_kernel<F_, 2>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;      \
-      default: hipLaunchKernelGGL((calib_mfma16q_kernel<F_, 4>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;     \
+      case 9: hipLaunchKernelGGL((calib_mfma16q_kernel<F_, 4>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;      \
+      case 10: hipLaunchKernelGGL((calib_mfma16a_kernel<F_, 0>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;     \
+      case 11: hipLaunchKernelGGL((calib_mfma16a_kernel<F_, 1>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;     \
+      case 12: hipLaunchKernelGGL((calib_mfma16a_kernel<F_, 2>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;     \
+      case 13: hipLaunchKernelGGL((calib_mfma16a_kernel<F_, 3>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;     \
+      default: hipLaunchKernelGGL((calib_mfma16a_kernel<F_, 4>), dim3(blocks), dim3(256), 0, st, pa, pb, o, steps); break;     \
     }                                                                                                                          \
   }
   if (dtype == MI355_BF16) MI355_CALIB(cbf16x8) else MI355_CALIB(cf16x8)

@@ -6,6 +6,9 @@
 //            are bank-conflict free.  A row-major B stays N-contiguous in LDS and is transposed
 //            by the LDS read itself (ds_read_b64_tr_b16).  Block -> tile map groups tiles per
 //            XCD so that one L2 serves neighbouring tiles.  By K:
+//              gemm_mfma_x16_kernel    (gemm_x16.hip) K % 128 == 0, K >= 512, a K-contiguous: four
+//                                      waves of 128x128 on v_mfma_f32_16x16x32, the form the power
+//                                      envelope favours;
 //              gemm_mfma_w4_kernel     K % 64 == 0, K >= 2048: four waves of 128x128, fragments
 //                                      read a step ahead, fills issued one at a time;
 //              gemm_mfma_dma64_kernel  K % 64 == 0: eight waves of 128x64 (two per SIMD), A
@@ -29,7 +32,8 @@ namespace mi355 {
 
 
 // v_mfma_f32_32x32x16: measured at ~96 % of the 2.5 PFLOP/s bf16 peak on MI355X when issued
-// back to back; the 16x16x32 form tops out near 60 %, so the 32x32 form is the only one used.
+// back to back on all-zero operands.  (The 16x16x32 form issues at the same rate and draws less power
+// on real operand data; the kernels of this file predate that measurement, gemm_x16.hip uses it.)
 // Operand layout: lane l holds 8 consecutive k (k = (l/32)*8 + e) of row/column l%32; the
 // 32x32 result puts column l%32 and rows 8*(r/4) + (l/32)*4 + r%4 in register r of lane l.
 template <typename T> struct Mfma;

@@ -168,6 +168,20 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave >> 1, wn = wave & 1;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+#ifdef MI355_GEMM_TRACE
+  // Diagnostic build only (-DMI355_GEMM_TRACE, libmi355_gemm_trace.so): shader-clock stamps (s_memtime,
+  // read behind the next barrier's wait, so no wait is added).  Lane 0 of every wave leaves 16 uint64 in
+  // the caller's workspace at ((block * 4 + wave) * 16), the layout of the stamps in gemm.hip:
+  //   [0..5]  sums over the half-stages that end in a wait and a barrier (all but the last two), for the
+  //           even and the odd ones: ticks issuing the half-stage's MFMAs / reads / requests, ticks in
+  //           s_waitcnt for the requests, ticks from there to behind the barrier;
+  //   [6] ticks in the K loop   [7] pairs of half-stages summed
+  //   [10] stamp at loop entry   [11] HW_ID   [12] stamp at tile entry   [13], [14] at the end of the
+  //   K loop   [15] when the tile's stores have completed.
+  const uint64_t tr_entry = __builtin_readcyclecounter();
+  uint64_t tr_sum[6] = {0, 0, 0, 0, 0, 0};
+  uint64_t tr_start[2] = {0, 0}, tr_p2_prev = 0, tr_pairs = 0;
+#endif
 
   // Fill addresses: a uniform base per operand (moved along k) plus one 32-bit byte offset per lane,
   // request and half (the host checks that they fit: leading dimensions below 4 M elements).  A wave
@@ -324,11 +338,36 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       quadrant(std::integral_constant<int, 1 - H>{}, I1{}, std::false_type{}, LB{}, I0{}, FILL_, pair, m0b, b_off[YF], fb);
       quadrant(std::integral_constant<int, H>{}, I1{}, std::false_type{}, LA{}, XRc{}, FILL_, pair, m0a, a_off[XF], fa);
     }
+#ifdef MI355_GEMM_TRACE
+    if constexpr (decltype(SYNC_)::value && WAIT >= 0) {
+      // wait, barrier and three stamps in one statement: the two stamps in front of the barrier have arrived
+      // behind its lgkmcnt(0); the one behind it is read a half-stage later (tr_start alternates between
+      // two scalars, so it is never copied before it has arrived)
+      constexpr int par = HH & 1;
+      uint64_t p1, p2;
+#define MI355_TR_END(N)                                                                                                 \
+  asm volatile("s_memtime %0\n\ts_waitcnt vmcnt(" #N ")\n\ts_memtime %1\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier\n\ts_memtime %2" \
+               : "=s"(p1), "=s"(p2), "=s"(tr_start[1 - par]) : "s"(tr_start[par]) : "memory");
+      if constexpr (WAIT == 24) MI355_TR_END(24)
+      if constexpr (WAIT == 16) MI355_TR_END(16)
+      if constexpr (WAIT == 8) MI355_TR_END(8)
+      if constexpr (WAIT == 0) MI355_TR_END(0)
+#undef MI355_TR_END
+      tr_sum[par * 3 + 0] += p1 - tr_start[par];
+      tr_sum[par * 3 + 1] += p2 - p1;
+      if (tr_p2_prev != 0) tr_sum[(1 - par) * 3 + 2] += tr_start[par] - tr_p2_prev;
+      tr_p2_prev = p2;
+      tr_pairs += par;
+    } else {
+      if constexpr (decltype(SYNC_)::value) __syncthreads();
+    }
+#else
     if constexpr (WAIT == 24 && !(MI355_X16_ABLATE & 8)) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
     if constexpr (WAIT == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     if constexpr (WAIT == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     if constexpr (WAIT == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     if constexpr (decltype(SYNC_)::value && !(MI355_X16_ABLATE & 2)) __syncthreads();
+#endif
     rd = bump(rd);
     fl = bump(fl);
   };
@@ -378,6 +417,10 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
   const int np = g.K / 32;  // pairs = half-stages; a multiple of 4 (K % 128 == 0), at least 8
   const unsigned char* fa = a_base + 2 * a_step;
   const unsigned char* fb = b_base + 2 * b_step;
+#ifdef MI355_GEMM_TRACE
+  const uint64_t tr_begin = __builtin_readcyclecounter();
+  tr_start[0] = tr_begin;
+#endif
   int t = 0;
   for (; t + 8 < np; t += 4) {
     half_stage(I0{}, Yes{}, Yes{}, W24{}, Yes{}, fa, fb);
@@ -399,7 +442,23 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
   // the last MFMA's result is read by VALU moves next; every wave is past its last LDS read (the barrier
   // that ended the half-stage before the last) and no request is in flight, so the ring is free
   asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#ifdef MI355_GEMM_TRACE
+  const uint64_t tr_end = __builtin_readcyclecounter();
+#endif
   store_tile_result16<T, NPQ>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS);
+#ifdef MI355_GEMM_TRACE
+  {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const uint64_t tr_stored = __builtin_readcyclecounter();
+    if (lane == 0 && g.ws != nullptr) {
+      uint64_t* o = reinterpret_cast<uint64_t*>(g.ws) + ((int64_t)blockIdx.x * 4 + wave) * 16;
+      for (int q = 0; q < 6; ++q) o[q] = tr_sum[q];
+      o[6] = tr_end - tr_begin; o[7] = tr_pairs; o[8] = 0; o[9] = 0; o[10] = tr_begin;
+      o[11] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));  // HW_REG_HW_ID (XCC / SE / CU of this wave)
+      o[12] = tr_entry; o[13] = tr_end; o[14] = tr_end; o[15] = tr_stored;
+    }
+  }
+#endif
 }
 
 template <typename T, bool B_NN>

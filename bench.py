@@ -50,8 +50,10 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy")
     ap.add_argument("--variant", type=int, default=0,
-                    help="with --only-op calib.mfma: 0 = the mm kernel's MFMA order, 1 = operands swapped between the "
-                         "ports, 2 = the other operand held across MFMAs, 3 = v_mfma_f32_16x16x32")
+                    help="with --only-op calib.mfma: 0 = the 32x32x16 mm kernels' MFMA order, 1 = operands swapped between the "
+                         "ports, 2 = the other operand held across MFMAs, 3 = v_mfma_f32_16x16x32, 4-9 = chained "
+                         "accumulator updates, 10 = the 16x16x32 mm kernel's stream, 11-14 = its reorderings "
+                         "(see mi355_calib_mfma in include/mi355_aten.h)")
     ap.add_argument("--trace", action="store_true",
                     help="with --only-op C3.mm_up|C3.mm_down: run the cycle-stamped diagnostic build of the GEMM "
                          "(libmi355_gemm_trace.so) and print where a tile's shader-clock ticks go")
@@ -341,10 +343,13 @@ def calib_mfma(dev, fill=None, variant=0, blocks=256, steps=2752, launches=20):
 
 
 def gemm_trace(case, dev, fill=None):
-    """One mm of this row through the stamped diagnostic build (see the MI355_GEMM_TRACE block in
-    csrc/gemm.hip for the record layout): mean shader-clock ticks per phase of a tile and per step
-    of the K loop, the gap between two tiles on one CU, and ticks per microsecond of kernel time
-    (the average shader clock, which is what moves with the operand data)."""
+    """One mm of this row through the stamped diagnostic build (see the MI355_GEMM_TRACE blocks in
+    csrc/gemm_x16.hip and csrc/gemm.hip for the record layout): mean shader-clock ticks per phase of a
+    tile and per pair of steps of the K loop (a step = 32 k: a half-stage of the 16x16x32 kernel, 64
+    MFMAs of 16 clocks, or a step of the 32x32x16 kernels, 32 MFMAs of 32 clocks), the gap between two
+    tiles on one CU, and ticks per microsecond of kernel time (the average shader clock, which is
+    what moves with the operand data).  MI355_GEMM_WAVES=4 in the environment selects the
+    32x32x16 four-wave kernel instead of the 16x16x32 one."""
     import ctypes
 
     import numpy as np

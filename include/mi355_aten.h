@@ -210,11 +210,15 @@ int mi355_gemm_tile_columns(int64_t M, int64_t N, int64_t K, int32_t* wide, int3
 
 /* Measurement only, no counterpart in the reference: the matrix-core instruction stream of the
  * large-tile mm kernel (per wave a 128 x 128 fp32 register tile, 32 v_mfma_f32_32x32x16 per 32-k
- * step) with no memory traffic in the loop.  `blocks` workgroups of four waves run `steps` (even)
- * steps on operand fragments loaded once from a and b (16 fragments of 16 bytes per thread each:
+ * step) with no memory traffic in the loop.  `blocks` workgroups of four waves run `steps` (a
+ * multiple of four) steps on operand fragments loaded once from a and b (16 fragments of 16 bytes per thread each:
  * blocks * 65536 bytes; the caller chooses the data), out receives blocks * 256 floats.  Work:
  * blocks * 4 * steps * 2 * 128 * 128 * 32 flop.  variant 0: the mm kernel's operand order; 1: operands
- * swapped between the two ports; 2: the other operand held across MFMAs; 3: v_mfma_f32_16x16x32.
+ * swapped between the two ports; 2: the other operand held across MFMAs; 3: v_mfma_f32_16x16x32;
+ * 4 / 5: 32x32x16 with the MFMAs on one accumulator block in chains of four / two; 6 - 9: 16x16x32 in
+ * chains (whole tile / quadrant by quadrant in chains of 1, 2, 4); 10 - 14: the 16x16x32 stream of the
+ * mm kernel in exactly the written order (asm statements): chains of two back to back (10), with one
+ * (11) or three (14) s_nop between the two, two blocks interleaved (12), first halves then second halves (13).
  * Its sustained rate on a given data distribution is the ceiling the power / clock envelope leaves to
  * mi355_gemm on that data. */
 int mi355_calib_mfma(const void* a, const void* b, void* out, int dtype, int blocks, int steps,
