@@ -2101,13 +2101,16 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
       // with 256x256 tiles when K is a multiple of 128: measured against the 32x32x16 form on
       // [4096,K]x[K,16384], it is level at K = 512 and 4 - 15 % faster from K = 768 on (C3: [4096,4096]x
-      // [4096,11008] 306 -> 279 us, [4096,11008]x[11008,4096] 270 -> 249 us).  MI355_GEMM_TILE=x16
-      // forces it for any tile count (=x16mixed: with the mixed-width grid at any K), =256x256 / =mixed keep
+      // [4096,11008] 306 -> 279 us, [4096,11008]x[11008,4096] 270 -> 249 us).  With a short K and output
+      // rows that do not start on 128-byte lines (N % 64 != 0) the eight-wave kernel's epilogue is the
+      // faster one ([4096,768]x[768,50264]: 404 us against 436 us here).  MI355_GEMM_TILE=x16 forces this
+      // form for any tile count (=x16mixed: with the mixed-width grid at any K), =256x256 / =mixed keep
       // the 32x32x16 form (test knobs).
       const bool x16_ok = K % 128 == 0 && K >= 256 && !a_t && ld32;
       const bool x16_mixed_forced = forced_tile != nullptr && strcmp(forced_tile, "x16mixed") == 0;  // mixed widths at any K
       const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced
-                                                         : K >= 512 && nblocks >= kNumCU * 3 / 4 && !mid && !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
+                                                         : K >= 512 && (K >= 2048 || N % 64 == 0) && nblocks >= kNumCU * 3 / 4 && !mid &&
+                                                               !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
       if (x16) {
         kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
         threads = 256;

@@ -66,11 +66,14 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
   const bool row_bias = use_c && g.c_vec && g.c_rs == 0;
   unsigned char* slab = lds + wave * (128 * 128);
   T* D = static_cast<T*>(g.out);
-#pragma unroll
-  for (int y = 0; y < 2; ++y) {
+  const bool inside = NPQ == 4 && m0 + 128 <= g.M && n0 + 128 <= g.N;  // no row or column of this wave's tile is cut
+  // MODE 0: alpha * acc; 1: + beta * a bias row (loaded once per 64 columns); 2: + beta * c.  The mode is
+  // chosen once per call, outside the loops over the accumulator blocks.
+  auto half = [&](auto MODE_, int y) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(MODE_)::value;
     const int nh = n0 + y * (16 * NPQ);
     float bias[NPQ][4];
-    if (row_bias) {
+    if constexpr (MODE == 1) {
 #pragma unroll
       for (int p = 0; p < NPQ; ++p) {
         const int n = nh + p * 16 + lg * 4;
@@ -79,56 +82,66 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
         for (int e = 0; e < 4; ++e) bias[p][e] = g.beta * static_cast<float>(t.v[e]);
       }
     }
+    unsigned char* wr = slab + lr * 128 + (lg & 1) * 8;
+    const int sx = (lr >> 1) & 7;  // = (row / 2) % 8 for every row 16 i + lr
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int row = i * 16 + lr;
-      const int m = m0 + row;
+      const int m = m0 + i * 16 + lr;
       const int mc = m < g.M ? m : g.M - 1;
 #pragma unroll
       for (int p = 0; p < NPQ; ++p) {
         const int nl = p * 16 + lg * 4;
         const int n = nh + nl;
-        const f32x4 v = acc[i][y * NPQ + p];
+        const f32x4 v = acc[i][(y ? NPQ : 0) + p];
         VecN4<T> r;
-        if (row_bias) {
+        if constexpr (MODE == 0) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) r.v[e] = static_cast<T>(g.alpha * v[e]);
+        } else if constexpr (MODE == 1) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) r.v[e] = static_cast<T>(g.alpha * v[e] + bias[p][e]);
         } else {
-          float cv[4] = {0.f, 0.f, 0.f, 0.f};  // columns past N are computed on valid addresses and never stored
-          if (use_c) {
-            if (g.c_vec) {
-              const int nv = n + 4 <= g.N ? n : 0;
-              const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (int64_t)mc * g.c_rs + nv);
+          float cv[4];  // columns past N are computed on valid addresses and never stored
+          if (g.c_vec) {
+            const int nv = n + 4 <= g.N ? n : 0;
+            const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (int64_t)mc * g.c_rs + nv);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(t.v[e]);
-            } else {
+            for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(t.v[e]);
+          } else {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int ne = n + e < g.N ? n + e : g.N - 1;
-                cv[e] = static_cast<float>(C[(int64_t)mc * g.c_rs + (int64_t)ne * g.c_cs]);
-              }
+            for (int e = 0; e < 4; ++e) {
+              const int ne = n + e < g.N ? n + e : g.N - 1;
+              cv[e] = static_cast<float>(C[(int64_t)mc * g.c_rs + (int64_t)ne * g.c_cs]);
             }
           }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float s = g.alpha * v[e];
-            r.v[e] = static_cast<T>(use_c ? s + g.beta * cv[e] : s);
-          }
+          for (int e = 0; e < 4; ++e) r.v[e] = static_cast<T>(g.alpha * v[e] + g.beta * cv[e]);
         }
-        const int slot = (nl >> 3) ^ ((row >> 1) & 7);
-        *reinterpret_cast<VecN4<T>*>(slab + row * 128 + slot * 16 + (lg & 1) * 8) = r;
+        *reinterpret_cast<VecN4<T>*>(wr + i * (16 * 128) + (((p * 2 + (lg >> 1)) ^ sx) << 4)) = r;
       }
     }
     // same wave wrote and reads: LDS operations of a wave complete in order
     if (g.out_vec) {
+      const int s = lane & 7, r0 = lane >> 3;  // 16-byte chunk s of rows r0 + 8 t
+      const unsigned char* rdp = slab + r0 * 128;
+      T* dst = D + (int64_t)(m0 + r0) * g.N + nh + s * 8;
+      if (inside) {
 #pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        const int chunk = t * kWave + lane;  // 1024 chunks of 16 bytes, 8 per row
-        const int row = chunk >> 3, s = chunk & 7;
-        const u32x4 v = *reinterpret_cast<const u32x4*>(slab + row * 128 + ((s ^ ((row >> 1) & 7)) << 4));
-        const int m = m0 + row, n = nh + s * 8;
-        if (m >= g.M || n >= g.N || s >= 2 * NPQ) continue;
-        *reinterpret_cast<u32x4*>(D + (int64_t)m * g.N + n) = v;
+        for (int t = 0; t < 16; ++t) {
+          const int row = r0 + 8 * t;  // (row / 2) % 8 = (r0 / 2 + 4 t) % 8
+          const u32x4 v = *reinterpret_cast<const u32x4*>(rdp + t * 1024 + ((s ^ (((r0 >> 1) + 4 * t) & 7)) << 4));
+          if ((MI355_X16_ABLATE & 16) && v[0] != 0x12345678u) continue;
+          *reinterpret_cast<u32x4*>(dst + (int64_t)(8 * t) * g.N) = v;
+          (void)row;
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+          const int row = r0 + 8 * t;
+          const u32x4 v = *reinterpret_cast<const u32x4*>(rdp + t * 1024 + ((s ^ ((row >> 1) & 7)) << 4));
+          if (m0 + row >= g.M || nh + s * 8 >= g.N || s >= 2 * NPQ) continue;
+          *reinterpret_cast<u32x4*>(dst + (int64_t)(8 * t) * g.N) = v;
+        }
       }
     } else {
       // output rows at any 2-byte offset (N % 8 != 0): one row per store instruction, lane l writes column l
@@ -140,6 +153,16 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
         if (n < g.N && lane < 16 * NPQ) D[(int64_t)(m0 + row) * g.N + n] = v;
       }
     }
+  };
+  if (!use_c) {
+    half(std::integral_constant<int, 0>{}, 0);
+    half(std::integral_constant<int, 0>{}, 1);
+  } else if (row_bias) {
+    half(std::integral_constant<int, 1>{}, 0);
+    half(std::integral_constant<int, 1>{}, 1);
+  } else {
+    half(std::integral_constant<int, 2>{}, 0);
+    half(std::integral_constant<int, 2>{}, 1);
   }
 }
 
@@ -445,6 +468,7 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
 #ifdef MI355_GEMM_TRACE
   const uint64_t tr_end = __builtin_readcyclecounter();
 #endif
+  if (!(MI355_X16_ABLATE & 32) || g.alpha == 12345.f)
   store_tile_result16<T, NPQ>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS);
 #ifdef MI355_GEMM_TRACE
   {
