@@ -2108,13 +2108,25 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // the 32x32x16 form (test knobs).
       const bool x16_ok = K % 128 == 0 && K >= 256 && !a_t && ld32;
       const bool x16_mixed_forced = forced_tile != nullptr && strcmp(forced_tile, "x16mixed") == 0;  // mixed widths at any K
-      const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced
+      const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced || strcmp(forced_tile, "x16persist") == 0
                                                          : K >= 512 && (K >= 2048 || N % 64 == 0) && nblocks >= kNumCU * 3 / 4 && !mid &&
                                                                !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
       if (x16) {
         kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
         threads = 256;
         lds_bytes = kX16Lds;
+        // More tiles than CUs, all of them whole: one workgroup per CU walks its tiles with the fill
+        // requests running on across them (gemm_mfma_x16_persistent_kernel).  MI355_GEMM_TILE=x16 keeps
+        // one workgroup per tile, =x16persist takes the walk for any tile count (test knobs).
+        const bool persist_forced = forced_tile != nullptr && strcmp(forced_tile, "x16persist") == 0;
+        bool persist = M % BM == 0 && N % BN == 0 && g.out_vec && K >= 512 && (forced_tile == nullptr ? nblocks > kNumCU : persist_forced);
+#ifdef MI355_GEMM_TRACE
+        persist = false;  // the stamps are per workgroup = per tile
+#endif
+        if (persist) {
+          kern = gemm_x16_persistent_kernel(std::is_same<T, bf16_t>::value, !b_nt);
+          if (nblocks > kNumCU) nblocks = kNumCU;
+        }
         // The mixed-width grid (192-wide tiles in the last round) is built for this form too, but it does not
         // pay here: [4096,4096]x[4096,11008] takes 284.6 us with it and 285.6 us without - a last round
         // that leaves CUs idle runs at a higher clock under the power limit, and a 192-wide tile issues the

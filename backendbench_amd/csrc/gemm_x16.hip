@@ -57,19 +57,21 @@ __device__ __forceinline__ int xswz_seg(int k) { return (k & 3) | (((k >> 3) & 1
 // Epilogue: the wave's 128 x 32 NPQ result, 16 NPQ columns at a time, through a 16 KB slab of the idle ring
 // (rows of 128 B, 16-byte slot s of row r at s ^ ((r / 2) % 8)) and out in whole 128-byte rows.
 // Register e of acc[i][j] in lane l is C[m0 + 16 i + l % 16][n0 + 16 j + 4 (l / 16) + e] (operands swapped).
-template <typename T, int NPQ>
+template <typename T, int NPQ, int RH = 1>
 __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32x4 (&acc)[8][2 * NPQ], unsigned char* lds,
                                                     int wave, int lane, int m0, int n0) {
+  static_assert(RH == 1 || RH == 2, "the slab holds all 128 rows of the wave's tile or 64 at a time");
+  constexpr int IB = 8 / RH;  // row blocks per pass
   const int lr = lane & 15, lg = lane >> 4;
   const T* C = static_cast<const T*>(g.c);
   const bool use_c = C != nullptr && g.beta != 0.f;
   const bool row_bias = use_c && g.c_vec && g.c_rs == 0;
-  unsigned char* slab = lds + wave * (128 * 128);
+  unsigned char* slab = lds + wave * (128 * 128 / RH);
   T* D = static_cast<T*>(g.out);
   const bool inside = NPQ == 4 && m0 + 128 <= g.M && n0 + 128 <= g.N;  // no row or column of this wave's tile is cut
   // MODE 0: alpha * acc; 1: + beta * a bias row (loaded once per 64 columns); 2: + beta * c.  The mode is
   // chosen once per call, outside the loops over the accumulator blocks.
-  auto half = [&](auto MODE_, int y) __attribute__((always_inline)) {
+  auto half = [&](auto MODE_, int y, int rh) __attribute__((always_inline)) {
     constexpr int MODE = decltype(MODE_)::value;
     const int nh = n0 + y * (16 * NPQ);
     float bias[NPQ][4];
@@ -85,7 +87,8 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
     unsigned char* wr = slab + lr * 128 + (lg & 1) * 8;
     const int sx = (lr >> 1) & 7;  // = (row / 2) % 8 for every row 16 i + lr
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int ii = 0; ii < IB; ++ii) {
+      const int i = rh * IB + ii;
       const int m = m0 + i * 16 + lr;
       const int mc = m < g.M ? m : g.M - 1;
 #pragma unroll
@@ -117,17 +120,17 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
 #pragma unroll
           for (int e = 0; e < 4; ++e) r.v[e] = static_cast<T>(g.alpha * v[e] + g.beta * cv[e]);
         }
-        *reinterpret_cast<VecN4<T>*>(wr + i * (16 * 128) + (((p * 2 + (lg >> 1)) ^ sx) << 4)) = r;
+        *reinterpret_cast<VecN4<T>*>(wr + ii * (16 * 128) + (((p * 2 + (lg >> 1)) ^ sx) << 4)) = r;
       }
     }
     // same wave wrote and reads: LDS operations of a wave complete in order
     if (g.out_vec) {
       const int s = lane & 7, r0 = lane >> 3;  // 16-byte chunk s of rows r0 + 8 t
       const unsigned char* rdp = slab + r0 * 128;
-      T* dst = D + (int64_t)(m0 + r0) * g.N + nh + s * 8;
+      T* dst = D + (int64_t)(m0 + rh * (16 * IB) + r0) * g.N + nh + s * 8;
       if (inside) {
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
+        for (int t = 0; t < 2 * IB; ++t) {
           const int row = r0 + 8 * t;  // (row / 2) % 8 = (r0 / 2 + 4 t) % 8
           const u32x4 v = *reinterpret_cast<const u32x4*>(rdp + t * 1024 + ((s ^ (((r0 >> 1) + 4 * t) & 7)) << 4));
           if ((MI355_X16_ABLATE & 16) && v[0] != 0x12345678u) continue;
@@ -136,34 +139,35 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
         }
       } else {
 #pragma unroll
-        for (int t = 0; t < 16; ++t) {
+        for (int t = 0; t < 2 * IB; ++t) {
           const int row = r0 + 8 * t;
           const u32x4 v = *reinterpret_cast<const u32x4*>(rdp + t * 1024 + ((s ^ ((row >> 1) & 7)) << 4));
-          if (m0 + row >= g.M || nh + s * 8 >= g.N || s >= 2 * NPQ) continue;
+          if (m0 + rh * (16 * IB) + row >= g.M || nh + s * 8 >= g.N || s >= 2 * NPQ) continue;
           *reinterpret_cast<u32x4*>(dst + (int64_t)(8 * t) * g.N) = v;
         }
       }
     } else {
       // output rows at any 2-byte offset (N % 8 != 0): one row per store instruction, lane l writes column l
       const int n = nh + lane;
-      const int rows = g.M - m0 < 128 ? g.M - m0 : 128;
+      const int mh = m0 + rh * (16 * IB);
+      const int rows = g.M - mh < 16 * IB ? g.M - mh : 16 * IB;
 #pragma unroll 8
       for (int row = 0; row < rows; ++row) {
         const T v = *reinterpret_cast<const T*>(slab + row * 128 + (((lane >> 3) ^ ((row >> 1) & 7)) << 4) + ((lane & 7) << 1));
-        if (n < g.N && lane < 16 * NPQ) D[(int64_t)(m0 + row) * g.N + n] = v;
+        if (n < g.N && lane < 16 * NPQ) D[(int64_t)(mh + row) * g.N + n] = v;
       }
     }
   };
-  if (!use_c) {
-    half(std::integral_constant<int, 0>{}, 0);
-    half(std::integral_constant<int, 0>{}, 1);
-  } else if (row_bias) {
-    half(std::integral_constant<int, 1>{}, 0);
-    half(std::integral_constant<int, 1>{}, 1);
-  } else {
-    half(std::integral_constant<int, 2>{}, 0);
-    half(std::integral_constant<int, 2>{}, 1);
-  }
+  auto all = [&](auto MODE_) __attribute__((always_inline)) {
+#pragma unroll
+    for (int rh = 0; rh < RH; ++rh) {
+      half(MODE_, 0, rh);
+      half(MODE_, 1, rh);
+    }
+  };
+  if (!use_c) all(std::integral_constant<int, 0>{});
+  else if (row_bias) all(std::integral_constant<int, 1>{});
+  else all(std::integral_constant<int, 2>{});
 }
 
 // Fill requests.  x16_set_m0 sets the LDS base of the requests behind it; request i of a group of four
@@ -182,9 +186,19 @@ constexpr int kXBias = 3072;  // the bases point this many bytes low, so that la
 // owns 96 columns, 48 per half, its quadrants are 4 x 3 blocks (24 MFMAs), and the 16 columns per
 // half-wave that the B sub-panels hold beyond that are fetched (the next columns, clamped at the matrix
 // edge) and not used.  Such tiles let a last, partly filled round of tiles be cut to fit the chip.
-template <typename T, bool B_NN, int NPQ>
-__device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, const int bm, const int bn) {
+//
+// PERSIST: the workgroup walks the tiles blockIdx.x, blockIdx.x + gridDim.x, ... (bm, bn are ignored) and
+// its fill requests run on as one stream across them: the last five half-stages of a tile request the
+// first five pairs of the next one, its last half-stage reads the next tile's first fragments, and the
+// next K loop starts the moment the epilogue has issued its stores - no prologue latency, no gap between
+// workgroups, and the stores drain while the next tile computes.  The epilogue borrows the one ring slot
+// that is free at that point (the pair just read), 64 rows of the wave's tile at a time.  For whole tiles
+// only (M, N multiples of 256: no clamped rows, so the lane offsets are the same for every tile) and
+// vector stores.
+template <typename T, bool B_NN, int NPQ, bool PERSIST = false>
+__device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, int bm, int bn) {
   static_assert(NPQ == 3 || NPQ == 4, "wave tile is 128 x 32 NPQ");
+  static_assert(!PERSIST || NPQ == 4, "the persistent form walks 256 x 256 tiles");
   using frag_t = typename Mfma16<T>::frag;
   constexpr int WCOLS = 32 * NPQ, HCOLS = 16 * NPQ;  // columns per wave and per half
   const int tid = threadIdx.x, lane = tid % kWave;
@@ -210,9 +224,21 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
   // request and half (the host checks that they fit: leading dimensions below 4 M elements).  A wave
   // fills the four consecutive 1 KB regions 4 wave .. 4 wave + 3 of a sub-panel: eight rows each of a
   // K-contiguous sub-panel (lane = row % 8 * 8 + chunk position), four k-rows of a row-major one.
-  const unsigned char* a_base = reinterpret_cast<const unsigned char*>(static_cast<const T*>(g.a) + (int64_t)bm * g.lda) - kXBias;
-  const unsigned char* b_base =
-      reinterpret_cast<const unsigned char*>(B_NN ? static_cast<const T*>(g.b) : static_cast<const T*>(g.b) + (int64_t)bn * g.ldb) - kXBias;
+  int pid = blockIdx.x, ptm = 0, ptn = 0;
+  if constexpr (PERSIST) {
+    tile_coords(g.tiles_m, g.tiles_n, pid, ptm, ptn);
+    bm = 0;  // the lane offsets below are relative to the tile (nothing is clamped: whole tiles only)
+    bn = 0;
+  }
+  // where a tile's operands start, kXBias bytes low (a row-major b: its first k-row at the tile's first column
+  // when PERSIST, else at column 0 with the columns in the lane offsets)
+  auto a_start = [&](int tm) { return reinterpret_cast<const unsigned char*>(static_cast<const T*>(g.a) + (int64_t)tm * g.lda) - kXBias; };
+  auto b_start = [&](int tn) {
+    const T* B = static_cast<const T*>(g.b);
+    return reinterpret_cast<const unsigned char*>(B_NN ? (PERSIST ? B + tn : B) : B + (int64_t)tn * g.ldb) - kXBias;
+  };
+  const unsigned char* a_base = a_start(PERSIST ? ptm * BM : bm);  // of the tile being computed
+  const unsigned char* b_base = b_start(PERSIST ? ptn * BN : bn);
   const int64_t a_step = 128;                                   // bytes per 64-k stage
   const int64_t b_step = B_NN ? (int64_t)128 * g.ldb : 128;
   uint32_t a_off[2][4], b_off[2][4];
@@ -371,6 +397,7 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
 #define MI355_TR_END(N)                                                                                                 \
   asm volatile("s_memtime %0\n\ts_waitcnt vmcnt(" #N ")\n\ts_memtime %1\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier\n\ts_memtime %2" \
                : "=s"(p1), "=s"(p2), "=s"(tr_start[1 - par]) : "s"(tr_start[par]) : "memory");
+      if constexpr (WAIT == 56) MI355_TR_END(56)
       if constexpr (WAIT == 24) MI355_TR_END(24)
       if constexpr (WAIT == 16) MI355_TR_END(16)
       if constexpr (WAIT == 8) MI355_TR_END(8)
@@ -385,6 +412,7 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       if constexpr (decltype(SYNC_)::value) __syncthreads();
     }
 #else
+    if constexpr (WAIT == 56) asm volatile("s_waitcnt vmcnt(56)" ::: "memory");
     if constexpr (WAIT == 24 && !(MI355_X16_ABLATE & 8)) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
     if constexpr (WAIT == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     if constexpr (WAIT == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
@@ -394,6 +422,7 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
     rd = bump(rd);
     fl = bump(fl);
   };
+  using W56 = std::integral_constant<int, 56>;
   using W24 = std::integral_constant<int, 24>;
   using W16 = std::integral_constant<int, 16>;
   using W8 = std::integral_constant<int, 8>;
@@ -419,7 +448,8 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
     fill_i(I2{}, b_off[second], b_base + s * b_step);
     fill_i(I3{}, b_off[second], b_base + s * b_step);
   }
-  asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+  if constexpr (PERSIST) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // all five: the first tile's waits assume what later tiles find
+  else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
@@ -438,6 +468,64 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
 
   // Half-stages t .. t + 3 request pairs t + 5 .. t + 8 = stages t / 2 + 2, + 3, + 3, + 4.
   const int np = g.K / 32;  // pairs = half-stages; a multiple of 4 (K % 128 == 0), at least 8
+  if constexpr (PERSIST) {
+    const int total = g.tiles_m * g.tiles_n;
+    for (;;) {
+      // the tile behind this one (the last tile requests its own first pairs once more: nobody reads them)
+      const int npid = pid + (int)gridDim.x;
+      const bool has_next = npid < total;
+      int ntm = ptm, ntn = ptn;
+      if (has_next) tile_coords(g.tiles_m, g.tiles_n, npid, ntm, ntn);
+      const unsigned char* na = a_start(ntm * BM);
+      const unsigned char* nb = b_start(ntn * BN);
+      const unsigned char* fa = a_base + 2 * a_step;
+      const unsigned char* fb = b_base + 2 * b_step;
+      // First four half-stages (np >= 16): pairs 2 .. 4 were requested before the previous tile's 32
+      // stores per lane, pair 5 behind them - only the wait for pair 5 has to see the stores out.
+      half_stage(I0{}, Yes{}, Yes{}, W56{}, Yes{}, fa, fb);
+      half_stage(I1{}, Yes{}, Yes{}, W56{}, Yes{}, fa + a_step, fb + b_step);
+      half_stage(I2{}, Yes{}, Yes{}, W56{}, Yes{}, fa + a_step, fb + b_step);
+      half_stage(I3{}, Yes{}, Yes{}, W24{}, Yes{}, fa + 2 * a_step, fb + 2 * b_step);
+      fa += 2 * a_step;
+      fb += 2 * b_step;
+      for (int t = 4; t + 8 < np; t += 4) {
+        half_stage(I0{}, Yes{}, Yes{}, W24{}, Yes{}, fa, fb);
+        half_stage(I1{}, Yes{}, Yes{}, W24{}, Yes{}, fa + a_step, fb + b_step);
+        half_stage(I2{}, Yes{}, Yes{}, W24{}, Yes{}, fa + a_step, fb + b_step);
+        half_stage(I3{}, Yes{}, Yes{}, W24{}, Yes{}, fa + 2 * a_step, fb + 2 * b_step);
+        fa += 2 * a_step;
+        fb += 2 * b_step;
+      }
+      // last eight: this tile's pairs np - 3 .. np - 1, then pairs 0 .. 4 of the next tile (stages 0, 0, 1, 1, 2)
+      half_stage(I0{}, Yes{}, Yes{}, W24{}, Yes{}, fa, fb);
+      half_stage(I1{}, Yes{}, Yes{}, W24{}, Yes{}, fa + a_step, fb + b_step);
+      half_stage(I2{}, Yes{}, Yes{}, W24{}, Yes{}, fa + a_step, fb + b_step);
+      half_stage(I3{}, Yes{}, Yes{}, W24{}, Yes{}, na, nb);
+      half_stage(I0{}, Yes{}, Yes{}, W24{}, Yes{}, na, nb);
+      half_stage(I1{}, Yes{}, Yes{}, W24{}, Yes{}, na + a_step, nb + b_step);
+      half_stage(I2{}, Yes{}, Yes{}, W24{}, Yes{}, na + a_step, nb + b_step);
+      half_stage(I3{}, Yes{}, Yes{}, W24{}, Yes{}, na + 2 * a_step, nb + 2 * b_step);  // reads the next tile's pair 0
+      // the last MFMA's result is read by VALU moves next; the slot of the pair just read (`fl`) is free
+      // until the next half-stage requests into it
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+      store_tile_result16<T, NPQ, 2>(g, acc, lds + fl, wave, lane, ptm * BM + wm * 128, ptn * BN + wn * 128);
+      __syncthreads();  // every wave is done with its slab before anyone requests into the slot
+      if (!has_next) break;
+      pid = npid; ptm = ntm; ptn = ntn;
+      a_base = na; b_base = nb;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 2 * NPQ; ++j) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+          asm volatile("" : "+a"(acc[i][j]));
+        }
+      asm volatile("s_nop 7" ::: "memory");  // the zeros are in before the first MFMA reads them
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the surplus requests of the last tile
+    return;
+  }
   const unsigned char* fa = a_base + 2 * a_step;
   const unsigned char* fb = b_base + 2 * b_step;
 #ifdef MI355_GEMM_TRACE
@@ -508,6 +596,18 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_mixed_kernel(GemmArgs g) {
     tile_coords(g.tiles_m, g.tail_n, blockIdx.x - wide, tm, tn);
     x16_tile<T, B_NN, 3>(g, lds, tm * BM, g.tiles_n * BN + tn * 192);
   }
+}
+
+// One workgroup per CU walks the tiles (x16_tile<..., PERSIST>): gridDim.x workgroups, tiles_m * tiles_n tiles.
+template <typename T, bool B_NN>
+__global__ __launch_bounds__(256) void gemm_mfma_x16_persistent_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  x16_tile<T, B_NN, 4, true>(g, lds, 0, 0);
+}
+
+const void* gemm_x16_persistent_kernel(bool is_bf16, bool b_nn) {
+  if (is_bf16) return b_nn ? (const void*)gemm_mfma_x16_persistent_kernel<bf16_t, true> : (const void*)gemm_mfma_x16_persistent_kernel<bf16_t, false>;
+  return b_nn ? (const void*)gemm_mfma_x16_persistent_kernel<f16_t, true> : (const void*)gemm_mfma_x16_persistent_kernel<f16_t, false>;
 }
 
 const void* gemm_x16_kernel(bool is_bf16, bool b_nn) {

@@ -246,6 +246,44 @@ def test_x16_gemm_every_k_loop_length(backend, layout, tile, monkeypatch):
         assert ev.bit_equal(ref16, half[rows.cuda()].cpu()), (layout, tile, K, "f16")
 
 
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+def test_x16_persistent_gemm_walks_its_tiles(backend, layout, monkeypatch):
+    """More whole 256x256 tiles than CUs: one workgroup per CU walks its tiles, with the fill requests running on
+    from one tile into the next.  [4096, K] x [K, 4352] has 16 x 17 = 272 tiles (sixteen workgroups get a second
+    tile), [2048, K] x [K, 12288] 8 x 48 = 384 (half of them), [256, K] x [K, 256] a single one (forced: a walk
+    of one tile).  K from the shortest loop the walk takes (512: the four special half-stages, one steady
+    iteration, the eight last ones) upwards.  Bit-equal to the one-workgroup-per-tile form of the same kernel
+    (same k order per element) and, on small-integer operands, to the oracle on sampled rows; bias row and a
+    full c through the epilogue's four passes."""
+    announce(f"persistent 16x16x32 GEMM, {layout}")
+    g = torch.Generator().manual_seed(14)
+    for (M, N) in ((4096, 4352), (2048, 12288), (256, 256)):
+        rows = torch.unique(torch.cat([torch.randint(0, M, (24,), generator=g), torch.tensor([0, 63, 64, 127, 128, 255, M - 1])]))
+        for K in (512, 640, 768, 1024, 2048):
+            a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+            if layout[1] == "t":
+                b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
+            else:
+                b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
+            bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
+            c = torch.randint(-2, 3, (M, N), generator=g).to(torch.bfloat16).cuda()
+            monkeypatch.setenv("MI355_GEMM_TILE", "x16persist")
+            walked = backend[aten.addmm.default](bias, a, b)
+            walked_c = backend[aten.addmm.default](c, a, b, beta=2.0)
+            walked_mm = backend[aten.mm.default](a, b)
+            monkeypatch.setenv("MI355_GEMM_TILE", "x16")
+            plain = backend[aten.addmm.default](bias, a, b)
+            monkeypatch.delenv("MI355_GEMM_TILE")
+            auto = backend[aten.addmm.default](bias, a, b)
+            assert ev.bit_equal(plain, walked), (layout, M, N, K)
+            assert ev.bit_equal(plain, auto), (layout, M, N, K, "planner's choice")
+            ref = aten_cpu.reference(aten.addmm.default, [bias, a[rows.cuda()], b])
+            assert ev.bit_equal(ref, walked[rows.cuda()].cpu()), (layout, M, N, K)
+            ref_c = aten_cpu.reference(aten.addmm.default, [c[rows.cuda()], a[rows.cuda()], b], {"beta": 2.0})
+            assert ev.bit_equal(ref_c, walked_c[rows.cuda()].cpu()), (layout, M, N, K, "full c")
+            assert ev.bit_equal((walked.float() - bias.float()).to(torch.bfloat16), walked_mm), (layout, M, N, K, "mm")
+
+
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
 @pytest.mark.parametrize("shape", [(704, 900), (2000, 2500)])
 def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
