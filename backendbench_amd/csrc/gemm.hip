@@ -2099,8 +2099,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                                                : (nb128 < kNumCU / 2 || (M <= 64 && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
                                                      (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2)));
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
-      // with 256x256 tiles when K is a multiple of 128: measured against the 32x32x16 form on
-      // [4096,K]x[K,16384], it is level at K = 512 and 4 - 15 % faster from K = 768 on (C3: [4096,4096]x
+      // with 256x256 tiles when K is a multiple of 128 (from 256 on): measured against the 32x32x16 forms on
+      // [4096,K]x[K,16384], it is 11 % faster at K = 256 and 4 - 15 % from K = 768 on (C3: [4096,4096]x
       // [4096,11008] 306 -> 279 us, [4096,11008]x[11008,4096] 270 -> 249 us).  With a short K and output
       // rows that do not start on 128-byte lines (N % 64 != 0) the eight-wave kernel's epilogue is the
       // faster one ([4096,768]x[768,50264]: 404 us against 436 us here).  MI355_GEMM_TILE=x16 forces this
@@ -2109,7 +2109,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool x16_ok = K % 128 == 0 && K >= 256 && !a_t && ld32;
       const bool x16_mixed_forced = forced_tile != nullptr && strcmp(forced_tile, "x16mixed") == 0;  // mixed widths at any K
       const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced || strcmp(forced_tile, "x16persist") == 0
-                                                         : K >= 512 && (K >= 2048 || N % 64 == 0) && nblocks >= kNumCU * 3 / 4 && !mid &&
+                                                         : (K >= 2048 || N % 64 == 0) && nblocks >= kNumCU * 3 / 4 && !mid &&
                                                                !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
       if (x16) {
         kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
@@ -2119,7 +2119,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         // requests running on across them (gemm_mfma_x16_persistent_kernel).  MI355_GEMM_TILE=x16 keeps
         // one workgroup per tile, =x16persist takes the walk for any tile count (test knobs).
         const bool persist_forced = forced_tile != nullptr && strcmp(forced_tile, "x16persist") == 0;
-        bool persist = M % BM == 0 && N % BN == 0 && g.out_vec && K >= 512 && (forced_tile == nullptr ? nblocks > kNumCU : persist_forced);
+        bool persist = M % BM == 0 && N % BN == 0 && g.out_vec && K >= 384 && (forced_tile == nullptr ? nblocks > kNumCU : persist_forced);
 #ifdef MI355_GEMM_TRACE
         persist = false;  // the stamps are per workgroup = per tile
 #endif

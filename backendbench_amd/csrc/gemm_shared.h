@@ -97,7 +97,7 @@ __device__ __forceinline__ void lds_dma16s(uint32_t lds_byte_offset, uint32_t la
 // a; b K-contiguous or row-major), its dynamic LDS size, and the host-side kernel handle.
 constexpr int kX16Lds = 5 * 32768;
 const void* gemm_x16_kernel(bool is_bf16, bool b_nn);
-const void* gemm_x16_persistent_kernel(bool is_bf16, bool b_nn);  // one workgroup per CU walks the tiles (whole tiles, K >= 512)
+const void* gemm_x16_persistent_kernel(bool is_bf16, bool b_nn);  // one workgroup per CU walks the tiles (whole tiles, K >= 384)
 const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn);  // 256-wide tile columns, then 192-wide ones (GemmArgs::tail_n)
 
 }  // namespace mi355

@@ -480,7 +480,7 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       const unsigned char* nb = b_start(ntn * BN);
       const unsigned char* fa = a_base + 2 * a_step;
       const unsigned char* fb = b_base + 2 * b_step;
-      // First four half-stages (np >= 16): pairs 2 .. 4 were requested before the previous tile's 32
+      // First four half-stages (np >= 12): pairs 2 .. 4 were requested before the previous tile's 32
       // stores per lane, pair 5 behind them - only the wait for pair 5 has to see the stores out.
       half_stage(I0{}, Yes{}, Yes{}, W56{}, Yes{}, fa, fb);
       half_stage(I1{}, Yes{}, Yes{}, W56{}, Yes{}, fa + a_step, fb + b_step);

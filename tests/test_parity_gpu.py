@@ -251,15 +251,15 @@ def test_x16_persistent_gemm_walks_its_tiles(backend, layout, monkeypatch):
     """More whole 256x256 tiles than CUs: one workgroup per CU walks its tiles, with the fill requests running on
     from one tile into the next.  [4096, K] x [K, 4352] has 16 x 17 = 272 tiles (sixteen workgroups get a second
     tile), [2048, K] x [K, 12288] 8 x 48 = 384 (half of them), [256, K] x [K, 256] a single one (forced: a walk
-    of one tile).  K from the shortest loop the walk takes (512: the four special half-stages, one steady
-    iteration, the eight last ones) upwards.  Bit-equal to the one-workgroup-per-tile form of the same kernel
+    of one tile).  K from the shortest loop the walk takes (384: the four special half-stages and the eight last
+    ones, no steady iteration) upwards.  Bit-equal to the one-workgroup-per-tile form of the same kernel
     (same k order per element) and, on small-integer operands, to the oracle on sampled rows; bias row and a
     full c through the epilogue's four passes."""
     announce(f"persistent 16x16x32 GEMM, {layout}")
     g = torch.Generator().manual_seed(14)
     for (M, N) in ((4096, 4352), (2048, 12288), (256, 256)):
         rows = torch.unique(torch.cat([torch.randint(0, M, (24,), generator=g), torch.tensor([0, 63, 64, 127, 128, 255, M - 1])]))
-        for K in (512, 640, 768, 1024, 2048):
+        for K in (384, 512, 640, 768, 1024, 2048):
             a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
             if layout[1] == "t":
                 b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
