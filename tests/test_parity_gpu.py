@@ -246,6 +246,40 @@ def test_x16_gemm_every_k_loop_length(backend, layout, tile, monkeypatch):
         assert ev.bit_equal(ref16, half[rows.cuda()].cpu()), (layout, tile, K, "f16")
 
 
+@pytest.mark.parametrize("tile", ["x16", "x16persist"])
+def test_x16_gemm_argument_forms(backend, tile, monkeypatch):
+    """What else reaches the 16x16x32 kernel besides dense operands: rows with a pitch (slices of wider tensors) on
+    both operands, a c that is a column ([M, 1]), a scalar-strided c (a transposed view), a c of NaNs under beta = 0
+    (never read), alpha and beta other than one, f16.  [512, 640] x [640, 768]: 2 x 3 tiles, forced onto the kernel
+    (one workgroup per tile, and the persistent walk).  Small-integer operands: bit-equal to the oracle."""
+    announce(f"16x16x32 GEMM argument forms, {tile}")
+    g = torch.Generator().manual_seed(15)
+    M, K, N = 512, 640, 768
+    ri = lambda *s, lo=-1, hi=2: torch.randint(lo, hi, s, generator=g)  # noqa: E731
+    for dtype in (torch.bfloat16, torch.float16):
+        wide_a = ri(M, K + 64).to(dtype).cuda()
+        wide_b = ri(K, N + 128).to(dtype).cuda()
+        wide_bt = ri(N, K + 8).to(dtype).cuda()
+        a = wide_a[:, 32:32 + K]            # 64-byte offset, pitch K + 64
+        b = wide_b[:, 64:64 + N]
+        bt = wide_bt[:, :K].t()
+        col = ri(M, 1, lo=-2, hi=3).to(dtype).cuda()
+        full_t = ri(N, M, lo=-2, hi=3).to(dtype).cuda().t()
+        nan_c = torch.full((M, N), float("nan"), dtype=dtype).cuda()
+        monkeypatch.setenv("MI355_GEMM_TILE", tile)
+        outs = {
+            "pitched nn": (backend[aten.mm.default](a, b), aten.mm.default, [a, b], {}),
+            "pitched nt": (backend[aten.mm.default](a, bt), aten.mm.default, [a, bt], {}),
+            "column c": (backend[aten.addmm.default](col, a, b), aten.addmm.default, [col, a, b], {}),
+            "transposed c": (backend[aten.addmm.default](full_t, a, bt, beta=2.0, alpha=3.0), aten.addmm.default, [full_t, a, bt], {"beta": 2.0, "alpha": 3.0}),
+            "nan c, beta 0": (backend[aten.addmm.default](nan_c, a, b, beta=0.0, alpha=2.0), aten.addmm.default, [nan_c, a, b], {"beta": 0.0, "alpha": 2.0}),
+        }
+        monkeypatch.delenv("MI355_GEMM_TILE")
+        for name, (got, op, args, kwargs) in outs.items():
+            ref = aten_cpu.reference(op, args, kwargs)
+            assert ev.bit_equal(ref, got.cpu()), (tile, dtype, name)
+
+
 @pytest.mark.parametrize("layout", ["nt", "nn"])
 def test_x16_persistent_gemm_walks_its_tiles(backend, layout, monkeypatch):
     """More whole 256x256 tiles than CUs: one workgroup per CU walks its tiles, with the fill requests running on
