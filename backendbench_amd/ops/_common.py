@@ -8,6 +8,7 @@ calls on tensors.
 """
 
 import functools
+import ctypes
 import os
 
 import torch
@@ -74,8 +75,10 @@ _entry = {}
 
 def launch(name, *args):
     """Call one C entry point with the current stream appended; raise on failure."""
-    if _pending:
-        poll_index_errors()
+    for w in _flag_words:
+        if w.value:
+            poll_index_errors()
+            break
     fn = _entry.get(name)
     if fn is None:
         fn = _entry[name] = getattr(_lib.load(), name)
@@ -137,27 +140,28 @@ def norm_dim(dim, ndim):
 
 
 # ---- out-of-range indices ----------------------------------------------------------
-# The indexing kernels never dereference a bad index; they zero the output there and set a
-# sticky device flag.  The error then surfaces the way a device-side assert of the stock
-# kernels does, asynchronously and without a device sync:
-#   * after an indexing launch the flag is copied to pinned host memory on the same stream
-#     (one copy in flight at a time) and an event is recorded;
-#   * every later call of any operator of this backend looks at that event; once it has completed
-#     and the flag is set, the call raises IndexError naming the earlier indexing call;
+# The indexing kernels never dereference a bad index; they zero the output there and store 1 into a
+# sticky int32 flag.  The flag lives in pinned host memory (device-accessible at its host address), so
+# the error surfaces the way a device-side assert of the stock kernels does - asynchronously, without a
+# device sync and without anything enqueued behind the kernel:
+#   * every later call of any operator of this backend reads the flag word (a plain host load); once a
+#     kernel has set it, that call raises IndexError naming the earlier indexing call;
 #   * check_index_errors() synchronises and raises at once (this repository's evaluator calls it
 #     after every test; MI355_SYNC_INDEX_CHECK=1 makes every indexing call do so, which is the
 #     CPU kernels' behaviour at the cost of a device sync per call).
-# Nothing is enqueued while the stream is being captured into a graph.
-_flags = {}
-_pending = []  # [(device key, pinned host int32, event)]: at most one entry per device
+# Nothing raises while the stream is being captured into a graph (the flag stays set).
+_flags = {}       # device key -> pinned int32 tensor (kept alive)
+_flag_words = []  # ctypes views of the same words, read on every launch
 
 
 def index_error_flag(device):
+    """Address of this device's flag word, as the kernels' err_flag argument."""
     key = device.index if device.index is not None else torch.cuda.current_device()
     f = _flags.get(key)
     if f is None:
-        f = torch.zeros(1, dtype=torch.int32, device=device)
+        f = torch.zeros(1, dtype=torch.int32, pin_memory=True)
         _flags[key] = f
+        _flag_words.append(ctypes.c_int32.from_address(f.data_ptr()))
     return f
 
 
@@ -165,36 +169,16 @@ def sync_index_check():
     return os.environ.get("MI355_SYNC_INDEX_CHECK", "0") == "1"
 
 
-def note_index_launch(device):
-    """Called behind every indexing launch: start the asynchronous read-back of the device flag
-    unless one is already in flight for this device or the stream is being captured."""
-    key = device.index if device.index is not None else torch.cuda.current_device()
-    for k, _, _ in _pending:
-        if k == key:
-            return
-    if torch.cuda.is_current_stream_capturing():
-        return
-    host = torch.empty(1, dtype=torch.int32, pin_memory=True)
-    host.copy_(_flags[key], non_blocking=True)
-    done = torch.cuda.Event()
-    done.record()
-    _pending.append((key, host, done))
-
-
 def poll_index_errors():
-    """Non-blocking: raise IndexError if a finished read-back shows that an earlier indexing call of
-    this backend met an out-of-range index.  Called at the start of every operator launch."""
+    """Non-blocking: raise IndexError if an earlier indexing call of this backend met an out-of-range
+    index and the device has run it.  Called at the start of every operator launch when a flag is set."""
     if torch.cuda.is_current_stream_capturing():
-        return  # no event queries inside a graph capture; the read-back stays pending
+        return  # not in the middle of a graph capture; the flag stays set
     bad = False
-    for entry in list(_pending):
-        key, host, done = entry
-        if not done.query():
-            continue
-        _pending.remove(entry)
-        if int(host[0]) != 0:
+    for w in _flag_words:
+        if w.value != 0:
             bad = True
-            _flags[key].zero_()
+            w.value = 0
     if bad:
         raise IndexError("index out of range in self (met by an earlier index_select / embedding / gather call of "
                          "this backend, whose output was zero-filled at that index)")
@@ -202,11 +186,13 @@ def poll_index_errors():
 
 def check_index_errors():
     """Synchronise and raise IndexError if any indexing kernel saw an out-of-range index since the last check."""
+    if not _flag_words:
+        return
+    torch.cuda.synchronize()
     bad = False
-    _pending.clear()
-    for f in _flags.values():
-        if int(f.item()) != 0:
+    for w in _flag_words:
+        if w.value != 0:
             bad = True
-            f.zero_()
+            w.value = 0
     if bad:
         raise IndexError("index out of range in self")

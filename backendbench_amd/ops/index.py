@@ -3,8 +3,8 @@
 import torch
 
 from .. import _lib
-from ._common import (check_index_errors, dense, device_managed, index_error_flag, launch, new_dense, norm_dim,
-                      note_index_launch, prod, sync_index_check)
+from ._common import (check_index_errors, dense, device_managed, index_error_flag, launch, new_dense, norm_dim, prod,
+                      sync_index_check)
 
 
 def _rows(src, outer, n_src, inner, index, out):
@@ -13,8 +13,6 @@ def _rows(src, outer, n_src, inner, index, out):
            _lib.dtype_code(index.dtype), index.numel(), out.data_ptr(), flag.data_ptr())
     if sync_index_check():
         check_index_errors()
-    else:
-        note_index_launch(src.device)
 
 
 def _check_index(index, name):
@@ -82,6 +80,4 @@ def gather(self, dim, index, *, sparse_grad=False):
     launch("mi355_gather", _lib.desc(src), d, _lib.desc(idx), _lib.desc(res), flag.data_ptr())
     if sync_index_check():
         check_index_errors()
-    else:
-        note_index_launch(self.device)
     return out

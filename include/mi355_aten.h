@@ -229,8 +229,8 @@ int mi355_calib_mfma(const void* a, const void* b, void* out, int dtype, int blo
 /* src dense [outer, n_src, inner], out dense [outer, n_idx, inner]:
  * out[o, j, :] = src[o, index[j], :].  elem_size in bytes (1, 2, 4, 8); idx_dtype
  * MI355_I32 or MI355_I64; index dense.  An index outside [0, n_src) is never
- * dereferenced: the row is zero-filled and *err_flag (device int32, may be NULL) is set
- * to 1 — the host decides when to read it.
+ * dereferenced: the row is zero-filled and *err_flag (an int32 the device can write: device
+ * memory or pinned host memory, may be NULL) is set to 1 — the host decides when to read it.
  * Slots: index_select__default (op_map.py:571), embedding__default (op_map.py:447). */
 int mi355_index_select(const void* src, int elem_size, int64_t outer, int64_t n_src,
                        int64_t inner, const void* index, int idx_dtype, int64_t n_idx,
