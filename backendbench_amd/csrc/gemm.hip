@@ -2101,7 +2101,11 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
       // with 256x256 tiles when K is a multiple of 128 (from 256 on): measured against the 32x32x16 forms on
       // [4096,K]x[K,16384], it is 11 % faster at K = 256 and 4 - 15 % from K = 768 on (C3: [4096,4096]x
-      // [4096,11008] 306 -> 279 us, [4096,11008]x[11008,4096] 270 -> 249 us).  With a short K and output
+      // [4096,11008] 306 -> 279 us, [4096,11008]x[11008,4096] 270 -> 249 us).  It also takes 129 - 191 tiles
+      // (and 96 - 128 at K >= 2048) unless they make one round of 256x128 tiles: a tile's time does not
+      // depend on how many CUs run one, while the 128x128 kernels need a second round of their four times
+      // as many tiles ([2304,4096]x[4096,4096], 144 tiles: 104 -> 78 us; [1280,4096]x[4096,7680]: 117 -> 82).
+      // With a short K and output
       // rows that do not start on 128-byte lines (N % 64 != 0) the eight-wave kernel's epilogue is the
       // faster one ([4096,768]x[768,50264]: 404 us against 436 us here).  MI355_GEMM_TILE=x16 forces this
       // form for any tile count (=x16mixed: with the mixed-width grid at any K), =256x256 / =mixed keep
@@ -2109,7 +2113,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool x16_ok = K % 128 == 0 && K >= 256 && !a_t && ld32;
       const bool x16_mixed_forced = forced_tile != nullptr && strcmp(forced_tile, "x16mixed") == 0;  // mixed widths at any K
       const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced || strcmp(forced_tile, "x16persist") == 0
-                                                         : (K >= 2048 || N % 64 == 0) && nblocks >= kNumCU * 3 / 4 && !mid &&
+                                                         : (K >= 2048 || N % 64 == 0) && (nblocks > kNumCU / 2 || (nblocks >= 96 && K >= 2048)) && !mid &&
                                                                !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
       if (x16) {
         kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
@@ -2155,6 +2159,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         kern = pick_w4(std::integral_constant<int, 2>{});
         threads = 256;
         lds_bytes = kGemmLds64;
+        // (The 16x16x32 kernel on 256x128 tiles was measured for this slot: with half the MFMAs per fill and
+        // per LDS read it is level with this form on a transposed b and 10 % behind on a row-major one.)
       } else if (!ktail && nblocks < kNumCU * 3 / 4) {  // 128x128 tiles, two workgroups per CU
         g.tiles_m = (int32_t)((M + SBM - 1) / SBM);
         g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
