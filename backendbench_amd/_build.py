@@ -89,6 +89,34 @@ def build_trace(verbose: bool = True) -> Path:
     return TRACE_LIB_PATH
 
 
+def ablate_lib_path(bits: int) -> Path:
+    return LIB_DIR / f"libmi355_gemm_ablate_{bits}.so"
+
+
+def build_ablate(bits: int, verbose: bool = True) -> Path:
+    """A measurement build of the GEMM sources with -DMI355_X16_ABLATE=<bits>: parts of the 16x16x32
+    kernel's K loop or epilogue left out (bit list beside the macro in csrc/gemm_x16.hip).  Its results
+    are wrong; `bench.py --only-op C3.mm_down --ablate <bits>` times it to show what each part costs."""
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    objs = []
+    for src, extra in (("gemm.hip", []), ("gemm_x16.hip", [f"-DMI355_X16_ABLATE={bits}"]), ("common.hip", [])):
+        obj = OBJ_DIR / (Path(src).stem + f".ablate{bits}.o")
+        proc = subprocess.run([HIPCC, *FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)], capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed for {src} (ablation build):\n{proc.stdout}\n{proc.stderr}")
+        objs.append(obj)
+    out = ablate_lib_path(bits)
+    tmp = out.with_suffix(".so.tmp")
+    proc = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"link failed (ablation build):\n{proc.stdout}\n{proc.stderr}")
+    os.replace(tmp, out)
+    if verbose:
+        print(f"built {out} ({out.stat().st_size // 1024} KiB)")
+    return out
+
+
 def build(verbose: bool = True, jobs: int = 8, incremental: bool = False) -> Path:
     """Compile every kernel source for gfx950 and link the shared library.  `incremental`
     (developer convenience, `--incremental` on the command line) keeps objects that are newer
@@ -110,6 +138,8 @@ def build(verbose: bool = True, jobs: int = 8, incremental: bool = False) -> Pat
 if __name__ == "__main__":
     if "--trace" in sys.argv[1:]:
         build_trace()
+    elif "--ablate" in sys.argv[1:]:
+        build_ablate(int(sys.argv[sys.argv.index("--ablate") + 1]))
     else:
         build(incremental="--incremental" in sys.argv[1:])
     sys.exit(0)

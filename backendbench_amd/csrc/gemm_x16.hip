@@ -24,6 +24,10 @@
 
 #include "gemm_shared.h"
 
+// Timing-only ablations for measurement builds (python -m backendbench_amd._build --ablate N, bench.py
+// --only-op C3.mm_down --ablate N): results are wrong, the product library is built with 0.  Bits: 1 no fill
+// requests in the K loop, 2 no barriers, 4 no LDS fragment reads, 8 no wait for the fills, 16 no global
+// stores in the epilogue, 32 no epilogue.
 #ifndef MI355_X16_ABLATE
 #define MI355_X16_ABLATE 0
 #endif

@@ -54,6 +54,10 @@ def parse():
                          "ports, 2 = the other operand held across MFMAs, 3 = v_mfma_f32_16x16x32, 4-9 = chained "
                          "accumulator updates, 10 = the 16x16x32 mm kernel's stream, 11-14 = its reorderings "
                          "(see mi355_calib_mfma in include/mi355_aten.h)")
+    ap.add_argument("--ablate", type=int, default=None,
+                    help="with --only-op C3.mm_up|C3.mm_down: time the GEMM through the measurement build that leaves "
+                         "parts of the 16x16x32 kernel out (python -m backendbench_amd._build --ablate N; bits: 1 fills, "
+                         "2 barriers, 4 LDS fragment reads, 8 fill waits, 16 epilogue stores, 32 epilogue); wrong results")
     ap.add_argument("--trace", action="store_true",
                     help="with --only-op C3.mm_up|C3.mm_down: run the cycle-stamped diagnostic build of the GEMM "
                          "(libmi355_gemm_trace.so) and print where a tile's shader-clock ticks go")
@@ -98,6 +102,9 @@ def main():
         return
     if args.only_op and args.trace:
         print(json.dumps(gemm_trace(by_key[args.only_op], dev, args.fill)))
+        return
+    if args.only_op and args.ablate is not None:
+        print(json.dumps(gemm_ablate(by_key[args.only_op], dev, args.ablate, args.fill)))
         return
     if args.only_op:
         if args.only_op == "calib.copy":
@@ -340,6 +347,50 @@ def calib_mfma(dev, fill=None, variant=0, blocks=256, steps=2752, launches=20):
     return {"only_op": "calib.mfma", "variant": variant, "fill": fill or "N(0,1) x N(0,0.02)", "ms": round(ms, 4),
             "flops": flops, "tflops": round(tf, 1), "frac_of_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
             "timing": f"{launches} launches of {blocks} x 4 waves x {steps} steps, events around the loop"}
+
+
+def gemm_ablate(case, dev, bits, fill=None, launches=40):
+    """The row's mm through the ablation build `bits` (see csrc/gemm_x16.hip): events around `launches`
+    back-to-back launches after a warm-up.  Timing only - the build leaves work out, its results are wrong.
+    MI355_GEMM_TILE in the environment applies as usual (x16 = one workgroup per tile)."""
+    import ctypes
+
+    import torch
+
+    from backendbench_amd import _build, _lib
+
+    path = _build.ablate_lib_path(bits)
+    if not path.exists():
+        raise RuntimeError(f"{path} is missing: python -m backendbench_amd._build --ablate {bits}")
+    lib = ctypes.CDLL(str(path))
+    fn = lib.mi355_gemm
+    fn.restype, fn.argtypes = _lib.SIGNATURES["mi355_gemm"]
+    (a, b), _ = case.make(dev)
+    if fill:
+        for t in (a, b):
+            t.copy_(torch.randint(-1, 2, t.shape, device=dev).to(t.dtype)) if fill == "sign" else t.fill_(0.0 if fill == "zeros" else 1.0)
+    M, K = a.shape
+    N = b.shape[1]
+    out = torch.empty(M, N, dtype=a.dtype, device=dev)
+
+    def run():
+        _lib.check(fn(a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), None, 0, 0,
+                      out.data_ptr(), M, N, K, 1.0, 0.0, _lib.dtype_code(a.dtype), None, 0, _lib.current_stream_handle()))
+
+    for _ in range(3 * launches):  # the first dozens of launches of a process run slower (clocks, power state)
+        run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(launches):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / launches
+    flops = 2.0 * M * N * K
+    return {"only_op": case.key, "ablate": bits, "fill": fill or "as configured", "ms": round(ms, 5),
+            "tflops_nominal": round(flops / (ms * 1e-3) / 1e12, 1),
+            "timing": f"events around {launches} back-to-back launches; results are wrong by construction"}
 
 
 def gemm_trace(case, dev, fill=None):
