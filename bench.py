@@ -479,7 +479,12 @@ def graph_bench(fn, args, kwargs, pool_bytes=768 * 2**20, target_ms=60.0):
     import torch
 
     nbytes = sum(a.numel() * a.element_size() for a in args if isinstance(a, torch.Tensor))
-    copies = max(2, min(24, math.ceil(pool_bytes / max(nbytes, 1))))
+    # at least four copies while they fit 6 GiB (inputs of a gigabyte: the gathers), else two (the 4.2 GB argmax)
+    copies = max(4 if 4 * nbytes <= 6 * 2**30 else 2, min(24, math.ceil(pool_bytes / max(nbytes, 1))))
+    # A replay costs about 2.3 us on top of its kernels (two launches per graph: + 1.2 us each, twelve: + 0.2):
+    # a graph of few copies walks its pool more than once, so that every row carries about the same share.
+    rounds = math.ceil(6 / copies)
+    launches = copies * rounds
     clone = lambda seq: [x.clone() if isinstance(x, torch.Tensor) else x for x in seq]
     pool = [list(args)] + [clone(args) for _ in range(copies - 1)]
     for p in pool[:2]:
@@ -488,8 +493,8 @@ def graph_bench(fn, args, kwargs, pool_bytes=768 * 2**20, target_ms=60.0):
     try:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            held = [fn(*p, **kwargs) for p in pool]
-        run, per_run, how = graph.replay, copies, f"hip graph of {copies} launches over {copies} input copies, events around replays"
+            held = [fn(*p, **kwargs) for _ in range(rounds) for p in pool]
+        run, per_run, how = graph.replay, launches, f"hip graph of {launches} launches over {copies} input copies, events around replays"
     except Exception as exc:  # noqa: BLE001
         print(f"bench.py: graph capture failed for this op ({exc}); eager launches", file=sys.stderr)
         run, per_run, how = (lambda: [fn(*p, **kwargs) for p in pool]), copies, "eager launches over input copies, events around the loop"
