@@ -173,7 +173,7 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
   unsigned char* slab = lds + wave * (MI * 32 * 128);  // MI * 32 rows x 128 bytes
   // A bias row (c broadcast along m: the Linear-layer addmm) is the same for every row of the
   // tile: its 8 groups of four columns are loaded once, scaled by beta, and reused for all rows.
-  const bool row_bias = use_c && g.c_vec && g.c_rs == 0;
+  const bool row_bias = use_c && g.bias_vec;
   float bias[NB][4][4];
   if (row_bias) {
 #pragma unroll
@@ -184,6 +184,10 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
         const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (n + 4 <= g.N ? n : 0));
 #pragma unroll
         for (int e = 0; e < 4; ++e) bias[j][q][e] = g.beta * static_cast<float>(t.v[e]);
+        if (n < g.N && n + 4 > g.N) {  // the last columns of an N that is no multiple of 4
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bias[j][q][e] = g.beta * static_cast<float>(C[n + e < g.N ? n + e : g.N - 1]);
+        }
       }
   }
   // 16-byte slot s of row r lives at slot s ^ ((r/2) % 8): two-way conflicts at most on both sides
@@ -248,15 +252,10 @@ __device__ __forceinline__ void store_tile_result(const GemmArgs& g, const f32x1
     }
   } else {
     // N not a multiple of 8 (e.g. a 50257-wide vocabulary): the rows of out start at any 2-byte
-    // offset.  One row per store instruction, lane l writes column l: the 64 element stores of an
-    // instruction fall into the same one or two 128-byte lines.
-    const int n = n0 + lane;
+    // offset; the lanes walk the 16-byte grid of the destination (store_slab_rows_shifted).
     const int rows = g.M - m0 < MI * 32 ? g.M - m0 : MI * 32;
-#pragma unroll 8
-    for (int row = 0; row < rows; ++row) {
-      const T v = *reinterpret_cast<const T*>(slab + row * 128 + (((lane >> 3) ^ ((row >> 1) & 7)) << 4) + ((lane & 7) << 1));
-      if (n < g.N && lane < NB * 32) D[(int64_t)(m0 + row) * g.N + n] = v;
-    }
+    const int cols = g.N - n0 < NB * 32 ? g.N - n0 : NB * 32;
+    store_slab_rows_shifted<T, MI * 32>(slab, D, g.N, m0, rows, n0, cols, lane);
   }
 }
 
@@ -1094,7 +1093,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   int tm, tn;
   tile_coords(g, tm, tn);
-  w4_tile<T, B_NN, NJ, A_T>(g, lds, tm * BM, tn * (NJ * 64));
+  // the fill requests take their bases in SGPRs: the tile origin is uniform, say so
+  w4_tile<T, B_NN, NJ, A_T>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * (NJ * 64)));
 }
 
 // The same tiles in two widths in one launch: blocks [0, tiles_m * tiles_n) are 256 x 256 tiles of the
@@ -1109,10 +1109,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_mixed_kernel(GemmArgs g) {
   int tm, tn;
   if ((int)blockIdx.x < wide) {
     tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
-    w4_tile<T, B_NN, 4, A_T, 4>(g, lds, tm * BM, tn * 256);
+    w4_tile<T, B_NN, 4, A_T, 4>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * 256));
   } else {
     tile_coords(g.tiles_m, g.tail_n, blockIdx.x - wide, tm, tn);
-    w4_tile<T, B_NN, 4, A_T, 3>(g, lds, tm * BM, g.tiles_n * 256 + tn * 192);
+    w4_tile<T, B_NN, 4, A_T, 3>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(g.tiles_n * 256 + tn * 192));
   }
 }
 
@@ -2051,6 +2051,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       g.c_rs = c_rs; g.c_cs = c_cs;
       g.c_vec = c != nullptr && c_cs == 1 && c_rs % 4 == 0 && reinterpret_cast<uintptr_t>(c) % 8 == 0 && N % 4 == 0;
       g.out_vec = N % 8 == 0 && aligned16(out);
+      g.bias_vec = c != nullptr && c_rs == 0 && c_cs == 1 && reinterpret_cast<uintptr_t>(c) % 8 == 0;
       g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
       g.alpha = (float)alpha; g.beta = (float)beta;
       g.tiles_m = (int32_t)((M + BM - 1) / BM);
@@ -2105,15 +2106,13 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // (and 96 - 128 at K >= 2048) unless they make one round of 256x128 tiles: a tile's time does not
       // depend on how many CUs run one, while the 128x128 kernels need a second round of their four times
       // as many tiles ([2304,4096]x[4096,4096], 144 tiles: 104 -> 78 us; [1280,4096]x[4096,7680]: 117 -> 82).
-      // With a short K and output
-      // rows that do not start on 128-byte lines (N % 64 != 0) the eight-wave kernel's epilogue is the
-      // faster one ([4096,768]x[768,50264]: 404 us against 436 us here).  MI355_GEMM_TILE=x16 forces this
-      // form for any tile count (=x16mixed: with the mixed-width grid at any K), =256x256 / =mixed keep
+      // Output rows that do not start on 128-byte lines (N % 64 != 0) get its whole-tile-row epilogue.
+      // MI355_GEMM_TILE=x16 forces this form for any tile count (=x16mixed: with the mixed-width grid at any K), =256x256 / =mixed keep
       // the 32x32x16 form (test knobs).
       const bool x16_ok = K % 128 == 0 && K >= 256 && !a_t && ld32;
       const bool x16_mixed_forced = forced_tile != nullptr && strcmp(forced_tile, "x16mixed") == 0;  // mixed widths at any K
       const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced || strcmp(forced_tile, "x16persist") == 0
-                                                         : (K >= 2048 || N % 64 == 0) && (nblocks > kNumCU / 2 || (nblocks >= 96 && K >= 2048)) && !mid &&
+                                                         : (nblocks > kNumCU / 2 || (nblocks >= 96 && K >= 2048)) && !mid &&
                                                                !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
       if (x16) {
         kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
@@ -2123,7 +2122,13 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         // requests running on across them (gemm_mfma_x16_persistent_kernel).  MI355_GEMM_TILE=x16 keeps
         // one workgroup per tile, =x16persist takes the walk for any tile count (test knobs).
         const bool persist_forced = forced_tile != nullptr && strcmp(forced_tile, "x16persist") == 0;
-        bool persist = M % BM == 0 && N % BN == 0 && g.out_vec && K >= 384 && (forced_tile == nullptr ? nblocks > kNumCU : persist_forced);
+        // The walk pays from four rounds of tiles on, or with a long K: with a short K and one to three
+        // rounds the workgroups that start late or run on a slower CU get as many tiles as the others,
+        // where the dispatcher hands a tile to whichever CU is free first ([8192,768]x[768,2304], 288
+        // tiles: 46.2 us against 43.4; [12544,768]x[768,3072], 588 tiles: 75.8 against 71.1; level at
+        // exactly two and three rounds; 24.5 rounds at K = 768: 592 against 636).
+        bool persist = M % BM == 0 && N % BN == 0 && g.out_vec && K >= 384 &&
+                       (forced_tile == nullptr ? nblocks > kNumCU && (K >= 2048 || nblocks >= 4 * kNumCU) : persist_forced);
 #ifdef MI355_GEMM_TRACE
         persist = false;  // the stamps are per workgroup = per tile
 #endif
@@ -2144,6 +2149,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
             kern = gemm_x16_mixed_kernel(std::is_same<T, bf16_t>::value, !b_nt);
           }
         }
+        // Output rows off the 128-byte lines: whole tile rows per store instruction (store_tile_rows16).
+        g.out_rows = !persist && g.tail_n == 0 && (N % 64 != 0 || reinterpret_cast<uintptr_t>(out) % 128 != 0);
       } else if (t64) {
         g.tiles_m = (int32_t)((M + TBM - 1) / TBM);
         g.tiles_n = (int32_t)((N + TBN - 1) / TBN);

@@ -31,6 +31,8 @@ struct GemmArgs {
   int32_t tail_n;  // gemm_mfma_w4_mixed_kernel: 192-wide tile columns behind the tiles_n 256-wide ones
   int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
   int32_t out_vec;  // out rows start on 16-byte boundaries (N a multiple of the vector width): vector stores
+  int32_t out_rows;  // gemm_mfma_x16_kernel: out rows do not start on 128-byte lines (N % 64 != 0), stage whole tile rows
+  int32_t bias_vec;  // c is one unit-stride row broadcast along m (a Linear layer's bias), 8-byte aligned: any N
   // Split-K (128x128 kernels only): blockIdx.y = split, which covers k in [split * ksplit,
   // min(K, (split + 1) * ksplit)) and writes its raw fp32 tile to ws[split][M][ws_ld], ws_ld = N
   // rounded up to a multiple of 4 (rows of every plane start on 16-byte boundaries for any N).
@@ -59,6 +61,57 @@ __device__ __forceinline__ void tile_coords(const int tiles_m, const int tiles_n
 }
 __device__ __forceinline__ void tile_coords(const GemmArgs& g, int& tm, int& tn) {
   tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
+}
+
+// Epilogue of the MFMA kernels for output rows that start at any 2-byte offset (N % 8 != 0: a 50257-wide
+// vocabulary projection).  `slab` holds `rows` result rows of SLOTS 16-byte slots (8 SLOTS elements; slot s
+// of row r at s ^ ((r / 2) % 8) for 128-byte rows, at s ^ (r % SLOTS) otherwise), of which the first `cols`
+// columns go to D[m_first + row][n_first ...].  A store instruction costs the memory pipeline the same
+// whether its lanes carry 2 or 16 bytes, so the lanes walk the 16-byte grid of the destination, not the
+// columns: SLOTS lanes per row, lane s stores the s-th whole 16-byte unit that lies inside the row segment
+// (its eight elements gathered from the two LDS slots they straddle), and the up to seven elements in front
+// of the first unit and behind the last one go out as single elements (they share their 16-byte units with
+// the neighbouring tiles' columns).
+template <typename T, int ROWS, int SLOTS = 8>
+__device__ __forceinline__ void store_slab_rows_shifted(const unsigned char* slab, T* D, int64_t N, int m_first, int rows,
+                                                        int n_first, int cols, int lane) {
+  constexpr int RPI = 64 / SLOTS;  // rows per store instruction
+  static_assert(sizeof(T) == 2 && (SLOTS == 8 || SLOTS == 32) && ROWS % (4 * RPI) == 0, "two-byte elements, batches of four instructions");
+  if (cols <= 0) return;
+  const int s = lane % SLOTS;
+  auto elem = [&](int row, int e) -> uint32_t {
+    const int x = SLOTS == 8 ? (row >> 1) & 7 : row & (SLOTS - 1);
+    return *reinterpret_cast<const uint16_t*>(slab + row * (SLOTS * 16) + (((e >> 3) ^ x) << 4) + ((e & 7) << 1));
+  };
+  // four store instructions' worth of rows at a time: all LDS reads of the batch are issued before its first store
+#pragma unroll
+  for (int t0 = 0; t0 < ROWS / RPI; t0 += 4) {
+    u32x4 v[4];
+    uint32_t hv[4], tv[4];
+    uint16_t* dst[4];
+    int head[4], nfull[4], tail0[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int row = (t0 + u) * RPI + lane / SLOTS;
+      dst[u] = reinterpret_cast<uint16_t*>(D) + ((int64_t)(m_first + row) * N + n_first);
+      const int to_unit = (int)((16 - (reinterpret_cast<uintptr_t>(dst[u]) & 15)) & 15) >> 1;  // elements up to the next 16-byte boundary
+      head[u] = row >= rows ? 0 : to_unit < cols ? to_unit : cols;
+      nfull[u] = row >= rows ? 0 : (cols - head[u]) >> 3;
+      tail0[u] = row >= rows ? cols : head[u] + 8 * nfull[u];
+      const int e0 = head[u] + 8 * (s < nfull[u] ? s : 0);  // clamped: the slab is read, nothing is stored
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        v[u][j] = elem(row, (e0 + 2 * j) & (SLOTS * 8 - 1)) | (elem(row, (e0 + 2 * j + 1) & (SLOTS * 8 - 1)) << 16);
+      hv[u] = elem(row, s);
+      tv[u] = elem(row, (tail0[u] + s) & (SLOTS * 8 - 1));
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (s < nfull[u]) *reinterpret_cast<u32x4*>(dst[u] + head[u] + 8 * s) = v[u];
+      if (s < head[u]) dst[u][s] = (uint16_t)hv[u];
+      if (tail0[u] + s < cols) dst[u][tail0[u] + s] = (uint16_t)tv[u];
+    }
+  }
 }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));

@@ -69,25 +69,35 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
   const int lr = lane & 15, lg = lane >> 4;
   const T* C = static_cast<const T*>(g.c);
   const bool use_c = C != nullptr && g.beta != 0.f;
-  const bool row_bias = use_c && g.c_vec && g.c_rs == 0;
+  const bool row_bias = use_c && g.bias_vec;
   unsigned char* slab = lds + wave * (128 * 128 / RH);
   T* D = static_cast<T*>(g.out);
   const bool inside = NPQ == 4 && m0 + 128 <= g.M && n0 + 128 <= g.N;  // no row or column of this wave's tile is cut
   // MODE 0: alpha * acc; 1: + beta * a bias row (loaded once per 64 columns); 2: + beta * c.  The mode is
   // chosen once per call, outside the loops over the accumulator blocks.
-  auto half = [&](auto MODE_, int y, int rh) __attribute__((always_inline)) {
-    constexpr int MODE = decltype(MODE_)::value;
-    const int nh = n0 + y * (16 * NPQ);
-    float bias[NPQ][4];
-    if constexpr (MODE == 1) {
+  // The bias row of the wave's 32 NPQ columns, loaded once for both halves and all passes (one exposed
+  // load latency per tile instead of one per half).
+  float bias2[2][NPQ][4];
+  if (row_bias) {
+#pragma unroll
+    for (int y = 0; y < 2; ++y)
 #pragma unroll
       for (int p = 0; p < NPQ; ++p) {
-        const int n = nh + p * 16 + lg * 4;
+        const int n = n0 + y * (16 * NPQ) + p * 16 + lg * 4;
         const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (n + 4 <= g.N ? n : 0));
 #pragma unroll
-        for (int e = 0; e < 4; ++e) bias[p][e] = g.beta * static_cast<float>(t.v[e]);
+        for (int e = 0; e < 4; ++e) bias2[y][p][e] = g.beta * static_cast<float>(t.v[e]);
+        if (n < g.N && n + 4 > g.N) {  // the last columns of an N that is no multiple of 4
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bias2[y][p][e] = g.beta * static_cast<float>(C[n + e < g.N ? n + e : g.N - 1]);
+        }
       }
-    }
+  }
+  auto half = [&](auto MODE_, auto Y_, int rh) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(MODE_)::value;
+    constexpr int y = decltype(Y_)::value;
+    const int nh = n0 + y * (16 * NPQ);
+    const float (&bias)[NPQ][4] = bias2[y];
     unsigned char* wr = slab + lr * 128 + (lg & 1) * 8;
     const int sx = (lr >> 1) & 7;  // = (row / 2) % 8 for every row 16 i + lr
 #pragma unroll
@@ -151,27 +161,124 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
         }
       }
     } else {
-      // output rows at any 2-byte offset (N % 8 != 0): one row per store instruction, lane l writes column l
-      const int n = nh + lane;
+      // output rows at any 2-byte offset (N % 8 != 0): the lanes walk the 16-byte grid of the destination
       const int mh = m0 + rh * (16 * IB);
       const int rows = g.M - mh < 16 * IB ? g.M - mh : 16 * IB;
-#pragma unroll 8
-      for (int row = 0; row < rows; ++row) {
-        const T v = *reinterpret_cast<const T*>(slab + row * 128 + (((lane >> 3) ^ ((row >> 1) & 7)) << 4) + ((lane & 7) << 1));
-        if (n < g.N && lane < 16 * NPQ) D[(int64_t)(mh + row) * g.N + n] = v;
-      }
+      const int cols = g.N - nh < 16 * NPQ ? g.N - nh : 16 * NPQ;
+      store_slab_rows_shifted<T, 16 * IB>(slab, D, g.N, mh, rows, nh, cols, lane);
     }
   };
   auto all = [&](auto MODE_) __attribute__((always_inline)) {
 #pragma unroll
     for (int rh = 0; rh < RH; ++rh) {
-      half(MODE_, 0, rh);
-      half(MODE_, 1, rh);
+      half(MODE_, std::integral_constant<int, 0>{}, rh);
+      half(MODE_, std::integral_constant<int, 1>{}, rh);
     }
   };
   if (!use_c) all(std::integral_constant<int, 0>{});
   else if (row_bias) all(std::integral_constant<int, 1>{});
   else all(std::integral_constant<int, 2>{});
+}
+
+// Epilogue of the one-workgroup-per-tile kernel for output rows that do not start on 128-byte lines
+// (N % 64 != 0: a 50264- or 50257-wide vocabulary).  With one slab per wave every store instruction writes
+// 128-byte pieces that straddle two lines of the destination, each line is completed by another wave's
+// stores later, and the 4 MB of L2 behind the 32 CUs of an XCD write many of them back half-filled in
+// between (WRITE_SIZE reads 1.34 x the output bytes, [8192,768]x[768,50264] takes 812 us against 620 us at
+// N = 50240).  Here the four waves park the whole 256 x 256 tile in the (idle) ring as rows of 512 bytes
+// (16-byte slot s of row r at s ^ (r % 32)) and every store instruction then writes two whole tile rows:
+// three complete lines and the two pieces a row shares with the neighbouring tiles.  Rows at any 2-byte
+// offset (N % 8 != 0) go out along the destination's 16-byte grid (store_slab_rows_shifted).
+template <typename T>
+__device__ __forceinline__ void store_tile_rows16(const GemmArgs& g, const f32x4 (&acc)[8][8], unsigned char* lds, int wave,
+                                                  int lane, int bm, int bn) {
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lr = lane & 15, lg = lane >> 4;
+  const T* C = static_cast<const T*>(g.c);
+  const bool use_c = C != nullptr && g.beta != 0.f;
+  const bool row_bias = use_c && g.bias_vec;
+  auto stage = [&](auto MODE_) __attribute__((always_inline)) {
+    constexpr int MODE = decltype(MODE_)::value;
+    float bias2[2][4][4];  // the bias row of the wave's 128 columns, loaded before anything is staged
+    if constexpr (MODE == 1) {
+#pragma unroll
+      for (int y = 0; y < 2; ++y)
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const int n = bn + wn * 128 + y * 64 + p * 16 + lg * 4;
+          const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (n + 4 <= g.N ? n : 0));
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bias2[y][p][e] = g.beta * static_cast<float>(t.v[e]);
+          if (n < g.N && n + 4 > g.N) {  // the last columns of an N that is no multiple of 4
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bias2[y][p][e] = g.beta * static_cast<float>(C[n + e < g.N ? n + e : g.N - 1]);
+          }
+        }
+    }
+#pragma unroll
+    for (int y = 0; y < 2; ++y) {
+      const int nh = bn + wn * 128 + y * 64;
+      const float (&bias)[4][4] = bias2[y];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int row = wm * 128 + i * 16 + lr;
+        const int m = bm + row;
+        const int mc = m < g.M ? m : g.M - 1;
+        unsigned char* wr = lds + row * 512 + (lg & 1) * 8;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const int n = nh + p * 16 + lg * 4;
+          const f32x4 v = acc[i][y * 4 + p];
+          VecN4<T> r;
+          if constexpr (MODE == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r.v[e] = static_cast<T>(g.alpha * v[e]);
+          } else if constexpr (MODE == 1) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r.v[e] = static_cast<T>(g.alpha * v[e] + bias[p][e]);
+          } else {
+            float cv[4];  // columns past N are computed on valid addresses and never stored
+            if (g.c_vec) {
+              const int nv = n + 4 <= g.N ? n : 0;
+              const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (int64_t)mc * g.c_rs + nv);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) cv[e] = static_cast<float>(t.v[e]);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const int ne = n + e < g.N ? n + e : g.N - 1;
+                cv[e] = static_cast<float>(C[(int64_t)mc * g.c_rs + (int64_t)ne * g.c_cs]);
+              }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r.v[e] = static_cast<T>(g.alpha * v[e] + g.beta * cv[e]);
+          }
+          const int slot = wn * 16 + (y * 4 + p) * 2 + (lg >> 1);
+          *reinterpret_cast<VecN4<T>*>(wr + ((slot ^ (row & 31)) << 4)) = r;
+        }
+      }
+    }
+  };
+  if (!use_c) stage(std::integral_constant<int, 0>{});
+  else if (row_bias) stage(std::integral_constant<int, 1>{});
+  else stage(std::integral_constant<int, 2>{});
+  __syncthreads();
+  // wave w stores rows 64 w .. 64 w + 63 of the tile, two per instruction
+  T* D = static_cast<T*>(g.out);
+  const int r0 = wave * 64;
+  const int rows = g.M - (bm + r0) < 64 ? g.M - (bm + r0) : 64;
+  const int cols = g.N - bn < 256 ? g.N - bn : 256;
+  if (g.out_vec) {
+    const int s = lane & 31;
+#pragma unroll 8
+    for (int t = 0; t < 32; ++t) {
+      const int row = r0 + 2 * t + (lane >> 5);
+      const u32x4 v = *reinterpret_cast<const u32x4*>(lds + row * 512 + ((s ^ (row & 31)) << 4));
+      if (2 * t + (lane >> 5) < rows && 8 * s < cols) *reinterpret_cast<u32x4*>(D + (int64_t)(bm + row) * g.N + bn + 8 * s) = v;
+    }
+  } else {
+    store_slab_rows_shifted<T, 64, 32>(lds + r0 * 512, D, g.N, bm + r0, rows, bn, cols, lane);
+  }
 }
 
 // Fill requests.  x16_set_m0 sets the LDS base of the requests behind it; request i of a group of four
@@ -231,6 +338,8 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
   int pid = blockIdx.x, ptm = 0, ptn = 0;
   if constexpr (PERSIST) {
     tile_coords(g.tiles_m, g.tiles_n, pid, ptm, ptn);
+    ptm = __builtin_amdgcn_readfirstlane(ptm);  // uniform: the fill requests take their bases in SGPRs
+    ptn = __builtin_amdgcn_readfirstlane(ptn);
     bm = 0;  // the lane offsets below are relative to the tile (nothing is clamped: whole tiles only)
     bn = 0;
   }
@@ -480,6 +589,8 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       const bool has_next = npid < total;
       int ntm = ptm, ntn = ptn;
       if (has_next) tile_coords(g.tiles_m, g.tiles_n, npid, ntm, ntn);
+      ntm = __builtin_amdgcn_readfirstlane(ntm);
+      ntn = __builtin_amdgcn_readfirstlane(ntn);
       const unsigned char* na = a_start(ntm * BM);
       const unsigned char* nb = b_start(ntn * BN);
       const unsigned char* fa = a_base + 2 * a_step;
@@ -560,8 +671,14 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
 #ifdef MI355_GEMM_TRACE
   const uint64_t tr_end = __builtin_readcyclecounter();
 #endif
-  if (!(MI355_X16_ABLATE & 32) || g.alpha == 12345.f)
-  store_tile_result16<T, NPQ>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS);
+  if (!(MI355_X16_ABLATE & 32) || g.alpha == 12345.f) {
+    if constexpr (NPQ == 4) {
+      if (g.out_rows) store_tile_rows16<T>(g, acc, lds, wave, lane, bm, bn);
+      else store_tile_result16<T, NPQ>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS);
+    } else {
+      store_tile_result16<T, NPQ>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS);
+    }
+  }
 #ifdef MI355_GEMM_TRACE
   {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -582,7 +699,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   int tm, tn;
   tile_coords(g, tm, tn);
-  x16_tile<T, B_NN, 4>(g, lds, tm * BM, tn * BN);
+  x16_tile<T, B_NN, 4>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * BN));
 }
 
 // Two tile widths in one launch: blocks [0, tiles_m * tiles_n) are 256 x 256 tiles of the columns
@@ -595,10 +712,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_mixed_kernel(GemmArgs g) {
   int tm, tn;
   if ((int)blockIdx.x < wide) {
     tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
-    x16_tile<T, B_NN, 4>(g, lds, tm * BM, tn * BN);
+    x16_tile<T, B_NN, 4>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * BN));
   } else {
     tile_coords(g.tiles_m, g.tail_n, blockIdx.x - wide, tm, tn);
-    x16_tile<T, B_NN, 3>(g, lds, tm * BM, g.tiles_n * BN + tn * 192);
+    x16_tile<T, B_NN, 3>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(g.tiles_n * BN + tn * 192));
   }
 }
 

@@ -204,6 +204,46 @@ def test_mixed_width_tile_grid(backend, layout, monkeypatch):
         assert ev.bit_equal(ref[:, edge - 8:edge + 200], mixed[rows.cuda()][:, edge - 8:edge + 200].cpu())  # across the seam
 
 
+@pytest.mark.parametrize("form", ["planner", "x16", "x16mixed", "256x128", "mixed", "w4", "w8", "64x64", "128x128"])
+def test_gemm_output_rows_off_16_byte_boundaries(backend, form, monkeypatch):
+    """An output width that is no multiple of 8 (a 50257-wide vocabulary) puts every row of the result at
+    another 2-byte offset; the MFMA kernels then store along the destination's 16-byte grid: whole units
+    inside a tile's row segment, single elements at its two ends (those units are shared with the
+    neighbouring tile's columns).  Every residue of N mod 8 (and two widths that are multiples of 8 but not
+    of 64: rows on 16-byte boundaries off the 128-byte lines), ragged last tile rows and columns, each
+    kernel form (forced by its knob), with and without a bias row.  Small-integer operands: bit-equal to
+    the oracle.  The C entry point is also handed an output one element into a larger buffer, whose
+    guard elements in front and behind must come back untouched."""
+    from backendbench_amd import _lib
+    from backendbench_amd.ops._common import launch
+    announce(f"GEMM output rows off 16-byte boundaries, {form}")
+    if form in ("w4", "w8"):
+        monkeypatch.setenv("MI355_GEMM_WAVES", form[1])
+    elif form != "planner":
+        monkeypatch.setenv("MI355_GEMM_TILE", form)
+        if form == "mixed":   # the mixed-width grid belongs to the four-wave 32x32x16 kernel
+            monkeypatch.setenv("MI355_GEMM_WAVES", "4")
+    g = torch.Generator().manual_seed(23)
+    M, K = (1000, 256) if form in ("64x64", "128x128") else (2300, 256)
+    widths = (257, 1026, 1283, 2052, 2309, 2566, 2823, 301) if form in ("64x64", "128x128") else (4097, 4098, 4355, 4100, 4613, 4358, 4103, 4104, 4376)
+    a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
+    for N in widths:
+        b = torch.randint(-1, 2, (N, K), generator=g).to(torch.bfloat16).cuda().t()
+        bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
+        ref = aten_cpu.reference(aten.mm.default, [a, b])
+        out = backend[aten.mm.default](a, b)
+        assert ev.bit_equal(ref, out.cpu()), (form, N)
+        out2 = backend[aten.addmm.default](bias, a, b)
+        assert ev.bit_equal((ref.float() + bias.cpu().float()).to(torch.bfloat16), out2.cpu()), (form, N, "bias")
+        # one element into the storage (rows at every 2-byte offset, guard elements around the result)
+        big = torch.full((M * N + 64,), 77.0, dtype=torch.bfloat16, device="cuda")
+        view = big[33:33 + M * N].view(M, N)
+        launch("mi355_gemm", a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), None, 0, 0,
+               view.data_ptr(), M, N, K, 1.0, 0.0, _lib.dtype_code(a.dtype), None, 0)
+        assert ev.bit_equal(ref, view.cpu()), (form, N, "offset view")
+        assert bool((big[:33] == 77.0).all()) and bool((big[33 + M * N:] == 77.0).all()), (form, N, "guard elements")
+
+
 @pytest.mark.parametrize("tile", ["x16", "x16mixed", "planner"])
 @pytest.mark.parametrize("layout", ["nt", "nn"])
 def test_x16_gemm_every_k_loop_length(backend, layout, tile, monkeypatch):
