@@ -7,6 +7,7 @@
 //             along the innermost dim when every operand is unit-stride or broadcast there;
 //   strided64 the same with 64-bit index math for > 2^31 work items.
 #pragma once
+#include <type_traits>
 #include "common.h"
 
 namespace mi355 {
@@ -70,12 +71,24 @@ struct EwPtrs {
   void* out;
 };
 
+// A functor with `static constexpr bool kPair = true` also has pair(a, b, c, r): the same operation on two
+// neighbouring elements at once (packed f16: v_pk_maximum3_f16 / v_pk_minimum3_f16 take two elements per
+// instruction and no round trip through fp32).
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <typename F, typename = void> struct HasPair : std::false_type {};
+template <typename F> struct HasPair<F, std::enable_if_t<F::kPair>> : std::true_type {};
+
 template <typename F, int V, typename VA, typename VB, typename VC>
 __device__ __forceinline__ VecN<typename F::out_t, V> ew_apply(const F& f, const VA& a, const VB& b,
                                                               const VC& c) {
   VecN<typename F::out_t, V> r;
+  if constexpr (HasPair<F>::value && V % 2 == 0) {
 #pragma unroll
-  for (int j = 0; j < V; ++j) r.v[j] = f(a.v[j], b.v[j], c.v[j]);
+    for (int j = 0; j < V; j += 2) f.pair(a.v + j, b.v + j, c.v + j, r.v + j);
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j) r.v[j] = f(a.v[j], b.v[j], c.v[j]);
+  }
   return r;
 }
 

@@ -58,6 +58,12 @@ template <typename T> struct MaximumF {
   using out_t = T; using in0_t = T; using in1_t = T; using in2_t = Unused;
   static constexpr int NIN = 2;
   using M = typename OpMath<T>::type;
+  static constexpr bool kPair = std::is_same<T, f16_t>::value;  // v_pk_maximum3_f16: IEEE 754-2019 maximum of two pairs
+  __device__ __forceinline__ void pair(const T* a, const T* b, const Unused*, T* r) const {
+    const f16x2_t m = __builtin_elementwise_maximum(f16x2_t{(_Float16)a[0], (_Float16)a[1]}, f16x2_t{(_Float16)b[0], (_Float16)b[1]});
+    r[0] = (T)m[0];
+    r[1] = (T)m[1];
+  }
   __device__ __forceinline__ T operator()(T a, T b, Unused) const {
     const M x = static_cast<M>(a), y = static_cast<M>(b);
     if constexpr (IsFloat<T>::value) {
@@ -72,6 +78,12 @@ template <typename T> struct MinimumF {
   using out_t = T; using in0_t = T; using in1_t = T; using in2_t = Unused;
   static constexpr int NIN = 2;
   using M = typename OpMath<T>::type;
+  static constexpr bool kPair = std::is_same<T, f16_t>::value;
+  __device__ __forceinline__ void pair(const T* a, const T* b, const Unused*, T* r) const {
+    const f16x2_t m = __builtin_elementwise_minimum(f16x2_t{(_Float16)a[0], (_Float16)a[1]}, f16x2_t{(_Float16)b[0], (_Float16)b[1]});
+    r[0] = (T)m[0];
+    r[1] = (T)m[1];
+  }
   __device__ __forceinline__ T operator()(T a, T b, Unused) const {
     const M x = static_cast<M>(a), y = static_cast<M>(b);
     if constexpr (IsFloat<T>::value) {
@@ -99,6 +111,16 @@ template <typename T> struct ClampF {
   using M = typename OpMath<T>::type;
   M lo, hi;  // floating point: a missing bound is -inf / +inf, a NaN bound is kept (it makes everything NaN)
   bool has_lo, has_hi;
+  // f16: the bounds rounded to f16 (as ATen rounds them to the tensor's dtype), then the NaN-propagating
+  // packed pair - a NaN input or bound gives NaN, hi applied last
+  static constexpr bool kPair = std::is_same<T, f16_t>::value;
+  __device__ __forceinline__ void pair(const T* a, const Unused*, const Unused*, T* r) const {
+    const _Float16 l = (_Float16)lo, h = (_Float16)hi;
+    const f16x2_t m = __builtin_elementwise_minimum(
+        __builtin_elementwise_maximum(f16x2_t{(_Float16)a[0], (_Float16)a[1]}, f16x2_t{l, l}), f16x2_t{h, h});
+    r[0] = (T)m[0];
+    r[1] = (T)m[1];
+  }
   __device__ __forceinline__ T operator()(T a, Unused, Unused) const {
     M x = static_cast<M>(a);
     if constexpr (IsFloat<T>::value) {
@@ -365,6 +387,14 @@ extern "C" int mi355_where(const mi355_tensor* cond, const mi355_tensor* a, cons
 template <typename T> struct ClampTensorF {
   using out_t = T; using in0_t = T; using in1_t = T; using in2_t = T;
   static constexpr int NIN = 3;
+  static constexpr bool kPair = std::is_same<T, f16_t>::value;
+  __device__ __forceinline__ void pair(const T* x, const T* lo, const T* hi, T* r) const {
+    const f16x2_t m = __builtin_elementwise_minimum(
+        __builtin_elementwise_maximum(f16x2_t{(_Float16)x[0], (_Float16)x[1]}, f16x2_t{(_Float16)lo[0], (_Float16)lo[1]}),
+        f16x2_t{(_Float16)hi[0], (_Float16)hi[1]});
+    r[0] = (T)m[0];
+    r[1] = (T)m[1];
+  }
   __device__ __forceinline__ T operator()(T x, T lo, T hi) const {
     if constexpr (IsFloat<T>::value) {
       using M = typename OpMath<T>::type;
