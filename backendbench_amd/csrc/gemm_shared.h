@@ -31,14 +31,14 @@ struct GemmArgs {
   int32_t tail_n;  // gemm_mfma_w4_mixed_kernel: 192-wide tile columns behind the tiles_n 256-wide ones
   int32_t c_vec;  // c is unit-stride along n with 8-byte aligned rows: read it as vectors
   int32_t out_vec;  // out rows start on 16-byte boundaries (N a multiple of the vector width): vector stores
-  int32_t out_rows;  // gemm_mfma_x16_kernel: out rows do not start on 128-byte lines (N % 64 != 0), stage whole tile rows
-  int32_t bias_vec;  // c is one unit-stride row broadcast along m (a Linear layer's bias), 8-byte aligned: any N
   // Split-K (128x128 kernels only): blockIdx.y = split, which covers k in [split * ksplit,
   // min(K, (split + 1) * ksplit)) and writes its raw fp32 tile to ws[split][M][ws_ld], ws_ld = N
   // rounded up to a multiple of 4 (rows of every plane start on 16-byte boundaries for any N).
   float* ws;
   int32_t ksplit;
   int32_t ws_ld;
+  int32_t out_rows;  // gemm_mfma_x16_kernel: out rows do not start on 128-byte lines (N % 64 != 0), stage whole tile rows
+  int32_t bias_vec;  // c is one unit-stride row broadcast along m (a Linear layer's bias), 8-byte aligned: any N
 };
 
 // Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous

@@ -69,35 +69,42 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
   const int lr = lane & 15, lg = lane >> 4;
   const T* C = static_cast<const T*>(g.c);
   const bool use_c = C != nullptr && g.beta != 0.f;
-  const bool row_bias = use_c && g.bias_vec;
+  const bool row_bias = use_c && (RH == 1 ? g.bias_vec != 0 : g.c_vec && g.c_rs == 0);  // (whole tiles in the persistent form: N % 4 == 0)
   unsigned char* slab = lds + wave * (128 * 128 / RH);
   T* D = static_cast<T*>(g.out);
   const bool inside = NPQ == 4 && m0 + 128 <= g.M && n0 + 128 <= g.N;  // no row or column of this wave's tile is cut
   // MODE 0: alpha * acc; 1: + beta * a bias row (loaded once per 64 columns); 2: + beta * c.  The mode is
   // chosen once per call, outside the loops over the accumulator blocks.
-  // The bias row of the wave's 32 NPQ columns, loaded once for both halves and all passes (one exposed
-  // load latency per tile instead of one per half).
-  float bias2[2][NPQ][4];
-  if (row_bias) {
+  // The bias row of a half's 16 NPQ columns.  One workgroup per tile (RH == 1): both halves are loaded before
+  // anything is staged, one exposed load latency per tile instead of two.  The persistent form (RH == 2)
+  // keeps the next tile's first fragments in registers across its epilogue and has no room for that.
+  auto load_bias = [&](int y, float (&bias)[NPQ][4]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int y = 0; y < 2; ++y)
+    for (int p = 0; p < NPQ; ++p) {
+      const int n = n0 + y * (16 * NPQ) + p * 16 + lg * 4;
+      const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (n + 4 <= g.N ? n : 0));
 #pragma unroll
-      for (int p = 0; p < NPQ; ++p) {
-        const int n = n0 + y * (16 * NPQ) + p * 16 + lg * 4;
-        const VecN4<T> t = *reinterpret_cast<const VecN4<T>*>(C + (n + 4 <= g.N ? n : 0));
-#pragma unroll
-        for (int e = 0; e < 4; ++e) bias2[y][p][e] = g.beta * static_cast<float>(t.v[e]);
+      for (int e = 0; e < 4; ++e) bias[p][e] = g.beta * static_cast<float>(t.v[e]);
+      if constexpr (RH == 1) {  // (the persistent form walks whole tiles)
         if (n < g.N && n + 4 > g.N) {  // the last columns of an N that is no multiple of 4
 #pragma unroll
-          for (int e = 0; e < 4; ++e) bias2[y][p][e] = g.beta * static_cast<float>(C[n + e < g.N ? n + e : g.N - 1]);
+          for (int e = 0; e < 4; ++e) bias[p][e] = g.beta * static_cast<float>(C[n + e < g.N ? n + e : g.N - 1]);
         }
       }
+    }
+  };
+  float bias2[RH == 1 ? 2 : 1][NPQ][4];
+  if constexpr (RH == 1) {
+    if (row_bias) {
+      load_bias(0, bias2[0]);
+      load_bias(1, bias2[1]);
+    }
   }
-  auto half = [&](auto MODE_, auto Y_, int rh) __attribute__((always_inline)) {
+  auto half = [&](auto MODE_, int y, int rh) __attribute__((always_inline)) {
     constexpr int MODE = decltype(MODE_)::value;
-    constexpr int y = decltype(Y_)::value;
     const int nh = n0 + y * (16 * NPQ);
-    const float (&bias)[NPQ][4] = bias2[y];
+    float (&bias)[NPQ][4] = bias2[RH == 1 ? y : 0];
+    if constexpr (MODE == 1 && RH != 1) load_bias(y, bias);
     unsigned char* wr = slab + lr * 128 + (lg & 1) * 8;
     const int sx = (lr >> 1) & 7;  // = (row / 2) % 8 for every row 16 i + lr
 #pragma unroll
@@ -160,7 +167,7 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
           *reinterpret_cast<u32x4*>(dst + (int64_t)(8 * t) * g.N) = v;
         }
       }
-    } else {
+    } else if constexpr (RH == 1) {  // (the persistent form is only launched on vector stores)
       // output rows at any 2-byte offset (N % 8 != 0): the lanes walk the 16-byte grid of the destination
       const int mh = m0 + rh * (16 * IB);
       const int rows = g.M - mh < 16 * IB ? g.M - mh : 16 * IB;
@@ -171,8 +178,8 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
   auto all = [&](auto MODE_) __attribute__((always_inline)) {
 #pragma unroll
     for (int rh = 0; rh < RH; ++rh) {
-      half(MODE_, std::integral_constant<int, 0>{}, rh);
-      half(MODE_, std::integral_constant<int, 1>{}, rh);
+      half(MODE_, 0, rh);
+      half(MODE_, 1, rh);
     }
   };
   if (!use_c) all(std::integral_constant<int, 0>{});
@@ -338,8 +345,6 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
   int pid = blockIdx.x, ptm = 0, ptn = 0;
   if constexpr (PERSIST) {
     tile_coords(g.tiles_m, g.tiles_n, pid, ptm, ptn);
-    ptm = __builtin_amdgcn_readfirstlane(ptm);  // uniform: the fill requests take their bases in SGPRs
-    ptn = __builtin_amdgcn_readfirstlane(ptn);
     bm = 0;  // the lane offsets below are relative to the tile (nothing is clamped: whole tiles only)
     bn = 0;
   }
@@ -589,8 +594,6 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       const bool has_next = npid < total;
       int ntm = ptm, ntn = ptn;
       if (has_next) tile_coords(g.tiles_m, g.tiles_n, npid, ntm, ntn);
-      ntm = __builtin_amdgcn_readfirstlane(ntm);
-      ntn = __builtin_amdgcn_readfirstlane(ntn);
       const unsigned char* na = a_start(ntm * BM);
       const unsigned char* nb = b_start(ntn * BN);
       const unsigned char* fa = a_base + 2 * a_step;
