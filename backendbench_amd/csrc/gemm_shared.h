@@ -76,41 +76,46 @@ template <typename T, int ROWS, int SLOTS = 8>
 __device__ __forceinline__ void store_slab_rows_shifted(const unsigned char* slab, T* D, int64_t N, int m_first, int rows,
                                                         int n_first, int cols, int lane) {
   constexpr int RPI = 64 / SLOTS;  // rows per store instruction
-  static_assert(sizeof(T) == 2 && (SLOTS == 8 || SLOTS == 32) && ROWS % (4 * RPI) == 0, "two-byte elements, batches of four instructions");
+  static_assert(sizeof(T) == 2 && (SLOTS == 8 || SLOTS == 32) && ROWS % RPI == 0, "two-byte elements");
   if (cols <= 0) return;
   const int s = lane % SLOTS;
-  auto elem = [&](int row, int e) -> uint32_t {
+  const int s1 = s + 1 < SLOTS ? s + 1 : s;
+#pragma unroll 2
+  for (int t = 0; t < ROWS / RPI; ++t) {
+    const int row = t * RPI + lane / SLOTS;
     const int x = SLOTS == 8 ? (row >> 1) & 7 : row & (SLOTS - 1);
-    return *reinterpret_cast<const uint16_t*>(slab + row * (SLOTS * 16) + (((e >> 3) ^ x) << 4) + ((e & 7) << 1));
-  };
-  // four store instructions' worth of rows at a time: all LDS reads of the batch are issued before its first store
-#pragma unroll
-  for (int t0 = 0; t0 < ROWS / RPI; t0 += 4) {
-    u32x4 v[4];
-    uint32_t hv[4], tv[4];
-    uint16_t* dst[4];
-    int head[4], nfull[4], tail0[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int row = (t0 + u) * RPI + lane / SLOTS;
-      dst[u] = reinterpret_cast<uint16_t*>(D) + ((int64_t)(m_first + row) * N + n_first);
-      const int to_unit = (int)((16 - (reinterpret_cast<uintptr_t>(dst[u]) & 15)) & 15) >> 1;  // elements up to the next 16-byte boundary
-      head[u] = row >= rows ? 0 : to_unit < cols ? to_unit : cols;
-      nfull[u] = row >= rows ? 0 : (cols - head[u]) >> 3;
-      tail0[u] = row >= rows ? cols : head[u] + 8 * nfull[u];
-      const int e0 = head[u] + 8 * (s < nfull[u] ? s : 0);  // clamped: the slab is read, nothing is stored
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        v[u][j] = elem(row, (e0 + 2 * j) & (SLOTS * 8 - 1)) | (elem(row, (e0 + 2 * j + 1) & (SLOTS * 8 - 1)) << 16);
-      hv[u] = elem(row, s);
-      tv[u] = elem(row, (tail0[u] + s) & (SLOTS * 8 - 1));
+    const unsigned char* rp = slab + row * (SLOTS * 16);
+    // Unit s = elements head + 8 s .. + 7: the upper 8 - head elements of slot s and the lower head elements of
+    // slot s + 1, read whole (16-byte reads: no bank conflicts) and shifted into place - by head / 2 dwords
+    // through two rounds of selects, by head % 2 halves through v_alignbit.
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(rp + ((s ^ x) << 4));
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(rp + ((s1 ^ x) << 4));
+    uint16_t* dst = reinterpret_cast<uint16_t*>(D) + ((int64_t)(m_first + row) * N + n_first);
+    const int to_unit = (int)((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15) >> 1;  // elements up to the next 16-byte boundary
+    const int head = row >= rows ? 0 : to_unit < cols ? to_unit : cols;
+    const int nfull = row >= rows ? 0 : (cols - head) >> 3;
+    const int tail0 = row >= rows ? cols : head + 8 * nfull;
+    const bool q2 = (to_unit & 4) != 0, q1 = (to_unit & 2) != 0;
+    const uint32_t a0 = q2 ? lo[2] : lo[0], a1 = q2 ? lo[3] : lo[1], a2 = q2 ? hi[0] : lo[2], a3 = q2 ? hi[1] : lo[3],
+                   a4 = q2 ? hi[2] : hi[0], a5 = q2 ? hi[3] : hi[1];
+    const uint32_t b0 = q1 ? a1 : a0, b1 = q1 ? a2 : a1, b2 = q1 ? a3 : a2, b3 = q1 ? a4 : a3, b4 = q1 ? a5 : a4;
+    const uint32_t sh = (uint32_t)(to_unit & 1) * 16u;
+    if (s < nfull) {
+      u32x4 v;
+      v[0] = __builtin_amdgcn_alignbit(b1, b0, sh);
+      v[1] = __builtin_amdgcn_alignbit(b2, b1, sh);
+      v[2] = __builtin_amdgcn_alignbit(b3, b2, sh);
+      v[3] = __builtin_amdgcn_alignbit(b4, b3, sh);
+      *reinterpret_cast<u32x4*>(dst + head + 8 * s) = v;
     }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      if (s < nfull[u]) *reinterpret_cast<u32x4*>(dst[u] + head[u] + 8 * s) = v[u];
-      if (s < head[u]) dst[u][s] = (uint16_t)hv[u];
-      if (tail0[u] + s < cols) dst[u][tail0[u] + s] = (uint16_t)tv[u];
-    }
+    // The elements in front of the first unit are the first `head` of slot 0; those behind the last unit start
+    // at element tail0 = head + 8 nfull, i.e. at position `head` of slot nfull: lane s of the row takes element
+    // s of either run from the slots it has (lanes 0 and nfull hold them).
+    const int e_tail = tail0 + s;
+    if (s < head)
+      dst[s] = *reinterpret_cast<const uint16_t*>(rp + ((0 ^ x) << 4) + (s << 1));
+    if (e_tail < cols)
+      dst[e_tail] = *reinterpret_cast<const uint16_t*>(rp + ((((e_tail >> 3) & (SLOTS - 1)) ^ x) << 4) + ((e_tail & 7) << 1));
   }
 }
 
