@@ -26,6 +26,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include <atomic>
 #include "gemm_shared.h"
 
 namespace mi355 {
@@ -1955,6 +1956,29 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   return p;
 }
 
+// Split-K inside one launch of the 16x16x32 kernel (gemm_mfma_x16_splitk_kernel): for products with 65 - 128
+// tiles of 256x256 (a quarter to half of the CUs) and K >= 3072, two workgroups per tile, each with half of K.
+// The caller's workspace holds one fp32 plane of 256 KB per tile and a 64-bit flag per plane.  Measured
+// against the kernels these products took before ([M,K]x[N,K]^T, us): 96 tiles at K = 3072 63 -> 58, at
+// K = 4096 77 -> 64; 86 tiles at K = 4096 78 -> 65; 128 tiles at K = 4096 76 -> 73, at K = 11008 205 -> 153
+// (the stock kernel: 173).  It does not pay at K = 2048 (128 tiles: 44 -> 51) nor with more workgroups per
+// tile (the summing workgroup reads the other planes one after the other: 64 tiles in four parts 45 -> 85,
+// 24 tiles 27 -> 74), which is why the plan knows only two; the kernel takes up to four.
+struct X16SplitPlan {
+  int splits, tiles8;
+  int64_t ws_bytes;
+};
+constexpr int64_t kX16SplitMinK = 3072;
+static X16SplitPlan plan_x16_split(int64_t M, int64_t N, int64_t K) {
+  X16SplitPlan p{1, 0, 0};
+  const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  if (K % kX16SplitUnit != 0 || K < kX16SplitMinK || tiles <= kNumCU / 4 || tiles > kNumCU / 2) return p;
+  p.splits = 2;
+  p.tiles8 = (int)((tiles + 7) / 8 * 8);
+  p.ws_bytes = (p.splits - 1) * tiles * (int64_t)(BM * BN * 4 + 8);
+  return p;
+}
+
 // Widths for the four-wave kernel's tile columns: `wide` columns of 256 followed by `narrow` columns
 // of 192 (gemm_mfma_w4_mixed_kernel), chosen to minimise the time of the launch when workgroups
 // go to the CUs in block order, one per CU; narrow == 0 is the plain 256-wide grid.  A 192-wide
@@ -2114,7 +2138,28 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced || strcmp(forced_tile, "x16persist") == 0
                                                          : (nblocks > kNumCU / 2 || (nblocks >= 96 && K >= 2048)) && !mid &&
                                                                !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
-      if (x16) {
+      // Too few tiles for the chip and a long K: the same kernel with two workgroups per tile that share K
+      // and meet in the workspace (plan_x16_split).  Any value of MI355_GEMM_TILE but x16split keeps it off.
+      X16SplitPlan xs = plan_x16_split(M, N, K);
+#ifdef MI355_GEMM_TRACE
+      xs.splits = 1;  // the stamps use the workspace
+#endif
+      const bool x16_split = x16_ok && xs.splits > 1 && workspace != nullptr && workspace_bytes >= xs.ws_bytes &&
+                             reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+                             (forced_tile != nullptr ? strcmp(forced_tile, "x16split") == 0 : getenv("MI355_GEMM_WAVES") == nullptr);
+      if (x16_split) {
+        static std::atomic<unsigned long long> epoch{0x5bd1e9955bd1e995ull};
+        kern = gemm_x16_splitk_kernel(std::is_same<T, bf16_t>::value, !b_nt);
+        threads = 256;
+        lds_bytes = kX16Lds;
+        g.ws = static_cast<float*>(workspace);
+        g.sk_splits = xs.splits;
+        g.sk_tiles8 = xs.tiles8;
+        g.sk_epoch = epoch.fetch_add(1) | 1ull;  // never 0: a flag is 0 between launches
+        g.sk_flags = reinterpret_cast<unsigned long long*>(static_cast<unsigned char*>(workspace) + (int64_t)(xs.splits - 1) * nblocks * (BM * BN * 4));
+        g.out_rows = N % 64 != 0 || reinterpret_cast<uintptr_t>(out) % 128 != 0;
+        nblocks = (int64_t)xs.splits * xs.tiles8;
+      } else if (x16) {
         kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
         threads = 256;
         lds_bytes = kX16Lds;
@@ -2326,7 +2371,9 @@ extern "C" int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
   if (M <= 0 || N <= 0 || K <= 0 || (es != 2 && es != 4)) return 0;
   if (dtype != MI355_BF16 && dtype != MI355_F16 && dtype != MI355_F32) return 0;
   const SplitPlan p = plan_splitk(M, N, K, es);
-  return p.nsplit > 1 ? (int64_t)p.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
+  const int64_t two_launch = p.nsplit > 1 ? (int64_t)p.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
+  const int64_t one_launch = es == 2 ? plan_x16_split(M, N, K).ws_bytes : 0;
+  return two_launch > one_launch ? two_launch : one_launch;
 }
 
 extern "C" int mi355_gemm_tile_columns(int64_t M, int64_t N, int64_t K, int32_t* wide, int32_t* narrow) {

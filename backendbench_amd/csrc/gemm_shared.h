@@ -39,6 +39,13 @@ struct GemmArgs {
   int32_t ws_ld;
   int32_t out_rows;  // gemm_mfma_x16_kernel: out rows do not start on 128-byte lines (N % 64 != 0), stage whole tile rows
   int32_t bias_vec;  // c is one unit-stride row broadcast along m (a Linear layer's bias), 8-byte aligned: any N
+  // gemm_mfma_x16_splitk_kernel: sk_splits workgroups share a tile's K range and meet in the caller's
+  // workspace: (sk_splits - 1) fp32 planes of 256 x 256 per tile at ws, behind them one 64-bit flag per plane
+  // (sk_flags), which holds sk_epoch (a value no earlier launch used) once the plane is complete.
+  int32_t sk_splits;
+  int32_t sk_tiles8;  // tiles rounded up to a multiple of 8: blocks [r * sk_tiles8, (r + 1) * sk_tiles8) have one role
+  unsigned long long sk_epoch;
+  unsigned long long* sk_flags;
 };
 
 // Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous
@@ -156,6 +163,8 @@ __device__ __forceinline__ void lds_dma16s(uint32_t lds_byte_offset, uint32_t la
 constexpr int kX16Lds = 5 * 32768;
 const void* gemm_x16_kernel(bool is_bf16, bool b_nn);
 const void* gemm_x16_persistent_kernel(bool is_bf16, bool b_nn);  // one workgroup per CU walks the tiles (whole tiles, K >= 384)
-const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn);  // 256-wide tile columns, then 192-wide ones (GemmArgs::tail_n)
+const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn);
+const void* gemm_x16_splitk_kernel(bool is_bf16, bool b_nn);  // 2 - 4 workgroups per tile split K and meet in the workspace
+constexpr int kX16SplitUnit = 128;        // K shares are multiples of this  // 256-wide tile columns, then 192-wide ones (GemmArgs::tail_n)
 
 }  // namespace mi355

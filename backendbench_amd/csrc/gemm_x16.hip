@@ -58,12 +58,60 @@ __device__ __forceinline__ int xswz_k(int r, int c) { return r * 128 + ((c ^ ((r
 // land in eight distinct segments.
 __device__ __forceinline__ int xswz_seg(int k) { return (k & 3) | (((k >> 3) & 1) << 2); }
 
+// Split-K inside one launch (gemm_mfma_x16_splitk_kernel): `role` 1 .. nprod are the producers of a tile -
+// each leaves its raw fp32 accumulators in its plane (register order, x16_plane_store), then raises its flag; role 0 sums
+// the planes into its own accumulators and runs the epilogue.  Producers never wait and sit in front of the
+// summing workgroups in block order, so whatever shares the chip with this launch cannot make it wait for a
+// workgroup that has not been dispatched.
+struct X16Split {
+  f32x4* planes;              // this tile's planes (role 0) or this producer's plane (role > 0)
+  unsigned long long* flags;  // likewise
+  unsigned long long epoch;
+  int role, nprod;
+  float poison;  // -0 (x + -0 == x), or NaN when a producer never arrived
+};
+constexpr int kX16PartRows = 2;  // rows of accumulator blocks whose plane values are in flight at once (4 blocks of 4 VGPRs each per row)
+constexpr int kX16SpinLimit = 1 << 21;  // polls (about 1 us each) before the summing workgroup gives up and writes NaNs
+
+// Plane accesses are agent-scope accesses (the sc1 bit on the instruction: relaxed atomics of 8 bytes), not
+// plain ones between agent-scope fences: a fence writes back / invalidates the whole L2 of the XCD, under the
+// feet of the workgroups that are still in their K loops (measured: 89 us instead of 64 for the product it
+// was meant to speed up).  Block (i, j) of wave w: 1 KB at f32x4 index (w * 64 + 8 i + j) * 64, elements 0, 1
+// of the 64 lanes in its first half, elements 2, 3 in the second (512 contiguous bytes per instruction).
+__device__ __forceinline__ void x16_plane_store(f32x4* block, int lane, const f32x4& v) {
+  unsigned long long* q = reinterpret_cast<unsigned long long*>(block) + lane;
+  const float e0 = v[0], e1 = v[1], e2 = v[2], e3 = v[3];  // (a bit cast straight from v[i] reads element 0 for every i)
+  const unsigned long long lo = (unsigned long long)__builtin_bit_cast(uint32_t, e0) | ((unsigned long long)__builtin_bit_cast(uint32_t, e1) << 32);
+  const unsigned long long hi = (unsigned long long)__builtin_bit_cast(uint32_t, e2) | ((unsigned long long)__builtin_bit_cast(uint32_t, e3) << 32);
+  __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(q + 64, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f32x4 x16_plane_load(const f32x4* block, int lane) {
+  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(block) + lane;
+  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long hi = __hip_atomic_load(q + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  f32x4 v;
+  v[0] = __builtin_bit_cast(float, (uint32_t)lo);
+  v[1] = __builtin_bit_cast(float, (uint32_t)(lo >> 32));
+  v[2] = __builtin_bit_cast(float, (uint32_t)hi);
+  v[3] = __builtin_bit_cast(float, (uint32_t)(hi >> 32));
+  return v;
+}
+// The producers' values of accumulator block (i, j) of this wave, summed (role 0, once the flags are up).
+__device__ __forceinline__ f32x4 x16_split_partial(const X16Split& sk, int wave, int lane, int i, int j) {
+  const f32x4* p = sk.planes + (wave * 64 + i * 8 + j) * 64;
+  f32x4 v = x16_plane_load(p, lane);
+  for (int q = 1; q < sk.nprod; ++q) v += x16_plane_load(p + (size_t)q * 16384, lane);
+  v[0] += sk.poison;
+  return v;
+}
+
 // Epilogue: the wave's 128 x 32 NPQ result, 16 NPQ columns at a time, through a 16 KB slab of the idle ring
 // (rows of 128 B, 16-byte slot s of row r at s ^ ((r / 2) % 8)) and out in whole 128-byte rows.
 // Register e of acc[i][j] in lane l is C[m0 + 16 i + l % 16][n0 + 16 j + 4 (l / 16) + e] (operands swapped).
-template <typename T, int NPQ, int RH = 1>
+template <typename T, int NPQ, int RH = 1, bool SPLITK = false>
 __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32x4 (&acc)[8][2 * NPQ], unsigned char* lds,
-                                                    int wave, int lane, int m0, int n0) {
+                                                    int wave, int lane, int m0, int n0, const X16Split& sk = X16Split{}) {
   static_assert(RH == 1 || RH == 2, "the slab holds all 128 rows of the wave's tile or 64 at a time");
   constexpr int IB = 8 / RH;  // row blocks per pass
   const int lr = lane & 15, lg = lane >> 4;
@@ -107,16 +155,27 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
     if constexpr (MODE == 1 && RH != 1) load_bias(y, bias);
     unsigned char* wr = slab + lr * 128 + (lg & 1) * 8;
     const int sx = (lr >> 1) & 7;  // = (row / 2) % 8 for every row 16 i + lr
+    // split K: what the producers hold for kX16PartRows rows of this half's blocks at a time
+    f32x4 part[kX16PartRows][SPLITK ? NPQ : 1];
 #pragma unroll
     for (int ii = 0; ii < IB; ++ii) {
       const int i = rh * IB + ii;
+      if constexpr (SPLITK) {
+        if (ii % kX16PartRows == 0) {
+#pragma unroll
+          for (int u = 0; u < kX16PartRows; ++u)
+#pragma unroll
+            for (int p = 0; p < NPQ; ++p) part[u][p] = x16_split_partial(sk, wave, lane, i + u, (y ? NPQ : 0) + p);
+        }
+      }
       const int m = m0 + i * 16 + lr;
       const int mc = m < g.M ? m : g.M - 1;
 #pragma unroll
       for (int p = 0; p < NPQ; ++p) {
         const int nl = p * 16 + lg * 4;
         const int n = nh + nl;
-        const f32x4 v = acc[i][(y ? NPQ : 0) + p];
+        f32x4 v = acc[i][(y ? NPQ : 0) + p];
+        if constexpr (SPLITK) v += part[ii % kX16PartRows][p];
         VecN4<T> r;
         if constexpr (MODE == 0) {
 #pragma unroll
@@ -196,9 +255,9 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
 // (16-byte slot s of row r at s ^ (r % 32)) and every store instruction then writes two whole tile rows:
 // three complete lines and the two pieces a row shares with the neighbouring tiles.  Rows at any 2-byte
 // offset (N % 8 != 0) go out along the destination's 16-byte grid (store_slab_rows_shifted).
-template <typename T>
+template <typename T, bool SPLITK = false>
 __device__ __forceinline__ void store_tile_rows16(const GemmArgs& g, const f32x4 (&acc)[8][8], unsigned char* lds, int wave,
-                                                  int lane, int bm, int bn) {
+                                                  int lane, int bm, int bn, const X16Split& sk = X16Split{}) {
   const int wm = wave >> 1, wn = wave & 1;
   const int lr = lane & 15, lg = lane >> 4;
   const T* C = static_cast<const T*>(g.c);
@@ -226,8 +285,17 @@ __device__ __forceinline__ void store_tile_rows16(const GemmArgs& g, const f32x4
     for (int y = 0; y < 2; ++y) {
       const int nh = bn + wn * 128 + y * 64;
       const float (&bias)[4][4] = bias2[y];
+      f32x4 part[kX16PartRows][SPLITK ? 4 : 1];  // split K: what the producers hold for kX16PartRows rows of this half's blocks at a time
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
+        if constexpr (SPLITK) {
+          if (i % kX16PartRows == 0) {
+#pragma unroll
+            for (int u = 0; u < kX16PartRows; ++u)
+#pragma unroll
+              for (int p = 0; p < 4; ++p) part[u][p] = x16_split_partial(sk, wave, lane, i + u, y * 4 + p);
+          }
+        }
         const int row = wm * 128 + i * 16 + lr;
         const int m = bm + row;
         const int mc = m < g.M ? m : g.M - 1;
@@ -235,7 +303,8 @@ __device__ __forceinline__ void store_tile_rows16(const GemmArgs& g, const f32x4
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
           const int n = nh + p * 16 + lg * 4;
-          const f32x4 v = acc[i][y * 4 + p];
+          f32x4 v = acc[i][y * 4 + p];
+          if constexpr (SPLITK) v += part[i % kX16PartRows][p];
           VecN4<T> r;
           if constexpr (MODE == 0) {
 #pragma unroll
@@ -313,8 +382,8 @@ constexpr int kXBias = 3072;  // the bases point this many bytes low, so that la
 // that is free at that point (the pair just read), 64 rows of the wave's tile at a time.  For whole tiles
 // only (M, N multiples of 256: no clamped rows, so the lane offsets are the same for every tile) and
 // vector stores.
-template <typename T, bool B_NN, int NPQ, bool PERSIST = false>
-__device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, int bm, int bn) {
+template <typename T, bool B_NN, int NPQ, bool PERSIST = false, bool SPLITK = false>
+__device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, int bm, int bn, const X16Split& sk = X16Split{}) {
   static_assert(NPQ == 3 || NPQ == 4, "wave tile is 128 x 32 NPQ");
   static_assert(!PERSIST || NPQ == 4, "the persistent form walks 256 x 256 tiles");
   using frag_t = typename Mfma16<T>::frag;
@@ -674,6 +743,48 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
 #ifdef MI355_GEMM_TRACE
   const uint64_t tr_end = __builtin_readcyclecounter();
 #endif
+  if constexpr (SPLITK) {
+    // Two paths read the accumulators from here on.  Pin them to their AGPRs at this point: without it the
+    // compiler copies them out early - between the last MFMA statements, whose wait states it does not know -
+    // to have them at hand for both paths.
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 2 * NPQ; ++j) asm volatile("" : "+a"(acc[i][j]));
+    if (sk.role > 0) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x16_plane_store(sk.planes + (wave * 64 + i * 8 + j) * 64, lane, acc[i][j]);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this wave's stores have completed (no cache-wide write-back)
+      __syncthreads();
+      if (tid == 0) __hip_atomic_store(sk.flags, sk.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    volatile uint32_t* gave_up = reinterpret_cast<volatile uint32_t*>(lds);  // the ring is idle
+    if (tid == 0) {
+      uint32_t bad = 0;
+      for (int q = 0; q < sk.nprod; ++q) {
+        int polls = 0;
+        while (__hip_atomic_load(sk.flags + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != sk.epoch) {
+          if (++polls > kX16SpinLimit) { bad = 1; break; }
+          __builtin_amdgcn_s_sleep(8);
+        }
+      }
+      *gave_up = bad;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the plane loads stay behind the polls
+    __syncthreads();
+    X16Split skc = sk;
+    skc.poison = *gave_up != 0 ? __builtin_nanf("") : -0.f;
+    __syncthreads();  // everyone has read *gave_up: the epilogue reuses the ring
+    if (g.out_rows) store_tile_rows16<T, true>(g, acc, lds, wave, lane, bm, bn, skc);
+    else store_tile_result16<T, NPQ, 1, true>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS, skc);
+    __syncthreads();  // every wave has read the planes
+    if (tid == 0)
+      for (int q = 0; q < sk.nprod; ++q) __hip_atomic_store(sk.flags + q, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return;
+  }
   if (!(MI355_X16_ABLATE & 32) || g.alpha == 12345.f) {
     if constexpr (NPQ == 4) {
       if (g.out_rows) store_tile_rows16<T>(g, acc, lds, wave, lane, bm, bn);
@@ -703,6 +814,49 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
   int tm, tn;
   tile_coords(g, tm, tn);
   x16_tile<T, B_NN, 4>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * BN));
+}
+
+// Fewer tiles than half the CUs and a long K: sk_splits workgroups per tile, each with its share of K.
+// Blocks [r * sk_tiles8, (r + 1) * sk_tiles8) have one role: r < sk_splits - 1 the producers r + 1, the
+// last group the summing workgroups (blocks are dispatched in order: a summing workgroup only ever waits
+// for workgroups in front of it).  Block t of a group works on tile t; sk_tiles8 is a multiple of 8, so the
+// workgroups of one tile share an XCD and its L2 (blocks go to the XCDs round robin), and blocks past the
+// tile count have nothing to do.  K is shared out in units of 128, the summing workgroup gets the largest
+// share: what it does with the planes only starts when the last producer is done, so a producer should not
+// be the one that finishes its K loop last.
+template <typename T, bool B_NN>
+__global__ __launch_bounds__(256) void gemm_mfma_x16_splitk_kernel(GemmArgs g) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const int S = g.sk_splits, tiles = g.tiles_m * g.tiles_n;
+  const int grp = __builtin_amdgcn_readfirstlane((int)blockIdx.x / g.sk_tiles8);
+  const int t = __builtin_amdgcn_readfirstlane((int)blockIdx.x % g.sk_tiles8);
+  if (t >= tiles) return;
+  const int role = grp == S - 1 ? 0 : grp + 1;
+  int tm, tn;
+  tile_coords(g.tiles_m, g.tiles_n, t, tm, tn);
+  const int units = g.K / kX16SplitUnit;
+  const int cu = (units + S - 1) / S;
+  const int pu = units - cu, pbase = pu / (S - 1), prem = pu % (S - 1);
+  int k0 = 0, ku = cu;
+  if (role > 0) {
+    const int q = role - 1;
+    k0 = cu + q * pbase + (q < prem ? q : prem);
+    ku = pbase + (q < prem ? 1 : 0);
+  }
+  GemmArgs gs = g;
+  const T* A = static_cast<const T*>(g.a);
+  const T* B = static_cast<const T*>(g.b);
+  gs.a = A + (int64_t)k0 * kX16SplitUnit;
+  gs.b = B_NN ? B + (int64_t)k0 * kX16SplitUnit * g.ldb : B + (int64_t)k0 * kX16SplitUnit;
+  gs.K = ku * kX16SplitUnit;
+  X16Split sk;
+  const int64_t first = (int64_t)t * (S - 1) + (role > 0 ? role - 1 : 0);  // plane / flag index
+  sk.planes = reinterpret_cast<f32x4*>(g.ws) + first * 16384;
+  sk.flags = g.sk_flags + first;
+  sk.epoch = g.sk_epoch;
+  sk.role = role;
+  sk.nprod = S - 1;
+  x16_tile<T, B_NN, 4, false, true>(gs, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * BN), sk);
 }
 
 // Two tile widths in one launch: blocks [0, tiles_m * tiles_n) are 256 x 256 tiles of the columns
@@ -737,6 +891,11 @@ const void* gemm_x16_persistent_kernel(bool is_bf16, bool b_nn) {
 const void* gemm_x16_kernel(bool is_bf16, bool b_nn) {
   if (is_bf16) return b_nn ? (const void*)gemm_mfma_x16_kernel<bf16_t, true> : (const void*)gemm_mfma_x16_kernel<bf16_t, false>;
   return b_nn ? (const void*)gemm_mfma_x16_kernel<f16_t, true> : (const void*)gemm_mfma_x16_kernel<f16_t, false>;
+}
+
+const void* gemm_x16_splitk_kernel(bool is_bf16, bool b_nn) {
+  if (is_bf16) return b_nn ? (const void*)gemm_mfma_x16_splitk_kernel<bf16_t, true> : (const void*)gemm_mfma_x16_splitk_kernel<bf16_t, false>;
+  return b_nn ? (const void*)gemm_mfma_x16_splitk_kernel<f16_t, true> : (const void*)gemm_mfma_x16_splitk_kernel<f16_t, false>;
 }
 
 const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn) {

@@ -6,7 +6,7 @@ from .. import _lib
 from ._common import cast, copy_into, dense, device_managed, launch, new_dense
 
 _GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32, torch.float64)
-_SPLITK_MAX_OUT = 128 * 128 * 256  # the planner never splits problems with 256 or more 128x128 tiles
+_SPLITK_MAX_OUT = 256 * 256 * 128 + 1  # the planner never splits problems with more than 128 tiles of 256x256
 _ws_fn = None
 
 

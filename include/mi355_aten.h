@@ -182,7 +182,10 @@ int mi355_layer_norm(const void* x, int dtype, const void* weight, const void* b
 
 /* Bytes of scratch mi355_gemm can use for a problem of this size and dtype (0 = none).  The
  * scratch holds fp32 partial products when a problem with few output tiles and a long K is
- * split along K over the chip; it only has to live until the kernels of that call have run. */
+ * split along K over the chip (by a second, summing launch, or inside one launch whose
+ * workgroups meet in the scratch through flag words kept there); it only has to live until the
+ * kernels of that call have run, its contents are undefined before and after, and two calls
+ * that may run at the same time must not share it. */
 int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype);
 
 /* out[M,N] = beta * c + alpha * (a[M,K] @ b[K,N]), fp32 accumulate, out dense row-major

@@ -204,6 +204,67 @@ def test_mixed_width_tile_grid(backend, layout, monkeypatch):
         assert ev.bit_equal(ref[:, edge - 8:edge + 200], mixed[rows.cuda()][:, edge - 8:edge + 200].cpu())  # across the seam
 
 
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gemm_split_k_inside_one_launch(backend, layout, dtype):
+    """Products with 65 - 128 tiles of 256x256 and K >= 3072: two workgroups per tile take half of K each, one
+    leaves its fp32 accumulators in the workspace and raises a flag, the other adds them to its own and runs
+    the epilogue.  Tile counts at both ends of the range and off the multiples of 8, ragged last tile rows and
+    columns, output rows off the 128-byte lines and (transposed b) off the 16-byte units, unit counts of K
+    that do not halve, plain / bias row / full c epilogues.  Small-integer operands make the two-part sum
+    exact: bit-equal to the oracle.  A HIP graph of such products is replayed with eager work in between -
+    the flags must be back at zero after every run, whoever used the workspace memory in the meantime."""
+    import ctypes
+
+    from backendbench_amd import _lib
+    announce(f"GEMM split K inside one launch, {layout}, {dtype}")
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(31)
+    shapes = [(2048, 3072, 2304), (2100, 3200, 2500), (3584, 3072, 2048 + 8), (1536, 4224, 2816), (1000, 3072, 5000)]
+    if layout == "nt":
+        shapes += [(1792, 3072, 4097), (2304, 3456, 2818)]
+    for M, K, N in shapes:
+        tiles = -(-M // 256) * -(-N // 256)
+        assert 64 < tiles <= 128, (M, N, tiles)
+        assert lib.mi355_gemm_workspace_bytes(M, N, K, _lib.dtype_code(dtype)) >= tiles * (256 * 256 * 4 + 8)
+        # one in four entries of a is non-zero: every |sum| stays far below 256, exact in bf16 as well
+        a = (torch.randint(-1, 2, (M, K), generator=g) * (torch.randint(0, 4, (M, K), generator=g) == 0)).to(dtype).cuda()
+        if layout == "nt":
+            b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t()
+        else:
+            b = torch.randint(-1, 2, (K, N), generator=g).to(dtype).cuda()
+        bias = torch.randint(-2, 3, (N,), generator=g).to(dtype).cuda()
+        full = torch.randint(-2, 3, (M, N), generator=g).to(dtype).cuda()
+        ref = aten_cpu.reference(aten.mm.default, [a, b])
+        assert float(ref.abs().max()) <= 192
+        out = backend[aten.mm.default](a, b)
+        assert ev.bit_equal(ref, out.cpu()), (layout, M, K, N)
+        out = backend[aten.addmm.default](bias, a, b)
+        assert ev.bit_equal((ref.float() + bias.cpu().float()).to(dtype), out.cpu()), (layout, M, K, N, "bias row")
+        out = backend[aten.addmm.default](full, a, b, beta=2, alpha=0.5)
+        assert ev.bit_equal((0.5 * ref.float() + 2 * full.cpu().float()).to(dtype), out.cpu()), (layout, M, K, N, "full c")
+    # graph replays: the same launches (same flag value) on the same workspace memory, run after run
+    M, K, N = shapes[1]
+    a = torch.randint(-1, 2, (M, K), generator=g).to(dtype).cuda()
+    b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t() if layout == "nt" else torch.randint(-1, 2, (K, N), generator=g).to(dtype).cuda()
+    a2 = torch.randint(-1, 2, (M, K), generator=g).to(dtype).cuda()
+    want, want2 = backend[aten.mm.default](a, b), backend[aten.mm.default](a2, b)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got = backend[aten.mm.default](a, b)
+        got2 = backend[aten.mm.default](a2, b)
+    for rep in range(4):
+        got.zero_()
+        got2.zero_()
+        junk = torch.full((64 << 20,), float(rep), device="cuda")   # eager work that may land on the freed workspace
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert ev.bit_equal(want, got) and ev.bit_equal(want2, got2), (layout, "replay", rep)
+        del junk
+
+
 @pytest.mark.parametrize("form", ["planner", "x16", "x16mixed", "256x128", "mixed", "w4", "w8", "64x64", "128x128"])
 def test_gemm_output_rows_off_16_byte_boundaries(backend, form, monkeypatch):
     """An output width that is no multiple of 8 (a 50257-wide vocabulary) puts every row of the result at
