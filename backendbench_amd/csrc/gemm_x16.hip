@@ -756,7 +756,9 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) x16_plane_store(sk.planes + (wave * 64 + i * 8 + j) * 64, lane, acc[i][j]);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // this wave's stores have completed (no cache-wide write-back)
+      // this wave's stores have completed before the barrier (a workgroup-scope fence leaves the counter
+      // alone here, an agent-scope one writes back the whole L2)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0) __hip_atomic_store(sk.flags, sk.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return;
