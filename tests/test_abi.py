@@ -102,6 +102,16 @@ def test_workspace_planners_run_on_the_host():
     assert odd > 0 and odd % (24 * 1004 * 4) == 0
     tiny = lib.mi355_gemm_workspace_bytes(64, 250, 1040, _lib.F32)           # fp32, 64x64 tiles
     assert tiny > 0 and tiny % (64 * 252 * 4) == 0
+    # 65 - 128 tiles of 256x256 with K >= 3072 (a multiple of 128): split K inside one launch, one fp32 plane
+    # of 256 KB and one 8-byte flag per tile; not for fp32, a shorter K, a K off the unit, or other tile counts
+    plane = 256 * 256 * 4 + 8
+    assert lib.mi355_gemm_workspace_bytes(2048, 4096, 4096, _lib.BF16) == 128 * plane
+    assert lib.mi355_gemm_workspace_bytes(2100, 2500, 3200, _lib.F16) == 90 * plane       # ragged tiles count whole
+    assert lib.mi355_gemm_workspace_bytes(2048, 4096, 4096, _lib.F32) == 0
+    assert lib.mi355_gemm_workspace_bytes(2048, 4096, 2944, _lib.BF16) == 0
+    assert lib.mi355_gemm_workspace_bytes(2048, 4096, 3136, _lib.BF16) == 0
+    assert lib.mi355_gemm_workspace_bytes(2304, 4096, 4096, _lib.BF16) == 0               # 144 tiles
+    assert lib.mi355_gemm_workspace_bytes(4096, 4096, 4096, _lib.BF16) == 0
 
 
 def _tile_columns(M, N, K=4096):
