@@ -1552,7 +1552,9 @@ __device__ __forceinline__ int swz_n64(int k, int u) {
   return k * 128 + ((((u >> 2) ^ ((k >> 1) & 1))) << 6) + ((u & 3) << 4);
 }
 
-template <typename T, bool B_NN, int S>
+// SPLIT: blockIdx.y owns the k range [blockIdx.y * ksplit, + ksplit) (whole 64-k stages) and leaves its raw fp32
+// tile in plane blockIdx.y of the workspace, as the 128x128 kernels do; gemm_splitk_finish_kernel sums the planes.
+template <typename T, bool B_NN, int S, bool SPLIT = false>
 __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using frag_t = typename Mfma<T>::frag;
@@ -1562,8 +1564,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
   int tm, tn;
   tile_coords(g, tm, tn);
   const int bm = tm * TBM, bn = tn * TBN;
-  const T* a_base = static_cast<const T*>(g.a) + (int64_t)bm * g.lda;
-  const T* b_base = static_cast<const T*>(g.b) + (B_NN ? 0 : (int64_t)bn * g.ldb);
+  const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
+  const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
+  const T* a_base = static_cast<const T*>(g.a) + (int64_t)bm * g.lda + kbeg;
+  const T* b_base = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)bn * g.ldb + kbeg);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
   // Region q = wave + 4 i (i < 2) of a panel is LDS bytes [q * 1024, q * 1024 + 1024): eight rows of 128 B.
@@ -1620,7 +1624,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[0][0][e] = acc_odd[e] = 0.f;
 
-  const int nk = g.K / 64;
+  const int nk = (kend - kbeg) / 64;
   for (int t = 0; t < S - 1 && t < nk; ++t) request_stage(t);
   for (int t = 0; t < nk; ++t) {
     const int last_requested = t + S - 2 < nk - 1 ? t + S - 2 : nk - 1;
@@ -1650,6 +1654,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
   }
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[0][0][e] += acc_odd[e];
+  if constexpr (SPLIT) {
+    store_partial_tile<1, 1>(g, acc, lane, bm + wm * 32, bn + wn * 32);
+    return;
+  }
   __syncthreads();  // the ring becomes the epilogue's staging area
   store_tile_result<T, 1, 0, 1>(g, acc, lds, wave, lane, bm + wm * 32, bn + wn * 32);
 }
@@ -1956,6 +1964,33 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   return p;
 }
 
+// Split-K for the 64x64-tile kernel: a handful of tiles with a long K (one image's 197 tokens against a
+// 3072 x 768 weight) leave most CUs idle and walk K at about 0.3 us per 64-k stage.  Splits of whole stages, at
+// least four each; the cost model is the one of plan_splitk with this kernel's figures (2 us to get going,
+// 0.3 us per stage, 1.3 x that with two workgroups on a CU, 3 us and the partial planes for the summing launch).
+static SplitPlan plan_t64_split(int64_t M, int64_t N, int64_t K) {
+  SplitPlan p{1, (int)K};
+  const int64_t tiles = ((M + TBM - 1) / TBM) * ((N + TBN - 1) / TBN);
+  if (K % 64 != 0 || K < 1024 || tiles > kNumCU / 2) return p;
+  const int64_t stages = K / 64;
+  double best = 0;
+  int64_t best_ks = stages;
+  for (int64_t ns = 1; ns <= stages / 4 && ns <= 64; ++ns) {
+    const int64_t ks = (stages + ns - 1) / ns;
+    if ((stages + ks - 1) / ks != ns || stages - (ns - 1) * ks < 4) continue;
+    const int64_t per_cu = (tiles * ns + kNumCU - 1) / kNumCU;
+    double t = 2000.0 + 300.0 * (double)ks * (per_cu >= 2 ? 1.3 * (double)((per_cu + 1) / 2) : 1.0);
+    if (ns > 1) t += 3000.0 + (double)ns * (double)M * (double)N * 8.0 / 4000.0;
+    if (ns == 1 || t < best) {
+      best = t;
+      best_ks = ks;
+    }
+  }
+  p.ksplit = (int)(best_ks * 64);
+  p.nsplit = (int)((stages + best_ks - 1) / best_ks);
+  return p;
+}
+
 // Split-K inside one launch of the 16x16x32 kernel (gemm_mfma_x16_splitk_kernel): for products with 65 - 128
 // tiles of 256x256 (a quarter to half of the CUs) and K >= 3072, two workgroups per tile, each with half of K.
 // The caller's workspace holds one fp32 plane of 256 KB per tile and a 64-bit flag per plane.  Measured
@@ -2119,10 +2154,17 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // tile would be padding ([32,768]x[768,32000]: 17.5 -> 13.3 us).  MI355_GEMM_TILE=64x64 forces them, =128x128 keeps them off: test knobs.
       const int64_t nb128 = ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN);
       const int64_t nb64 = ((M + TBM - 1) / TBM) * ((N + TBN - 1) / TBN);
+      // With scratch for its split-K form (plan_t64_split) they also take the few tiles with a long K
+      // ([197,3072]x[3072,768]: 15.4 -> 12.1 us, [64,4096]x[4096,4096]: 17.6 -> 15.2, [64,11008]x[11008,4096]: 32.8 ->
+      // 28.4; not a handful of rows against a weight that takes longer to stream than to multiply:
+      // [8,8192]x[8192,8192] 32.1 us on the 128x128 kernels, 35.8 here).
+      const SplitPlan ts = plan_t64_split(M, N, K);
+      const bool t64_split = ts.nsplit > 1 && M >= 16 && workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+                             workspace_bytes >= (int64_t)ts.nsplit * M * ((N + 3) / 4 * 4) * 4;
       const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
                                                : (nb128 < kNumCU / 2 || (M <= 64 && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
-                                                     (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2)));
+                                                     (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2) || t64_split));
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
       // with 256x256 tiles when K is a multiple of 128 (from 256 on): measured against the 32x32x16 forms on
       // [4096,K]x[K,16384], it is 11 % faster at K = 256 and 4 - 15 % from K = 768 on (C3: [4096,4096]x
@@ -2201,10 +2243,21 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         g.tiles_n = (int32_t)((N + TBN - 1) / TBN);
         nblocks = nb64;
         threads = 256;
-        const bool deep = nblocks <= kNumCU;
+        if (t64_split) {
+          nsplit = ts.nsplit;
+          g.ws = static_cast<float*>(workspace);
+          g.ksplit = ts.ksplit;
+          g.ws_ld = (int32_t)((N + 3) / 4 * 4);
+        }
+        const bool deep = nblocks * nsplit <= kNumCU;
         lds_bytes = (deep ? 8 : 4) * kTStage;
-        if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8> : (const void*)gemm_mfma_t64_kernel<T, true, 8>;
-        else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4> : (const void*)gemm_mfma_t64_kernel<T, true, 4>;
+        if (nsplit > 1) {
+          if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8, true> : (const void*)gemm_mfma_t64_kernel<T, true, 8, true>;
+          else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4, true> : (const void*)gemm_mfma_t64_kernel<T, true, 4, true>;
+        } else {
+          if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8> : (const void*)gemm_mfma_t64_kernel<T, true, 8>;
+          else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4> : (const void*)gemm_mfma_t64_kernel<T, true, 4>;
+        }
       } else if (mid) {
         g.tiles_n = (int32_t)((N + 127) / 128);
         nblocks = tiles_mid;
@@ -2371,7 +2424,12 @@ extern "C" int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
   if (M <= 0 || N <= 0 || K <= 0 || (es != 2 && es != 4)) return 0;
   if (dtype != MI355_BF16 && dtype != MI355_F16 && dtype != MI355_F32) return 0;
   const SplitPlan p = plan_splitk(M, N, K, es);
-  const int64_t two_launch = p.nsplit > 1 ? (int64_t)p.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
+  int64_t two_launch = p.nsplit > 1 ? (int64_t)p.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
+  if (es == 2) {  // the 64x64-tile kernel's own split
+    const SplitPlan t = plan_t64_split(M, N, K);
+    const int64_t t64 = t.nsplit > 1 ? (int64_t)t.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
+    two_launch = t64 > two_launch ? t64 : two_launch;
+  }
   const int64_t one_launch = es == 2 ? plan_x16_split(M, N, K).ws_bytes : 0;
   return two_launch > one_launch ? two_launch : one_launch;
 }

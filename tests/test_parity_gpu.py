@@ -235,8 +235,10 @@ def test_gemm_split_k_inside_one_launch(backend, layout, dtype):
             b = torch.randint(-1, 2, (K, N), generator=g).to(dtype).cuda()
         bias = torch.randint(-2, 3, (N,), generator=g).to(dtype).cuda()
         full = torch.randint(-2, 3, (M, N), generator=g).to(dtype).cuda()
-        ref = aten_cpu.reference(aten.mm.default, [a, b])
+        # the oracle on the fp32 copies (its f16 kernel takes a minute here): exact integer sums, exact in `dtype`
+        ref = aten_cpu.reference(aten.mm.default, [a.float(), b.float()])
         assert float(ref.abs().max()) <= 192
+        ref = ref.to(dtype)
         out = backend[aten.mm.default](a, b)
         assert ev.bit_equal(ref, out.cpu()), (layout, M, K, N)
         out = backend[aten.addmm.default](bias, a, b)
@@ -491,6 +493,36 @@ def test_split_k_with_ragged_k(backend, dtype):
             out = backend[aten.mm.default](a, b)
             ref = aten_cpu.reference(aten.mm.default, [a, b])
             assert ev.bit_equal(ref, out.cpu()), (M, N, K, nt)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_split_k_on_64x64_tiles(backend, dtype, monkeypatch):
+    """A handful of 64x64 tiles with a long K (one image's 197 tokens against a 3072 x 768 weight) split K in
+    whole 64-k stages over the chip: blockIdx.y owns a k range, leaves its raw fp32 tile in its plane, and the
+    summing launch applies alpha / beta / bias.  Stage counts that do not divide by the split count, ragged
+    and odd-N outputs, both layouts of b, every epilogue; MI355_GEMM_TILE=64x64 forces the kernel where the
+    planner would take another one.  Small-integer operands: bit-equal to the oracle."""
+    announce(f"split-K on 64x64 tiles, {dtype}")
+    g = torch.Generator().manual_seed(43)
+    for forced in (False, True):
+        if forced:
+            monkeypatch.setenv("MI355_GEMM_TILE", "64x64")
+        for M, N, K in [(197, 768, 3072), (128, 768, 3136), (16, 4096, 4096), (70, 1001, 2112), (256, 4096, 4032), (64, 520, 11008), (300, 200, 1088)]:
+            for nt in (True, False):
+                if not nt and N % 8:
+                    continue
+                a = (torch.randint(-1, 2, (M, K), generator=g) * (torch.randint(0, 4, (M, K), generator=g) == 0)).to(dtype).cuda()
+                b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t() if nt else torch.randint(-1, 2, (K, N), generator=g).to(dtype).cuda()
+                bias = torch.randint(-2, 3, (N,), generator=g).to(dtype).cuda()
+                full = torch.randint(-2, 3, (M, N), generator=g).to(dtype).cuda()
+                ref = aten_cpu.reference(aten.mm.default, [a.float(), b.float()])   # exact integer sums (the f16 CPU kernel is slow)
+                assert float(ref.abs().max()) <= 192
+                ref = ref.to(dtype)
+                assert ev.bit_equal(ref, backend[aten.mm.default](a, b).cpu()), (forced, M, N, K, nt)
+                out = backend[aten.addmm.default](bias, a, b)
+                assert ev.bit_equal((ref.float() + bias.cpu().float()).to(dtype), out.cpu()), (forced, M, N, K, nt, "bias row")
+                out = backend[aten.addmm.default](full, a, b, beta=2, alpha=0.5)
+                assert ev.bit_equal((0.5 * ref.float() + 2 * full.cpu().float()).to(dtype), out.cpu()), (forced, M, N, K, nt, "full c")
 
 
 def test_f64_addmm_keeps_alpha_and_beta_in_f64(backend):
