@@ -2214,7 +2214,17 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         // where the dispatcher hands a tile to whichever CU is free first ([8192,768]x[768,2304], 288
         // tiles: 46.2 us against 43.4; [12544,768]x[768,3072], 588 tiles: 75.8 against 71.1; level at
         // exactly two and three rounds; 24.5 rounds at K = 768: 592 against 636).
-        bool persist = M % BM == 0 && N % BN == 0 && g.out_vec && K >= 384 &&
+        // M or N off the multiples of 256: the walk moves its last row / column of tiles back to the edge and
+        // computes the overlap twice - for output rows on 128-byte lines, and never when c shares memory with
+        // out (an element of the overlap would take beta * c twice).
+        const unsigned char* c_lo = static_cast<const unsigned char*>(c);
+        const unsigned char* o_lo = static_cast<const unsigned char*>(out);
+        const int64_t c_span = ((M - 1) * c_rs + (N - 1) * c_cs + 1) * (int64_t)sizeof(T);  // (non-negative strides)
+        const bool c_apart = c == nullptr || beta == 0.0 ||
+                             (c_rs >= 0 && c_cs >= 0 && (c_lo + c_span <= o_lo || o_lo + M * N * (int64_t)sizeof(T) <= c_lo));
+        const bool whole = M % BM == 0 && N % BN == 0;
+        const bool edge_ok = M >= BM && N >= BN && N % 64 == 0 && reinterpret_cast<uintptr_t>(out) % 128 == 0 && c_apart;
+        bool persist = (whole || edge_ok) && g.out_vec && K >= 384 &&
                        (forced_tile == nullptr ? nblocks > kNumCU && (K >= 2048 || nblocks >= 4 * kNumCU) : persist_forced);
 #ifdef MI355_GEMM_TRACE
         persist = false;  // the stamps are per workgroup = per tile

@@ -379,9 +379,9 @@ constexpr int kXBias = 3072;  // the bases point this many bytes low, so that la
 // first five pairs of the next one, its last half-stage reads the next tile's first fragments, and the
 // next K loop starts the moment the epilogue has issued its stores - no prologue latency, no gap between
 // workgroups, and the stores drain while the next tile computes.  The epilogue borrows the one ring slot
-// that is free at that point (the pair just read), 64 rows of the wave's tile at a time.  For whole tiles
-// only (M, N multiples of 256: no clamped rows, so the lane offsets are the same for every tile) and
-// vector stores.
+// that is free at that point (the pair just read), 64 rows of the wave's tile at a time.  Every tile is
+// whole (no clamped rows, so the lane offsets are the same for every tile): when M or N is no multiple of 256
+// the last row / column of tiles overlaps its neighbour.  Vector stores only.
 template <typename T, bool B_NN, int NPQ, bool PERSIST = false, bool SPLITK = false>
 __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, int bm, int bn, const X16Split& sk = X16Split{}) {
   static_assert(NPQ == 3 || NPQ == 4, "wave tile is 128 x 32 NPQ");
@@ -424,8 +424,13 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
     const T* B = static_cast<const T*>(g.b);
     return reinterpret_cast<const unsigned char*>(B_NN ? (PERSIST ? B + tn : B) : B + (int64_t)tn * g.ldb) - kXBias;
   };
-  const unsigned char* a_base = a_start(PERSIST ? ptm * BM : bm);  // of the tile being computed
-  const unsigned char* b_base = b_start(PERSIST ? ptn * BN : bn);
+  // PERSIST: a last row or column of tiles that would stick out of the matrix is moved back so that it ends
+  // at the edge (M, N >= 256): every tile stays whole, and the rows / columns it shares with its neighbour are
+  // computed - from the same k sequence - and stored twice with the same values.
+  auto row0 = [&](int tm) { const int m = tm * BM; return m + BM <= g.M ? m : g.M - BM; };
+  auto col0 = [&](int tn) { const int n = tn * BN; return n + BN <= g.N ? n : g.N - BN; };
+  const unsigned char* a_base = a_start(PERSIST ? row0(ptm) : bm);  // of the tile being computed
+  const unsigned char* b_base = b_start(PERSIST ? col0(ptn) : bn);
   const int64_t a_step = 128;                                   // bytes per 64-k stage
   const int64_t b_step = B_NN ? (int64_t)128 * g.ldb : 128;
   uint32_t a_off[2][4], b_off[2][4];
@@ -663,8 +668,8 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       const bool has_next = npid < total;
       int ntm = ptm, ntn = ptn;
       if (has_next) tile_coords(g.tiles_m, g.tiles_n, npid, ntm, ntn);
-      const unsigned char* na = a_start(ntm * BM);
-      const unsigned char* nb = b_start(ntn * BN);
+      const unsigned char* na = a_start(row0(ntm));
+      const unsigned char* nb = b_start(col0(ntn));
       const unsigned char* fa = a_base + 2 * a_step;
       const unsigned char* fb = b_base + 2 * b_step;
       // First four half-stages (np >= 12): pairs 2 .. 4 were requested before the previous tile's 32
@@ -695,7 +700,7 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       // the last MFMA's result is read by VALU moves next; the slot of the pair just read (`fl`) is free
       // until the next half-stage requests into it
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-      store_tile_result16<T, NPQ, 2>(g, acc, lds + fl, wave, lane, ptm * BM + wm * 128, ptn * BN + wn * 128);
+      store_tile_result16<T, NPQ, 2>(g, acc, lds + fl, wave, lane, row0(ptm) + wm * 128, col0(ptn) + wn * 128);
       __syncthreads();  // every wave is done with its slab before anyone requests into the slot
       if (!has_next) break;
       pid = npid; ptm = ntm; ptn = ntn;

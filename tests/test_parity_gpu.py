@@ -385,16 +385,20 @@ def test_x16_gemm_argument_forms(backend, tile, monkeypatch):
 
 @pytest.mark.parametrize("layout", ["nt", "nn"])
 def test_x16_persistent_gemm_walks_its_tiles(backend, layout, monkeypatch):
-    """More whole 256x256 tiles than CUs: one workgroup per CU walks its tiles, with the fill requests running on
+    """More 256x256 tiles than CUs: one workgroup per CU walks its tiles, with the fill requests running on
     from one tile into the next.  [4096, K] x [K, 4352] has 16 x 17 = 272 tiles (sixteen workgroups get a second
     tile), [2048, K] x [K, 12288] 8 x 48 = 384 (half of them), [256, K] x [K, 256] a single one (forced: a walk
     of one tile).  K from the shortest loop the walk takes (384: the four special half-stages and the eight last
     ones, no steady iteration) upwards.  Bit-equal to the one-workgroup-per-tile form of the same kernel
     (same k order per element) and, on small-integer operands, to the oracle on sampled rows; bias row and a
     full c through the epilogue's four passes."""
+    from backendbench_amd import _lib
+    from backendbench_amd.ops._common import launch
     announce(f"persistent 16x16x32 GEMM, {layout}")
     g = torch.Generator().manual_seed(14)
-    for (M, N) in ((4096, 4352), (2048, 12288), (256, 256)):
+    # (4000, 4416), (2100, 12352), (300, 320): M and N off the multiples of 256 (N a multiple of 64) - the walk moves
+    # its last row / column of tiles back to the matrix edge and stores the overlap twice
+    for (M, N) in ((4096, 4352), (2048, 12288), (256, 256), (4000, 4416), (2100, 12352), (300, 320)):
         rows = torch.unique(torch.cat([torch.randint(0, M, (24,), generator=g), torch.tensor([0, 63, 64, 127, 128, 255, M - 1])]))
         for K in (384, 512, 640, 768, 1024, 2048):
             a = torch.randint(-1, 2, (M, K), generator=g).to(torch.bfloat16).cuda()
@@ -419,6 +423,14 @@ def test_x16_persistent_gemm_walks_its_tiles(backend, layout, monkeypatch):
             ref_c = aten_cpu.reference(aten.addmm.default, [c[rows.cuda()], a[rows.cuda()], b], {"beta": 2.0})
             assert ev.bit_equal(ref_c, walked_c[rows.cuda()].cpu()), (layout, M, N, K, "full c")
             assert ev.bit_equal((walked.float() - bias.float()).to(torch.bfloat16), walked_mm), (layout, M, N, K, "mm")
+            if (M % 256 or N % 256) and K == 768:
+                # c in the memory of out (the C entry point allows it): no element may take beta * c twice
+                monkeypatch.setenv("MI355_GEMM_TILE", "x16persist")
+                acc = c.clone()
+                launch("mi355_gemm", a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), acc.data_ptr(), N, 1,
+                       acc.data_ptr(), M, N, K, 1.0, 2.0, _lib.dtype_code(a.dtype), None, 0)
+                monkeypatch.delenv("MI355_GEMM_TILE")
+                assert ev.bit_equal(walked_c, acc), (layout, M, N, K, "c in place")
 
 
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
