@@ -2157,14 +2157,14 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // With scratch for its split-K form (plan_t64_split) they also take the few tiles with a long K
       // ([197,3072]x[3072,768]: 15.4 -> 12.1 us, [64,4096]x[4096,4096]: 17.6 -> 15.2, [64,11008]x[11008,4096]: 32.8 ->
       // 28.4; not a handful of rows against a weight that takes longer to stream than to multiply:
-      // [8,8192]x[8192,8192] 32.1 us on the 128x128 kernels, 35.8 here).
+      // [8,8192]x[8192,8192] 32.1 us on the 128x128 kernels, 35.8 here split, 42.4 unsplit).
       const SplitPlan ts = plan_t64_split(M, N, K);
       const bool t64_split = ts.nsplit > 1 && M >= 16 && workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
                              workspace_bytes >= (int64_t)ts.nsplit * M * ((N + 3) / 4 * 4) * 4;
       const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
                                                : (nb128 < kNumCU / 2 || (M <= 64 && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
-                                                     (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2) || t64_split));
+                                                     (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2 && M >= 16) || t64_split));
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
       // with 256x256 tiles when K is a multiple of 128 (from 256 on): measured against the 32x32x16 forms on
       // [4096,K]x[K,16384], it is 11 % faster at K = 256 and 4 - 15 % from K = 768 on (C3: [4096,4096]x
