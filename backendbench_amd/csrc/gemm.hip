@@ -2159,12 +2159,17 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // 28.4; not a handful of rows against a weight that takes longer to stream than to multiply:
       // [8,8192]x[8192,8192] 32.1 us on the 128x128 kernels, 35.8 here split, 42.4 unsplit).
       const SplitPlan ts = plan_t64_split(M, N, K);
-      const bool t64_split = ts.nsplit > 1 && M >= 16 && workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+      // ... nor 16 - 32 rows against 128 MB of weight ([16,8192]x[8192,8192]: 32.4 us there, 35.8 here).
+      const bool light_b = (int64_t)N * K * (int64_t)sizeof(T) <= 100000000;
+      const bool t64_split = ts.nsplit > 1 && M >= 16 && light_b && workspace != nullptr &&
+                             reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
                              workspace_bytes >= (int64_t)ts.nsplit * M * ((N + 3) / 4 * 4) * 4;
       const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
                                                : (nb128 < kNumCU / 2 || (M <= 64 && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
-                                                     (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2 && M >= 16) || t64_split));
+                                                     (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2 && M >= 16 && light_b) || t64_split ||
+                                                      nb64 >= 160));  // enough 64x64 tiles for the chip: no need to split a long K
+                                                                      // (a few rows against a 32000 x 4096 vocabulary: 48 us, 128x128 tiles 55)
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
       // with 256x256 tiles when K is a multiple of 128 (from 256 on): measured against the 32x32x16 forms on
       // [4096,K]x[K,16384], it is 11 % faster at K = 256 and 4 - 15 % from K = 768 on (C3: [4096,4096]x
@@ -2175,10 +2180,14 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // Output rows that do not start on 128-byte lines (N % 64 != 0) get its whole-tile-row epilogue.
       // MI355_GEMM_TILE=x16 forces this form for any tile count (=x16mixed: with the mixed-width grid at any K), =256x256 / =mixed keep
       // the 32x32x16 form (test knobs).
+      // Fewer tiles than CUs: only when the tiles are mostly output (a few rows against a wide weight make
+      // 125 tiles of 256 rows that are 99 % padding: [8,4096]x[4096,32000] took 83 us here, 48 on 64x64 tiles).
+      const bool well_filled = (double)M * (double)N >= 0.75 * (double)nblocks * BM * BN;
       const bool x16_ok = K % 128 == 0 && K >= 256 && !a_t && ld32;
+      const bool x16_pays = nblocks > kNumCU || well_filled;  // (the planner's rule; the knobs force the kernel regardless)
       const bool x16_mixed_forced = forced_tile != nullptr && strcmp(forced_tile, "x16mixed") == 0;  // mixed widths at any K
       const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced || strcmp(forced_tile, "x16persist") == 0
-                                                         : (nblocks > kNumCU / 2 || (nblocks >= 96 && K >= 2048)) && !mid &&
+                                                         : x16_pays && (nblocks > kNumCU / 2 || (nblocks >= 96 && K >= 2048)) && !mid &&
                                                                !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
       // Too few tiles for the chip and a long K: the same kernel with two workgroups per tile that share K
       // and meet in the workspace (plan_x16_split).  Any value of MI355_GEMM_TILE but x16split keeps it off.
@@ -2188,7 +2197,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
 #endif
       const bool x16_split = x16_ok && xs.splits > 1 && workspace != nullptr && workspace_bytes >= xs.ws_bytes &&
                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
-                             (forced_tile != nullptr ? strcmp(forced_tile, "x16split") == 0 : getenv("MI355_GEMM_WAVES") == nullptr);
+                             (forced_tile != nullptr ? strcmp(forced_tile, "x16split") == 0 : x16_pays && getenv("MI355_GEMM_WAVES") == nullptr);
       if (x16_split) {
         static std::atomic<unsigned long long> epoch{0x5bd1e9955bd1e995ull};
         kern = gemm_x16_splitk_kernel(std::is_same<T, bf16_t>::value, !b_nt);
