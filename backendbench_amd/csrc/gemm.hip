@@ -2146,7 +2146,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const char* forced_tile = getenv("MI355_GEMM_TILE");
       const bool mid = !ktail && K % 64 == 0 && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "256x128") == 0
-                                               : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > (K >= 2048 ? 228 : 248) && tiles_mid <= kNumCU);
+                                               : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > (K >= 2048 ? 228 : 248) && tiles_mid <= kNumCU &&
+                                                     4 * M >= 3 * (int64_t)g.tiles_m * BM);  // rows that are mostly output ([128,4096]x[4096,32000]: 74 us here, 61 on 128x128 tiles)
       // Fewer 128x128 tiles than half the CUs: 64x64 tiles reach four times as many (measured on this
       // chip: [197,768]x[768,768] 11.6 -> 7.5 us, 1024^3 14.6 -> 9.4 us).  A 64x64 workgroup walks K at
       // about 0.3 us per 64 k, so a few tiles with a long K stay on the 128x128 kernels, which split K
@@ -2166,7 +2167,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                              workspace_bytes >= (int64_t)ts.nsplit * M * ((N + 3) / 4 * 4) * 4;
       const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
-                                               : (nb128 < kNumCU / 2 || (M <= 64 && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
+                                               : (nb128 < kNumCU / 2 || ((M <= 64 || N <= 64) && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
                                                      (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2 && M >= 16 && light_b) || t64_split ||
                                                       nb64 >= 160));  // enough 64x64 tiles for the chip: no need to split a long K
                                                                       // (a few rows against a 32000 x 4096 vocabulary: 48 us, 128x128 tiles 55)
@@ -2197,7 +2198,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
 #endif
       const bool x16_split = x16_ok && xs.splits > 1 && workspace != nullptr && workspace_bytes >= xs.ws_bytes &&
                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
-                             (forced_tile != nullptr ? strcmp(forced_tile, "x16split") == 0 : x16_pays && getenv("MI355_GEMM_WAVES") == nullptr);
+                             (forced_tile != nullptr ? strcmp(forced_tile, "x16split") == 0
+                                                     : x16_pays && M >= 512 && getenv("MI355_GEMM_WAVES") == nullptr);  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
       if (x16_split) {
         static std::atomic<unsigned long long> epoch{0x5bd1e9955bd1e995ull};
         kern = gemm_x16_splitk_kernel(std::is_same<T, bf16_t>::value, !b_nt);
