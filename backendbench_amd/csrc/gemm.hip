@@ -19,8 +19,9 @@
 //            Problems with few tiles run on 128x128 tiles (two workgroups per CU), split along
 //            K over the chip when the caller provides a workspace.
 //   mfma f32 v_mfma_f32_32x32x2_f32, 128x128 tiles.
-//   generic  any strides and dtypes (f64 accumulates in f64): 64x64 LDS tile, FMA inner loop.
+//   generic  any strides, the dtypes but f64: 64x64 LDS tile, FMA inner loop.
 //            Correctness path for shapes the MFMA kernels do not take.
+//   f64      gemm_f64.hip: v_mfma_f64_16x16x4_f64, any strides.
 #include <stdlib.h>
 #include <string.h>
 #include <type_traits>
@@ -1842,11 +1843,11 @@ __global__ __launch_bounds__(256) void gemm_mfma_f32_kernel(GemmArgs g) {
 }
 
 // ---------------------------------------------------------------- generic fallback
-// Any strides; fp64 accumulates in fp64, the other dtypes in fp32.  A block of 256 threads owns
+// Any strides; accumulates in fp32 (fp64 products run on the MFMA kernel of gemm_f64.hip; instantiated
+// for double, this kernel would accumulate in fp64).  A block of 256 threads owns
 // a (16 TT) x (16 TT) tile, TT x TT outputs per thread (rows ty TT + i, columns tx + 16 j: lanes
 // along n, so LDS reads of B and the stores are conflict-free and coalesced), GK-k steps.  TT = 4:
-// 64x64 tiles, 32-k steps; TT = 8: 128x128 tiles, 16-k steps, half the LDS reads per FMA (large
-// fp64 products).  The loads of step t + 1 are issued into registers before the FMAs of step t,
+// 64x64 tiles, 32-k steps; TT = 8: 128x128 tiles, 16-k steps, half the LDS reads per FMA.  The loads of step t + 1 are issued into registers before the FMAs of step t,
 // so a step costs its arithmetic and not a round trip to memory; the element-to-thread mapping
 // of each operand's loads follows its contiguous dim.
 template <typename T, int TT>
@@ -2419,21 +2420,25 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       return finish_splitk<float>(g, nsplit, st);
     }
   }
-  // 128x128 tiles once they still give every CU a block, else 64x64
-  const bool big = ((M + 127) / 128) * ((N + 127) / 128) >= kNumCU && K >= 64;
-  const int64_t gt = big ? 128 : 64;
-  const int64_t gx = (N + gt - 1) / gt, gy = (M + gt - 1) / gt;
-  MI355_REQUIRE(gy < 65536 && gx < (int64_t(1) << 31), "mi355_gemm: generic path needs M < 4M rows");
-  using GA = typename std::conditional<std::is_same<T, double>::value, double, float>::type;  // f64 keeps alpha / beta in f64
-  if (big)
-    hipLaunchKernelGGL((gemm_generic_kernel<T, 8>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                       static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
-                       static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (GA)alpha, (GA)beta);
-  else
-    hipLaunchKernelGGL((gemm_generic_kernel<T, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
-                       static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
-                       static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (GA)alpha, (GA)beta);
-  return check_launch("mi355_gemm(generic)");
+  if constexpr (std::is_same<T, double>::value) {  // fp64: the MFMA kernel of gemm_f64.hip
+    return launch_gemm_f64(static_cast<const double*>(a), a_rs, a_cs, static_cast<const double*>(b), b_rs, b_cs,
+                           static_cast<const double*>(c), c_rs, c_cs, static_cast<double*>(out), M, N, K, alpha, beta, st);
+  } else {
+    // 128x128 tiles once they still give every CU a block, else 64x64
+    const bool big = ((M + 127) / 128) * ((N + 127) / 128) >= kNumCU && K >= 64;
+    const int64_t gt = big ? 128 : 64;
+    const int64_t gx = (N + gt - 1) / gt, gy = (M + gt - 1) / gt;
+    MI355_REQUIRE(gy < 65536 && gx < (int64_t(1) << 31), "mi355_gemm: generic path needs M < 4M rows");
+    if (big)
+      hipLaunchKernelGGL((gemm_generic_kernel<T, 8>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+                         static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
+                         static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (float)alpha, (float)beta);
+    else
+      hipLaunchKernelGGL((gemm_generic_kernel<T, 4>), dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, st,
+                         static_cast<const T*>(a), a_rs, a_cs, static_cast<const T*>(b), b_rs, b_cs,
+                         static_cast<const T*>(c), c_rs, c_cs, static_cast<T*>(out), M, N, K, (float)alpha, (float)beta);
+    return check_launch("mi355_gemm(generic)");
+  }
 }
 
 }  // namespace mi355

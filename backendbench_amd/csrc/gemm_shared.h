@@ -167,4 +167,9 @@ const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn);
 const void* gemm_x16_splitk_kernel(bool is_bf16, bool b_nn);  // 2 - 4 workgroups per tile split K and meet in the workspace
 constexpr int kX16SplitUnit = 128;        // K shares are multiples of this  // 256-wide tile columns, then 192-wide ones (GemmArgs::tail_n)
 
+// gemm_f64.hip: fp64 products on v_mfma_f64_16x16x4_f64, any strides (c may be null).
+int launch_gemm_f64(const double* a, int64_t a_rs, int64_t a_cs, const double* b, int64_t b_rs, int64_t b_cs, const double* c,
+                    int64_t c_rs, int64_t c_cs, double* out, int64_t M, int64_t N, int64_t K, double alpha, double beta,
+                    hipStream_t st);
+
 }  // namespace mi355

@@ -195,7 +195,8 @@ int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int dtype);
  * Fast (MFMA) layouts, all with 16-byte aligned base and row starts: a with unit column stride,
  * or for bf16 / f16 with unit row stride (a transposed view) when K % 64 == 0 and M % 8 == 0;
  * b with unit row stride (weight.t()) or unit column stride with N a multiple of 8 (fp32: 4).
- * Any other strides, and f64, run on a plain FMA kernel: correct, far slower.
+ * Any other strides run on a plain FMA kernel: correct, far slower.  f64 runs on its own MFMA kernel
+ * (v_mfma_f64_16x16x4_f64) for any strides.
  * workspace: device memory, 16-byte aligned, of at least mi355_gemm_workspace_bytes() bytes,
  * or NULL / smaller — then the call is not split along K (same result, slower on skinny shapes).
  * Slots: mm__default (op_map.py:739), addmm__default (op_map.py:270). */

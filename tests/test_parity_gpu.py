@@ -553,6 +553,39 @@ def test_f64_addmm_keeps_alpha_and_beta_in_f64(backend):
     assert torch.allclose(tiny, c, rtol=1e-12, atol=1e-12)
 
 
+def test_f64_products_on_the_mfma_kernel(backend):
+    """fp64 mm / addmm run on v_mfma_f64_16x16x4_f64 (64x64 tiles, 128x128 from 256 tiles on) for every
+    combination of operand layouts: shapes off the tile and step sizes, K down to 1, the three addmm
+    forms.  1e-12 against the oracle, relative to the largest element; integer-valued operands (sums
+    below 2^53) must come out exactly."""
+    announce("f64 mfma products")
+    g = torch.Generator().manual_seed(11)
+    shapes = [(1, 1, 1), (3, 5, 7), (16, 4, 16), (17, 33, 65), (65, 17, 63), (129, 1000, 257), (200, 100, 300),
+              (2100, 70, 2100), (1, 515, 300), (300, 16, 1)]
+    for (M, K, N) in shapes:
+        for a_t in (False, True):
+            for b_t in (False, True):
+                a = torch.randn(K, M, generator=g, dtype=torch.float64).t() if a_t else torch.randn(M, K, generator=g, dtype=torch.float64)
+                b = torch.randn(N, K, generator=g, dtype=torch.float64).t() if b_t else torch.randn(K, N, generator=g, dtype=torch.float64)
+                ref = aten_cpu.reference(aten.mm.default, [a, b])
+                got = backend[aten.mm.default](a.cuda(), b.cuda()).cpu()
+                assert got.shape == ref.shape
+                assert (got - ref).abs().max() <= 1e-12 * max(ref.abs().max().item(), 1.0), (M, K, N, a_t, b_t)
+        a = torch.randn(M, K, generator=g, dtype=torch.float64)
+        b = torch.randn(K, N, generator=g, dtype=torch.float64)
+        for c, kw in ((torch.randn(N, generator=g, dtype=torch.float64), {"beta": 0.3, "alpha": 0.1}),
+                      (torch.randn(M, N, generator=g, dtype=torch.float64).t().contiguous().t(), {"beta": -2.0, "alpha": 0.5}),
+                      (torch.randn(M, 1, generator=g, dtype=torch.float64), {})):
+            ref = aten_cpu.reference(aten.addmm.default, [c, a, b], kw)
+            got = backend[aten.addmm.default](c.cuda(), a.cuda(), b.cuda(), **kw).cpu()
+            assert (got - ref).abs().max() <= 1e-12 * max(ref.abs().max().item(), 1.0), (M, K, N, kw)
+    # integers: every partial sum is exact in fp64, whatever the order of the additions
+    ai = torch.randint(-1000, 1000, (300, 700), generator=g).double()
+    bi = torch.randint(-1000, 1000, (700, 2100), generator=g).double()
+    assert torch.equal(backend[aten.mm.default](ai.cuda(), bi.cuda()).cpu(), aten_cpu.reference(aten.mm.default, [ai, bi]))
+    assert torch.equal(backend[aten.mm.default](bi.t().cuda(), ai.t().cuda()).cpu(), aten_cpu.reference(aten.mm.default, [bi.t(), ai.t()]))
+
+
 @pytest.mark.parametrize("layout", ["nn", "nt"])
 @pytest.mark.parametrize("shape", [(200, 330), (1700, 1752), (2100, 2064)])
 def test_fp32_gemm_every_k_loop_length(backend, layout, shape):
