@@ -554,14 +554,14 @@ def test_f64_addmm_keeps_alpha_and_beta_in_f64(backend):
 
 
 def test_f64_products_on_the_mfma_kernel(backend):
-    """fp64 mm / addmm run on v_mfma_f64_16x16x4_f64 (64x64 tiles, 128x128 from 256 tiles on) for every
-    combination of operand layouts: shapes off the tile and step sizes, K down to 1, the three addmm
-    forms.  1e-12 against the oracle, relative to the largest element; integer-valued operands (sums
+    """fp64 mm / addmm run on v_mfma_f64_16x16x4_f64 (32x32 tiles for a few dozen tiles, 64x64, 128x128
+    from 256 tiles on) for every combination of operand layouts: shapes off the tile and step sizes, K
+    down to 1, the three addmm forms.  1e-12 against the oracle, relative to the largest element; integer-valued operands (sums
     below 2^53) must come out exactly."""
     announce("f64 mfma products")
     g = torch.Generator().manual_seed(11)
     shapes = [(1, 1, 1), (3, 5, 7), (16, 4, 16), (17, 33, 65), (65, 17, 63), (129, 1000, 257), (200, 100, 300),
-              (2100, 70, 2100), (1, 515, 300), (300, 16, 1)]
+              (2100, 70, 2100), (1000, 40, 1030), (1, 515, 300), (300, 16, 1)]
     for (M, K, N) in shapes:
         for a_t in (False, True):
             for b_t in (False, True):
