@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink factor for every shape (debug only)")
     ap.add_argument("--ops", default="all", help="comma-separated substrings of per-op rows to time, or 'none'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy, 'calib.mm' = a bf16 product of --shape")
+    ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy, 'calib.mm' = a product of --shape in --dtype")
     ap.add_argument("--variant", type=int, default=0,
                     help="with --only-op calib.mfma: 0 = the 32x32x16 mm kernels' MFMA order, 1 = operands swapped between the "
                          "ports, 2 = the other operand held across MFMAs, 3 = v_mfma_f32_16x16x32, 4-9 = chained "
@@ -62,8 +62,10 @@ def parse():
                     help="with --only-op C3.mm_up|C3.mm_down: run the cycle-stamped diagnostic build of the GEMM "
                          "(libmi355_gemm_trace.so) and print where a tile's shader-clock ticks go")
     ap.add_argument("--shape", default=None,
-                    help="with --only-op calib.mm: M,K,N of a bf16 product [M,K] x [K,N] timed like a C3 row, operands "
+                    help="with --only-op calib.mm: M,K,N of a product [M,K] x [K,N] (--dtype, default bf16) timed like a C3 row, operands "
                          "drawn like C3's (how the time of a K = 4096 product moves with the number of 256x256 tiles)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32", "f64"],
+                    help="with --only-op calib.mm: the operands' dtype")
     ap.add_argument("--fill", default=None, choices=["zeros", "ones", "sign"],
                     help="with --only-op: overwrite the floating-point inputs with zeros, ones or values from "
                          "{-1, 0, 1} (shows how far a kernel's time depends on the data through the power/clock envelope)")
@@ -105,11 +107,12 @@ def main():
         return
     if args.only_op == "calib.mm":
         M, K, N = (int(v) for v in args.shape.split(","))
-        a = torch.randn(M, K, device=dev).to(torch.bfloat16)
-        b = (torch.randn(K, N, device=dev) * 0.02).to(torch.bfloat16)
+        dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32, "f64": torch.float64}[args.dtype]
+        a = torch.randn(M, K, device=dev).to(dt)
+        b = (torch.randn(K, N, device=dev) * 0.02).to(dt)
         ms, how = graph_bench(backend[torch.ops.aten.mm.default], [a, b], {})
         tiles = -(-M // 256) * -(-N // 256)
-        print(json.dumps({"only_op": "calib.mm", "shape": [M, K, N], "ms": round(ms, 5),
+        print(json.dumps({"only_op": "calib.mm", "shape": [M, K, N], "dtype": args.dtype, "ms": round(ms, 5),
                           "tflops": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1), "tiles_256x256": tiles,
                           "rounds_of_256_cus": round(tiles / 256, 3), "timing": how}))
         return
