@@ -261,6 +261,26 @@ __global__ __launch_bounds__(256) void calib_mfma16a_kernel(const F* __restrict_
   out[lane_slot] = sum;
 }
 
+// fp64: WAVES waves per workgroup, each issuing `steps` rounds of eight independent v_mfma_f64_16x16x4_f64
+// (2048 flop each) on one operand value per lane.
+typedef double calib_f64x4 __attribute__((ext_vector_type(4)));
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void calib_mfma_f64_kernel(const double* __restrict__ a, const double* __restrict__ b,
+                                                                  float* __restrict__ out, int steps) {
+  calib_f64x4 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = calib_f64x4{0.0, 0.0, 0.0, 0.0};
+  const double av = a[threadIdx.x % 256], bv = b[threadIdx.x % 256];
+  for (int s = 0; s < steps; ++s) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(av, bv, acc[i], 0, 0, 0);
+  }
+  double t = 0.0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) t += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  if (threadIdx.x < 256) out[blockIdx.x * 256 + threadIdx.x] = static_cast<float>(t);
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -277,7 +297,21 @@ extern "C" int mi355_calib_mfma(const void* a, const void* b, void* out, int dty
                                 void* stream) {
   MI355_REQUIRE(a != nullptr && b != nullptr && out != nullptr, "mi355_calib_mfma: NULL buffer");
   MI355_REQUIRE(blocks > 0 && steps > 0 && steps % 4 == 0, "mi355_calib_mfma: blocks > 0 and a number of steps divisible by four");
-  MI355_REQUIRE(dtype == MI355_BF16 || dtype == MI355_F16, "mi355_calib_mfma: bf16 or f16");
+  if (dtype == MI355_F64) {  // variant = waves per workgroup; a, b: 256 doubles each
+    const double* pa = static_cast<const double*>(a);
+    const double* pb = static_cast<const double*>(b);
+    float* of = static_cast<float*>(out);
+    hipStream_t sf = static_cast<hipStream_t>(stream);
+    switch (variant) {
+      case 1: hipLaunchKernelGGL((calib_mfma_f64_kernel<1>), dim3(blocks), dim3(64), 0, sf, pa, pb, of, steps); break;
+      case 4: hipLaunchKernelGGL((calib_mfma_f64_kernel<4>), dim3(blocks), dim3(256), 0, sf, pa, pb, of, steps); break;
+      case 8: hipLaunchKernelGGL((calib_mfma_f64_kernel<8>), dim3(blocks), dim3(512), 0, sf, pa, pb, of, steps); break;
+      case 16: hipLaunchKernelGGL((calib_mfma_f64_kernel<16>), dim3(blocks), dim3(1024), 0, sf, pa, pb, of, steps); break;
+      default: return set_error(MI355_ERR_INVALID, "mi355_calib_mfma: f64 takes 1, 4, 8 or 16 waves per workgroup as variant");
+    }
+    return check_launch("mi355_calib_mfma(f64)");
+  }
+  MI355_REQUIRE(dtype == MI355_BF16 || dtype == MI355_F16, "mi355_calib_mfma: bf16, f16 or f64");
   MI355_REQUIRE(variant >= 0 && variant <= 14, "mi355_calib_mfma: variant 0..14");
   hipStream_t st = static_cast<hipStream_t>(stream);
   float* o = static_cast<float*>(out);

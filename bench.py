@@ -65,7 +65,8 @@ def parse():
                     help="with --only-op calib.mm: M,K,N of a product [M,K] x [K,N] (--dtype, default bf16) timed like a C3 row, operands "
                          "drawn like C3's (how the time of a K = 4096 product moves with the number of 256x256 tiles)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32", "f64"],
-                    help="with --only-op calib.mm: the operands' dtype")
+                    help="with --only-op calib.mm: the operands' dtype; with --only-op calib.mfma: f64 times the fp64 MFMA "
+                         "(--variant = waves per workgroup: 1, 4, 8, 16)")
     ap.add_argument("--fill", default=None, choices=["zeros", "ones", "sign"],
                     help="with --only-op: overwrite the floating-point inputs with zeros, ones or values from "
                          "{-1, 0, 1} (shows how far a kernel's time depends on the data through the power/clock envelope)")
@@ -103,7 +104,7 @@ def main():
     # covers the same launches.  "calib.copy" is a plain 128 MiB -> 128 MiB copy with the
     # library's copy kernel (known traffic, for scaling hardware byte counters).
     if args.only_op == "calib.mfma":
-        print(json.dumps(calib_mfma(dev, args.fill, args.variant)))
+        print(json.dumps(calib_mfma_f64(dev, args.variant or 16) if args.dtype == "f64" else calib_mfma(dev, args.fill, args.variant)))
         return
     if args.only_op == "calib.mm":
         M, K, N = (int(v) for v in args.shape.split(","))
@@ -363,6 +364,40 @@ def calib_mfma(dev, fill=None, variant=0, blocks=256, steps=2752, launches=20):
     return {"only_op": "calib.mfma", "variant": variant, "fill": fill or "N(0,1) x N(0,0.02)", "ms": round(ms, 4),
             "flops": flops, "tflops": round(tf, 1), "frac_of_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
             "timing": f"{launches} launches of {blocks} x 4 waves x {steps} steps, events around the loop"}
+
+
+def calib_mfma_f64(dev, waves, blocks=256, steps=20000, launches=5):
+    """Issue rate of v_mfma_f64_16x16x4_f64 with `waves` waves per workgroup, one workgroup per CU, eight
+    independent accumulator blocks per wave, no memory traffic (mi355_calib_mfma with dtype f64)."""
+    import torch
+
+    from backendbench_amd import _lib
+
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(0)
+    a = torch.randn(256, generator=g, dtype=torch.float64).to(dev)
+    b = torch.randn(256, generator=g, dtype=torch.float64).to(dev)
+    out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
+    stream = _lib.current_stream_handle()
+
+    def run():
+        _lib.check(lib.mi355_calib_mfma(a.data_ptr(), b.data_ptr(), out.data_ptr(), _lib.F64, blocks, steps, waves, stream))
+
+    run()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(launches):
+        run()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / launches
+    flops = blocks * waves * steps * 8 * 2048
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"only_op": "calib.mfma", "dtype": "f64", "waves_per_workgroup": waves, "ms": round(ms, 4), "flops": flops,
+            "tflops": round(tf, 1), "frac_of_peak": round(tf / 78.6, 4),
+            "ns_per_mfma_and_wave": round(ms * 1e6 / (steps * 8), 1),
+            "timing": f"{launches} launches of {blocks} x {waves} waves x {steps} rounds of 8 MFMAs, events around the loop"}
 
 
 def gemm_ablate(case, dev, bits, fill=None, launches=40):

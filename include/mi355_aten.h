@@ -224,7 +224,11 @@ int mi355_gemm_tile_columns(int64_t M, int64_t N, int64_t K, int32_t* wide, int3
  * mm kernel in exactly the written order (asm statements): chains of two back to back (10), with one
  * (11) or three (14) s_nop between the two, two blocks interleaved (12), first halves then second halves (13).
  * Its sustained rate on a given data distribution is the ceiling the power / clock envelope leaves to
- * mi355_gemm on that data. */
+ * mi355_gemm on that data.
+ * dtype MI355_F64: `variant` is the number of waves per workgroup (1, 4, 8 or 16), every wave issues
+ * `steps` rounds of eight independent v_mfma_f64_16x16x4_f64 on one value per lane (a, b: 256 doubles
+ * each): blocks * variant * steps * 8 * 2048 flop - how the issue rate of that instruction depends on
+ * the waves per SIMD. */
 int mi355_calib_mfma(const void* a, const void* b, void* out, int dtype, int blocks, int steps,
                      int variant, void* stream);
 
