@@ -13,7 +13,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libmi355_aten.so"
-ABI_VERSION = 7
+ABI_VERSION = 8
 MAX_DIMS = 8
 
 # mi355_dtype
@@ -59,6 +59,8 @@ _PAD = (0,) * MAX_DIMS
 SIGNATURES = {
     "mi355_abi_version": (c_int, []),
     "mi355_last_error": (c_char_p, []),
+    "mi355_init": (c_int, []),
+    "mi355_set_knob": (c_int, [c_char_p, c_char_p]),
     "mi355_binary": (c_int, [c_int, _P, _P, c_double, c_int64, _P, c_void_p]),
     "mi355_unary": (c_int, [c_int, _P, c_int, c_double, c_double, c_int64, c_int64, _P, c_void_p]),
     "mi355_where": (c_int, [_P, _P, _P, _P, c_void_p]),
@@ -88,6 +90,12 @@ SIGNATURES = {
         [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
          c_int64, c_int64, c_double, c_double, c_int, c_void_p, c_int64, c_void_p],
     ),
+    "mi355_gemm_f32out": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int64,
+         c_int64, c_int64, c_double, c_double, c_int, c_void_p],
+    ),
+    "mi355_gemm_status": (c_int, []),
     "mi355_gemm_tile_columns": (c_int, [c_int64, c_int64, c_int64, ctypes.POINTER(c_int32), ctypes.POINTER(c_int32)]),
     "mi355_calib_mfma": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mi355_index_select": (
@@ -120,6 +128,25 @@ def load():
         raise RuntimeError(f"libmi355_aten.so has ABI {got}, the Python side expects {ABI_VERSION}")
     _lib = lib
     return lib
+
+
+_initialised = set()
+
+
+def init_device(index):
+    """mi355_init() once per device: refuses anything but a 256-CU gfx950 part and resolves the
+    library's per-device addresses.  Called from the first launch on a device."""
+    if index in _initialised:
+        return
+    rc = load().mi355_init()
+    if rc != 0:
+        check(rc)
+    _initialised.add(index)
+
+
+def set_knob(name, value=None):
+    """Test / measurement hook: override (or, with None, restore) one of the library's knobs."""
+    check(load().mi355_set_knob(name.encode(), None if value is None else str(value).encode()))
 
 
 def check(rc):

@@ -16,6 +16,17 @@ namespace mi355 {
 int set_error(int code, const char* fmt, ...);
 int check_launch(const char* what);
 
+// Test and measurement knobs, read from the environment once per process (MI355_GEMM_TILE,
+// MI355_GEMM_WAVES) and changed afterwards only through mi355_set_knob(): no entry point calls
+// getenv on its way to a launch.
+struct Knobs {
+  char gemm_tile[16];   // "" = the planner decides; see mi355_set_knob in include/mi355_aten.h
+  char gemm_waves[8];   // "" / "4" / "8"
+  int x16_spin_limit;   // polls of the in-launch split-K's bounded wait before it gives up
+};
+const Knobs& knobs();
+constexpr int kX16SpinLimitDefault = 1 << 21;  // about 1 us per poll
+
 #define MI355_REQUIRE(cond, ...)                                  \
   do {                                                            \
     if (!(cond)) return ::mi355::set_error(MI355_ERR_INVALID, __VA_ARGS__); \

@@ -4,7 +4,10 @@
 
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
 #include <algorithm>
+#include <mutex>
 
 namespace mi355 {
 
@@ -16,6 +19,26 @@ int set_error(int code, const char* fmt, ...) {
   vsnprintf(g_error, sizeof(g_error), fmt, ap);
   va_end(ap);
   return code;
+}
+
+static Knobs g_knobs;
+static std::once_flag g_knobs_once;
+
+static void copy_knob(char* dst, size_t cap, const char* src) {
+  if (src == nullptr) src = "";
+  strncpy(dst, src, cap - 1);
+  dst[cap - 1] = 0;
+}
+
+static void knobs_from_env() {
+  copy_knob(g_knobs.gemm_tile, sizeof(g_knobs.gemm_tile), getenv("MI355_GEMM_TILE"));
+  copy_knob(g_knobs.gemm_waves, sizeof(g_knobs.gemm_waves), getenv("MI355_GEMM_WAVES"));
+  g_knobs.x16_spin_limit = kX16SpinLimitDefault;
+}
+
+const Knobs& knobs() {
+  std::call_once(g_knobs_once, knobs_from_env);
+  return g_knobs;
 }
 
 int check_launch(const char* what) {
@@ -67,4 +90,46 @@ bool same_dense_layout(const mi355_tensor* const* ts, int nt) {
 }  // namespace mi355
 
 extern "C" int mi355_abi_version(void) { return MI355_ABI_VERSION; }
+
+extern "C" int mi355_set_knob(const char* name, const char* value) {
+  using namespace mi355;
+  knobs();  // the environment first, so that a later call cannot overwrite this one
+  if (name == nullptr) return set_error(MI355_ERR_INVALID, "mi355_set_knob: name is NULL");
+  if (strcmp(name, "gemm_tile") == 0) {
+    copy_knob(g_knobs.gemm_tile, sizeof(g_knobs.gemm_tile), value);
+  } else if (strcmp(name, "gemm_waves") == 0) {
+    copy_knob(g_knobs.gemm_waves, sizeof(g_knobs.gemm_waves), value);
+  } else if (strcmp(name, "x16_spin_limit") == 0) {
+    const long v = (value == nullptr || value[0] == 0) ? kX16SpinLimitDefault : strtol(value, nullptr, 10);
+    if (v < 0 || v > (1L << 30)) return set_error(MI355_ERR_INVALID, "mi355_set_knob: x16_spin_limit %ld out of range", v);
+    g_knobs.x16_spin_limit = (int)v;
+  } else {
+    return set_error(MI355_ERR_INVALID, "mi355_set_knob: unknown knob '%s'", name);
+  }
+  return MI355_OK;
+}
+
+// Defined next to the state they cover.
+namespace mi355 {
+int reduce_static_init();   // reduce.hip: address of the built-in scratch array on the current device
+}
+
+extern "C" int mi355_init(void) {
+  using namespace mi355;
+  knobs();
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_init: hipGetDevice failed: %s", hipGetErrorString(e));
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_init: hipGetDeviceProperties failed: %s", hipGetErrorString(e));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return set_error(MI355_ERR_UNSUPPORTED, "mi355_init: device %d is %s; this library holds gfx950 code only", dev, prop.gcnArchName);
+  // The persistent and split-K grids, the tile planner and the streaming kernels' grids are sized for
+  // this many CUs; a partitioned or cut-down part would run them with idle or oversubscribed CUs.
+  if (prop.multiProcessorCount != kNumCU)
+    return set_error(MI355_ERR_UNSUPPORTED, "mi355_init: device %d has %d compute units, the launch heuristics are built for %d",
+                     dev, prop.multiProcessorCount, kNumCU);
+  return reduce_static_init();
+}
 extern "C" const char* mi355_last_error(void) { return mi355::g_error; }

@@ -2144,7 +2144,9 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       // with it; measured crossover at about 230 tiles for K = 3072 and 250 for K = 1024.
       // MI355_GEMM_TILE=256x128 forces it (a test knob).
       const int64_t tiles_mid = (int64_t)g.tiles_m * ((N + 127) / 128);
-      const char* forced_tile = getenv("MI355_GEMM_TILE");
+      const Knobs& kn = knobs();
+      const char* forced_tile = kn.gemm_tile[0] ? kn.gemm_tile : nullptr;
+      const char* forced_waves = kn.gemm_waves[0] ? kn.gemm_waves : nullptr;
       const bool mid = !ktail && K % 64 == 0 && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "256x128") == 0
                                                : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > (K >= 2048 ? 228 : 248) && tiles_mid <= kNumCU &&
@@ -2190,7 +2192,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool x16_mixed_forced = forced_tile != nullptr && strcmp(forced_tile, "x16mixed") == 0;  // mixed widths at any K
       const bool x16 = x16_ok && (forced_tile != nullptr ? strcmp(forced_tile, "x16") == 0 || x16_mixed_forced || strcmp(forced_tile, "x16persist") == 0
                                                          : x16_pays && (nblocks > kNumCU / 2 || (nblocks >= 96 && K >= 2048)) && !mid &&
-                                                               !t64 && getenv("MI355_GEMM_WAVES") == nullptr);
+                                                               !t64 && forced_waves == nullptr);
       // Too few tiles for the chip and a long K: the same kernel with two workgroups per tile that share K
       // and meet in the workspace (plan_x16_split).  Any value of MI355_GEMM_TILE but x16split keeps it off.
       X16SplitPlan xs = plan_x16_split(M, N, K);
@@ -2200,16 +2202,17 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool x16_split = x16_ok && xs.splits > 1 && workspace != nullptr && workspace_bytes >= xs.ws_bytes &&
                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
                              (forced_tile != nullptr ? strcmp(forced_tile, "x16split") == 0
-                                                     : x16_pays && M >= 512 && getenv("MI355_GEMM_WAVES") == nullptr);  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
+                                                     : x16_pays && M >= 512 && forced_waves == nullptr);  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
       if (x16_split) {
-        static std::atomic<unsigned long long> epoch{0x5bd1e9955bd1e995ull};
+        static std::atomic<unsigned long long> epoch{0x5bd1e9955bd1e995ull};  // odd, and stepped by two: odd for ever
         kern = gemm_x16_splitk_kernel(std::is_same<T, bf16_t>::value, !b_nt);
         threads = 256;
         lds_bytes = kX16Lds;
         g.ws = static_cast<float*>(workspace);
         g.sk_splits = xs.splits;
         g.sk_tiles8 = xs.tiles8;
-        g.sk_epoch = epoch.fetch_add(1) | 1ull;  // never 0: a flag is 0 between launches
+        g.sk_epoch = epoch.fetch_add(2);  // a value of its own per launch, never 0 (a flag is 0 between launches)
+        g.sk_spin_limit = kn.x16_spin_limit;
         g.sk_flags = reinterpret_cast<unsigned long long*>(static_cast<unsigned char*>(workspace) + (int64_t)(xs.splits - 1) * nblocks * (BM * BN * 4));
         g.out_rows = N % 64 != 0 || reinterpret_cast<uintptr_t>(out) % 128 != 0;
         nblocks = (int64_t)xs.splits * xs.tiles8;
@@ -2313,7 +2316,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       } else if (K % 64 == 0) {
         // Four waves of 128x128 run the steady state 3-5 % faster and pay ~2 us more per tile
         // (two-pass epilogue), which evens out near K = 2048.  MI355_GEMM_WAVES=4|8 forces one form.
-        const char* forced = getenv("MI355_GEMM_WAVES");
+        const char* forced = forced_waves;
         const bool w4 = a_t || (ld32 && (forced != nullptr ? forced[0] == '4' : K >= 2048));  // the eight-wave kernels have no M-contiguous-A form
         lds_bytes = kGemmLds64;
         if (w4) {
@@ -2441,6 +2444,78 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
   }
 }
 
+
+// out (fp32) = alpha * ws + beta * c in place over a dense [M, N] fp32 matrix, N % 4 == 0 (mm.dtype / addmm.dtype:
+// the 128x128 kernels' SPLIT form has left the raw fp32 product in `out` itself).
+template <typename T>
+__global__ __launch_bounds__(256) void gemm_f32out_finish_kernel(GemmArgs g) {
+  const int64_t quads = (int64_t)g.M * g.N / 4;
+  const int qpr = g.N / 4;
+  const T* C = static_cast<const T*>(g.c);
+  const bool use_c = C != nullptr && g.beta != 0.f;
+  float* D = static_cast<float*>(g.out);
+  for (int64_t qd = (int64_t)blockIdx.x * 256 + threadIdx.x; qd < quads; qd += (int64_t)gridDim.x * 256) {
+    f32x4 v = *reinterpret_cast<const f32x4*>(D + qd * 4);
+    const int64_t m = qd / qpr, n = (qd - m * qpr) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float r = g.alpha * v[e];
+      if (use_c) r += g.beta * static_cast<float>(C[m * g.c_rs + (n + e) * g.c_cs]);
+      v[e] = r;
+    }
+    *reinterpret_cast<f32x4*>(D + qd * 4) = v;
+  }
+}
+
+// bf16 / f16 operands, fp32 result: the 128x128 MFMA kernels in their SPLIT form with a single split whose
+// "plane" is the output itself - the fp32 accumulators go to memory as they are, never rounded to T.
+template <typename T>
+static int run_gemm_f32out(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs, const void* c,
+                           int64_t c_rs, int64_t c_cs, float* out, int64_t M, int64_t N, int64_t K, double alpha, double beta,
+                           hipStream_t st) {
+  const bool a_ok = a_cs == 1 && a_rs % 8 == 0 && aligned16(a);
+  const bool b_nt = b_rs == 1 && b_cs % 8 == 0 && aligned16(b);
+  const bool b_nn = b_cs == 1 && b_rs % 8 == 0 && aligned16(b) && N % 8 == 0;
+  const bool fits = M < (1 << 30) && N < (1 << 30) && K < (1 << 30);
+  if (!(a_ok && (b_nt || b_nn) && K > 0 && K % BK3 == 0 && N % 4 == 0 && aligned16(out) && fits))
+    return set_error(MI355_ERR_UNSUPPORTED,
+                     "mi355_gemm_f32out: layout not taken (needs K-contiguous a, b K-contiguous or row-major with N %% 8 == 0, "
+                     "K %% 32 == 0, N %% 4 == 0, 16-byte aligned bases): widen the operands and call mi355_gemm in f32");
+  GemmArgs g{};
+  g.a = a; g.b = b; g.c = c; g.out = out;
+  g.lda = a_rs;
+  g.ldb = b_nt ? b_cs : b_rs;
+  g.c_rs = c_rs; g.c_cs = c_cs;
+  g.M = (int32_t)M; g.N = (int32_t)N; g.K = (int32_t)K;
+  g.alpha = (float)alpha; g.beta = (float)beta;
+  g.tiles_m = (int32_t)((M + SBM - 1) / SBM);
+  g.tiles_n = (int32_t)((N + SBN - 1) / SBN);
+  const int64_t nblocks = (int64_t)g.tiles_m * g.tiles_n;
+  MI355_REQUIRE(nblocks < (int64_t(1) << 31), "mi355_gemm_f32out: too many tiles");
+  g.ws = out;
+  g.ksplit = (int32_t)K;
+  g.ws_ld = (int32_t)N;
+  const bool pairs = nblocks <= kNumCU && K % 64 == 0;  // at most one workgroup per CU: the deep-ring kernel
+  const int lds_bytes = pairs ? kSmall2Lds : kSmallLds;
+  const void* kern;
+  if (pairs) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, true, false> : (const void*)gemm_mfma_small2_kernel<T, true, true, false>;
+  else kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, true, false> : (const void*)gemm_mfma_small_kernel<T, true, true, false>;
+  hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  if (e != hipSuccess)
+    return set_error(MI355_ERR_LAUNCH, "mi355_gemm_f32out: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
+  void* params[] = {&g};
+  e = hipLaunchKernel(kern, dim3((unsigned)nblocks, 1), dim3(256), params, lds_bytes, st);
+  if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm_f32out: launch failed: %s", hipGetErrorString(e));
+  int rc = check_launch("mi355_gemm_f32out");
+  if (rc) return rc;
+  if (alpha != 1.0 || (c != nullptr && beta != 0.0)) {
+    const int grid = grid_for(M * N / 4, 256, kNumCU * 8);
+    hipLaunchKernelGGL((gemm_f32out_finish_kernel<T>), dim3(grid), dim3(256), 0, st, g);
+    rc = check_launch("mi355_gemm_f32out(finish)");
+  }
+  return rc;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -2485,5 +2560,20 @@ extern "C" int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void*
     case MI355_F32: return run_gemm<float>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
     case MI355_F64: return run_gemm<double>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
     default: return set_error(MI355_ERR_UNSUPPORTED, "mi355_gemm: unsupported dtype %s", dtype_name(dtype));
+  }
+}
+
+extern "C" int mi355_gemm_f32out(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs,
+                                 const void* c, int64_t c_rs, int64_t c_cs, void* out, int64_t M, int64_t N, int64_t K,
+                                 double alpha, double beta, int dtype, void* stream) {
+  MI355_REQUIRE(M >= 0 && N >= 0 && K >= 0, "mi355_gemm_f32out: negative extent");
+  if (M == 0 || N == 0) return MI355_OK;
+  MI355_REQUIRE(out != nullptr, "mi355_gemm_f32out: NULL out");
+  MI355_REQUIRE(K == 0 || (a != nullptr && b != nullptr), "mi355_gemm_f32out: NULL operand");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case MI355_BF16: return run_gemm_f32out<bf16_t>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, static_cast<float*>(out), M, N, K, alpha, beta, st);
+    case MI355_F16: return run_gemm_f32out<f16_t>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, static_cast<float*>(out), M, N, K, alpha, beta, st);
+    default: return set_error(MI355_ERR_UNSUPPORTED, "mi355_gemm_f32out: operands must be bf16 or f16, got %s", dtype_name(dtype));
   }
 }

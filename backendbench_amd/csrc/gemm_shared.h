@@ -41,11 +41,12 @@ struct GemmArgs {
   int32_t bias_vec;  // c is one unit-stride row broadcast along m (a Linear layer's bias), 8-byte aligned: any N
   // gemm_mfma_x16_splitk_kernel: sk_splits workgroups share a tile's K range and meet in the caller's
   // workspace: (sk_splits - 1) fp32 planes of 256 x 256 per tile at ws, behind them one 64-bit flag per plane
-  // (sk_flags), which holds sk_epoch (a value no earlier launch used) once the plane is complete.
+  // (sk_flags), which holds sk_epoch (a value of this launch alone) once the plane is complete.
   int32_t sk_splits;
   int32_t sk_tiles8;  // tiles rounded up to a multiple of 8: blocks [r * sk_tiles8, (r + 1) * sk_tiles8) have one role
   unsigned long long sk_epoch;
   unsigned long long* sk_flags;
+  int32_t sk_spin_limit;  // polls of a flag before the summing workgroup gives up (Knobs::x16_spin_limit)
 };
 
 // Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous

@@ -68,10 +68,13 @@ struct X16Split {
   unsigned long long* flags;  // likewise
   unsigned long long epoch;
   int role, nprod;
+  int spin_limit;  // polls of one flag before the summing workgroup gives up
   float poison;  // -0 (x + -0 == x), or NaN when a producer never arrived
 };
 constexpr int kX16PartRows = 2;  // rows of accumulator blocks whose plane values are in flight at once (4 blocks of 4 VGPRs each per row)
-constexpr int kX16SpinLimit = 1 << 21;  // polls (about 1 us each) before the summing workgroup gives up and writes NaNs
+// Set by a summing workgroup whose bounded wait ran out (it then writes NaNs into its tile): the launch
+// still reports success, so this word is how the host learns of it (mi355_gemm_status).  Sticky until read.
+static __device__ unsigned int x16_gave_up_word;
 
 // Plane accesses are agent-scope accesses (the sc1 bit on the instruction: relaxed atomics of 8 bytes), not
 // plain ones between agent-scope fences: a fence writes back / invalidates the whole L2 of the XCD, under the
@@ -774,11 +777,12 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
       for (int q = 0; q < sk.nprod; ++q) {
         int polls = 0;
         while (__hip_atomic_load(sk.flags + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != sk.epoch) {
-          if (++polls > kX16SpinLimit) { bad = 1; break; }
+          if (++polls > sk.spin_limit) { bad = 1; break; }
           __builtin_amdgcn_s_sleep(8);
         }
       }
       *gave_up = bad;
+      if (bad) __hip_atomic_store(&x16_gave_up_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the plane loads stay behind the polls
     __syncthreads();
@@ -861,6 +865,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_splitk_kernel(GemmArgs g) {
   sk.planes = reinterpret_cast<f32x4*>(g.ws) + first * 16384;
   sk.flags = g.sk_flags + first;
   sk.epoch = g.sk_epoch;
+  sk.spin_limit = g.sk_spin_limit;
   sk.role = role;
   sk.nprod = S - 1;
   x16_tile<T, B_NN, 4, false, true>(gs, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * BN), sk);
@@ -911,3 +916,15 @@ const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn) {
 }
 
 }  // namespace mi355
+
+extern "C" int mi355_gemm_status(void) {
+  unsigned int word = 0;
+  hipError_t e = hipMemcpyFromSymbol(&word, HIP_SYMBOL(mi355::x16_gave_up_word), sizeof(word));
+  if (e != hipSuccess) return mi355::set_error(MI355_ERR_LAUNCH, "mi355_gemm_status: reading the status word failed: %s", hipGetErrorString(e));
+  if (word == 0) return MI355_OK;
+  const unsigned int zero = 0;
+  e = hipMemcpyToSymbol(HIP_SYMBOL(mi355::x16_gave_up_word), &zero, sizeof(zero));
+  if (e != hipSuccess) return mi355::set_error(MI355_ERR_LAUNCH, "mi355_gemm_status: clearing the status word failed: %s", hipGetErrorString(e));
+  return mi355::set_error(MI355_ERR_LAUNCH,
+                          "mi355_gemm: a split-K launch gave up waiting for a partial product (its output tile holds NaNs)");
+}

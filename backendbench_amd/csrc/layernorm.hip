@@ -157,89 +157,188 @@ __global__ __launch_bounds__(BLOCK) void layernorm_tile_kernel(const T* __restri
 // with the NEXT row's loads issued before the current row is reduced, so the memory system
 // always holds a row per wave in flight while the reductions and the normalisation run.  One wave
 // per row: both all-reduces stay inside the wave (DPP + bpermute), no barrier in the loop.
-// gamma / beta are staged once per block in LDS (2 n elements of dynamic shared memory).  Same
-// statistics as the tile kernel (mean, then the centred second moment from the registers).
-template <typename T, typename S, int NV, bool HW, bool HB>
-__global__ __launch_bounds__(kLnBlock) __attribute__((amdgpu_waves_per_eu(4, 8))) void layernorm_stream_kernel(const T* __restrict__ x, const T* __restrict__ w,
+// gamma / beta are staged once per block in LDS (2 n elements of dynamic shared memory, as floats
+// for bf16).  Same statistics as the tile kernel (mean, then the centred second moment of the
+// same values).
+// Both rows stay in the registers as loaded (NV 16-byte vectors each) and are widened to fp32
+// anew in each pass: 2 x 4 NV registers of row data instead of 4 NV + NV V floats, which keeps a
+// 4096-element row with gamma and beta under 96 registers - five waves per SIMD and nothing
+// spilled to scratch memory (the fp32 register tile spilled two to five registers per lane, 3 %
+// extra HBM traffic).  The row sum takes v_dot2_f32_{bf16,f16} against (1, 1); FULL (the row
+// fills all NV slabs) drops the per-slab masks.
+typedef uint32_t ln_raw16 __attribute__((ext_vector_type(4)));
+typedef __bf16 ln_bf2 __attribute__((ext_vector_type(2)));
+typedef _Float16 ln_h2 __attribute__((ext_vector_type(2)));
+
+// Sum of the V elements of one 16-byte vector, accumulated in fp32 onto `acc`.  Two-byte types take
+// v_dot2_f32_{bf16,f16} against (1, 1): two elements per instruction, no widening first.
+template <typename T> __device__ __forceinline__ float ln_vec_sum(ln_raw16 r, float acc) {
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    const ln_bf2 one = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { const uint32_t wd = r[i]; acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(ln_bf2, wd), one, acc, false); }
+  } else if constexpr (std::is_same<T, f16_t>::value) {
+    const ln_h2 one = {(_Float16)1.0f, (_Float16)1.0f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { const uint32_t wd = r[i]; acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(ln_h2, wd), one, acc, false); }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { const uint32_t wd = r[i]; acc += __builtin_bit_cast(float, wd); }
+  }
+  return acc;
+}
+// The V elements of a 16-byte vector as floats.
+template <typename T, int V> __device__ __forceinline__ void ln_widen(ln_raw16 r, float (&f)[V]) {
+  if constexpr (std::is_same<T, bf16_t>::value) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __builtin_bit_cast(float, r[i] << 16);
+      f[2 * i + 1] = __builtin_bit_cast(float, r[i] & 0xffff0000u);
+    }
+  } else {
+    const VecN<T, V> xv = __builtin_bit_cast(VecN<T, V>, r);
+#pragma unroll
+    for (int j = 0; j < V; ++j) f[j] = static_cast<float>(xv.v[j]);
+  }
+}
+
+// Half h (0, 1) of a 16-byte vector as H = V / 2 floats.
+template <typename T, int H> __device__ __forceinline__ void ln_widen_half(ln_raw16 r, int h, float (&f)[H]) {
+  const uint32_t w0 = h ? r[2] : r[0], w1 = h ? r[3] : r[1];
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    f[0] = __builtin_bit_cast(float, w0 << 16);
+    f[1] = __builtin_bit_cast(float, w0 & 0xffff0000u);
+    f[2] = __builtin_bit_cast(float, w1 << 16);
+    f[3] = __builtin_bit_cast(float, w1 & 0xffff0000u);
+  } else if constexpr (std::is_same<T, f16_t>::value) {
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 a = __builtin_bit_cast(h2, w0), b = __builtin_bit_cast(h2, w1);
+    f[0] = static_cast<float>(a[0]); f[1] = static_cast<float>(a[1]);
+    f[2] = static_cast<float>(b[0]); f[3] = static_cast<float>(b[1]);
+  } else {
+    f[0] = __builtin_bit_cast(float, w0);
+    f[1] = __builtin_bit_cast(float, w1);
+  }
+}
+
+// V elements of gamma / beta from global memory into their LDS form (widened to P when P is wider than T).
+template <typename T, typename P, int V> __device__ __forceinline__ void ln_stage(P* dst, const T* src) {
+  const VecN<T, V> v = ld<T, V>(src);
+  VecN<P, V> o;
+#pragma unroll
+  for (int j = 0; j < V; ++j) o.v[j] = static_cast<P>(v.v[j]);
+  st<P, V>(dst, o);
+}
+// H consecutive staged parameters as floats (one LDS read of H * sizeof(P) bytes).
+template <typename P, int H> __device__ __forceinline__ void ln_params_half(const P* p, float (&f)[H]) {
+  const VecN<P, H> v = ld<P, H>(p);
+#pragma unroll
+  for (int j = 0; j < H; ++j) f[j] = static_cast<float>(v.v[j]);
+}
+
+template <typename T, typename S, int NV, bool HW, bool HB, bool FULL>
+__global__ __launch_bounds__(kLnBlock) void layernorm_stream_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                                    const T* __restrict__ b, T* __restrict__ y,
                                                                    S* __restrict__ mean_out, S* __restrict__ rstd_out,
                                                                    int64_t rows, int64_t n, float eps) {
   constexpr int V = Vec<T>::N;
+  static_assert(sizeof(T) * V == 16, "one 16-byte vector per lane and slab");
   extern __shared__ __attribute__((aligned(32))) unsigned char ln_smem[];  // gamma, then beta: 2 n elements
-  T* gl = reinterpret_cast<T*>(ln_smem);
-  T* bl = gl + n;
+  // bf16 has no mixed-precision FMA (f16 has v_fma_mix_f32): its gamma / beta are widened once, when
+  // they are staged, instead of once per row and element.
+  using P = typename std::conditional<std::is_same<T, bf16_t>::value, float, T>::type;
+  P* gl = reinterpret_cast<P*>(ln_smem);
+  P* bl = gl + n;
   const int lane = threadIdx.x % kWave;
   const int64_t waves = (int64_t)gridDim.x * (kLnBlock / kWave);
-  int64_t row = (int64_t)blockIdx.x * (kLnBlock / kWave) + threadIdx.x / kWave;
+  int64_t row = (int64_t)blockIdx.x * (kLnBlock / kWave) + __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   bool in[NV];
-  VecN<T, V> nxt[NV];
+  ln_raw16 ra[NV], rb[NV];
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int64_t c = ((int64_t)k * kWave + lane) * V;
-    in[k] = c < n;  // n % V == 0: a vector is inside the row or past it
-    if (in[k] && row < rows) nxt[k] = ld_nt<T, V>(x + row * n + c);
+    in[k] = FULL || c < n;  // n % V == 0: a vector is inside the row or past it
+    ra[k] = rb[k] = ln_raw16{0u, 0u, 0u, 0u};  // slabs past the row stay zeros (+0 in every float type)
+    if (in[k] && row < rows) ra[k] = __builtin_nontemporal_load(reinterpret_cast<const ln_raw16*>(x + row * n + c));
   }
-  // gamma / beta once per block into LDS, behind the first row's loads
   if constexpr (HW || HB) {
     for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kLnBlock * V) {
-      if constexpr (HW) st<T, V>(gl + c, ld<T, V>(w + c));
-      if constexpr (HB) st<T, V>(bl + c, ld<T, V>(b + c));
+      if constexpr (HW) ln_stage<T, P, V>(gl + c, w + c);
+      if constexpr (HB) ln_stage<T, P, V>(bl + c, b + c);
     }
     __syncthreads();
   }
   const float inv_n = 1.f / (float)n;
-  for (; row < rows; row += waves) {
-    float v[NV][V];
-#pragma unroll
-    for (int k = 0; k < NV; ++k)
-#pragma unroll
-      for (int j = 0; j < V; ++j) v[k][j] = in[k] ? static_cast<float>(nxt[k].v[j]) : 0.f;
+  // One row: request the row after it into `nxt`, then three passes over `cur` as loaded.
+  auto one_row = [&](ln_raw16 (&cur)[NV], ln_raw16 (&nxt)[NV]) {
     const int64_t ahead = row + waves;
     if (ahead < rows) {
 #pragma unroll
       for (int k = 0; k < NV; ++k)
-        if (in[k]) nxt[k] = ld_nt<T, V>(x + ahead * n + ((int64_t)k * kWave + lane) * V);
+        if (in[k])
+          nxt[k] = __builtin_nontemporal_load(reinterpret_cast<const ln_raw16*>(x + ahead * n + ((int64_t)k * kWave + lane) * V));
     }
     float s = 0.f;
 #pragma unroll
-    for (int k = 0; k < NV; ++k)
-#pragma unroll
-      for (int j = 0; j < V; ++j) s += v[k][j];
+    for (int k = 0; k < NV; ++k) s = ln_vec_sum<T>(cur[k], s);
     const float mean = wave_allreduce(s, SumOp()) * inv_n;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) asm volatile("" : "+v"(cur[k]));
     float q = 0.f;
 #pragma unroll
     for (int k = 0; k < NV; ++k)
       if (in[k]) {
+        float f[V];
+        ln_widen<T, V>(cur[k], f);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-          const float d = v[k][j] - mean;
-          v[k][j] = d;
+          const float d = f[j] - mean;
           q += d * d;
         }
       }
     const float rstd = rsqrtf(wave_allreduce(q, SumOp()) * inv_n + eps);
+#pragma unroll
+    for (int k = 0; k < NV; ++k) asm volatile("" : "+v"(cur[k]));
     if (lane == 0) {
       mean_out[row] = static_cast<S>(mean);
       rstd_out[row] = static_cast<S>(rstd);
     }
+    const float shift = -mean * rstd;
     T* out = y + row * n;
 #pragma unroll
     for (int k = 0; k < NV; ++k)
       if (in[k]) {
         const int64_t c = ((int64_t)k * kWave + lane) * V;
-        VecN<T, V> g, be, r;
-        if constexpr (HW) g = ld<T, V>(gl + c);
-        if constexpr (HB) be = ld<T, V>(bl + c);
+        // half a vector at a time: 4 + 4 + 4 widened values live instead of 3 V
+        VecN<T, V> r;
 #pragma unroll
-        for (int j = 0; j < V; ++j) {
-          float f = v[k][j] * rstd;
-          if constexpr (HW && HB) f = f * static_cast<float>(g.v[j]) + static_cast<float>(be.v[j]);
-          else if constexpr (HW) f *= static_cast<float>(g.v[j]);
-          else if constexpr (HB) f += static_cast<float>(be.v[j]);
-          r.v[j] = static_cast<T>(f);
+        for (int h = 0; h < 2; ++h) {
+          constexpr int H = V / 2;
+          float f[H], g[H], be[H];
+          ln_widen_half<T, H>(cur[k], h, f);
+          if constexpr (HW) ln_params_half<P, H>(gl + c + h * H, g);
+          if constexpr (HB) ln_params_half<P, H>(bl + c + h * H, be);
+#pragma unroll
+          for (int j = 0; j < H; ++j) {
+            float t = __builtin_fmaf(f[j], rstd, shift);  // (x - mean) * rstd
+            if constexpr (HW && HB) t = __builtin_fmaf(t, g[j], be[j]);
+            else if constexpr (HW) t *= g[j];
+            else if constexpr (HB) t += be[j];
+            r.v[h * H + j] = static_cast<T>(t);
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
         st_nt<T, V>(out + c, r);
+        __builtin_amdgcn_sched_barrier(0);
       }
+  };
+  // Two rows per trip, the two register sets trading places, so no row is copied between them.
+  while (row < rows) {
+    one_row(ra, rb);
+    row += waves;
+    if (row >= rows) break;
+    one_row(rb, ra);
+    row += waves;
   }
 }
 
@@ -353,7 +452,7 @@ template <typename T, typename W, typename S, bool VEC>
 __global__ __launch_bounds__(kLnBlock) void layernorm_block_kernel(const T* __restrict__ x, const W* __restrict__ w,
                                                                   const W* __restrict__ b, T* __restrict__ y,
                                                                   S* __restrict__ mean_out, S* __restrict__ rstd_out,
-                                                                  int64_t n, float eps) {
+                                                                  int64_t n, double eps) {
   using A = typename LnAcc<T>::type;
   constexpr int V = Vec<T>::N;
   __shared__ WF<A> smem[kLnBlock / kWave];
@@ -378,7 +477,7 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_block_kernel(const T* __re
   const A mean = a.mean;
   A rstd;
   if constexpr (std::is_same<A, double>::value) rstd = 1.0 / sqrt(a.m2 / (double)n + (double)eps);
-  else rstd = rsqrtf(a.m2 / (float)n + eps);
+  else rstd = rsqrtf(a.m2 / (float)n + (float)eps);
   if (threadIdx.x == 0) {
     mean_out[blockIdx.x] = static_cast<S>(mean);
     rstd_out[blockIdx.x] = static_cast<S>(rstd);
@@ -429,7 +528,7 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_split_finish_kernel(const 
                                                                          const W* __restrict__ b, T* __restrict__ y,
                                                                          S* __restrict__ mean_out, S* __restrict__ rstd_out,
                                                                          const unsigned char* __restrict__ ws, int64_t n,
-                                                                         int64_t chunk, float eps) {
+                                                                         int64_t chunk, double eps) {
   using A = typename LnAcc<T>::type;
   constexpr int V = Vec<T>::N;
   __shared__ WF<A> smem[kLnBlock / kWave];
@@ -445,7 +544,7 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_split_finish_kernel(const 
   const A mean = a.mean;
   A rstd;
   if constexpr (std::is_same<A, double>::value) rstd = 1.0 / sqrt(a.m2 / (double)n + (double)eps);
-  else rstd = rsqrtf(a.m2 / (float)n + eps);
+  else rstd = rsqrtf(a.m2 / (float)n + (float)eps);
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     mean_out[blockIdx.y] = static_cast<S>(mean);
     rstd_out[blockIdx.y] = static_cast<S>(rstd);
@@ -498,10 +597,10 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
       const bool xv16 = N % V == 0 && aligned16(x) && aligned16(y);
       if (xv16) {
         hipLaunchKernelGGL((layernorm_split_partial_kernel<T, true>), grid, dim3(kLnBlock), 0, st, x, wsp, N, sp.chunk);
-        hipLaunchKernelGGL((layernorm_split_finish_kernel<T, W, S, true>), grid, dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, wsp, N, sp.chunk, (float)eps);
+        hipLaunchKernelGGL((layernorm_split_finish_kernel<T, W, S, true>), grid, dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, wsp, N, sp.chunk, eps);
       } else {
         hipLaunchKernelGGL((layernorm_split_partial_kernel<T, false>), grid, dim3(kLnBlock), 0, st, x, wsp, N, sp.chunk);
-        hipLaunchKernelGGL((layernorm_split_finish_kernel<T, W, S, false>), grid, dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, wsp, N, sp.chunk, (float)eps);
+        hipLaunchKernelGGL((layernorm_split_finish_kernel<T, W, S, false>), grid, dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, wsp, N, sp.chunk, eps);
       }
       return check_launch("mi355_layer_norm(split rows)");
     }
@@ -527,28 +626,38 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
     // that every wave gets the same number of rows when M allows it.
     auto launch = [&](auto nv) {
       constexpr int NV = decltype(nv)::value;
-      auto go = [&](auto hw, auto hb) {
-        constexpr bool HW_ = decltype(hw)::value, HB_ = decltype(hb)::value;
-        const void* kern = (const void*)layernorm_stream_kernel<T, S, NV, HW_, HB_>;
+      auto go = [&](auto hw, auto hb, auto full) {
+        constexpr bool HW_ = decltype(hw)::value, HB_ = decltype(hb)::value, FULL_ = decltype(full)::value;
+        const void* kern = (const void*)layernorm_stream_kernel<T, S, NV, HW_, HB_, FULL_>;
+        // gamma and beta in LDS: as floats for bf16 (widened once at staging)
+        const size_t smem = has_params ? 2 * (size_t)N * (std::is_same<T, bf16_t>::value ? sizeof(float) : sizeof(T)) : 0;
         static thread_local int resident = 0;  // blocks per CU, per instantiation
-        if (resident == 0) {
+        static thread_local size_t resident_smem = 0;
+        if (resident == 0 || resident_smem != smem) {
           int nb = 0;
-          if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, kLnBlock, has_params ? param_bytes : 0) != hipSuccess || nb < 1) nb = 2;
+          if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kern, kLnBlock, smem) != hipSuccess || nb < 1) nb = 2;
           resident = nb;
+          resident_smem = smem;
         }
         const int64_t max_waves = (int64_t)kNumCU * resident * (kLnBlock / kWave);
         const int64_t per_wave = (M + max_waves - 1) / max_waves;
         const int64_t nwaves = (M + per_wave - 1) / per_wave;
         const unsigned nblk = (unsigned)((nwaves + kLnBlock / kWave - 1) / (kLnBlock / kWave));
-        hipLaunchKernelGGL((layernorm_stream_kernel<T, S, NV, HW_, HB_>), dim3(nblk), dim3(kLnBlock), has_params ? param_bytes : 0, st, x,
+        hipLaunchKernelGGL((layernorm_stream_kernel<T, S, NV, HW_, HB_, FULL_>), dim3(nblk), dim3(kLnBlock), smem, st, x,
                            reinterpret_cast<const T*>(w), reinterpret_cast<const T*>(b), y, mean, rstd, M, N, (float)eps);
       };
       using std::true_type;
       using std::false_type;
-      if (w && b) go(true_type(), true_type());
-      else if (w) go(true_type(), false_type());
-      else if (b) go(false_type(), true_type());
-      else go(false_type(), false_type());
+      // Rows that fill every slab run without the per-slab masks (two-byte types; for fp32 the masked
+      // form measured 2 % faster, 23.1 against 23.5 us on [8192, 2048]).
+      auto pick = [&](auto full) {
+        if (w && b) go(true_type(), true_type(), full);
+        else if (w) go(true_type(), false_type(), full);
+        else if (b) go(false_type(), true_type(), full);
+        else go(false_type(), false_type(), full);
+      };
+      if (sizeof(T) == 2 && N == (int64_t)NV * kWave * V) pick(true_type());
+      else pick(false_type());
     };
     if (N <= 4 * kWave * V) launch(std::integral_constant<int, 4>());
     else launch(std::integral_constant<int, 8>());
@@ -595,8 +704,8 @@ static int run_ln(const void* xv, const void* wv, const void* bv, void* yv, void
     }
   }, 16);
   if (!done) {
-    if (vec) hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, true>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, (float)eps);
-    else hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, false>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, (float)eps);
+    if (vec) hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, true>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, eps);
+    else hipLaunchKernelGGL((layernorm_block_kernel<T, W, S, false>), dim3((unsigned)M), dim3(kLnBlock), 0, st, x, w, b, y, mean, rstd, N, eps);
   }
   return check_launch("mi355_layer_norm");
 }

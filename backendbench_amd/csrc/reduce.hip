@@ -675,6 +675,15 @@ static int scratch_address(void** ptr) {
   return MI355_OK;
 }
 
+// Called by mi355_init(): resolves the address on the current device ahead of the first call, so that
+// a mi355_reduce_static recorded into a HIP graph does no runtime query during the capture.
+namespace mi355 {
+int reduce_static_init() {
+  void* ptr = nullptr;
+  return scratch_address(&ptr);
+}
+}  // namespace mi355
+
 extern "C" int64_t mi355_reduce_static_max_bytes(void) { return kStaticScratchBytes; }
 
 extern "C" int mi355_reduce_static(int op, const void* x, int in_dtype, int64_t outer, int64_t red, int64_t inner,

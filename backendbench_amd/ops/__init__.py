@@ -12,7 +12,7 @@ from .elementwise import (_inplace_from, add, add_, clamp, clamp_, clamp_max, cl
                           clamp_min_, clamp_min_tensor, clamp_tensor, maximum, minimum, mul, mul_, out_variant, relu,
                           relu_, tuple_out_variant, where)
 from .index import embedding, gather, index_select
-from .matmul import addmm, mm
+from .matmul import addmm, addmm_dtype, mm, mm_dtype
 from .reduce import (amax, argmax, log_softmax, mean_default, mean_dim, native_layer_norm, softmax, sum_default,
                      sum_dim)
 
@@ -60,6 +60,8 @@ VARIANT_SLOTS = {
     "mul__Scalar": mul,
     "clamp_min__Tensor": clamp_min_tensor,
     "clamp_max__Tensor": clamp_max_tensor,
+    "mm__dtype": mm_dtype,        # bf16 / f16 operands, fp32 result (BackendBench/scripts/op_map.py:740)
+    "addmm__dtype": addmm_dtype,  # (op_map.py:271)
     # out= overloads
     "add__out": out_variant(add),
     "mul__out": out_variant(mul),
@@ -87,6 +89,8 @@ VARIANT_SLOTS = {
     "mean__dtype_out": out_variant(mean_default),
     "embedding__out": out_variant(embedding),
     "native_layer_norm__out": tuple_out_variant(native_layer_norm, 3),
+    "mm__dtype_out": out_variant(mm_dtype),
+    "addmm__dtype_out": out_variant(addmm_dtype),
 }
 
 SLOTS = {**CORE_SLOTS, **VARIANT_SLOTS}

@@ -71,6 +71,8 @@ def device_managed(fn):
 
 
 _entry = {}
+_ready = set()  # devices mi355_init() has accepted
+_current_device = getattr(torch._C, "_cuda_getDevice", None) or torch.cuda.current_device
 
 
 def launch(name, *args):
@@ -82,6 +84,10 @@ def launch(name, *args):
     fn = _entry.get(name)
     if fn is None:
         fn = _entry[name] = getattr(_lib.load(), name)
+    dev = _current_device()
+    if dev not in _ready:
+        _lib.init_device(dev)  # refuses a GPU the launch heuristics are not built for
+        _ready.add(dev)
     rc = fn(*args, _lib.current_stream_handle())
     if rc != 0:
         _lib.check(rc)
@@ -97,6 +103,50 @@ def row_major_strides(shape):
 def new_dense(shape, dtype, device):
     """Uninitialised row-major tensor (empty_strided parses its arguments faster than empty)."""
     return torch.empty_strided(shape, row_major_strides(shape), dtype=dtype, device=device)
+
+
+# ---- out= overloads write in place ---------------------------------------------------
+# An out= overload offers its `out` tensor(s) here before it calls the functional wrapper; the
+# wrapper asks for its result buffer with new_result() / result_like() and gets `out` itself when
+# shape, dtype, device and layout are the ones it would have allocated.  The kernel then writes
+# straight into `out`: no temporary, no second pass.  Anything else (a resize, a cast, an `out`
+# that shares memory with an input) leaves the offer untaken and the overload copies as before.
+_offered = []
+
+
+def offer_out(*outs):
+    _offered[:] = outs
+
+
+def withdraw_out():
+    _offered.clear()
+
+
+def _take(shape, dtype, device, strides):
+    for i, t in enumerate(_offered):
+        if t.dtype == dtype and t.device == device and tuple(t.shape) == tuple(shape) and t.stride() == tuple(strides):
+            return _offered.pop(i)
+    return None
+
+
+def new_result(shape, dtype, device):
+    """Row-major buffer for an operator's result: the offered out= tensor when it fits, else a new one."""
+    if _offered:
+        t = _take(shape, dtype, device, row_major_strides(shape))
+        if t is not None:
+            return t
+    return torch.empty_strided(shape, row_major_strides(shape), dtype=dtype, device=device)
+
+
+def result_like(lead, dtype):
+    """Result buffer with the (permuted-dense) layout of `lead`: the offered out= tensor when it has exactly
+    that layout, else torch.empty_like's."""
+    out = torch.empty_like(lead) if lead.dtype == dtype else torch.empty_like(lead, dtype=dtype)
+    if _offered:
+        t = _take(out.shape, dtype, out.device, out.stride())
+        if t is not None:
+            return t
+    return out
 
 
 def copy_into(dst, src):
@@ -150,6 +200,9 @@ def norm_dim(dim, ndim):
 #     after every test; MI355_SYNC_INDEX_CHECK=1 makes every indexing call do so, which is the
 #     CPU kernels' behaviour at the cost of a device sync per call).
 # Nothing raises while the stream is being captured into a graph (the flag stays set).
+# Which call raises is therefore a matter of timing, as with a device-side assert: the first launch of this
+# backend that finds the word set - any operator, possibly an unrelated one, which is then not launched -
+# raises for every out-of-range index met up to that point; the words are cleared behind a device sync.
 _flags = {}       # device key -> pinned int32 tensor (kept alive)
 _flag_words = []  # ctypes views of the same words, read on every launch
 
@@ -174,6 +227,12 @@ def poll_index_errors():
     index and the device has run it.  Called at the start of every operator launch when a flag is set."""
     if torch.cuda.is_current_stream_capturing():
         return  # not in the middle of a graph capture; the flag stays set
+    if not any(w.value for w in _flag_words):
+        return
+    # Everything enqueued so far runs to its end before the words are cleared: a second indexing kernel
+    # that is still storing 1 cannot slip its error past the clear and have it reported against some later,
+    # innocent call (the error path may cost a device sync; the check above does not).
+    torch.cuda.synchronize()
     bad = False
     for w in _flag_words:
         if w.value != 0:

@@ -10,7 +10,8 @@ import math
 import torch
 
 from .. import _lib
-from ._common import cast, copy_into, dense, device_managed, launch, new_dense
+from ._common import (cast, copy_into, dense, device_managed, launch, new_dense, new_result, offer_out, result_like,
+                      withdraw_out)
 
 
 def _out_like_inputs(shape, dtype, inputs):
@@ -25,10 +26,10 @@ def _out_like_inputs(shape, dtype, inputs):
                 lead = None
                 break
     if lead is not None:
-        out = torch.empty_like(lead) if lead.dtype == dtype else torch.empty_like(lead, dtype=dtype)
+        out = result_like(lead, dtype)
         if lead.is_contiguous() or out.stride() == lead.stride():  # preserve_format: dense permutations survive
             return out
-    return new_dense(shape, dtype, inputs[0].device)
+    return new_result(shape, dtype, inputs[0].device)
 
 
 def _is_permuted_dense(t):
@@ -255,7 +256,7 @@ _C_NAMES = {torch.uint8: "uint8_t", torch.int8: "int8_t", torch.int16: "int16_t"
 
 def _unary(op, x, out_dtype, bounds=0, lo=None, hi=None, inplace=False):
     x = cast(x, out_dtype)
-    out = x if inplace else torch.empty_like(x)  # preserve_format: dense permutations keep their layout
+    out = x if inplace else result_like(x, out_dtype)  # preserve_format: dense permutations keep their layout
     if out.numel() == 0:
         return out
     if out_dtype.is_floating_point:
@@ -438,25 +439,56 @@ def clamp_max_tensor(self, max):
     return minimum(self, max)
 
 
+def _shares_memory(out, args, kwargs):
+    """True when `out` lives in the storage of some tensor argument (conservative: same storage = overlap)."""
+    base = out.untyped_storage().data_ptr()
+    for a in list(args) + list(kwargs.values()):
+        if isinstance(a, torch.Tensor) and a.device == out.device and a.numel() and a.untyped_storage().data_ptr() == base:
+            return True
+    return False
+
+
+def _call_into(functional, outs, args, kwargs):
+    """functional(*args, **kwargs) with `outs` offered as result buffers (see _common.offer_out): GPU tensors
+    that share no storage with an argument - a kernel writing its result over an operand it is still
+    reading would be a race the functional form does not have."""
+    direct = [o for o in outs if o.is_cuda and not _shares_memory(o, args, kwargs)]
+    if len(direct) != len(outs):
+        return functional(*args, **kwargs)
+    offer_out(*direct)
+    try:
+        return functional(*args, **kwargs)
+    finally:
+        withdraw_out()
+
+
+def _store_result(out, res):
+    """`res` into `out` as ATen's out= overloads do: castable dtype, `out` resized when its shape differs."""
+    if res is out:
+        return out  # the kernel wrote into `out` itself
+    if not torch.can_cast(res.dtype, out.dtype):
+        raise RuntimeError(f"result type {str(res.dtype).replace('torch.', '').capitalize()} can't be cast to "
+                           f"the desired output type {str(out.dtype).replace('torch.', '').capitalize()}")
+    if tuple(out.shape) != tuple(res.shape):
+        out.resize_(res.shape)
+    if res.device != out.device:
+        res = res.to(out.device)
+    return copy_into_any(out, res)
+
+
 def tuple_out_variant(functional, n):
-    """`<op>.out(..., out0=, out1=, ...)` of an operator with `n` results (native_layer_norm.out):
-    each result goes into its own out tensor, resized and cast as in out_variant; returns them."""
+    """`<op>.out(..., out0=, out1=, ...)` of an operator with `n` results (native_layer_norm.out): each result
+    lands in its own out tensor - written there by the kernel when that tensor already has the result's shape,
+    dtype and a dense layout, resized / cast by a copy otherwise; returns the out tensors."""
 
     def impl(*args, **kwargs):
         outs = [kwargs.pop(f"out{i}") for i in range(n)]
-        results = functional(*args, **kwargs)
+        results = _call_into(functional, outs, args, kwargs)
         for res, out in zip(results, outs):
-            if not torch.can_cast(res.dtype, out.dtype):
+            if res is not out and not torch.can_cast(res.dtype, out.dtype):
                 raise RuntimeError(f"result type {str(res.dtype).replace('torch.', '').capitalize()} can't be cast to "
                                    f"the desired output type {str(out.dtype).replace('torch.', '').capitalize()}")
-        done = []
-        for res, out in zip(results, outs):
-            if tuple(out.shape) != tuple(res.shape):
-                out.resize_(res.shape)
-            if res.device != out.device:
-                res = res.to(out.device)
-            done.append(copy_into_any(out, res))
-        return tuple(done)
+        return tuple(_store_result(out, res) for res, out in zip(results, outs))
 
     impl.__name__ = functional.__name__ + "_out"
     impl.__doc__ = f"out= variant of {functional.__name__} ({n} results)"
@@ -464,19 +496,13 @@ def tuple_out_variant(functional, n):
 
 
 def out_variant(functional):
-    """`<op>.out(..., out=Tensor)` from the functional wrapper: compute, resize `out` if its
-    shape differs (as ATen does), then store with a cast into `out`'s dtype and return `out`."""
+    """`<op>.out(..., out=Tensor)` from the functional wrapper.  When `out` already has the result's shape and
+    dtype, a dense layout and no memory in common with an argument, the kernel writes into it directly (the
+    common case: same traffic as the functional form).  Otherwise the result is computed into a temporary,
+    `out` is resized if its shape differs (as ATen does) and the copy kernel stores it with a cast."""
 
     def impl(*args, out, **kwargs):
-        res = functional(*args, **kwargs)
-        if not torch.can_cast(res.dtype, out.dtype):
-            raise RuntimeError(f"result type {str(res.dtype).replace('torch.', '').capitalize()} can't be cast to "
-                               f"the desired output type {str(out.dtype).replace('torch.', '').capitalize()}")
-        if tuple(out.shape) != tuple(res.shape):
-            out.resize_(res.shape)
-        if res.device != out.device:
-            res = res.to(out.device)
-        return copy_into_any(out, res)
+        return _store_result(out, _call_into(functional, [out], args, kwargs))
 
     impl.__name__ = functional.__name__ + "_out"
     impl.__doc__ = f"out= variant of {functional.__name__}"

@@ -3,7 +3,7 @@
 import torch
 
 from .. import _lib
-from ._common import (check_index_errors, dense, device_managed, index_error_flag, launch, new_dense, norm_dim, prod,
+from ._common import (check_index_errors, dense, device_managed, index_error_flag, launch, new_dense, new_result, norm_dim, prod,
                       sync_index_check)
 
 
@@ -35,7 +35,7 @@ def index_select(self, dim, index):
     else:
         shape = tuple(self.shape)
         out_shape = shape[:d] + (index.numel(),) + shape[d + 1 :]
-    out = new_dense(out_shape, self.dtype, self.device)
+    out = new_result(out_shape, self.dtype, self.device)
     if out.numel() == 0:
         return out
     _rows(dense(self), prod(shape[:d]), shape[d], prod(shape[d + 1 :]), dense(index), out)
@@ -49,7 +49,7 @@ def embedding(weight, indices, padding_idx=-1, scale_grad_by_freq=False, sparse=
     if weight.dim() != 2:
         raise RuntimeError("'weight' must be 2-D")
     _lib.dtype_code(weight.dtype)
-    out = new_dense(tuple(indices.shape) + (weight.shape[1],), weight.dtype, weight.device)
+    out = new_result(tuple(indices.shape) + (weight.shape[1],), weight.dtype, weight.device)
     if out.numel() == 0:
         return out
     _rows(dense(weight), 1, weight.shape[0], weight.shape[1], dense(indices), out)
@@ -63,7 +63,7 @@ def gather(self, dim, index, *, sparse_grad=False):
         raise RuntimeError("gather(): Expected dtype int64 for index")
     _lib.dtype_code(self.dtype)
     d = norm_dim(dim, self.dim())
-    out = new_dense(index.shape, self.dtype, self.device)
+    out = new_result(index.shape, self.dtype, self.device)
     if index.numel() == 0:
         return out
     # 0-d operands behave as one-element vectors

@@ -3,7 +3,7 @@
 import torch
 
 from .. import _lib
-from ._common import cast, copy_into, dense, device_managed, launch, new_dense
+from ._common import cast, copy_into, dense, device_managed, launch, new_dense, new_result
 
 _GEMM_DTYPES = (torch.bfloat16, torch.float16, torch.float32, torch.float64)
 _SPLITK_MAX_OUT = 256 * 256 * 128 + 1  # the planner never splits problems with more than 128 tiles of 256x256
@@ -29,7 +29,7 @@ def _gemm(a, b, c, alpha, beta):
         raise NotImplementedError(f"mi355 backend: matmul on {a.dtype} is not supported")
     M, K = a.shape
     N = b.shape[1]
-    out = new_dense((M, N), a.dtype, a.device)
+    out = new_result((M, N), a.dtype, a.device)
     if M == 0 or N == 0:
         return out
     if c is not None:
@@ -76,6 +76,74 @@ def _gemm(a, b, c, alpha, beta):
            c_rs, c_cs, out.data_ptr(), M, N, K, float(alpha), float(beta), code,
            ws.data_ptr() if ws is not None else None, ws_bytes)
     return out
+
+
+_HALF = (torch.bfloat16, torch.float16)
+_UNSUPPORTED = -2  # MI355_ERR_UNSUPPORTED
+_f32out_fn = None
+
+
+def _check_out_dtype(a, out_dtype):
+    """ATen's rule for the .dtype overloads: the operands' own dtype, or fp32 for f16 / bf16 operands."""
+    if not (out_dtype == a.dtype or (out_dtype == torch.float32 and a.dtype in _HALF)):
+        raise RuntimeError("out_dtype must be the same as input dtype or fp32 for fp16/bf16 inputs")
+
+
+def _gemm_f32out(a, b, c, alpha, beta):
+    """bf16 / f16 operands, fp32 result (mm.dtype / addmm.dtype with out_dtype=float32): the MFMA kernels
+    store their fp32 accumulators unrounded (mi355_gemm_f32out).  Layouts that entry point does not take
+    (odd K or N, misaligned views) run as an fp32 product of the widened operands instead: the products of
+    two bf16 / f16 values are exact in fp32, so both paths add up the same terms in fp32."""
+    global _f32out_fn
+    if a.dim() != 2 or b.dim() != 2:
+        raise RuntimeError(f"mat1 and mat2 must be matrices, got {a.dim()}-D and {b.dim()}-D tensors")
+    if a.shape[1] != b.shape[0]:
+        raise RuntimeError(f"mat1 and mat2 shapes cannot be multiplied ({a.shape[0]}x{a.shape[1]} and "
+                           f"{b.shape[0]}x{b.shape[1]})")
+    if a.dtype != b.dtype:
+        raise RuntimeError(f"expected m1 and m2 to have the same dtype, but got: {a.dtype} != {b.dtype}")
+    M, K = a.shape
+    N = b.shape[1]
+    if c is not None:
+        if c.dtype != a.dtype:
+            raise RuntimeError(f"self and mat2 must have the same dtype, but got {c.dtype} and {a.dtype}")
+        c = c.expand(M, N)
+    if M and N and K:
+        if a.stride(1) != 1:
+            a = dense(a)
+        if b.stride(1) != 1 and b.stride(0) != 1:
+            b = dense(b)
+        out = new_result((M, N), torch.float32, a.device)
+        if _f32out_fn is None:
+            _f32out_fn = _lib.load().mi355_gemm_f32out
+        c_args = (c.data_ptr(), c.stride(0), c.stride(1)) if c is not None else (None, 0, 0)
+        rc = _f32out_fn(a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), *c_args,
+                        out.data_ptr(), M, N, K, float(alpha), float(beta), _lib.dtype_code(a.dtype),
+                        _lib.current_stream_handle())
+        if rc == 0:
+            return out
+        if rc != _UNSUPPORTED:
+            _lib.check(rc)
+    wide_c = cast(c, torch.float32) if c is not None else None
+    return _gemm(cast(a, torch.float32), cast(b, torch.float32), wide_c, alpha, beta)
+
+
+@device_managed
+def mm_dtype(self, mat2, out_dtype):
+    """aten.mm.dtype: mm with the result in `out_dtype` (fp32 from bf16 / f16 operands, or the operands' dtype)."""
+    _check_out_dtype(self, out_dtype)
+    if out_dtype == self.dtype:
+        return _gemm(self, mat2, None, 1.0, 0.0)
+    return _gemm_f32out(self, mat2, None, 1.0, 0.0)
+
+
+@device_managed
+def addmm_dtype(self, mat1, mat2, out_dtype, *, beta=1, alpha=1):
+    """aten.addmm.dtype: beta * self + alpha * (mat1 @ mat2) in `out_dtype`; self has the operands' dtype."""
+    _check_out_dtype(mat1, out_dtype)
+    if out_dtype == mat1.dtype:
+        return _gemm(mat1, mat2, self, alpha, beta)
+    return _gemm_f32out(mat1, mat2, self, alpha, beta)
 
 
 @device_managed

@@ -8,7 +8,7 @@ with the copy kernel.
 import torch
 
 from .. import _lib
-from ._common import cast, copy_into, dense, device_managed, launch, new_dense, norm_dim, prod
+from ._common import cast, copy_into, dense, device_managed, launch, new_dense, new_result, norm_dim, prod
 
 _NATIVE_IN = (torch.float32, torch.float16, torch.bfloat16, torch.float64, torch.int32, torch.int64)
 _SMALL_INT = (torch.int16, torch.int8, torch.uint8, torch.bool)
@@ -123,7 +123,7 @@ def _run_reduce(op, x, dims, keepdim, out_dtype):
         # 732 us on the column kernel).  Indices along the reduced axis are unchanged by it.
         xd = dense(xd.as_strided((outer, red, inner), (red * inner, inner, 1)).transpose(1, 2))  # xd's memory is dense in this order
         outer, inner = outer * inner, 1
-    out = new_dense(_out_shape(x, dims, keepdim), out_dtype, x.device)
+    out = new_result(_out_shape(x, dims, keepdim), out_dtype, x.device)
     lib = _lib.load()
     in_code, out_code = _lib.dtype_code(xd.dtype), _lib.dtype_code(out_dtype)
     ws_bytes = lib.mi355_reduce_workspace_bytes(op, in_code, outer, red, inner)
@@ -238,7 +238,7 @@ def _softmax_impl(self, dim, half_to_float, log):
         raise RuntimeError("conversion is supported for Half and BFloat16 type only")
     out_dtype = torch.float32 if half_to_float else self.dtype
     d = norm_dim(dim, self.dim())
-    out = new_dense(self.shape, out_dtype, self.device)
+    out = new_result(self.shape, out_dtype, self.device)
     if self.numel() == 0:
         return out
     x = dense(self)
@@ -294,9 +294,9 @@ def native_layer_norm(input, normalized_shape, weight, bias, eps):
     lead = list(input.shape[: input.dim() - k])
     M, N = prod(lead), prod(normalized_shape)
     stat_dtype = torch.float64 if input.dtype == torch.float64 else torch.float32
-    y = new_dense(input.shape, input.dtype, input.device)
-    mean = new_dense(lead + [1] * k, stat_dtype, input.device)
-    rstd = new_dense(lead + [1] * k, stat_dtype, input.device)
+    y = new_result(input.shape, input.dtype, input.device)
+    mean = new_result(lead + [1] * k, stat_dtype, input.device)
+    rstd = new_result(lead + [1] * k, stat_dtype, input.device)
     if M == 0:
         return y, mean, rstd
     if N == 0:

@@ -1,10 +1,12 @@
 """Result files of an evaluation run.
 
-Writes the same four files, with the same fields, as BackendBench/output.py:116-288:
-full_results.json (every test result, sorted by op then args), operator_summary.csv (one
-row per operator), failed_tests.json and OVERALL_SUMMARY.md.  Beyond the reference's fields,
-performance records and operator rows carry roofline columns (algorithmic_work, bound,
-achieved, achieved_unit, roofline_frac) when the suite declares the work of a timed case.
+Writes the same four files, with the same fields in the same order, as
+BackendBench/output.py:116-288: full_results.json (every test result, sorted by op then args),
+operator_summary.csv (one row per operator), failed_tests.json and OVERALL_SUMMARY.md - a
+consumer of the reference's schema reads them unchanged.  What this build measures beyond the
+reference (algorithmic work of a timed case, GB/s or TFLOP/s, fraction of the MI355X peak) goes
+to a fifth file of its own, roofline_summary.csv, written only when the suite declared the work
+of some timed case.
 """
 
 import csv
@@ -25,10 +27,32 @@ def _geomean(xs):
     return torch.tensor(xs, dtype=torch.float64).log().mean().exp().item() if xs else 0.0
 
 
+ROOFLINE_FIELDS = ("algorithmic_work", "bound", "achieved", "achieved_unit", "roofline_frac")
+
+
+def _reference_record(result):
+    """asdict() of a result with exactly the reference's fields (BackendBench/eval.py:24-46)."""
+    rec = asdict(result)
+    for name in ROOFLINE_FIELDS:
+        rec.pop(name, None)
+    return rec
+
+
+def roofline_rows(performance_results):
+    """One row per timed case whose suite declared its algorithmic work: what roofline_summary.csv holds."""
+    rows = []
+    for r in performance_results or []:
+        if r.successfully_ran and getattr(r, "roofline_frac", None) is not None:
+            rows.append({"operator": r.op_name, "args": r.args, "benchmark_time_ms": r.benchmark_time_ms,
+                         "speedup": r.speedup, **{name: getattr(r, name) for name in ROOFLINE_FIELDS}})
+    rows.sort(key=lambda row: (row["operator"], -row["algorithmic_work"], row["args"]))
+    return rows
+
+
 def prepare_results(correctness_results, performance_results):
     """(all results as dicts, failed tests as dicts, {op: summary row})."""
     order = lambda r: (r["op_name"], r["args"])
-    all_results = sorted([asdict(r) for r in correctness_results] + [asdict(r) for r in performance_results], key=order)
+    all_results = sorted([_reference_record(r) for r in correctness_results] + [_reference_record(r) for r in performance_results], key=order)
     by_op = defaultdict(lambda: ([], []))
     for r in correctness_results:
         by_op[r.op_name][0].append(r)
@@ -55,20 +79,8 @@ def prepare_results(correctness_results, performance_results):
             "max_absolute_error": max((e[0] for e in errs), default=0.0),
             "max_relative_error": max((e[1] for e in errs), default=0.0),
         }
-        # Roofline columns, beyond the reference's (BackendBench/output.py:151-176): present when the
-        # suite declared the algorithmic work of its timed cases.  With several timed cases the row
-        # carries the one with the most work (the headline shape).
-        roof = [r for r in ps if r.successfully_ran and getattr(r, "roofline_frac", None) is not None]
-        top = max(roof, key=lambda r: r.algorithmic_work) if roof else None
-        summaries[op_name].update({
-            "algorithmic_work": top.algorithmic_work if top else "",
-            "bound": top.bound if top else "",
-            "achieved": top.achieved if top else "",
-            "achieved_unit": top.achieved_unit if top else "",
-            "roofline_frac": top.roofline_frac if top else "",
-        })
-    failed = sorted([asdict(r) for r in correctness_results if not r.is_correct]
-                    + [asdict(r) for r in performance_results if not r.successfully_ran], key=order)
+    failed = sorted([_reference_record(r) for r in correctness_results if not r.is_correct]
+                    + [_reference_record(r) for r in performance_results if not r.successfully_ran], key=order)
     return all_results, failed, summaries
 
 
@@ -129,6 +141,12 @@ def save_results(correctness_results, performance_results, output_path, command=
             w.writeheader()
             w.writerows(rows)
     (base / "failed_tests.json").write_text(json.dumps(failed, indent=2))
+    roof = roofline_rows(performance_results)
+    if roof:
+        with open(base / "roofline_summary.csv", "w", newline="") as f:
+            w = csv.DictWriter(f, fieldnames=list(roof[0].keys()))
+            w.writeheader()
+            w.writerows(roof)
     if all(x is not None for x in (command, mean_correctness, geomean_perf, perf_at_p_score)):
         (base / "OVERALL_SUMMARY.md").write_text(
             overall_summary_text(command, mean_correctness, geomean_perf, perf_at_p_score, p,

@@ -30,11 +30,10 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
-MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, TFLOP/s
 # HBM bytes per launch from hardware counters (FETCH_SIZE + WRITE_SIZE, each scaled by what the
-# same counter reads for a plain 128 MiB copy); measured once per kernel with rocprofv3 --pmc,
-# summary in profiles/C2_row_kernels__softmax_layer_norm.md.  Not re-measured by this script.
+# same counter reads for a plain 128 MiB copy): rocprofv3 --pmc runs of `bench.py --only-op <row>`,
+# commands and tables in profiles/C2_row_kernels__softmax_layer_norm.md.  A profiler cannot run inside
+# this script, so the figures are carried here and named as such in the output ("traffic_source").
 MEASURED_TRAFFIC_BYTES = {"C2.layer_norm": 138_790_000, "C2.softmax": 134_300_000}
 
 
@@ -48,6 +47,7 @@ def parse():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink factor for every shape (debug only)")
     ap.add_argument("--ops", default="all", help="comma-separated substrings of per-op rows to time, or 'none'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-calib", action="store_true", help="skip the calibration block (plain copies, MFMA streams)")
     ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy, 'calib.mm' = a product of --shape in --dtype")
     ap.add_argument("--variant", type=int, default=0,
                     help="with --only-op calib.mfma: 0 = the 32x32x16 mm kernels' MFMA order, 1 = operands swapped between the "
@@ -99,50 +99,12 @@ def main():
     def impl_of(case):
         return backend[case.op]
 
-    # ------------------------------------------------------------ profiler mode
-    # One op only, timed exactly like its per_op row, so that a profiler's per-kernel average
-    # covers the same launches.  "calib.copy" is a plain 128 MiB -> 128 MiB copy with the
-    # library's copy kernel (known traffic, for scaling hardware byte counters).
-    if args.only_op == "calib.mfma":
-        print(json.dumps(calib_mfma_f64(dev, args.variant or 16) if args.dtype == "f64" else calib_mfma(dev, args.fill, args.variant)))
-        return
-    if args.only_op == "calib.mm":
-        M, K, N = (int(v) for v in args.shape.split(","))
-        dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32, "f64": torch.float64}[args.dtype]
-        a = torch.randn(M, K, device=dev).to(dt)
-        b = (torch.randn(K, N, device=dev) * 0.02).to(dt)
-        ms, how = graph_bench(backend[torch.ops.aten.mm.default], [a, b], {})
-        tiles = -(-M // 256) * -(-N // 256)
-        print(json.dumps({"only_op": "calib.mm", "shape": [M, K, N], "dtype": args.dtype, "ms": round(ms, 5),
-                          "tflops": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1), "tiles_256x256": tiles,
-                          "rounds_of_256_cus": round(tiles / 256, 3), "timing": how}))
-        return
-    if args.only_op and args.trace:
-        print(json.dumps(gemm_trace(by_key[args.only_op], dev, args.fill)))
-        return
-    if args.only_op and args.ablate is not None:
-        print(json.dumps(gemm_ablate(by_key[args.only_op], dev, args.ablate, args.fill)))
-        return
-    if args.only_op:
-        if args.only_op == "calib.copy":
-            from backendbench_amd.ops._common import copy_into
+    from backendbench_amd import measure
+    from backendbench_amd.measure import HBM_PEAK_GBS, MFMA_BF16_PEAK_TFLOPS, copy_ms_for, cpu_time_ms, graph_bench
 
-            src = torch.empty(32 * 2**20, dtype=torch.float32, device=dev).normal_()
-            f, a, kw, work = (lambda s: copy_into(torch.empty_like(s), s)), [src], {}, 2 * src.numel() * 4
-        else:
-            case = by_key[args.only_op]
-            a, kw = case.make(dev)
-            f, work = impl_of(case), case.work
-            if args.fill:
-                for t in a:
-                    if isinstance(t, torch.Tensor) and t.dtype.is_floating_point:
-                        if args.fill == "sign":
-                            t.copy_(torch.randint(-1, 2, t.shape, device=t.device).to(t.dtype))
-                        else:
-                            t.fill_(0.0 if args.fill == "zeros" else 1.0)
-        ms, how = graph_bench(f, a, kw)
-        print(json.dumps({"only_op": args.only_op, "ms": round(ms, 5), "work": work, "timing": how,
-                          **({"fill": args.fill} if args.fill else {})}))
+    # One op only (profilers, calibrations, diagnostics): backendbench_amd/measure.py
+    if args.only_op:
+        measure.only_op(args, backend, by_key, dev)
         return
 
     # ------------------------------------------------------------ headline step loop (C2)
@@ -264,6 +226,20 @@ def main():
         del a, kw
         torch.cuda.empty_cache()
 
+    # What the chip sustains in this very run: plain copies over five sizes and the GEMM kernels' MFMA
+    # streams without memory traffic.  Every row is then also stated against that measured ceiling.
+    calib = None
+    if not args.no_calib and args.scale == 1.0:
+        calib = measure.calib_block(dev)
+        fit = calib["copy_fit"]
+        stream = calib["mfma"]["x16_stream_gemm_data"]["tflops"]
+        for r in per_op:
+            if r["bound"] == "hbm":
+                fit_ms = fit["intercept_us"] * 1e-3 + r["bytes"] / (fit["asymptote_gbs"] * 1e9) * 1e3
+                r["copy_fit_ms"] = round(fit_ms, 5)          # a plain copy of this many bytes, from the fitted line
+                r["vs_copy_fit"] = round(fit_ms / r["ms"], 3)
+            else:
+                r["frac_of_measured_stream"] = round(r["tflops"] / stream, 4)  # of the 16x16x32 MFMA stream on this data
     rows = {r["op"]: r for r in per_op}
     # dominant kernel of the step = the op with the largest share of a step's GPU time
     roofline = None
@@ -273,6 +249,7 @@ def main():
         roofline = {"bound": "hbm", "kernel": dom["op"], "achieved": dom["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(dom["gbs"] / HBM_PEAK_GBS, 4),
                     "traffic": MEASURED_TRAFFIC_BYTES.get(dom["op"]) if args.scale == 1.0 else None,
+                    "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --only-op " + dom["op"] + "`, scaled by a 128 MiB copy's (profiles/)",
                     "bytes_per_launch": dom["bytes"], "avg_launch_ms": dom["ms"],
                     "timing": dom["timing"]}
     cpu_baseline = None
@@ -298,283 +275,10 @@ def main():
                                "sum(dim=-1) + amax(dim=-1), one call each per step, each on its own copy of the input",
                    "bytes_per_step": int(step_bytes), "launch": launch_mode, "input_pool": pool_n,
                    "scale": args.scale},
-        "roofline": roofline, "cpu_baseline": cpu_baseline,
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "calib": calib,
         "geomean_speedup_vs_cpu": geomean, "per_op": per_op,
     }
     print(json.dumps(line))
-
-
-def copy_ms_for(nbytes, dev, cache):
-    """Mean ms per launch of the library's flat copy kernel moving `nbytes` in total (half read,
-    half written), with graph_bench's recipe: the size-matched ceiling of a memory-bound row
-    (launch ramp and tail included, which dominate rows of a few tens of megabytes)."""
-    import torch
-
-    from backendbench_amd.ops._common import copy_into
-
-    n = max(1024, (nbytes // 2) // 4096 * 1024)  # fp32 elements of the source
-    if n not in cache:
-        src = torch.empty(n, dtype=torch.float32, device=dev).normal_()
-        cache[n] = graph_bench(lambda s: copy_into(torch.empty_like(s), s), [src], {})[0]
-        del src
-    return cache[n]
-
-
-def calib_mfma(dev, fill=None, variant=0, blocks=256, steps=2752, launches=20):
-    """Sustained rate of the mm kernel's MFMA stream with no memory traffic (mi355_calib_mfma): one
-    workgroup of four waves per CU, each wave a 128 x 128 register tile, `steps` 32-k steps per
-    launch (eight times the K loop of the [4096,11008] x [11008,4096] product).  Operand data as
-    the GEMM configuration prescribes (left N(0,1), right N(0,0.02), bf16) unless `fill` overrides
-    it: what this loop sustains is the ceiling the power / clock envelope leaves a GEMM on that data."""
-    import torch
-
-    from backendbench_amd import _lib
-
-    lib = _lib.load()
-    g = torch.Generator().manual_seed(0)
-    n = blocks * 256 * 16 * 8  # bf16 elements per operand buffer
-    a = torch.randn(n, generator=g).bfloat16()
-    b = (torch.randn(n, generator=g) * 0.02).bfloat16()
-    if fill == "zeros":
-        a.zero_(), b.zero_()
-    elif fill == "ones":
-        a.fill_(1.0), b.fill_(1.0)
-    elif fill == "sign":
-        a = torch.randint(-1, 2, (n,), generator=g).bfloat16()
-        b = torch.randint(-1, 2, (n,), generator=g).bfloat16()
-    a, b = a.to(dev), b.to(dev)
-    out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
-    stream = _lib.current_stream_handle()
-
-    def run():
-        _lib.check(lib.mi355_calib_mfma(a.data_ptr(), b.data_ptr(), out.data_ptr(), _lib.BF16, blocks, steps, variant, stream))
-
-    for _ in range(3):
-        run()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(launches):
-        run()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / launches
-    flops = blocks * 4 * steps * 2 * 128 * 128 * 32
-    tf = flops / (ms * 1e-3) / 1e12
-    return {"only_op": "calib.mfma", "variant": variant, "fill": fill or "N(0,1) x N(0,0.02)", "ms": round(ms, 4),
-            "flops": flops, "tflops": round(tf, 1), "frac_of_peak": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-            "timing": f"{launches} launches of {blocks} x 4 waves x {steps} steps, events around the loop"}
-
-
-def calib_mfma_f64(dev, waves, blocks=256, steps=20000, launches=5):
-    """Issue rate of v_mfma_f64_16x16x4_f64 with `waves` waves per workgroup, one workgroup per CU, eight
-    independent accumulator blocks per wave, no memory traffic (mi355_calib_mfma with dtype f64)."""
-    import torch
-
-    from backendbench_amd import _lib
-
-    lib = _lib.load()
-    g = torch.Generator().manual_seed(0)
-    a = torch.randn(256, generator=g, dtype=torch.float64).to(dev)
-    b = torch.randn(256, generator=g, dtype=torch.float64).to(dev)
-    out = torch.empty(blocks * 256, dtype=torch.float32, device=dev)
-    stream = _lib.current_stream_handle()
-
-    def run():
-        _lib.check(lib.mi355_calib_mfma(a.data_ptr(), b.data_ptr(), out.data_ptr(), _lib.F64, blocks, steps, waves, stream))
-
-    run()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(launches):
-        run()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / launches
-    flops = blocks * waves * steps * 8 * 2048
-    tf = flops / (ms * 1e-3) / 1e12
-    return {"only_op": "calib.mfma", "dtype": "f64", "waves_per_workgroup": waves, "ms": round(ms, 4), "flops": flops,
-            "tflops": round(tf, 1), "frac_of_peak": round(tf / 78.6, 4),
-            "ns_per_mfma_and_wave": round(ms * 1e6 / (steps * 8), 1),
-            "timing": f"{launches} launches of {blocks} x {waves} waves x {steps} rounds of 8 MFMAs, events around the loop"}
-
-
-def gemm_ablate(case, dev, bits, fill=None, launches=40):
-    """The row's mm through the ablation build `bits` (see csrc/gemm_x16.hip): events around `launches`
-    back-to-back launches after a warm-up.  Timing only - the build leaves work out, its results are wrong.
-    MI355_GEMM_TILE in the environment applies as usual (x16 = one workgroup per tile)."""
-    import ctypes
-
-    import torch
-
-    from backendbench_amd import _build, _lib
-
-    path = _build.ablate_lib_path(bits)
-    if not path.exists():
-        raise RuntimeError(f"{path} is missing: python -m backendbench_amd._build --ablate {bits}")
-    lib = ctypes.CDLL(str(path))
-    fn = lib.mi355_gemm
-    fn.restype, fn.argtypes = _lib.SIGNATURES["mi355_gemm"]
-    (a, b), _ = case.make(dev)
-    if fill:
-        for t in (a, b):
-            t.copy_(torch.randint(-1, 2, t.shape, device=dev).to(t.dtype)) if fill == "sign" else t.fill_(0.0 if fill == "zeros" else 1.0)
-    M, K = a.shape
-    N = b.shape[1]
-    out = torch.empty(M, N, dtype=a.dtype, device=dev)
-
-    def run():
-        _lib.check(fn(a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), None, 0, 0,
-                      out.data_ptr(), M, N, K, 1.0, 0.0, _lib.dtype_code(a.dtype), None, 0, _lib.current_stream_handle()))
-
-    for _ in range(3 * launches):  # the first dozens of launches of a process run slower (clocks, power state)
-        run()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(launches):
-        run()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / launches
-    flops = 2.0 * M * N * K
-    return {"only_op": case.key, "ablate": bits, "fill": fill or "as configured", "ms": round(ms, 5),
-            "tflops_nominal": round(flops / (ms * 1e-3) / 1e12, 1),
-            "timing": f"events around {launches} back-to-back launches; results are wrong by construction"}
-
-
-def gemm_trace(case, dev, fill=None):
-    """One mm of this row through the stamped diagnostic build (see the MI355_GEMM_TRACE blocks in
-    csrc/gemm_x16.hip and csrc/gemm.hip for the record layout): mean shader-clock ticks per phase of a
-    tile and per pair of steps of the K loop (a step = 32 k: a half-stage of the 16x16x32 kernel, 64
-    MFMAs of 16 clocks, or a step of the 32x32x16 kernels, 32 MFMAs of 32 clocks), the gap between two
-    tiles on one CU, and ticks per microsecond of kernel time (the average shader clock, which is
-    what moves with the operand data).  MI355_GEMM_WAVES=4 in the environment selects the
-    32x32x16 four-wave kernel instead of the 16x16x32 one."""
-    import ctypes
-
-    import numpy as np
-    import torch
-
-    from backendbench_amd import _build, _lib
-
-    if not _build.TRACE_LIB_PATH.exists():
-        raise RuntimeError(f"{_build.TRACE_LIB_PATH} is missing: python -m backendbench_amd._build --trace")
-    lib = ctypes.CDLL(str(_build.TRACE_LIB_PATH))
-    fn = lib.mi355_gemm
-    fn.restype, fn.argtypes = _lib.SIGNATURES["mi355_gemm"]
-    (a, b), _ = case.make(dev)
-    if fill:
-        for t in (a, b):
-            t.copy_(torch.randint(-1, 2, t.shape, device=dev).to(t.dtype)) if fill == "sign" else t.fill_(0.0 if fill == "zeros" else 1.0)
-    M, K = a.shape
-    N = b.shape[1]
-    out = torch.empty(M, N, dtype=a.dtype, device=dev)
-    ws = torch.zeros(1 << 20, dtype=torch.int64, device=dev)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(3):
-        ws.zero_()
-        e0.record()
-        _lib.check(fn(a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), None, 0, 0,
-                      out.data_ptr(), M, N, K, 1.0, 0.0, _lib.dtype_code(a.dtype), ws.data_ptr(), ws.numel() * 8,
-                      _lib.current_stream_handle()))
-        e1.record()
-        torch.cuda.synchronize()
-    us = e0.elapsed_time(e1) * 1e3
-    rec = ws.cpu().numpy().reshape(-1, 4, 16)
-    rec = rec[rec[:, 0, 7] > 0]
-    w0 = rec[:, 0, :].astype(np.float64)
-    iters = w0[:, 7]
-    entry, begin, end, drained, stored = w0[:, 12], w0[:, 10], w0[:, 13], w0[:, 14], w0[:, 15]
-    hw = rec[:, 0, 11]
-    cu_key = (np.arange(len(rec)) % 8) * 4096 + (hw & 0xFF00)  # XCD (block % 8), SE / SH / CU bits of HW_ID
-    gaps = []
-    for k in np.unique(cu_key):
-        idx = np.where(cu_key == k)[0]
-        idx = idx[np.argsort(entry[idx])]
-        gaps += list(entry[idx[1:]] - stored[idx[:-1]])
-    per_step = (w0[:, :6] / iters[:, None]).mean(axis=0)
-    names = ["even_issue", "even_fill_wait", "even_barrier", "odd_issue", "odd_fill_wait", "odd_barrier_and_back_edge"]
-    whole = float(np.mean(stored - entry))
-    return {"only_op": case.key, "trace": True, "fill": fill or "as configured", "kernel_us": round(us, 1), "tiles": int(len(rec)),
-            "ticks_per_step_pair": {n: round(float(v), 1) for n, v in zip(names, per_step)},
-            "mfma_ticks_per_step_pair_at_full_rate": 2048,
-            "ticks_per_tile": {"prologue": round(float(np.mean(begin - entry))), "steady_loop": round(float(np.mean(end - begin))),
-                               "remainder_and_drain": round(float(np.mean(drained - end))),
-                               "epilogue_until_stored": round(float(np.mean(stored - drained))), "whole_tile": round(whole)},
-            "ticks_between_tiles_on_a_cu": round(float(np.median(gaps))) if gaps and len(rec) > 256 else None,
-            "rounds_of_tiles": round(len(rec) / 256, 3),
-            "approx_ticks_per_us": round(whole * max(1.0, np.ceil(len(rec) / 256)) / us) if us > 0 else None}
-
-
-def graph_bench(fn, args, kwargs, pool_bytes=768 * 2**20, target_ms=60.0):
-    """Mean ms per launch of `fn`: a HIP graph holds one launch per member of a pool of
-    argument copies (pool larger than the last-level cache, so no launch finds its inputs
-    cached); the graph is replayed back to back and the whole run is bracketed by one pair of
-    events on the launch stream.  Per-launch time = elapsed / launches: kernel time plus the
-    graph's inter-kernel gap, without per-launch event or Python overhead."""
-    import torch
-
-    nbytes = sum(a.numel() * a.element_size() for a in args if isinstance(a, torch.Tensor))
-    # at least four copies while they fit 6 GiB (inputs of a gigabyte: the gathers), else two (the 4.2 GB argmax)
-    copies = max(4 if 4 * nbytes <= 6 * 2**30 else 2, min(24, math.ceil(pool_bytes / max(nbytes, 1))))
-    # A replay costs about 2.3 us on top of its kernels (two launches per graph: + 1.2 us each, twelve: + 0.2):
-    # a graph of few copies walks its pool more than once, so that every row carries about the same share.
-    rounds = math.ceil(6 / copies)
-    launches = copies * rounds
-    clone = lambda seq: [x.clone() if isinstance(x, torch.Tensor) else x for x in seq]
-    pool = [list(args)] + [clone(args) for _ in range(copies - 1)]
-    for p in pool[:2]:
-        fn(*p, **kwargs)
-    torch.cuda.synchronize()
-    try:
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            held = [fn(*p, **kwargs) for _ in range(rounds) for p in pool]
-        run, per_run, how = graph.replay, launches, f"hip graph of {launches} launches over {copies} input copies, events around replays"
-    except Exception as exc:  # noqa: BLE001
-        print(f"bench.py: graph capture failed for this op ({exc}); eager launches", file=sys.stderr)
-        run, per_run, how = (lambda: [fn(*p, **kwargs) for p in pool]), copies, "eager launches over input copies, events around the loop"
-    run()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    run()
-    e1.record()
-    torch.cuda.synchronize()
-    once = max(e0.elapsed_time(e1), 1e-3)
-    reps = max(3, min(2000, int(target_ms / once)))
-    e0.record()
-    for _ in range(reps):
-        run()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / (reps * per_run), how
-
-
-def cpu_time_ms(case, args, kwargs, budget_s=2.0):
-    """Mean ms per call of ATen on the host CPU for this row (the oracle), at full size, with the
-    reference's CPU recipe (BackendBench/eval.py:149-159: 10 warm-up calls, then 100 timed calls
-    with perf_counter, mean).  Rows that cost more than 10 ms per call (the GEMMs, the 4.2 GB
-    argmax) keep the full-size call and run fewer repetitions, as many as fit `budget_s`; the
-    counts are reported."""
-    import torch
-
-    from oracle import aten_cpu
-
-    a = aten_cpu.to_cpu(list(args))
-    kw = aten_cpu.to_cpu(dict(kwargs))
-    t0 = time.perf_counter()
-    case.op(*a, **kw)
-    first = time.perf_counter() - t0
-    if first < 0.010:
-        warm, runs = 10, 100
-    else:
-        runs = max(3, min(100, int(budget_s / first)))
-        warm = max(1, min(10, runs // 3))
-    sec = aten_cpu.time_call(case.op, a, kw, warmup=warm, runs=runs)
-    return round(sec * 1e3, 4), f"full size, {warm} warm-up + {runs} timed runs, {torch.get_num_threads()} threads"
 
 
 if __name__ == "__main__":

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define MI355_ABI_VERSION 7
+#define MI355_ABI_VERSION 8
 #define MI355_MAX_DIMS 8
 
 typedef enum mi355_dtype {
@@ -66,6 +66,28 @@ typedef struct mi355_tensor {
 
 int mi355_abi_version(void);
 const char* mi355_last_error(void);
+
+/* Once per process and GPU, with that GPU current, before the first kernel call (the Python
+ * binding does it on the first launch on a device).  No counterpart in the reference, which
+ * holds no device code.  Checks that the device is a gfx950 part with the 256 compute units
+ * the launch heuristics are sized for (persistent GEMM grids, split-K grids, streaming row
+ * kernels) and refuses any other with MI355_ERR_UNSUPPORTED; resolves the address of the
+ * built-in scratch array of mi355_reduce_static on this device, so that a later call of it
+ * makes no runtime query (a caller may be recording a HIP graph by then). */
+int mi355_init(void);
+
+/* Test and measurement knobs; no counterpart in the reference.  The planner's choice of GEMM
+ * kernel can be overridden so that a test reaches every kernel form on a shape of its choosing:
+ *   "gemm_tile":  "x16" | "x16persist" | "x16split" | "x16mixed" | "256x256" | "mixed" | "256x128" |
+ *                 "128x128" | "64x64"       (initial value: the environment's MI355_GEMM_TILE)
+ *   "gemm_waves": "4" | "8"                  (initial value: MI355_GEMM_WAVES)
+ *   "x16_spin_limit": polls of the in-launch split-K's bounded wait for a partial product
+ *                 before it gives up (default 2^21, about two seconds); a test sets it to 0
+ *                 to walk the give-up path while every kernel still runs to its end.
+ * value NULL or "" restores the default.  The environment is read once, at the first call
+ * of any entry point that looks at a knob; afterwards only this function changes them.
+ * Not thread-safe against concurrent mi355_gemm calls. */
+int mi355_set_knob(const char* name, const char* value);
 
 /* ---- elementwise -------------------------------------------------------------- */
 
@@ -149,6 +171,8 @@ int mi355_reduce(int op, const void* x, int in_dtype, int64_t outer, int64_t red
  * mi355_reduce_workspace_bytes() exceeds the buffer is refused with MI355_ERR_INVALID.
  * All calls on one GPU share that GPU's buffer: calls that may overlap in time on one GPU
  * (different streams, different threads) race; calls ordered on one stream do not. */
+/* Under HIP graph capture call mi355_init() beforehand: the first mi355_reduce_static on a
+ * device otherwise asks the runtime for the buffer's address (hipGetSymbolAddress). */
 int64_t mi355_reduce_static_max_bytes(void);
 int mi355_reduce_static(int op, const void* x, int in_dtype, int64_t outer, int64_t red,
                         int64_t inner, void* out, int out_dtype, void* stream);
@@ -204,6 +228,27 @@ int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t
                int64_t b_cs, const void* c, int64_t c_rs, int64_t c_cs, void* out,
                int64_t M, int64_t N, int64_t K, double alpha, double beta, int dtype,
                void* workspace, int64_t workspace_bytes, void* stream);
+
+/* out[M,N] in FP32 (dense row-major) = beta * c + alpha * (a[M,K] @ b[K,N]) for bf16 / f16 a, b, c
+ * (`dtype`): the fp32 accumulators are stored as they are, never rounded to the operand type.
+ * Takes the MFMA layouts only - a with unit column stride, b with unit row stride or with unit
+ * column stride and N % 8 == 0, K % 32 == 0, N % 4 == 0, 16-byte aligned bases and row starts -
+ * and returns MI355_ERR_UNSUPPORTED without launching anything for every other problem: the
+ * caller then widens a, b, c to fp32 (mi355_copy) and calls mi355_gemm with MI355_F32, which
+ * computes the same sums of exact products.  No workspace.
+ * Slots: mm__dtype (op_map.py:740), addmm__dtype (op_map.py:271) and their out= forms. */
+int mi355_gemm_f32out(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs,
+                      int64_t b_cs, const void* c, int64_t c_rs, int64_t c_cs, void* out,
+                      int64_t M, int64_t N, int64_t K, double alpha, double beta, int dtype,
+                      void* stream);
+
+/* Reads and clears the sticky status word of the GEMM kernels; no counterpart in the reference.
+ * A split-K launch whose summing workgroup ran out of polls (see "x16_spin_limit") fills its
+ * output tile with NaNs and sets the word; mi355_gemm itself has long returned MI355_OK by then.
+ * Returns MI355_ERR_LAUNCH with a message if the word was set since the last call, else 0.
+ * Synchronous (two small copies from / to the device): synchronise the streams that ran GEMMs
+ * first, and do not call it while a stream is being captured. */
+int mi355_gemm_status(void);
 
 /* How the large-tile bf16 / f16 kernel cuts the N columns of an [M, N] output (K a multiple of 64):
  * `wide` tile columns of 256 followed by `narrow` tile columns of 192.  narrow > 0 when K >= 4096,

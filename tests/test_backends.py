@@ -114,7 +114,7 @@ def test_repo_kernel_directory_layout(repo_root):
     for folder in SLOTS:
         assert os.path.isfile(os.path.join(base, folder, f"{folder}_implementation_v1.py"))
     b = DirectoryBackend(base)
-    assert len(b.compiled_kernels) == len(SLOTS) == 64
+    assert len(b.compiled_kernels) == len(SLOTS) == 68
     expected = {"add.Tensor", "mul.Tensor", "maximum.default", "relu.default", "clamp.default", "where.self",
                 "sum.dim_IntList", "sum.default", "mean.dim", "mean.default", "amax.default", "argmax.default",
                 "_softmax.default", "native_layer_norm.default", "mm.default", "addmm.default",

@@ -54,64 +54,7 @@ def test_documented_special_values():
 
 
 # ---- 2. numpy restatement over the whole edge suite --------------------------------------
-def np_of(t):
-    if isinstance(t, torch.Tensor):
-        if t.dtype in (torch.bfloat16, torch.float16, torch.float32):
-            return t.double().numpy()
-        return t.numpy()
-    return t
-
-
-def numpy_result(case, args, kwargs):
-    n = case.op.__name__
-    a = [np_of(x) for x in args]
-    if n in ("add.Tensor", "add.Scalar"):
-        return numpy_ref.add(a[0], a[1], kwargs.get("alpha", 1))
-    if n in ("mul.Tensor", "mul.Scalar"):
-        return numpy_ref.mul(a[0], a[1])
-    if n in ("maximum.default", "clamp_min.Tensor"):
-        return numpy_ref.maximum(*np.broadcast_arrays(a[0], a[1]))
-    if n in ("minimum.default", "clamp_max.Tensor"):
-        return numpy_ref.minimum(*np.broadcast_arrays(a[0], a[1]))
-    if n == "clamp_min.default":
-        return numpy_ref.clamp(a[0], a[1], None)
-    if n == "clamp_max.default":
-        return numpy_ref.clamp(a[0], None, a[1])
-    if n == "clamp.Tensor":
-        return numpy_ref.clamp_tensor(a[0], a[1], a[2] if len(a) > 2 else None)
-    if n == "_log_softmax.default":
-        return numpy_ref.log_softmax(a[0], a[1])
-    if n == "relu.default":
-        return numpy_ref.relu(a[0])
-    if n == "clamp.default":
-        return numpy_ref.clamp(a[0], *(a[1:] + [None, None])[:2])
-    if n == "where.self":
-        return numpy_ref.where(a[0], a[1], a[2])
-    if n in ("sum.dim_IntList", "mean.dim", "amax.default"):
-        fn = {"sum.dim_IntList": numpy_ref.sum_, "mean.dim": numpy_ref.mean, "amax.default": numpy_ref.amax}[n]
-        dim = a[1] if len(a) > 1 else ([] if n == "amax.default" else None)
-        return fn(a[0], dim, a[2] if len(a) > 2 else False)
-    if n in ("sum.default", "mean.default"):
-        return (numpy_ref.sum_ if n == "sum.default" else numpy_ref.mean)(a[0], None)
-    if n == "argmax.default":
-        return numpy_ref.argmax(a[0], a[1] if len(a) > 1 else None, a[2] if len(a) > 2 else False)
-    if n == "_softmax.default":
-        return numpy_ref.softmax(a[0], a[1]) if a[0].ndim else np.ones(())
-    if n == "native_layer_norm.default":
-        return numpy_ref.layer_norm(a[0], a[1], a[2], a[3], a[4])
-    if n == "mm.default":
-        return numpy_ref.mm(a[0], a[1])
-    if n == "addmm.default":
-        return numpy_ref.addmm(a[0], a[1], a[2], kwargs.get("beta", 1), kwargs.get("alpha", 1))
-    if n == "index_select.default":
-        return numpy_ref.index_select(a[0], a[1], a[2])
-    if n == "embedding.default":
-        return numpy_ref.embedding(a[0], a[1])
-    if n == "gather.default":
-        if a[0].ndim == 0:
-            return a[0]
-        return numpy_ref.gather(a[0], a[1], a[2])
-    raise AssertionError(n)
+from tight import np_of, numpy_result  # noqa: E402  (shared with the GPU suites' second, tighter bar)
 
 
 def tolerance(args, out):
@@ -296,3 +239,69 @@ def test_oracle_matches_golden(case):
             assert (g["nan"], g["pinf"], g["ninf"]) == (w["nan"], w["pinf"], w["ninf"])
             assert g["l1"] == pytest.approx(w["l1"], rel=2e-3, abs=1e-3)
             assert g["total"] == pytest.approx(w["total"], rel=2e-3, abs=2e-3 * max(1.0, w["l1"]))
+
+
+# ---- 5. the tighter per-dtype bar tells accumulator widths apart (CPU mock of the comparer) -----------
+class _Case:
+    def __init__(self, op):
+        self.op = op
+
+
+def _narrow_sum(terms, dtype, chunk=128):
+    """Sum along the last axis in chunks of `chunk` terms (each chunk in fp32) with the running total rounded
+    to `dtype` after every chunk: an accumulator that is only partly as wide as advertised."""
+    acc = torch.zeros(terms.shape[:-1], dtype=dtype)
+    for i in range(0, terms.shape[-1], chunk):
+        acc = (acc.float() + terms[..., i : i + chunk].float().sum(-1)).to(dtype)
+    return acc
+
+
+def test_tight_bar_separates_fp32_from_bf16_accumulation():
+    from tight import tight_check
+
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(8, 512, generator=g).bfloat16()
+    b = (torch.randn(512, 6, generator=g) * 0.02).bfloat16()
+    case = _Case(aten.mm.default)
+    terms = a.float()[:, None, :] * b.float().t()[None, :, :]          # [8, 6, 512] exact products
+    fp32_acc = terms.sum(-1).bfloat16()
+    bf16_acc = _narrow_sum(terms, torch.bfloat16)
+    assert ev_allclose(fp32_acc, bf16_acc)                              # the reference's 1e-2 bar sees no difference
+    assert tight_check(case, [a, b], {}, fp32_acc) is None
+    assert "mm.default" in tight_check(case, [a, b], {}, bf16_acc)
+    # fp32 results: an fp32 accumulator passes, an f16 one does not
+    af, bf_ = torch.randn(4, 2048, generator=g), torch.randn(2048, 3, generator=g)
+    t32 = af[:, None, :] * bf_.t()[None, :, :]
+    assert tight_check(case, [af, bf_], {}, t32.sum(-1)) is None
+    assert tight_check(case, [af, bf_], {}, _narrow_sum(t32, torch.float16).float()) is not None
+
+
+def test_tight_bar_separates_fp64_from_fp32_arithmetic():
+    from tight import tight_check
+
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(5, 300, generator=g, dtype=torch.float64) * 3
+    sm = _Case(aten._softmax.default)
+    assert tight_check(sm, [x, -1, False], {}, torch.softmax(x, -1)) is None
+    assert tight_check(sm, [x, -1, False], {}, torch.softmax(x.float(), -1).double()) is not None
+    ln = _Case(aten.native_layer_norm.default)
+    w, b = torch.randn(300, generator=g, dtype=torch.float64), torch.randn(300, generator=g, dtype=torch.float64)
+    good = torch.ops.aten.native_layer_norm(x, [300], w, b, 1e-5)
+    assert tight_check(ln, [x, [300], w, b, 1e-5], {}, good) is None
+    low = tuple(t.double() for t in torch.ops.aten.native_layer_norm(x.float(), [300], w.float(), b.float(), 1e-5))
+    assert tight_check(ln, [x, [300], w, b, 1e-5], {}, low) is not None
+    # half outputs: one rounding of the fp32 result passes, a second rounding through a coarser type does not
+    xs = torch.randn(64, 1000, generator=g).bfloat16()
+    sm_out = torch.softmax(xs.float(), -1)
+    assert tight_check(sm, [xs, -1, False], {}, sm_out.bfloat16()) is None
+    assert tight_check(sm, [xs, -1, False], {}, (sm_out * 1.02).bfloat16()) is not None   # 2 % off: inside 1e-2 + 1e-2 |x|
+    sums = _Case(aten.sum.dim_IntList)
+    big = (torch.randn(16, 4096, generator=g) * 4).bfloat16()
+    assert tight_check(sums, [big, [-1]], {}, big.float().sum(-1).bfloat16()) is None
+    assert tight_check(sums, [big, [-1]], {}, _narrow_sum(big, torch.bfloat16)) is not None
+
+
+def ev_allclose(a, b):
+    from backendbench_amd import eval as ev
+
+    return ev.allclose(a, b)

@@ -5,7 +5,7 @@ import csv
 import json
 
 from backendbench_amd.eval import CorrectnessTestResult, PerformanceTestResult
-from backendbench_amd.output import overall_summary_text, prepare_results, save_results, summary_rows
+from backendbench_amd.output import overall_summary_text, prepare_results, roofline_rows, save_results, summary_rows
 
 
 def results():
@@ -30,9 +30,14 @@ def test_prepare_results():
     assert summary["relu.default"]["passed_performance_tests"] == 0 and summary["relu.default"]["geomean_speedup"] == 0.0
     assert list(s) == ["operator", "total_tests", "correctness_tests", "performance_tests", "passed_correctness_tests",
                        "passed_performance_tests", "failed_correctness_tests", "failed_performance_tests",
-                       "correctness_rate", "avg_speedup", "geomean_speedup", "max_absolute_error", "max_relative_error",
-                       "algorithmic_work", "bound", "achieved", "achieved_unit", "roofline_frac"]
-    assert s["roofline_frac"] == "" and s["bound"] == ""       # no declared work: the columns stay empty
+                       "correctness_rate", "avg_speedup", "geomean_speedup", "max_absolute_error", "max_relative_error"]
+    # exactly the reference's record fields (BackendBench/eval.py:24-46), nothing of this build's on top
+    perf = [r for r in everything if r["test_type"] == "performance"][0]
+    assert list(perf) == ["op_name", "args", "speedup", "benchmark_time_ms", "reference_time_ms", "error_msg",
+                          "successfully_ran", "test_type"]
+    corr = [r for r in everything if r["test_type"] == "correctness"][0]
+    assert list(corr) == ["op_name", "args", "is_correct", "error_msg", "error_type", "traceback", "max_abs_error",
+                          "max_rel_error", "test_type"]
 
 
 def test_roofline_columns():
@@ -55,10 +60,13 @@ def test_roofline_columns():
     p = [PerformanceTestResult("mm.default", "small", 1.5, 0.01, 0.015, successfully_ran=True,
                                **roofline_columns(SimpleNamespace(case=SimpleNamespace(work=1e9, bound="mfma")), 0.01, True)),
          PerformanceTestResult("mm.default", "big", 1.2, 0.25, 0.3, successfully_ran=True, **cols)]
-    _, _, summary = prepare_results([], p)
-    row = summary["mm.default"]
-    assert row["algorithmic_work"] == 369367187456.0 and row["bound"] == "mfma" and row["achieved_unit"] == "TFLOP/s"
-    assert abs(row["roofline_frac"] - 0.5909874999296) < 1e-9
+    everything, _, summary = prepare_results([], p)
+    assert "roofline_frac" not in summary["mm.default"] and all("bound" not in r for r in everything)
+    rows = roofline_rows(p)                                      # the fifth file: the case with the most work first
+    assert [r["args"] for r in rows] == ["big", "small"] and rows[0]["operator"] == "mm.default"
+    assert rows[0]["algorithmic_work"] == 369367187456.0 and rows[0]["bound"] == "mfma" and rows[0]["achieved_unit"] == "TFLOP/s"
+    assert abs(rows[0]["roofline_frac"] - 0.5909874999296) < 1e-9
+    assert roofline_rows(results()[1]) == []                     # no declared work: no rows, no file
 
 
 def test_summary_rows_and_text():
@@ -80,3 +88,13 @@ def test_save_results_writes_four_files(tmp_path):
     assert {r["operator"] for r in rows} == {"add.Tensor", "relu.default"}
     save_results(c, p, str(tmp_path / "bare"))
     assert not (tmp_path / "bare" / "OVERALL_SUMMARY.md").exists()
+    from types import SimpleNamespace
+
+    from backendbench_amd.eval import roofline_columns
+
+    cols = roofline_columns(SimpleNamespace(case=SimpleNamespace(work=134217728.0, bound="hbm")), 0.024, True)
+    p2 = p + [PerformanceTestResult("_softmax.default", "s0", 1.3, 0.024, 0.031, successfully_ran=True, **cols)]
+    save_results(c, p2, str(tmp_path / "roof"))
+    rows = list(csv.DictReader(open(tmp_path / "roof" / "roofline_summary.csv")))
+    assert len(rows) == 1 and rows[0]["operator"] == "_softmax.default" and rows[0]["bound"] == "hbm"
+    assert abs(float(rows[0]["roofline_frac"]) - 134217728 / 0.024e-3 / 1e9 / 8000.0) < 1e-9

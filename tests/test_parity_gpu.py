@@ -18,6 +18,8 @@ from backendbench_amd.backends import DirectoryBackend
 from backendbench_amd.suite import SmokeTestSuite, edge_cases, perf_cases
 from oracle import aten_cpu
 
+from tight import tight_check  # noqa: E402
+
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -30,7 +32,7 @@ PERF = perf_cases()
 def backend():
     assert torch.cuda.is_available(), "these tests need the MI355X"
     b = DirectoryBackend(os.path.join(ROOT, "generated_kernels"))
-    assert len(b.compiled_kernels) == 64
+    assert len(b.compiled_kernels) == 68
     return b
 
 
@@ -55,6 +57,9 @@ def run_case(backend, case):
     if not ok:
         a, r = ev.compute_errors(ref, res_cpu)
         pytest.fail(f"{case.key}: mismatch (max abs {a}, max rel {r}); ref={ref!r:.400} res={res_cpu!r:.400}")
+    # the second, per-dtype bar: against the numpy float64 restatement (tests/tight.py)
+    msg = tight_check(case, aten_cpu.to_cpu(list(args)), aten_cpu.to_cpu(dict(kwargs)), res_cpu)
+    assert msg is None, f"{case.key}: {msg}"
 
 
 @pytest.mark.parametrize("case", EDGE, ids=[c.key for c in EDGE])
@@ -130,7 +135,7 @@ def test_headline_gemm_full_size(backend, key):
 
 @pytest.mark.parametrize("waves", ["4", "8", "256x128"])
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
-def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch):
+def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, gemm_knobs):
     """The 256x256-tile kernels only run when a problem has enough tiles to fill the chip, so the
     small K-step cases of the edge suite never reach them.  A [3500, K] x [K, 3600] product has
     14 x 15 tiles (ragged last row and column of tiles); K walks through every prologue / steady /
@@ -141,9 +146,9 @@ def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch
     forces the four-wave kernel on 256x128 tiles for every K that is a multiple of 64."""
     announce(f"large-tile GEMM K loop lengths, {layout}, {waves}")
     if waves == "256x128":   # the four-wave kernel on 256x128 tiles, otherwise chosen for mid-sized problems
-        monkeypatch.setenv("MI355_GEMM_TILE", waves)
+        gemm_knobs.tile(waves)
     else:
-        monkeypatch.setenv("MI355_GEMM_WAVES", waves)
+        gemm_knobs.waves(waves)
     g = torch.Generator().manual_seed(5)
     M, N = (3504, 3600) if layout[0] == "t" else (3500, 3600)   # an M-contiguous operand needs M % 8 == 0
     rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 127, 128, 255, 256, 3327, 3328, 3499])]))
@@ -165,7 +170,7 @@ def test_large_tile_gemm_every_k_loop_length(backend, layout, waves, monkeypatch
 
 
 @pytest.mark.parametrize("layout", ["nt", "nn", "tn", "tt"])
-def test_mixed_width_tile_grid(backend, layout, monkeypatch):
+def test_mixed_width_tile_grid(backend, layout, gemm_knobs):
     """More than one round of 256x256 tiles with a ragged last round: the four-wave kernel cuts the last
     columns into 192-wide tiles (one launch, two tile widths).  [4104, K] x [K, 4500] has 17 x 18 tiles of
     256x256; the planner must choose a mixed grid for it, the result must be bit-equal to the plain grid's
@@ -179,7 +184,7 @@ def test_mixed_width_tile_grid(backend, layout, monkeypatch):
     wide, narrow = ctypes.c_int32(), ctypes.c_int32()
     assert _lib.load().mi355_gemm_tile_columns(M, N, 4096, ctypes.byref(wide), ctypes.byref(narrow)) == 0
     assert narrow.value > 0, "this shape is meant to take the mixed grid"
-    monkeypatch.setenv("MI355_GEMM_WAVES", "4")
+    gemm_knobs.waves("4")
     g = torch.Generator().manual_seed(11)
     edge = wide.value * 256
     rows = torch.unique(torch.cat([torch.randint(0, M, (40,), generator=g), torch.tensor([0, 255, 256, 4095, 4096, 4103])]))
@@ -193,11 +198,11 @@ def test_mixed_width_tile_grid(backend, layout, monkeypatch):
         else:
             b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
         bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
-        monkeypatch.setenv("MI355_GEMM_TILE", "mixed")      # the mixed grid whatever K is (by itself: K >= 4096)
+        gemm_knobs.tile("mixed")      # the mixed grid whatever K is (by itself: K >= 4096)
         mixed = backend[aten.addmm.default](bias, a, b)
-        monkeypatch.setenv("MI355_GEMM_TILE", "256x256")
+        gemm_knobs.tile("256x256")
         plain = backend[aten.addmm.default](bias, a, b)
-        monkeypatch.delenv("MI355_GEMM_TILE")
+        gemm_knobs.tile(None)
         assert ev.bit_equal(plain, mixed), (layout, K)
         ref = aten_cpu.reference(aten.addmm.default, [bias, a[rows.cuda()], b])
         assert ev.bit_equal(ref, mixed[rows.cuda()].cpu()), (layout, K)
@@ -268,7 +273,7 @@ def test_gemm_split_k_inside_one_launch(backend, layout, dtype):
 
 
 @pytest.mark.parametrize("form", ["planner", "x16", "x16mixed", "256x128", "mixed", "w4", "w8", "64x64", "128x128"])
-def test_gemm_output_rows_off_16_byte_boundaries(backend, form, monkeypatch):
+def test_gemm_output_rows_off_16_byte_boundaries(backend, form, gemm_knobs):
     """An output width that is no multiple of 8 (a 50257-wide vocabulary) puts every row of the result at
     another 2-byte offset; the MFMA kernels then store along the destination's 16-byte grid: whole units
     inside a tile's row segment, single elements at its two ends (those units are shared with the
@@ -281,11 +286,11 @@ def test_gemm_output_rows_off_16_byte_boundaries(backend, form, monkeypatch):
     from backendbench_amd.ops._common import launch
     announce(f"GEMM output rows off 16-byte boundaries, {form}")
     if form in ("w4", "w8"):
-        monkeypatch.setenv("MI355_GEMM_WAVES", form[1])
+        gemm_knobs.waves(form[1])
     elif form != "planner":
-        monkeypatch.setenv("MI355_GEMM_TILE", form)
+        gemm_knobs.tile(form)
         if form == "mixed":   # the mixed-width grid belongs to the four-wave 32x32x16 kernel
-            monkeypatch.setenv("MI355_GEMM_WAVES", "4")
+            gemm_knobs.waves("4")
     g = torch.Generator().manual_seed(23)
     M, K = (1000, 256) if form in ("64x64", "128x128") else (2300, 256)
     widths = (257, 1026, 1283, 2052, 2309, 2566, 2823, 301) if form in ("64x64", "128x128") else (4097, 4098, 4355, 4100, 4613, 4358, 4103, 4104, 4376)
@@ -309,7 +314,7 @@ def test_gemm_output_rows_off_16_byte_boundaries(backend, form, monkeypatch):
 
 @pytest.mark.parametrize("tile", ["x16", "x16mixed", "planner"])
 @pytest.mark.parametrize("layout", ["nt", "nn"])
-def test_x16_gemm_every_k_loop_length(backend, layout, tile, monkeypatch):
+def test_x16_gemm_every_k_loop_length(backend, layout, tile, gemm_knobs):
     """The 256x256-tile kernel on v_mfma_f32_16x16x32 (the planner's choice for products that fill the chip
     when K is a multiple of 128 from 512 on): [4104, K] x [K, 4500] has 17 x 18 tiles with a ragged last tile
     row and column; K walks from the shortest loop the kernel takes (two pairs of stages: only the peeled
@@ -337,11 +342,11 @@ def test_x16_gemm_every_k_loop_length(backend, layout, tile, monkeypatch):
             b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
         bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
         if tile != "planner":
-            monkeypatch.setenv("MI355_GEMM_TILE", tile)
+            gemm_knobs.tile(tile)
         out = backend[aten.addmm.default](bias, a, b)
         half = backend[aten.mm.default](a.half(), b.half())
         if tile != "planner":
-            monkeypatch.delenv("MI355_GEMM_TILE")
+            gemm_knobs.tile(None)
         ref = aten_cpu.reference(aten.addmm.default, [bias, a[rows.cuda()], b])
         assert ev.bit_equal(ref, out[rows.cuda()].cpu()), (layout, tile, K)
         assert ev.bit_equal(ref[:, edge - 8:edge + 200], out[rows.cuda()][:, edge - 8:edge + 200].cpu()), (layout, tile, K, "seam")
@@ -350,7 +355,7 @@ def test_x16_gemm_every_k_loop_length(backend, layout, tile, monkeypatch):
 
 
 @pytest.mark.parametrize("tile", ["x16", "x16persist"])
-def test_x16_gemm_argument_forms(backend, tile, monkeypatch):
+def test_x16_gemm_argument_forms(backend, tile, gemm_knobs):
     """What else reaches the 16x16x32 kernel besides dense operands: rows with a pitch (slices of wider tensors) on
     both operands, a c that is a column ([M, 1]), a scalar-strided c (a transposed view), a c of NaNs under beta = 0
     (never read), alpha and beta other than one, f16.  [512, 640] x [640, 768]: 2 x 3 tiles, forced onto the kernel
@@ -369,7 +374,7 @@ def test_x16_gemm_argument_forms(backend, tile, monkeypatch):
         col = ri(M, 1, lo=-2, hi=3).to(dtype).cuda()
         full_t = ri(N, M, lo=-2, hi=3).to(dtype).cuda().t()
         nan_c = torch.full((M, N), float("nan"), dtype=dtype).cuda()
-        monkeypatch.setenv("MI355_GEMM_TILE", tile)
+        gemm_knobs.tile(tile)
         outs = {
             "pitched nn": (backend[aten.mm.default](a, b), aten.mm.default, [a, b], {}),
             "pitched nt": (backend[aten.mm.default](a, bt), aten.mm.default, [a, bt], {}),
@@ -377,14 +382,14 @@ def test_x16_gemm_argument_forms(backend, tile, monkeypatch):
             "transposed c": (backend[aten.addmm.default](full_t, a, bt, beta=2.0, alpha=3.0), aten.addmm.default, [full_t, a, bt], {"beta": 2.0, "alpha": 3.0}),
             "nan c, beta 0": (backend[aten.addmm.default](nan_c, a, b, beta=0.0, alpha=2.0), aten.addmm.default, [nan_c, a, b], {"beta": 0.0, "alpha": 2.0}),
         }
-        monkeypatch.delenv("MI355_GEMM_TILE")
+        gemm_knobs.tile(None)
         for name, (got, op, args, kwargs) in outs.items():
             ref = aten_cpu.reference(op, args, kwargs)
             assert ev.bit_equal(ref, got.cpu()), (tile, dtype, name)
 
 
 @pytest.mark.parametrize("layout", ["nt", "nn"])
-def test_x16_persistent_gemm_walks_its_tiles(backend, layout, monkeypatch):
+def test_x16_persistent_gemm_walks_its_tiles(backend, layout, gemm_knobs):
     """More 256x256 tiles than CUs: one workgroup per CU walks its tiles, with the fill requests running on
     from one tile into the next.  [4096, K] x [K, 4352] has 16 x 17 = 272 tiles (sixteen workgroups get a second
     tile), [2048, K] x [K, 12288] 8 x 48 = 384 (half of them), [256, K] x [K, 256] a single one (forced: a walk
@@ -408,13 +413,13 @@ def test_x16_persistent_gemm_walks_its_tiles(backend, layout, monkeypatch):
                 b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
             bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
             c = torch.randint(-2, 3, (M, N), generator=g).to(torch.bfloat16).cuda()
-            monkeypatch.setenv("MI355_GEMM_TILE", "x16persist")
+            gemm_knobs.tile("x16persist")
             walked = backend[aten.addmm.default](bias, a, b)
             walked_c = backend[aten.addmm.default](c, a, b, beta=2.0)
             walked_mm = backend[aten.mm.default](a, b)
-            monkeypatch.setenv("MI355_GEMM_TILE", "x16")
+            gemm_knobs.tile("x16")
             plain = backend[aten.addmm.default](bias, a, b)
-            monkeypatch.delenv("MI355_GEMM_TILE")
+            gemm_knobs.tile(None)
             auto = backend[aten.addmm.default](bias, a, b)
             assert ev.bit_equal(plain, walked), (layout, M, N, K)
             assert ev.bit_equal(plain, auto), (layout, M, N, K, "planner's choice")
@@ -425,11 +430,11 @@ def test_x16_persistent_gemm_walks_its_tiles(backend, layout, monkeypatch):
             assert ev.bit_equal((walked.float() - bias.float()).to(torch.bfloat16), walked_mm), (layout, M, N, K, "mm")
             if (M % 256 or N % 256) and K == 768:
                 # c in the memory of out (the C entry point allows it): no element may take beta * c twice
-                monkeypatch.setenv("MI355_GEMM_TILE", "x16persist")
+                gemm_knobs.tile("x16persist")
                 acc = c.clone()
                 launch("mi355_gemm", a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), acc.data_ptr(), N, 1,
                        acc.data_ptr(), M, N, K, 1.0, 2.0, _lib.dtype_code(a.dtype), None, 0)
-                monkeypatch.delenv("MI355_GEMM_TILE")
+                gemm_knobs.tile(None)
                 assert ev.bit_equal(walked_c, acc), (layout, M, N, K, "c in place")
 
 
@@ -462,7 +467,7 @@ def test_small_tile_gemm_every_k_loop_length(backend, layout, shape):
 
 @pytest.mark.parametrize("layout", ["nt", "nn"])
 @pytest.mark.parametrize("shape", [(197, 776), (1000, 1080), (64, 64), (33, 4104)])
-def test_tile64_gemm_every_k_loop_length(backend, layout, shape, monkeypatch):
+def test_tile64_gemm_every_k_loop_length(backend, layout, shape, gemm_knobs):
     """The 64x64-tile kernel (products whose 128x128 tiles would leave most CUs idle): [197, K] x [K, 776] has
     4 x 13 tiles with ragged last row and column (one workgroup per CU: the eight-stage ring), [1000, K] x
     [K, 1080] has 16 x 17 = 272 (more than one per CU: the four-stage ring).  K walks from one stage to more
@@ -478,10 +483,10 @@ def test_tile64_gemm_every_k_loop_length(backend, layout, shape, monkeypatch):
         else:
             b = torch.randint(-1, 2, (K, N), generator=g).to(torch.bfloat16).cuda()
         bias = torch.randint(-2, 3, (N,), generator=g).to(torch.bfloat16).cuda()
-        monkeypatch.setenv("MI355_GEMM_TILE", "64x64")
+        gemm_knobs.tile("64x64")
         out = backend[aten.addmm.default](bias, a, b, beta=2.0)
         half = backend[aten.mm.default](a.half(), b.half())
-        monkeypatch.delenv("MI355_GEMM_TILE")
+        gemm_knobs.tile(None)
         ref = aten_cpu.reference(aten.addmm.default, [bias, a, b], {"beta": 2.0})
         assert ev.bit_equal(ref, out.cpu()), (layout, shape, K)
         assert ev.bit_equal(aten_cpu.reference(aten.mm.default, [a.half(), b.half()]), half.cpu()), (layout, shape, K, "f16")
@@ -508,7 +513,7 @@ def test_split_k_with_ragged_k(backend, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_split_k_on_64x64_tiles(backend, dtype, monkeypatch):
+def test_split_k_on_64x64_tiles(backend, dtype, gemm_knobs):
     """A handful of 64x64 tiles with a long K (one image's 197 tokens against a 3072 x 768 weight) split K in
     whole 64-k stages over the chip: blockIdx.y owns a k range, leaves its raw fp32 tile in its plane, and the
     summing launch applies alpha / beta / bias.  Stage counts that do not divide by the split count, ragged
@@ -518,7 +523,7 @@ def test_split_k_on_64x64_tiles(backend, dtype, monkeypatch):
     g = torch.Generator().manual_seed(43)
     for forced in (False, True):
         if forced:
-            monkeypatch.setenv("MI355_GEMM_TILE", "64x64")
+            gemm_knobs.tile("64x64")
         for M, N, K in [(197, 768, 3072), (128, 768, 3136), (16, 4096, 4096), (70, 1001, 2112), (256, 4096, 4032), (64, 520, 11008), (300, 200, 1088)]:
             for nt in (True, False):
                 if not nt and N % 8:
@@ -1205,7 +1210,7 @@ def test_misaligned_rows_see_exactly_their_own_elements(backend, n, dtype):
 @pytest.mark.parametrize("family", ["gpt2", "bert"])
 def test_transformers_model_under_the_dispatcher_override(backend, family):
     """A randomly initialised Hugging Face model (built from a config, nothing downloaded) gives
-    the same hidden states with the 64 slots overriding ATen's HIP kernels as without, in fp32
+    the same hidden states with the 68 slots overriding ATen's HIP kernels as without, in fp32
     and in bf16; the spy shows the model really runs through the C ABI."""
     transformers = pytest.importorskip("transformers")
     import backendbench_amd

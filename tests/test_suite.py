@@ -55,6 +55,9 @@ def test_baseline_suite_covers_every_slot():
         op for op in slot_ops
         if not op._overloadname.endswith("out") and not op._schema.name.endswith("_")
     }
+    # mm.dtype / addmm.dtype have no CPU kernel in ATen, so no suite built from the CPU oracle can hold them:
+    # tests/test_variants_gpu.py checks them against the fp32 product of the widened operands
+    functional -= {torch.ops.aten.mm.dtype, torch.ops.aten.addmm.dtype}
     assert len(functional) == 28 and ops == functional
     assert {c.key.split(".")[0] for c in perf_cases()} == {"C1", "C2", "C3", "C4", "C5"}
     assert len(edge_cases()) >= 250

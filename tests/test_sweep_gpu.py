@@ -18,6 +18,7 @@ import torch
 from backendbench_amd import eval as ev
 from backendbench_amd.backends import DirectoryBackend
 from oracle import aten_cpu
+from tight import tight_check  # noqa: E402
 
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -308,6 +309,11 @@ SWEEP = {
 }
 
 
+class _OpCase:
+    def __init__(self, op):
+        self.op = op
+
+
 def _seed(op, i):
     return sum(map(ord, op.__name__)) * 1000 + i
 
@@ -385,4 +391,8 @@ def test_random_sweep_matches_the_oracle(backend, op):
         if not ev.allclose(ref, got, exact=exact):
             a, r = ev.compute_errors(ref, got)
             failures.append(f"{what}\n    max abs {a}, max rel {r}\n    {_first_differences(ref, got)}")
+            continue
+        msg = tight_check(_OpCase(op), args, kwargs, got)   # the per-dtype bar against the fp64 restatement
+        if msg is not None:
+            failures.append(f"{what}\n    {msg}")
     assert not failures, f"{len(failures)} of {N_DRAWS} draws differ:\n" + "\n".join(failures)

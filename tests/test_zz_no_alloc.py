@@ -24,10 +24,14 @@ def _both(op, x, outer, red, inner, out_dtype):
     got = torch.full_like(ref, 77)  # poisoned: every element must be written
     _lib.check(lib.mi355_reduce(op, x.data_ptr(), in_code, outer, red, inner, ref.data_ptr(), out_code,
                                 ws.data_ptr(), need, stream))
-    before = torch.cuda.memory_allocated()
-    _lib.check(lib.mi355_reduce_static(op, x.data_ptr(), in_code, outer, red, inner, got.data_ptr(), out_code, stream))
-    assert torch.cuda.memory_allocated() == before
+    _lib.check(lib.mi355_init())  # resolves the built-in buffer's address on this device: nothing left to ask at call time
     torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    free_before, _ = torch.cuda.mem_get_info()   # hipMemGetInfo: sees every allocation on the device, not only torch's
+    _lib.check(lib.mi355_reduce_static(op, x.data_ptr(), in_code, outer, red, inner, got.data_ptr(), out_code, stream))
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before, "mi355_reduce_static changed the device's free memory"
     return need, ref, got
 
 
@@ -75,3 +79,34 @@ def test_static_scratch_refuses_what_does_not_fit():
     out = torch.zeros(8, dtype=torch.int64, device="cuda")
     rc = lib.mi355_reduce_static(_lib.ARGMAX, x.data_ptr(), _lib.F32, outer, red, inner, out.data_ptr(), _lib.I64, None)
     assert rc == -1 and b"built-in buffer" in lib.mi355_last_error()
+
+
+def test_static_scratch_under_graph_capture_and_replay():
+    """The callers this entry point is for: recorded into a HIP graph (after mi355_init(), so the capture
+    holds kernel launches only) and replayed with eager work in between; every replay gives the eager result."""
+    lib = _lib.load()
+    _lib.check(lib.mi355_init())
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(3, 1 << 20, generator=g).cuda()
+    in_code = _lib.dtype_code(x.dtype)
+    assert lib.mi355_reduce_workspace_bytes(_lib.SUM, in_code, 3, 1 << 20, 1) > 0
+    want = torch.empty(3, device="cuda")
+    _lib.check(lib.mi355_reduce_static(_lib.SUM, x.data_ptr(), in_code, 3, 1 << 20, 1, want.data_ptr(), _lib.F32,
+                                       _lib.current_stream_handle()))
+    torch.cuda.synchronize()
+    got = torch.zeros(3, device="cuda")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(lib.mi355_reduce_static(_lib.SUM, x.data_ptr(), in_code, 3, 1 << 20, 1, got.data_ptr(), _lib.F32,
+                                           _lib.current_stream_handle()))
+    for rep in range(4):
+        got.fill_(-1.0)
+        other = torch.randn(2, 70001, generator=g).cuda()          # an eager call in between shares the buffer
+        tmp = torch.empty(2, device="cuda")
+        _lib.check(lib.mi355_reduce_static(_lib.SUM, other.data_ptr(), in_code, 2, 70001, 1, tmp.data_ptr(), _lib.F32,
+                                           _lib.current_stream_handle()))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(want, got), rep
+    torch.testing.assert_close(got.cpu(), x.cpu().sum(-1), atol=1e-2, rtol=1e-2)
