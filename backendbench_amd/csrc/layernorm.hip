@@ -221,13 +221,20 @@ template <typename T, int H> __device__ __forceinline__ void ln_widen_half(ln_ra
   }
 }
 
-// V elements of gamma / beta from global memory into their LDS form (widened to P when P is wider than T).
-template <typename T, typename P, int V> __device__ __forceinline__ void ln_stage(P* dst, const T* src) {
-  const VecN<T, V> v = ld<T, V>(src);
-  VecN<P, V> o;
+// gamma / beta in LDS (widened to P when P is wider than T), in two planes: plane h holds half h (H = V / 2
+// elements) of every V-element vector, vector after vector.  A wave's read of one half of its lanes' vectors
+// is then one contiguous stretch of LDS - with the vectors stored whole, the halves sit 2 H elements apart
+// and every such read met a two-way bank conflict (SQ_LDS_BANK_CONFLICT: 48 % of the LDS cycles).
+template <typename T, typename P, int V> __device__ __forceinline__ void ln_stage(P* planes, int64_t half_elems, int64_t c, const T* src) {
+  constexpr int H = V / 2;
+  const VecN<T, V> v = ld<T, V>(src + c);
 #pragma unroll
-  for (int j = 0; j < V; ++j) o.v[j] = static_cast<P>(v.v[j]);
-  st<P, V>(dst, o);
+  for (int h = 0; h < 2; ++h) {
+    VecN<P, H> o;
+#pragma unroll
+    for (int j = 0; j < H; ++j) o.v[j] = static_cast<P>(v.v[h * H + j]);
+    st<P, H>(planes + h * half_elems + (c / V) * H, o);
+  }
 }
 // H consecutive staged parameters as floats (one LDS read of H * sizeof(P) bytes).
 template <typename P, int H> __device__ __forceinline__ void ln_params_half(const P* p, float (&f)[H]) {
@@ -263,8 +270,8 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_stream_kernel(const T* __r
   }
   if constexpr (HW || HB) {
     for (int64_t c = (int64_t)threadIdx.x * V; c < n; c += (int64_t)kLnBlock * V) {
-      if constexpr (HW) ln_stage<T, P, V>(gl + c, w + c);
-      if constexpr (HB) ln_stage<T, P, V>(bl + c, b + c);
+      if constexpr (HW) ln_stage<T, P, V>(gl, n / 2, c, w);
+      if constexpr (HB) ln_stage<T, P, V>(bl, n / 2, c, b);
     }
     __syncthreads();
   }
@@ -316,8 +323,8 @@ __global__ __launch_bounds__(kLnBlock) void layernorm_stream_kernel(const T* __r
           constexpr int H = V / 2;
           float f[H], g[H], be[H];
           ln_widen_half<T, H>(cur[k], h, f);
-          if constexpr (HW) ln_params_half<P, H>(gl + c + h * H, g);
-          if constexpr (HB) ln_params_half<P, H>(bl + c + h * H, be);
+          if constexpr (HW) ln_params_half<P, H>(gl + h * (n / 2) + (c / V) * H, g);
+          if constexpr (HB) ln_params_half<P, H>(bl + h * (n / 2) + (c / V) * H, be);
 #pragma unroll
           for (int j = 0; j < H; ++j) {
             float t = __builtin_fmaf(f[j], rstd, shift);  // (x - mean) * rstd

@@ -145,9 +145,16 @@ def _after_impl():
     check_index_errors()
 
 
+def _own_outs(kwargs):
+    """kwargs with every out= tensor (`out`, `out0`, ...) replaced by a clone.  The reference calls the operator
+    and the implementation with the same kwargs (BackendBench/eval.py:99-102), so for an out= overload both
+    would write into one tensor and the comparison would be of that tensor with itself."""
+    return {k: (v.clone() if isinstance(v, torch.Tensor) and k.startswith("out") else v) for k, v in kwargs.items()}
+
+
 def eval_correctness_test(op, impl, test) -> CorrectnessTestResult:
     args, kwargs = test.args, test.kwargs
-    ref = op(*args, **kwargs)
+    ref = op(*args, **_own_outs(kwargs))
     args_str = serialize_args(args, kwargs)
     try:
         res = impl(*args, **kwargs)

@@ -328,12 +328,134 @@ def calib_block(dev):
     return out
 
 
+def _gpt2_small(dev, dt, vocab=50257, width=768, layers=12, heads=12, positions=1024):
+    """GPT-2 small as plain torch modules (token + position embedding, 12 pre-norm blocks of causal
+    self-attention and a 4x GELU MLP, final layer norm, tied-shape vocabulary projection), randomly initialised.
+    Written out here so that nothing in the forward pass depends on the host (no data-dependent Python branches,
+    no .item()): the same call can be recorded into a HIP graph."""
+    import torch
+    from torch import nn
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.ln1, self.ln2 = nn.LayerNorm(width), nn.LayerNorm(width)
+            self.qkv, self.proj = nn.Linear(width, 3 * width), nn.Linear(width, width)
+            self.fc1, self.fc2 = nn.Linear(width, 4 * width), nn.Linear(4 * width, width)
+
+        def forward(self, x, mask):
+            B, T, C = x.shape
+            q, k, v = self.qkv(self.ln1(x).view(B * T, C)).view(B, T, 3, heads, C // heads).permute(2, 0, 3, 1, 4)
+            att = torch.matmul(q, k.transpose(-1, -2)) * (1.0 / (C // heads) ** 0.5)
+            att = torch.softmax(att + mask, dim=-1)
+            y = torch.matmul(att, v).transpose(1, 2).reshape(B * T, C)
+            x = x + self.proj(y).view(B, T, C)
+            h = torch.nn.functional.gelu(self.fc1(self.ln2(x).view(B * T, C)), approximate="tanh")
+            return x + self.fc2(h).view(B, T, C)
+
+    class GPT2(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.wte, self.wpe = nn.Embedding(vocab, width), nn.Embedding(positions, width)
+            self.blocks = nn.ModuleList(Block() for _ in range(layers))
+            self.ln_f = nn.LayerNorm(width)
+            self.head = nn.Linear(width, vocab, bias=False)
+
+        def forward(self, ids, pos, mask):
+            x = self.wte(ids) + self.wpe(pos)
+            for blk in self.blocks:
+                x = blk(x, mask)
+            B, T, C = x.shape
+            return self.head(self.ln_f(x).view(B * T, C)).view(B, T, -1)
+
+    torch.manual_seed(0)
+    model = GPT2()
+    for p in model.parameters():
+        if p.dim() > 1:
+            nn.init.normal_(p, std=0.02)
+    return model.to(device=dev, dtype=dt).eval()
+
+
+def e2e_gpt2(dev, dtype_name="bf16", batch=8, seq=1024, reps=10):
+    """One forward pass of a randomly initialised GPT-2 small (12 layers, 768 wide, 12 heads, 50257-token
+    vocabulary) on `batch` x `seq` tokens: ms per forward with this backend's kernels behind the dispatcher
+    (enable()) and with the stock ROCm kernels, launched eagerly from Python and replayed from a HIP graph.
+    Eager rows also give the host's share: the time the Python thread needs to enqueue one forward (no device
+    sync inside), which bounds the eager rate from below whenever it exceeds the GPU time.  The reference quotes
+    this kind of figure for its own kernels (docs/correctness.md:21: "about twice as slow as PyTorch eager")."""
+    import torch
+
+    import backendbench_amd
+
+    dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dtype_name]
+    model = _gpt2_small(dev, dt)
+    ids = torch.randint(0, 50257, (batch, seq), generator=torch.Generator().manual_seed(1)).to(dev)
+    pos = torch.arange(seq, device=dev).unsqueeze(0)
+    mask = torch.full((seq, seq), float("-inf"), device=dev, dtype=dt).triu(1)   # additive causal mask, built once
+
+    def forward():
+        with torch.no_grad():
+            return model(ids, pos, mask)
+
+    def timed(run, n):
+        for _ in range(3):
+            run()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(n):
+            run()
+        e1.record()
+        host = (time.perf_counter() - t0) * 1e3 / n       # enqueue only: nothing waits for the device in the loop
+        torch.cuda.synchronize()
+        return {"ms_per_forward": round(e0.elapsed_time(e1) / n, 3), "host_enqueue_ms": round(host, 3)}
+
+    def both_modes():
+        out = {"eager": timed(forward, reps)}
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):     # warm-up on the capture's kind of stream: lazy set-up happens here
+                forward()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                held = forward()
+            out["graph"] = timed(graph.replay, reps)
+            del held, graph
+        except Exception as exc:  # noqa: BLE001
+            out["graph"] = {"error": str(exc)[:300]}
+            torch.cuda.synchronize()
+        return out
+
+    ref = forward().float()
+    stock = both_modes()
+    kernel_dir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "generated_kernels")
+    with backendbench_amd.BackendBench.enable(kernel_dir=kernel_dir, dispatch_key="CUDA"):
+        got = forward().float()
+        ours = both_modes()
+        torch.cuda.synchronize()
+    err = float((got - ref).abs().max()) / max(float(ref.abs().max()), 1e-6)
+    res = {"only_op": "e2e.gpt2", "model": "GPT-2 small (12 x 768, 12 heads, vocabulary 50257), random weights", "dtype": dtype_name,
+           "tokens": [batch, seq], "stock": stock, "override": ours, "max_abs_diff_of_logits_over_scale": round(err, 5)}
+    for mode in ("eager", "graph"):
+        a, b = stock[mode].get("ms_per_forward"), ours[mode].get("ms_per_forward")
+        if a and b:
+            res[f"speedup_{mode}"] = round(a / b, 3)
+    return res
+
+
 def only_op(args, backend, by_key, dev):
     """`bench.py --only-op <row>` and its diagnostic forms; prints one JSON line."""
     import torch
 
     if args.only_op == "calib.mfma":
         print(json.dumps(calib_mfma_f64(dev, args.variant or 16) if args.dtype == "f64" else calib_mfma(dev, args.fill, args.variant)))
+        return
+    if args.only_op == "e2e.gpt2":
+        print(json.dumps(e2e_gpt2(dev, args.dtype if args.dtype in ("bf16", "f16", "f32") else "bf16")))
         return
     if args.only_op == "calib.all":
         print(json.dumps({"only_op": "calib.all", **calib_block(dev)}))

@@ -613,6 +613,47 @@ def sibling_perf_cases(scale: float = 1.0) -> List[Case]:
     ]
 
 
+# functional overload -> its out= overload (BackendBench/scripts/op_map.py lists both on one `canonical:` line)
+OUT_OVERLOADS = {
+    aten.add.Tensor: aten.add.out, aten.mul.Tensor: aten.mul.out, aten.maximum.default: aten.maximum.out,
+    aten.minimum.default: aten.minimum.out, aten.relu.default: aten.relu.out, aten.clamp.default: aten.clamp.out,
+    aten.clamp.Tensor: aten.clamp.Tensor_out, aten.clamp_min.default: aten.clamp_min.out, aten.clamp_max.default: aten.clamp_max.out,
+    aten.where.self: aten.where.self_out, aten.add.Scalar: aten.add.Scalar_out, aten.mul.Scalar: aten.mul.Scalar_out,
+    aten.sum.dim_IntList: aten.sum.IntList_out, aten.sum.default: aten.sum.out, aten.mean.dim: aten.mean.out,
+    aten.mean.default: aten.mean.dtype_out, aten.amax.default: aten.amax.out, aten.argmax.default: aten.argmax.out,
+    aten._softmax.default: aten._softmax.out, aten._log_softmax.default: aten._log_softmax.out,
+    aten.native_layer_norm.default: aten.native_layer_norm.out, aten.mm.default: aten.mm.out, aten.addmm.default: aten.addmm.out,
+    aten.index_select.default: aten.index_select.out, aten.embedding.default: aten.embedding.out, aten.gather.default: aten.gather.out,
+}
+
+
+def out_perf_cases(scale: float = 1.0) -> List[Case]:
+    """One timed case per out= overload: the headline row (or the sibling row) of its functional overload with
+    an `out` of the result's shape, dtype and layout added - the case in which the kernels write into `out`
+    directly, so the row should cost what the functional one does.  The result's shape comes from running the
+    functional overload on meta tensors: nothing is computed to build the case."""
+    seen, cases = set(), []
+    for case in perf_cases(scale) + sibling_perf_cases(scale):
+        out_op = OUT_OVERLOADS.get(case.op)
+        if out_op is None or out_op in seen:
+            continue
+        seen.add(out_op)
+
+        def make(device, case=case):
+            args, kwargs = case.make(device)
+            meta = lambda v: v.to("meta") if isinstance(v, torch.Tensor) else v
+            res = case.op(*[meta(a) for a in args], **{k: meta(v) for k, v in kwargs.items()})
+            dev = next(a.device for a in args if isinstance(a, torch.Tensor))
+            fresh = lambda r: torch.empty_strided(r.shape, r.stride(), dtype=r.dtype, device=dev)
+            if isinstance(res, (tuple, list)):
+                return args, {**kwargs, **{f"out{i}": fresh(r) for i, r in enumerate(res)}}
+            return args, {**kwargs, "out": fresh(res)}
+
+        cases.append(Case("O." + case.key.split(".", 1)[1] + "_out", out_op, make, work=case.work, bound=case.bound,
+                          exact=case.exact, note=f"out= form of {case.key}"))
+    return cases
+
+
 def _as_test(case, device):
     return CaseTest(case, device)
 
@@ -632,6 +673,11 @@ def BaselineTestSuite(device="cuda", scale=1.0, filter=None):
     for case in sibling_perf_cases(scale):
         if not per_op.setdefault(case.op, ([], []))[1]:
             per_op[case.op][1].append(case)
+    if device != "cpu":   # on the GPU only (the CPU suite is the oracle's; it pins functional overloads)
+        for case in out_perf_cases(scale):
+            per_op.setdefault(case.op, ([], []))[1].append(case)
+        for case in out_perf_cases(min(scale, 0.02)):   # the same call at a small size as the correctness test
+            per_op[case.op][0].append(case)
     optests = []
     for op, (edges, perfs) in per_op.items():
         name = op.__name__

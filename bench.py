@@ -48,7 +48,8 @@ def parse():
     ap.add_argument("--ops", default="all", help="comma-separated substrings of per-op rows to time, or 'none'")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-calib", action="store_true", help="skip the calibration block (plain copies, MFMA streams)")
-    ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy, 'calib.mm' = a product of --shape in --dtype")
+    ap.add_argument("--only-op", default=None, help="time just this per-op row (for profilers); 'calib.copy' = plain copy, 'calib.mm' = a product of --shape in --dtype, "
+                                                       "'calib.all' = the calibration block, 'e2e.gpt2' = a GPT-2-small forward with and without the override")
     ap.add_argument("--variant", type=int, default=0,
                     help="with --only-op calib.mfma: 0 = the 32x32x16 mm kernels' MFMA order, 1 = operands swapped between the "
                          "ports, 2 = the other operand held across MFMAs, 3 = v_mfma_f32_16x16x32, 4-9 = chained "
@@ -88,7 +89,7 @@ def main():
 
     from backendbench_amd import eval as ev
     from backendbench_amd.backends import DirectoryBackend
-    from backendbench_amd.suite import perf_cases
+    from backendbench_amd.suite import out_perf_cases, perf_cases
 
     torch.cuda.set_device(0)
     dev = torch.device("cuda", 0)
@@ -226,6 +227,21 @@ def main():
         del a, kw
         torch.cuda.empty_cache()
 
+    # out= overloads at four headline shapes: `out` has the result's shape and dtype, so the kernels write into
+    # it directly and the row should cost what the functional row does (vs_functional = functional ms / this ms).
+    by_ms = {r["op"]: r["ms"] for r in per_op}
+    out_rows = []
+    wanted_out = {"O.add_out": "C1.add", "O.relu_out": "C1.relu", "O.softmax_out": "C2.softmax", "O.mm_up_out": "C3.mm_up"}
+    for case in out_perf_cases(args.scale):
+        base = wanted_out.get(case.key)
+        if base is None or base not in by_ms:
+            continue
+        a, kw = case.make(dev)
+        ms, how = graph_bench(backend[case.op], a, kw)
+        out_rows.append({"op": case.key, "ms": round(ms, 5), "functional_row": base, "vs_functional": round(by_ms[base] / ms, 3), "timing": how})
+        del a, kw
+        torch.cuda.empty_cache()
+
     # What the chip sustains in this very run: plain copies over five sizes and the GEMM kernels' MFMA
     # streams without memory traffic.  Every row is then also stated against that measured ceiling.
     calib = None
@@ -276,7 +292,7 @@ def main():
                    "bytes_per_step": int(step_bytes), "launch": launch_mode, "input_pool": pool_n,
                    "scale": args.scale},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "calib": calib,
-        "geomean_speedup_vs_cpu": geomean, "per_op": per_op,
+        "geomean_speedup_vs_cpu": geomean, "per_op": per_op, "out_overloads": out_rows,
     }
     print(json.dumps(line))
 

@@ -1097,7 +1097,7 @@ def test_evaluator_scores_the_whole_gpu_suite(backend):
         assert c_score == 1.0 and not wrong, (test.op, wrong[:3])
         assert math.isfinite(float(p_score)) and float(p_score) > 0, test.op
         n_ops += 1
-    assert n_ops == 28
+    assert n_ops == 28 + 26   # functional overloads + one timed (and one checked) case per out= overload
     assert not any(c.extra.get("cpu_reference_only") for t in suite for c in [x.case for x in t.correctness_tests])
 
 
