@@ -5,6 +5,7 @@ and the ablation builds of the GEMM).  Nothing here is on the product path: the 
 import this module.
 """
 
+import collections
 import json
 import math
 import os
@@ -219,7 +220,7 @@ def gemm_trace(case, dev, fill=None):
             "approx_ticks_per_us": round(whole * max(1.0, np.ceil(len(rec) / 256)) / us) if us > 0 else None}
 
 
-def graph_bench(fn, args, kwargs, pool_bytes=768 * 2**20, target_ms=60.0):
+def graph_bench(fn, args, kwargs, pool_bytes=768 * 2**20, target_ms=60.0, min_launches=24, keep=None):
     """Mean ms per launch of `fn`: a HIP graph holds one launch per member of a pool of
     argument copies (pool larger than the last-level cache, so no launch finds its inputs
     cached); the graph is replayed back to back and the whole run is bracketed by one pair of
@@ -230,9 +231,11 @@ def graph_bench(fn, args, kwargs, pool_bytes=768 * 2**20, target_ms=60.0):
     nbytes = sum(a.numel() * a.element_size() for a in args if isinstance(a, torch.Tensor))
     # at least four copies while they fit 6 GiB (inputs of a gigabyte: the gathers), else two (the 4.2 GB argmax)
     copies = max(4 if 4 * nbytes <= 6 * 2**30 else 2, min(24, math.ceil(pool_bytes / max(nbytes, 1))))
-    # A replay costs about 2.3 us on top of its kernels (two launches per graph: + 1.2 us each, twelve: + 0.2):
-    # a graph of few copies walks its pool more than once, so that every row carries about the same share.
-    rounds = math.ceil(6 / copies)
+    # A replay costs about 2.3 us on top of its kernels (two launches per graph: + 1.2 us each, twelve: + 0.2,
+    # twenty-four: + 0.1): a graph of fewer than 24 copies walks its pool more than once, so that every row
+    # carries the same, small share of it (with six launches per graph the rows of 8 copies carried 0.3 us, those
+    # of 24 copies 0.1 us, and the figure read 1 - 2 % above rocprofv3's per-kernel average for the former).
+    rounds = math.ceil(min_launches / copies)
     launches = copies * rounds
     clone = lambda seq: [x.clone() if isinstance(x, torch.Tensor) else x for x in seq]
     pool = [list(args)] + [clone(args) for _ in range(copies - 1)]
@@ -242,7 +245,16 @@ def graph_bench(fn, args, kwargs, pool_bytes=768 * 2**20, target_ms=60.0):
     try:
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            held = [fn(*p, **kwargs) for _ in range(rounds) for p in pool]
+            # Results are dropped as a program's would be: the last `copies` stay alive (a result buffer comes round
+            # again only after `copies` other launches, a pool's worth of traffic), the older ones return to the
+            # graph's memory pool and are handed out again.  Holding all of them alive gave the row gathers 16 - 24
+            # distinct 134 MB outputs next to 4 GB of tables and cost them 7 - 14 % (address translation, not
+            # bandwidth: the same launches one at a time behind a cache flush take the same time wherever the
+            # buffers lie).
+            held = collections.deque(maxlen=copies if keep is None else keep)
+            for _ in range(rounds):
+                for p in pool:
+                    held.append(fn(*p, **kwargs))
         run, per_run, how = graph.replay, launches, f"hip graph of {launches} launches over {copies} input copies, events around replays"
     except Exception as exc:  # noqa: BLE001
         print(f"measure: graph capture failed for this op ({exc}); eager launches", file=sys.stderr)
