@@ -73,7 +73,7 @@ def build_trace(verbose: bool = True) -> Path:
     library carries no stamps."""
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     objs = []
-    for src, extra in (("gemm.hip", ["-DMI355_GEMM_TRACE"]), ("gemm_x16.hip", ["-DMI355_GEMM_TRACE"]), ("gemm_f64.hip", []), ("common.hip", [])):
+    for src, extra in (("gemm.hip", ["-DMI355_GEMM_TRACE"]), ("gemm_x16.hip", ["-DMI355_GEMM_TRACE"]), ("gemm_f64.hip", []), ("common.hip", ["-DMI355_GEMM_ONLY"])):
         obj = OBJ_DIR / (Path(src).stem + ".trace.o")
         proc = subprocess.run([HIPCC, *FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)], capture_output=True, text=True)
         if proc.returncode != 0:
@@ -100,7 +100,7 @@ def build_ablate(bits: int, verbose: bool = True) -> Path:
     are wrong; `bench.py --only-op C3.mm_down --ablate <bits>` times it to show what each part costs."""
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
     objs = []
-    for src, extra in (("gemm.hip", []), ("gemm_x16.hip", [f"-DMI355_X16_ABLATE={bits}"]), ("gemm_f64.hip", []), ("common.hip", [])):
+    for src, extra in (("gemm.hip", []), ("gemm_x16.hip", [f"-DMI355_X16_ABLATE={bits}"]), ("gemm_f64.hip", []), ("common.hip", ["-DMI355_GEMM_ONLY"])):
         obj = OBJ_DIR / (Path(src).stem + f".ablate{bits}.o")
         proc = subprocess.run([HIPCC, *FLAGS, *extra, "-c", str(CSRC / src), "-o", str(obj)], capture_output=True, text=True)
         if proc.returncode != 0:

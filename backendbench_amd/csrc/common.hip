@@ -109,9 +109,13 @@ extern "C" int mi355_set_knob(const char* name, const char* value) {
   return MI355_OK;
 }
 
-// Defined next to the state they cover.
+// Defined next to the state they cover.  (The GEMM-only measurement builds - MI355_GEMM_ONLY - hold no reduce.hip.)
 namespace mi355 {
+#ifndef MI355_GEMM_ONLY
 int reduce_static_init();   // reduce.hip: address of the built-in scratch array on the current device
+#else
+static int reduce_static_init() { return MI355_OK; }
+#endif
 }
 
 extern "C" int mi355_init(void) {

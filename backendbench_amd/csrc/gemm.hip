@@ -1993,23 +1993,38 @@ static SplitPlan plan_t64_split(int64_t M, int64_t N, int64_t K) {
 }
 
 // Split-K inside one launch of the 16x16x32 kernel (gemm_mfma_x16_splitk_kernel): for products with 65 - 128
-// tiles of 256x256 (a quarter to half of the CUs) and K >= 3072, two workgroups per tile, each with half of K.
-// The caller's workspace holds one fp32 plane of 256 KB per tile and a 64-bit flag per plane.  Measured
-// against the kernels these products took before ([M,K]x[N,K]^T, us): 96 tiles at K = 3072 63 -> 58, at
-// K = 4096 77 -> 64; 86 tiles at K = 4096 78 -> 65; 128 tiles at K = 4096 76 -> 73, at K = 11008 205 -> 153
-// (the stock kernel: 173).  It does not pay at K = 2048 (128 tiles: 44 -> 51) nor with more workgroups per
-// tile (the summing workgroup reads the other planes one after the other: 64 tiles in four parts 45 -> 85,
-// 24 tiles 27 -> 74), which is why the plan knows only two; the kernel takes up to four.
+// tiles of 256x256 (a quarter to half of the CUs) and K >= 2048 (3072 from 113 tiles on), two workgroups per tile,
+// each with about half of K.  The caller's workspace holds one fp32 plane of 256 KB per tile and a 64-bit flag per
+// plane.  Measured against one workgroup per tile ([M,K]x[N,K]^T, us; the stock kernel in brackets): 96 tiles at
+// K = 2048 44 -> 40 (33), at 3072 63 -> 50 (47), at 4096 77 -> 60 (58), at 8192 143 -> 97 (106); 128 tiles at K =
+// 2048 46 -> 45 (40), at 3072 65 -> 56 (56), at 4096 80 -> 69 (69), at 8192 148 -> 114 (126).  The exchange costs
+// a producer 3 us (its plane, 16 bytes a lane and instruction) and the summing workgroup 4 us on top of its
+// epilogue; a CU takes a plane in at 50 - 60 GB/s, so more workgroups per tile do not pay - the one that sums
+// reads all the other planes (48 tiles at K = 8192: two parts 86 us, three 78, four 83; the 128x128 kernels 90),
+// which is why the plan knows only two; the kernel takes up to four (a test knob: x16split3, x16split4).
 struct X16SplitPlan {
   int splits, tiles8;
   int64_t ws_bytes;
 };
-constexpr int64_t kX16SplitMinK = 3072;
+constexpr int64_t kX16SplitMinK = 2048, kX16SplitMinKFull = 3072;
+constexpr int kX16MaxSplits = 4;  // the summing workgroup's epilogue exists for one to three producers
 static X16SplitPlan plan_x16_split(int64_t M, int64_t N, int64_t K) {
   X16SplitPlan p{1, 0, 0};
   const int64_t tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-  if (K % kX16SplitUnit != 0 || K < kX16SplitMinK || tiles <= kNumCU / 4 || tiles > kNumCU / 2) return p;
-  p.splits = 2;
+  if (K % kX16SplitUnit != 0) return p;
+  const Knobs& kn = knobs();
+  int splits = 0;
+  if (strncmp(kn.gemm_tile, "x16split", 8) == 0 && kn.gemm_tile[8] >= '2' && kn.gemm_tile[8] <= '0' + kX16MaxSplits && kn.gemm_tile[9] == 0) {
+    splits = kn.gemm_tile[8] - '0';  // a test knob: this many workgroups per tile at any tile count
+  } else {
+    if (tiles <= kNumCU / 4 || tiles > kNumCU / 2 || K < (tiles <= 112 ? kX16SplitMinK : kX16SplitMinKFull)) return p;
+    splits = 2;
+  }
+  // every share is at least two units (the kernel's K loop needs 256): the producers share what the summing
+  // workgroup leaves
+  const int units = (int)(K / kX16SplitUnit);
+  if ((units - x16_split_summing_units(units, splits)) / (splits - 1) < 2) return p;
+  p.splits = splits;
   p.tiles8 = (int)((tiles + 7) / 8 * 8);
   p.ws_bytes = (p.splits - 1) * tiles * (int64_t)(BM * BN * 4 + 8);
   return p;
@@ -2170,10 +2185,14 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                              workspace_bytes >= (int64_t)ts.nsplit * M * ((N + 3) / 4 * 4) * 4;
       const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
-                                               : (nb128 < kNumCU / 2 || ((M <= 64 || N <= 64) && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
-                                                     (K <= (M <= 32 ? 1024 : 2048) || (nb128 > 32 && nb128 < kNumCU / 2 && M >= 16 && light_b) || t64_split ||
-                                                      nb64 >= 160));  // enough 64x64 tiles for the chip: no need to split a long K
-                                                                      // (a few rows against a 32000 x 4096 vocabulary: 48 us, 128x128 tiles 55)
+                                               : (nb128 < kNumCU / 2 || (nb128 == kNumCU / 2 && K <= 2048) ||  // (exactly 128 tiles, [1024,2048]x[2048,2048]: 26.4 -> 21.2 us, K = 512: 10.0 -> 7.0; level at K = 3072, behind from 4096 on)
+                                                  ((M <= 64 || N <= 64) && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
+                                                     (K <= (M <= 32 ? 1024 : 2048) || t64_split ||
+                                                      // enough 64x64 tiles for the chip: no need to split a long K (a few rows against a 32000 x 4096
+                                                      // vocabulary: 48 us, 128x128 tiles 55) - up to K = 4096 for more than one row of tiles: beyond, the
+                                                      // 128x128 kernels with K split over the chip are ahead ([512,8192]x[8192,1536]: 42 us here, 31 there;
+                                                      // [768,8192]x[8192,2048]: 62 against 52; at K = 4096 these are level or ahead: 23.4 against 27.5)
+                                                      ((K <= 4096 || M <= 64) && ((nb128 > 32 && nb128 < kNumCU / 2 && M >= 16 && light_b) || nb64 >= 160))));
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
       // with 256x256 tiles when K is a multiple of 128 (from 256 on): measured against the 32x32x16 forms on
       // [4096,K]x[K,16384], it is 11 % faster at K = 256 and 4 - 15 % from K = 768 on (C3: [4096,4096]x
@@ -2201,7 +2220,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
 #endif
       const bool x16_split = x16_ok && xs.splits > 1 && workspace != nullptr && workspace_bytes >= xs.ws_bytes &&
                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
-                             (forced_tile != nullptr ? strcmp(forced_tile, "x16split") == 0
+                             (forced_tile != nullptr ? strncmp(forced_tile, "x16split", 8) == 0
                                                      : x16_pays && M >= 512 && forced_waves == nullptr);  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
       if (x16_split) {
         static std::atomic<unsigned long long> epoch{0x5bd1e9955bd1e995ull};  // odd, and stepped by two: odd for ever

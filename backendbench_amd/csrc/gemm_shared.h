@@ -166,7 +166,13 @@ const void* gemm_x16_kernel(bool is_bf16, bool b_nn);
 const void* gemm_x16_persistent_kernel(bool is_bf16, bool b_nn);  // one workgroup per CU walks the tiles (whole tiles, K >= 384)
 const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn);
 const void* gemm_x16_splitk_kernel(bool is_bf16, bool b_nn);  // 2 - 4 workgroups per tile split K and meet in the workspace
-constexpr int kX16SplitUnit = 128;        // K shares are multiples of this  // 256-wide tile columns, then 192-wide ones (GemmArgs::tail_n)
+constexpr int kX16SplitUnit = 128;        // K shares are multiples of this
+// The summing workgroup's share of `units` K units among `splits` workgroups: an even share and, from eight units
+// each on, one more - a unit takes about 2.2 us, a producer's plane store 3 us (host and device agree through this).
+__host__ __device__ constexpr int x16_split_summing_units(int units, int splits) {
+  return (units + splits - 1) / splits + (units >= 8 * splits ? 1 : 0);
+}
+  // 256-wide tile columns, then 192-wide ones (GemmArgs::tail_n)
 
 // gemm_f64.hip: fp64 products on v_mfma_f64_16x16x4_f64, any strides (c may be null).
 int launch_gemm_f64(const double* a, int64_t a_rs, int64_t a_cs, const double* b, int64_t b_rs, int64_t b_cs, const double* c,

@@ -27,7 +27,10 @@
 // Timing-only ablations for measurement builds (python -m backendbench_amd._build --ablate N, bench.py
 // --only-op C3.mm_down --ablate N): results are wrong, the product library is built with 0.  Bits: 1 no fill
 // requests in the K loop, 2 no barriers, 4 no LDS fragment reads, 8 no wait for the fills, 16 no global
-// stores in the epilogue, 32 no epilogue.
+// stores in the epilogue, 32 no epilogue; split K: 64 producers store no plane, 128 the summing workgroup neither
+// waits nor reads planes, 1024 wall-clock stamps of
+// every workgroup's phases behind the flags (eight 64-bit words per block: entry, K loop done, plane stored /
+// flags seen, end, role, XCC id).
 #ifndef MI355_X16_ABLATE
 #define MI355_X16_ABLATE 0
 #endif
@@ -69,52 +72,58 @@ struct X16Split {
   unsigned long long epoch;
   int role, nprod;
   int spin_limit;  // polls of one flag before the summing workgroup gives up
-  float poison;  // -0 (x + -0 == x), or NaN when a producer never arrived
 };
-constexpr int kX16PartRows = 2;  // rows of accumulator blocks whose plane values are in flight at once (4 blocks of 4 VGPRs each per row)
 // Set by a summing workgroup whose bounded wait ran out (it then writes NaNs into its tile): the launch
 // still reports success, so this word is how the host learns of it (mi355_gemm_status).  Sticky until read.
 static __device__ unsigned int x16_gave_up_word;
 
-// Plane accesses are agent-scope accesses (the sc1 bit on the instruction: relaxed atomics of 8 bytes), not
-// plain ones between agent-scope fences: a fence writes back / invalidates the whole L2 of the XCD, under the
-// feet of the workgroups that are still in their K loops (measured: 89 us instead of 64 for the product it
-// was meant to speed up).  Block (i, j) of wave w: 1 KB at f32x4 index (w * 64 + 8 i + j) * 64, elements 0, 1
-// of the 64 lanes in its first half, elements 2, 3 in the second (512 contiguous bytes per instruction).
-__device__ __forceinline__ void x16_plane_store(f32x4* block, int lane, const f32x4& v) {
-  unsigned long long* q = reinterpret_cast<unsigned long long*>(block) + lane;
-  const float e0 = v[0], e1 = v[1], e2 = v[2], e3 = v[3];  // (a bit cast straight from v[i] reads element 0 for every i)
-  const unsigned long long lo = (unsigned long long)__builtin_bit_cast(uint32_t, e0) | ((unsigned long long)__builtin_bit_cast(uint32_t, e1) << 32);
-  const unsigned long long hi = (unsigned long long)__builtin_bit_cast(uint32_t, e2) | ((unsigned long long)__builtin_bit_cast(uint32_t, e3) << 32);
-  __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(q + 64, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Plane accesses are agent-scope accesses (the sc1 bit on the instruction), not plain ones between agent-scope
+// fences: a fence writes back / invalidates the whole L2 of the XCD, under the feet of the workgroups that
+// are still in their K loops (measured: 89 us instead of 64 for the product it was meant to speed up).
+// They are buffer instructions of 16 bytes per lane (bit 4 of the cache policy operand is sc1), ordered against the flag by
+// the producer's wait for its stores and the summing workgroup's barrier behind the poll.  Block (i, j) of wave
+// w: 1 KB at byte (w * 64 + 8 i + j) * 1024 of the plane, lane l's four values at 16 l (register order).
+constexpr int kX16Sc1 = 1 << 4;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t x16_plane_rsrc(f32x4* planes, int nplanes) {
+  return __builtin_amdgcn_make_buffer_rsrc(planes, 0, nplanes * (BM * BN * 4), 0x00020000);  // raw bytes, bounds-checked
 }
-__device__ __forceinline__ f32x4 x16_plane_load(const f32x4* block, int lane) {
-  const unsigned long long* q = reinterpret_cast<const unsigned long long*>(block) + lane;
-  const unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const unsigned long long hi = __hip_atomic_load(q + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  f32x4 v;
-  v[0] = __builtin_bit_cast(float, (uint32_t)lo);
-  v[1] = __builtin_bit_cast(float, (uint32_t)(lo >> 32));
-  v[2] = __builtin_bit_cast(float, (uint32_t)hi);
-  v[3] = __builtin_bit_cast(float, (uint32_t)(hi >> 32));
-  return v;
+__device__ __forceinline__ void x16_plane_store(__amdgpu_buffer_rsrc_t planes, int block, int lane, const f32x4& v) {
+  if constexpr ((MI355_X16_ABLATE & 64) != 0) return;
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), planes, lane * 16, block * 1024, kX16Sc1);
 }
-// The producers' values of accumulator block (i, j) of this wave, summed (role 0, once the flags are up).
-__device__ __forceinline__ f32x4 x16_split_partial(const X16Split& sk, int wave, int lane, int i, int j) {
-  const f32x4* p = sk.planes + (wave * 64 + i * 8 + j) * 64;
-  f32x4 v = x16_plane_load(p, lane);
-  for (int q = 1; q < sk.nprod; ++q) v += x16_plane_load(p + (size_t)q * 16384, lane);
-  v[0] += sk.poison;
-  return v;
+// The summing workgroup (role 0, once the flags are up) adds the producers' values to its own on the way out, in
+// the epilogue: what the NPROD producers hold for accumulator block (i, j) of this wave, summed.  The epilogue
+// asks for x16_part_rows<NPROD>() rows of a half's blocks at a time - as many as 128 VGPRs hold - and all their
+// loads are issued before the first value is used: the planes come over at the latency of one batch after the
+// other (1.4 us each, measured), so few large batches are what makes the exchange cheap (two rows at a time took
+// 11 us for one plane).  NPROD is a constant: with a run-time count every plane's load is waited for before the
+// next one is issued.  The accumulators stay in the AGPRs until their block's turn (pinned there at the use),
+// which is what leaves the VGPRs free for the values in flight.
+template <int NPROD>
+constexpr int x16_part_rows() { return NPROD <= 1 ? 8 : NPROD == 2 ? 4 : 2; }
+struct X16Planes {
+  __amdgpu_buffer_rsrc_t rsrc;
+  float poison;  // -0 (x + -0 == x), or NaN when a producer never arrived
+};
+template <int NPROD>
+__device__ __forceinline__ f32x4 x16_split_partial(const X16Planes& pl, int wave, int lane, int i, int j) {
+  const int block = (wave * 64 + i * 8 + j) * 1024;
+  f32x4 v[NPROD > 0 ? NPROD : 1];
+#pragma unroll
+  for (int q = 0; q < NPROD; ++q)
+    v[q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(pl.rsrc, lane * 16, block + q * (BM * BN * 4), kX16Sc1));
+#pragma unroll
+  for (int q = 1; q < NPROD; ++q) v[0] += v[q];
+  v[0][0] += pl.poison;
+  return v[0];
 }
 
 // Epilogue: the wave's 128 x 32 NPQ result, 16 NPQ columns at a time, through a 16 KB slab of the idle ring
 // (rows of 128 B, 16-byte slot s of row r at s ^ ((r / 2) % 8)) and out in whole 128-byte rows.
 // Register e of acc[i][j] in lane l is C[m0 + 16 i + l % 16][n0 + 16 j + 4 (l / 16) + e] (operands swapped).
-template <typename T, int NPQ, int RH = 1, bool SPLITK = false>
-__device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32x4 (&acc)[8][2 * NPQ], unsigned char* lds,
-                                                    int wave, int lane, int m0, int n0, const X16Split& sk = X16Split{}) {
+template <typename T, int NPQ, int RH = 1, int NPROD = 0>
+__device__ __forceinline__ void store_tile_result16(const GemmArgs& g, f32x4 (&acc)[8][2 * NPQ], unsigned char* lds,
+                                                    int wave, int lane, int m0, int n0, const X16Planes* pl = nullptr) {
   static_assert(RH == 1 || RH == 2, "the slab holds all 128 rows of the wave's tile or 64 at a time");
   constexpr int IB = 8 / RH;  // row blocks per pass
   const int lr = lane & 15, lg = lane >> 4;
@@ -158,17 +167,19 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
     if constexpr (MODE == 1 && RH != 1) load_bias(y, bias);
     unsigned char* wr = slab + lr * 128 + (lg & 1) * 8;
     const int sx = (lr >> 1) & 7;  // = (row / 2) % 8 for every row 16 i + lr
-    // split K: what the producers hold for kX16PartRows rows of this half's blocks at a time
-    f32x4 part[kX16PartRows][SPLITK ? NPQ : 1];
+    // split K: what the producers hold for PR rows of this half's blocks at a time
+    constexpr bool SPLITK = NPROD > 0;  // the summing workgroup of a K split over NPROD + 1 workgroups
+    constexpr int PR = SPLITK ? x16_part_rows<NPROD>() : 1;
+    f32x4 part[PR][SPLITK ? NPQ : 1];
 #pragma unroll
     for (int ii = 0; ii < IB; ++ii) {
       const int i = rh * IB + ii;
       if constexpr (SPLITK) {
-        if (ii % kX16PartRows == 0) {
+        if (ii % PR == 0) {
 #pragma unroll
-          for (int u = 0; u < kX16PartRows; ++u)
+          for (int u = 0; u < PR; ++u)
 #pragma unroll
-            for (int p = 0; p < NPQ; ++p) part[u][p] = x16_split_partial(sk, wave, lane, i + u, (y ? NPQ : 0) + p);
+            for (int p = 0; p < NPQ; ++p) part[u][p] = x16_split_partial<NPROD>(*pl, wave, lane, i + u, (y ? NPQ : 0) + p);
         }
       }
       const int m = m0 + i * 16 + lr;
@@ -177,8 +188,9 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
       for (int p = 0; p < NPQ; ++p) {
         const int nl = p * 16 + lg * 4;
         const int n = nh + nl;
+        if constexpr (SPLITK) asm volatile("" : "+a"(acc[i][(y ? NPQ : 0) + p]));
         f32x4 v = acc[i][(y ? NPQ : 0) + p];
-        if constexpr (SPLITK) v += part[ii % kX16PartRows][p];
+        if constexpr (SPLITK) v += part[ii % PR][p];
         VecN4<T> r;
         if constexpr (MODE == 0) {
 #pragma unroll
@@ -258,9 +270,9 @@ __device__ __forceinline__ void store_tile_result16(const GemmArgs& g, const f32
 // (16-byte slot s of row r at s ^ (r % 32)) and every store instruction then writes two whole tile rows:
 // three complete lines and the two pieces a row shares with the neighbouring tiles.  Rows at any 2-byte
 // offset (N % 8 != 0) go out along the destination's 16-byte grid (store_slab_rows_shifted).
-template <typename T, bool SPLITK = false>
-__device__ __forceinline__ void store_tile_rows16(const GemmArgs& g, const f32x4 (&acc)[8][8], unsigned char* lds, int wave,
-                                                  int lane, int bm, int bn, const X16Split& sk = X16Split{}) {
+template <typename T, int NPROD = 0>
+__device__ __forceinline__ void store_tile_rows16(const GemmArgs& g, f32x4 (&acc)[8][8], unsigned char* lds, int wave,
+                                                  int lane, int bm, int bn, const X16Planes* pl = nullptr) {
   const int wm = wave >> 1, wn = wave & 1;
   const int lr = lane & 15, lg = lane >> 4;
   const T* C = static_cast<const T*>(g.c);
@@ -288,15 +300,17 @@ __device__ __forceinline__ void store_tile_rows16(const GemmArgs& g, const f32x4
     for (int y = 0; y < 2; ++y) {
       const int nh = bn + wn * 128 + y * 64;
       const float (&bias)[4][4] = bias2[y];
-      f32x4 part[kX16PartRows][SPLITK ? 4 : 1];  // split K: what the producers hold for kX16PartRows rows of this half's blocks at a time
+      constexpr bool SPLITK = NPROD > 0;
+      constexpr int PR = SPLITK ? x16_part_rows<NPROD>() : 1;
+      f32x4 part[PR][SPLITK ? 4 : 1];  // split K: what the producers hold for PR rows of this half's blocks at a time
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if constexpr (SPLITK) {
-          if (i % kX16PartRows == 0) {
+          if (i % PR == 0) {
 #pragma unroll
-            for (int u = 0; u < kX16PartRows; ++u)
+            for (int u = 0; u < PR; ++u)
 #pragma unroll
-              for (int p = 0; p < 4; ++p) part[u][p] = x16_split_partial(sk, wave, lane, i + u, y * 4 + p);
+              for (int p = 0; p < 4; ++p) part[u][p] = x16_split_partial<NPROD>(*pl, wave, lane, i + u, y * 4 + p);
           }
         }
         const int row = wm * 128 + i * 16 + lr;
@@ -306,8 +320,9 @@ __device__ __forceinline__ void store_tile_rows16(const GemmArgs& g, const f32x4
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
           const int n = nh + p * 16 + lg * 4;
+          if constexpr (SPLITK) asm volatile("" : "+a"(acc[i][y * 4 + p]));
           f32x4 v = acc[i][y * 4 + p];
-          if constexpr (SPLITK) v += part[i % kX16PartRows][p];
+          if constexpr (SPLITK) v += part[i % PR][p];
           VecN4<T> r;
           if constexpr (MODE == 0) {
 #pragma unroll
@@ -395,6 +410,8 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave >> 1, wn = wave & 1;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+  [[maybe_unused]] uint64_t st_entry = 0, st_loop = 0, st_met = 0;
+  if constexpr (SPLITK && (MI355_X16_ABLATE & 1024) != 0) st_entry = __builtin_amdgcn_s_memrealtime();
 #ifdef MI355_GEMM_TRACE
   // Diagnostic build only (-DMI355_GEMM_TRACE, libmi355_gemm_trace.so): shader-clock stamps (s_memtime,
   // read behind the next barrier's wait, so no wait is added).  Lane 0 of every wave leaves 16 uint64 in
@@ -751,6 +768,17 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
 #ifdef MI355_GEMM_TRACE
   const uint64_t tr_end = __builtin_readcyclecounter();
 #endif
+  if constexpr (SPLITK && (MI355_X16_ABLATE & 1024) != 0) st_loop = __builtin_amdgcn_s_memrealtime();
+  [[maybe_unused]] auto stamp_out = [&]() {
+    if constexpr ((MI355_X16_ABLATE & 1024) != 0) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (tid == 0) {
+        unsigned long long* o = g.sk_flags + (int64_t)(g.sk_splits - 1) * g.tiles_m * g.tiles_n + 64 + (int64_t)blockIdx.x * 8;
+        o[0] = st_entry; o[1] = st_loop; o[2] = st_met; o[3] = __builtin_amdgcn_s_memrealtime(); o[4] = sk.role;
+        o[5] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (3 << 11));  // HW_REG_XCC_ID
+      }
+    }
+  };
   if constexpr (SPLITK) {
     // Two paths read the accumulators from here on.  Pin them to their AGPRs at this point: without it the
     // compiler copies them out early - between the last MFMA statements, whose wait states it does not know -
@@ -760,15 +788,22 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
 #pragma unroll
       for (int j = 0; j < 2 * NPQ; ++j) asm volatile("" : "+a"(acc[i][j]));
     if (sk.role > 0) {
+      const __amdgpu_buffer_rsrc_t plane = x16_plane_rsrc(sk.planes, 1);
 #pragma unroll
       for (int i = 0; i < 8; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) x16_plane_store(sk.planes + (wave * 64 + i * 8 + j) * 64, lane, acc[i][j]);
+        for (int j = 0; j < 8; ++j) x16_plane_store(plane, wave * 64 + i * 8 + j, lane, acc[i][j]);
       // this wave's stores have completed before the barrier (a workgroup-scope fence leaves the counter
       // alone here, an agent-scope one writes back the whole L2)
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0) __hip_atomic_store(sk.flags, sk.epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if constexpr ((MI355_X16_ABLATE & 1024) != 0) st_met = __builtin_amdgcn_s_memrealtime();
+      stamp_out();
+      return;
+    }
+    if constexpr ((MI355_X16_ABLATE & 128) != 0) {
+      store_tile_result16<T, NPQ>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS);
       return;
     }
     volatile uint32_t* gave_up = reinterpret_cast<volatile uint32_t*>(lds);  // the ring is idle
@@ -786,14 +821,25 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the plane loads stay behind the polls
     __syncthreads();
-    X16Split skc = sk;
-    skc.poison = *gave_up != 0 ? __builtin_nanf("") : -0.f;
+    if constexpr ((MI355_X16_ABLATE & 1024) != 0) st_met = __builtin_amdgcn_s_memrealtime();
+    X16Planes pl;
+    pl.rsrc = x16_plane_rsrc(sk.planes, sk.nprod);
+    pl.poison = *gave_up != 0 ? __builtin_nanf("") : -0.f;
     __syncthreads();  // everyone has read *gave_up: the epilogue reuses the ring
-    if (g.out_rows) store_tile_rows16<T, true>(g, acc, lds, wave, lane, bm, bn, skc);
-    else store_tile_result16<T, NPQ, 1, true>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS, skc);
+    auto finish = [&](auto NPROD_) __attribute__((always_inline)) {
+      constexpr int NPROD = decltype(NPROD_)::value;
+      if constexpr (NPQ == 4) {
+        if (g.out_rows) return store_tile_rows16<T, NPROD>(g, acc, lds, wave, lane, bm, bn, &pl);
+      }
+      store_tile_result16<T, NPQ, 1, NPROD>(g, acc, lds, wave, lane, bm + wm * 128, bn + wn * WCOLS, &pl);
+    };
+    if (sk.nprod == 1) finish(std::integral_constant<int, 1>{});
+    else if (sk.nprod == 2) finish(std::integral_constant<int, 2>{});
+    else finish(std::integral_constant<int, 3>{});  // (the host plans at most four workgroups per tile)
     __syncthreads();  // every wave has read the planes
     if (tid == 0)
       for (int q = 0; q < sk.nprod; ++q) __hip_atomic_store(sk.flags + q, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    stamp_out();
     return;
   }
   if (!(MI355_X16_ABLATE & 32) || g.alpha == 12345.f) {
@@ -833,8 +879,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
 // for workgroups in front of it).  Block t of a group works on tile t; sk_tiles8 is a multiple of 8, so the
 // workgroups of one tile share an XCD and its L2 (blocks go to the XCDs round robin), and blocks past the
 // tile count have nothing to do.  K is shared out in units of 128, the summing workgroup gets the largest
-// share: what it does with the planes only starts when the last producer is done, so a producer should not
-// be the one that finishes its K loop last.
+// share (x16_split_summing_units): what it does with the planes only starts when the last producer has stored
+// its plane, 3 us after its K loop, so the summing workgroup's own K loop should end about then.
 template <typename T, bool B_NN>
 __global__ __launch_bounds__(256) void gemm_mfma_x16_splitk_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -846,7 +892,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_x16_splitk_kernel(GemmArgs g) {
   int tm, tn;
   tile_coords(g.tiles_m, g.tiles_n, t, tm, tn);
   const int units = g.K / kX16SplitUnit;
-  const int cu = (units + S - 1) / S;
+  const int cu = x16_split_summing_units(units, S);
   const int pu = units - cu, pbase = pu / (S - 1), prem = pu % (S - 1);
   int k0 = 0, ku = cu;
   if (role > 0) {

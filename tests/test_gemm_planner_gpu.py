@@ -4,7 +4,7 @@
 (run_gemm in csrc/gemm.hip).  The other GEMM tests force each form with a knob on shapes of their
 choosing; this one walks shapes on both sides of every cut-off the planner itself applies -
 256x256-tile counts 64/65, 96, 128/129, 191/192, 228/229, 248/249, 256/257, K = 256, 384, 1024,
-2048, 3072, M = 16, 64, 512, a right operand under / over 100 MB, tiles three quarters full or
+2048, 3072, 4096 (a few tiles), M = 16, 64, 512, a right operand under / over 100 MB, tiles three quarters full or
 less - and checks whatever the planner chose against the oracle.
 
 Operands are small integers (one in four entries of a non-zero), so every sum is an integer far
@@ -84,6 +84,22 @@ def test_planner_boundaries_in_the_tile_count(backend, grid):
         M = 256 * tm - (40 if ragged else 0)
         N = 256 * tn - (64 if ragged else 0)
         _check(backend, M, K, N, layout, dtype, seed=1000 * tm + 10 * tn + i, with_bias=(i % 2 == 1))
+
+
+# Under half a round of 128x128 tiles the planner also looks at K: 64x64 tiles up to K = 4096 (at exactly 128
+# tiles of 128x128 up to 2048), the 128x128 kernels with K split over the chip beyond.
+_SMALL_GRIDS = [(4, 8), (2, 16), (3, 8), (2, 12), (2, 6)]
+
+
+@pytest.mark.parametrize("grid", _SMALL_GRIDS, ids=[f"{tm}x{tn}={tm * tn}tiles" for tm, tn in _SMALL_GRIDS])
+def test_planner_boundaries_in_k_for_a_few_tiles(backend, grid):
+    tm, tn = grid
+    print(f"\n[gpu-case] planner boundaries in K: {tm} x {tn} tiles of 256x256", flush=True)
+    sys.stdout.flush()
+    for i, K in enumerate([2048, 2112, 3072, 4096, 4160, 8192]):
+        layout = "nt" if (i + tm) % 2 else "nn"
+        dtype = torch.bfloat16 if (i + tn) % 2 == 0 else torch.float16
+        _check(backend, 256 * tm - (24 if i % 3 == 2 else 0), K, 256 * tn, layout, dtype, seed=31 * tm + 7 * tn + i, with_bias=(i % 2 == 0))
 
 
 @pytest.mark.parametrize("M", [15, 16, 17, 63, 64, 65, 200, 180, 511, 512, 513])

@@ -211,8 +211,8 @@ def test_mixed_width_tile_grid(backend, layout, gemm_knobs):
 
 @pytest.mark.parametrize("layout", ["nt", "nn"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_gemm_split_k_inside_one_launch(backend, layout, dtype):
-    """Products with 65 - 128 tiles of 256x256 and K >= 3072: two workgroups per tile take half of K each, one
+def test_gemm_split_k_inside_one_launch(backend, layout, dtype, gemm_knobs):
+    """Products with 65 - 128 tiles of 256x256 and K >= 2048 (3072 above 112 tiles): two workgroups per tile take about half of K each, one
     leaves its fp32 accumulators in the workspace and raises a flag, the other adds them to its own and runs
     the epilogue.  Tile counts at both ends of the range and off the multiples of 8, ragged last tile rows and
     columns, output rows off the 128-byte lines and (transposed b) off the 16-byte units, unit counts of K
@@ -225,13 +225,18 @@ def test_gemm_split_k_inside_one_launch(backend, layout, dtype):
     announce(f"GEMM split K inside one launch, {layout}, {dtype}")
     lib = _lib.load()
     g = torch.Generator().manual_seed(31)
-    shapes = [(2048, 3072, 2304), (2100, 3200, 2500), (3584, 3072, 2048 + 8), (1536, 4224, 2816), (1000, 3072, 5000)]
+    shapes = [(2048, 3072, 2304), (2100, 3200, 2500), (3584, 3072, 2048 + 8), (1536, 4224, 2816), (1000, 3072, 5000),
+              (2048, 2048, 2304), (2100, 2176, 2500)]          # (K at the lower bound; 17 units of K)
     if layout == "nt":
         shapes += [(1792, 3072, 4097), (2304, 3456, 2818)]
-    for M, K, N in shapes:
+    # three and four workgroups per tile (the summing one then reads two or three planes): a knob, at any tile count
+    forced = [("x16split3", 1536, 3200, 1024 + 8), ("x16split4", 700, 4096, 1280), ("x16split4", 2048, 2048 + 128, 2304)]
+    for knob, M, K, N in [(None, *sh) for sh in shapes] + forced:
         tiles = -(-M // 256) * -(-N // 256)
-        assert 64 < tiles <= 128, (M, N, tiles)
-        assert lib.mi355_gemm_workspace_bytes(M, N, K, _lib.dtype_code(dtype)) >= tiles * (256 * 256 * 4 + 8)
+        gemm_knobs.tile(knob)
+        parts = int(knob[-1]) if knob else 2
+        assert knob is not None or 64 < tiles <= 128, (M, N, tiles)
+        assert lib.mi355_gemm_workspace_bytes(M, N, K, _lib.dtype_code(dtype)) >= (parts - 1) * tiles * (256 * 256 * 4 + 8)
         # one in four entries of a is non-zero: every |sum| stays far below 256, exact in bf16 as well
         a = (torch.randint(-1, 2, (M, K), generator=g) * (torch.randint(0, 4, (M, K), generator=g) == 0)).to(dtype).cuda()
         if layout == "nt":
@@ -250,6 +255,7 @@ def test_gemm_split_k_inside_one_launch(backend, layout, dtype):
         assert ev.bit_equal((ref.float() + bias.cpu().float()).to(dtype), out.cpu()), (layout, M, K, N, "bias row")
         out = backend[aten.addmm.default](full, a, b, beta=2, alpha=0.5)
         assert ev.bit_equal((0.5 * ref.float() + 2 * full.cpu().float()).to(dtype), out.cpu()), (layout, M, K, N, "full c")
+    gemm_knobs.tile(None)
     # graph replays: the same launches (same flag value) on the same workspace memory, run after run
     M, K, N = shapes[1]
     a = torch.randint(-1, 2, (M, K), generator=g).to(dtype).cuda()
