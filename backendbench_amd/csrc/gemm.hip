@@ -1993,10 +1993,10 @@ static SplitPlan plan_t64_split(int64_t M, int64_t N, int64_t K) {
 }
 
 // Split-K inside one launch of the 16x16x32 kernel (gemm_mfma_x16_splitk_kernel): for products with 65 - 128
-// tiles of 256x256 (a quarter to half of the CUs) and K >= 2048 (3072 from 113 tiles on), two workgroups per tile,
+// tiles of 256x256 (a quarter to half of the CUs) and K >= 2048 (1536 for 96 - 112 tiles, 3072 from 113 on), two workgroups per tile,
 // each with about half of K.  The caller's workspace holds one fp32 plane of 256 KB per tile and a 64-bit flag per
 // plane.  Measured against one workgroup per tile ([M,K]x[N,K]^T, us; the stock kernel in brackets): 96 tiles at
-// K = 2048 44 -> 40 (33), at 3072 63 -> 50 (47), at 4096 77 -> 60 (58), at 8192 143 -> 97 (106); 128 tiles at K =
+// K = 1536 36.7 -> 34.6 (27.7; the 128x128 kernels 34.7; 72 tiles: 36.0 -> 32.5, the 128x128 kernels 30.4), at K = 2048 44 -> 40 (33), at 3072 63 -> 50 (47), at 4096 77 -> 60 (58), at 8192 143 -> 97 (106); 128 tiles at K =
 // 2048 46 -> 45 (40), at 3072 65 -> 56 (56), at 4096 80 -> 69 (69), at 8192 148 -> 114 (126).  The exchange costs
 // a producer 3 us (its plane, 16 bytes a lane and instruction) and the summing workgroup 4 us on top of its
 // epilogue; a CU takes a plane in at 50 - 60 GB/s, so more workgroups per tile do not pay - the one that sums
@@ -2006,7 +2006,7 @@ struct X16SplitPlan {
   int splits, tiles8;
   int64_t ws_bytes;
 };
-constexpr int64_t kX16SplitMinK = 2048, kX16SplitMinKFull = 3072;
+constexpr int64_t kX16SplitMinK = 2048, kX16SplitMinKMid = 1536, kX16SplitMinKFull = 3072;
 constexpr int kX16MaxSplits = 4;  // the summing workgroup's epilogue exists for one to three producers
 static X16SplitPlan plan_x16_split(int64_t M, int64_t N, int64_t K) {
   X16SplitPlan p{1, 0, 0};
@@ -2017,7 +2017,7 @@ static X16SplitPlan plan_x16_split(int64_t M, int64_t N, int64_t K) {
   if (strncmp(kn.gemm_tile, "x16split", 8) == 0 && kn.gemm_tile[8] >= '2' && kn.gemm_tile[8] <= '0' + kX16MaxSplits && kn.gemm_tile[9] == 0) {
     splits = kn.gemm_tile[8] - '0';  // a test knob: this many workgroups per tile at any tile count
   } else {
-    if (tiles <= kNumCU / 4 || tiles > kNumCU / 2 || K < (tiles <= 112 ? kX16SplitMinK : kX16SplitMinKFull)) return p;
+    if (tiles <= kNumCU / 4 || tiles > kNumCU / 2 || K < (tiles > 112 ? kX16SplitMinKFull : tiles >= 96 ? kX16SplitMinKMid : kX16SplitMinK)) return p;
     splits = 2;
   }
   // every share is at least two units (the kernel's K loop needs 256): the producers share what the summing

@@ -212,7 +212,7 @@ def test_mixed_width_tile_grid(backend, layout, gemm_knobs):
 @pytest.mark.parametrize("layout", ["nt", "nn"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_gemm_split_k_inside_one_launch(backend, layout, dtype, gemm_knobs):
-    """Products with 65 - 128 tiles of 256x256 and K >= 2048 (3072 above 112 tiles): two workgroups per tile take about half of K each, one
+    """Products with 65 - 128 tiles of 256x256 and K >= 2048 (1536 for 96 - 112 tiles, 3072 above): two workgroups per tile take about half of K each, one
     leaves its fp32 accumulators in the workspace and raises a flag, the other adds them to its own and runs
     the epilogue.  Tile counts at both ends of the range and off the multiples of 8, ragged last tile rows and
     columns, output rows off the 128-byte lines and (transposed b) off the 16-byte units, unit counts of K
@@ -226,7 +226,8 @@ def test_gemm_split_k_inside_one_launch(backend, layout, dtype, gemm_knobs):
     lib = _lib.load()
     g = torch.Generator().manual_seed(31)
     shapes = [(2048, 3072, 2304), (2100, 3200, 2500), (3584, 3072, 2048 + 8), (1536, 4224, 2816), (1000, 3072, 5000),
-              (2048, 2048, 2304), (2100, 2176, 2500)]          # (K at the lower bound; 17 units of K)
+              (2048, 2048, 2304), (2100, 2176, 2500),          # (K at the lower bound; 17 units of K)
+              (2048, 1536, 3072)]                              # (96 - 112 tiles: from K = 1536)
     if layout == "nt":
         shapes += [(1792, 3072, 4097), (2304, 3456, 2818)]
     # three and four workgroups per tile (the summing one then reads two or three planes): a knob, at any tile count
