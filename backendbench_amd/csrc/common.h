@@ -22,6 +22,7 @@ int check_launch(const char* what);
 struct Knobs {
   char gemm_tile[16];   // "" = the planner decides; see mi355_set_knob in include/mi355_aten.h
   char gemm_waves[8];   // "" / "4" / "8"
+  char gemm_split[12];  // "" = the planner decides how a split K meets; "launch2" a summing launch, "inlaunch" inside the one launch
   int x16_spin_limit;   // polls of the in-launch split-K's bounded wait before it gives up
 };
 const Knobs& knobs();

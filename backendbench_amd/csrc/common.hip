@@ -99,6 +99,8 @@ extern "C" int mi355_set_knob(const char* name, const char* value) {
     copy_knob(g_knobs.gemm_tile, sizeof(g_knobs.gemm_tile), value);
   } else if (strcmp(name, "gemm_waves") == 0) {
     copy_knob(g_knobs.gemm_waves, sizeof(g_knobs.gemm_waves), value);
+  } else if (strcmp(name, "gemm_split") == 0) {
+    copy_knob(g_knobs.gemm_split, sizeof(g_knobs.gemm_split), value);
   } else if (strcmp(name, "x16_spin_limit") == 0) {
     const long v = (value == nullptr || value[0] == 0) ? kX16SpinLimitDefault : strtol(value, nullptr, 10);
     if (v < 0 || v > (1L << 30)) return set_error(MI355_ERR_INVALID, "mi355_set_knob: x16_spin_limit %ld out of range", v);

@@ -86,6 +86,103 @@ __device__ __forceinline__ void store_partial_tile(const GemmArgs& g, const f32x
   }
 }
 
+// ---- split K inside one launch (the 128x128- and 64x64-tile kernels, SPLIT == 2)
+// blockIdx.y is the part of K, as in the two-launch form.  Parts 0 .. gridDim.y - 2 are producers: each
+// leaves its raw fp32 accumulators in its plane of the workspace (register order: 16-byte piece q of block b
+// of wave w at byte ((w NB + b) 4 + q) 1024 + 16 lane - one `buffer_store_dwordx4 ... sc1` per piece), waits for
+// the stores and raises its 64-bit flag.  The last part sums: it polls the flags (bounded), adds the planes
+// to its own accumulators, sets the flags back to 0 and runs the ordinary epilogue.  Blocks are dispatched
+// in order, x fastest, so a summing workgroup only ever waits for workgroups in front of it, and producers
+// never wait: nothing that shares the chip with the launch can make it wait for a workgroup that has not
+// been dispatched.  Agent-scope accesses (the sc1 bit), not fences: see gemm_x16.hip.  The flag value is the
+// launch's own (GemmArgs::sk_epoch), so stale workspace contents and graph replays are both safe.
+// A plane is NB x 16 KB (64 KB for a 128x128 tile): reading one costs the summing workgroup 1 - 2 us, where
+// a summing launch costs 3 us plus every plane written and read through HBM.
+constexpr int kSc1 = 1 << 4;  // bit 4 of a buffer instruction's cache policy operand
+static __device__ unsigned int insplit_gave_up_word;  // sticky, read and cleared by mi355_gemm_status
+
+template <int NB>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t insplit_rsrc(const GemmArgs& g, int64_t first_plane, int nplanes) {
+  return __builtin_amdgcn_make_buffer_rsrc(g.ws + first_plane * (NB * 4096), 0, nplanes * (NB * 16384), 0x00020000);
+}
+
+template <int MI, int NJ>
+__device__ __forceinline__ void insplit_leave(const GemmArgs& g, const f32x16 (&acc)[MI][NJ], int tid, int wave, int lane) {
+  constexpr int NB = MI * NJ;
+  const int nprod = (int)gridDim.y - 1;
+  const int64_t plane = (int64_t)blockIdx.x * nprod + blockIdx.y;
+  const __amdgpu_buffer_rsrc_t rsrc = insplit_rsrc<NB>(g, plane, 1);
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        f32x4 r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = acc[i][j][q * 4 + e];
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, r), rsrc, lane * 16, ((wave * NB + i * NJ + j) * 4 + q) * 1024, kSc1);
+      }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's plane is out before the barrier
+  __syncthreads();
+  if (tid == 0) __hip_atomic_store(g.sk_flags + plane, g.sk_epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int MI, int NJ>
+__device__ __forceinline__ void insplit_sum(const GemmArgs& g, f32x16 (&acc)[MI][NJ], unsigned char* lds, int tid, int wave, int lane) {
+  constexpr int NB = MI * NJ;
+  const int nprod = (int)gridDim.y - 1;
+  const int64_t first = (int64_t)blockIdx.x * nprod;
+  __syncthreads();  // every wave is past its last LDS read: the ring is idle
+  volatile uint32_t* gave_up = reinterpret_cast<volatile uint32_t*>(lds);
+  if (tid == 0) {
+    uint32_t bad = 0;
+    for (int p = 0; p < nprod; ++p) {
+      int polls = 0;
+      while (__hip_atomic_load(g.sk_flags + first + p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != g.sk_epoch) {
+        if (++polls > g.sk_spin_limit) { bad = 1; break; }
+        __builtin_amdgcn_s_sleep(8);
+      }
+    }
+    *gave_up = bad;
+    if (bad) __hip_atomic_store(&insplit_gave_up_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");  // the plane loads stay behind the polls
+  __syncthreads();
+  const float poison = *gave_up != 0 ? __builtin_nanf("") : -0.f;  // -0: x + -0 == x
+  const __amdgpu_buffer_rsrc_t rsrc = insplit_rsrc<NB>(g, first, nprod);
+  for (int p = 0; p < nprod; ++p) {
+    f32x4 part[NB][4];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        part[b][q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane * 16, p * (NB * 16384) + ((wave * NB + b) * 4 + q) * 1024, kSc1));
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] += part[i * NJ + j][q][e];
+  }
+  acc[0][0][0] += poison;  // NaN marks the tile of a producer that never arrived
+  __syncthreads();  // every wave has used what it read of the planes, and has read *gave_up: the epilogue reuses the ring
+  if (tid == 0)
+    for (int p = 0; p < nprod; ++p) __hip_atomic_store(g.sk_flags + first + p, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The in-launch split's status word for mi355_gemm_status: reads it into *word and clears it when set.
+int read_insplit_status(unsigned int* word) {
+  hipError_t e = hipMemcpyFromSymbol(word, HIP_SYMBOL(insplit_gave_up_word), sizeof(*word));
+  if (e == hipSuccess && *word != 0) {
+    const unsigned int zero = 0;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(insplit_gave_up_word), &zero, sizeof(zero));
+  }
+  return e == hipSuccess ? 0 : (int)e;
+}
+
 // out = alpha * sum over splits of ws + beta * c, four consecutive n per thread.  A group of
 // four columns that starts inside a row may end in its padding (N % 4 != 0): those output rows
 // are misaligned and are stored element by element.
@@ -1129,7 +1226,7 @@ constexpr int kSStage = 2 * kSPanel;              // 16 KB
 constexpr int kSmallLds = kStages3 * kSStage;     // 64 KB
 constexpr int kSmall2Lds = 5 * 2 * SBM * 64 * 2;  // 160 KB: five pairs of (A 128x64 + B 64x128)
 
-template <typename T, bool B_NN, bool SPLIT, bool A_T>
+template <typename T, bool B_NN, int SPLIT, bool A_T>
 __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
   constexpr int S = kStages3;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -1328,15 +1425,22 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing is in flight: the last steps issue no fills)
 
-  if constexpr (SPLIT) store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
-  else store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
+  if constexpr (SPLIT == 1) {
+    store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
+  } else {
+    if constexpr (SPLIT == 2) {  // the parts meet inside this launch: the last one sums and stores
+      if (blockIdx.y + 1 < gridDim.y) return insplit_leave(g, acc, tid, wave, lane);
+      insplit_sum(g, acc, lds, tid, wave, lane);
+    }
+    store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
+  }
 }
 
 // The 128x128 tile for launches with at most one workgroup per CU: nothing else hides a
 // workgroup's barrier, LDS and fill latencies there, so it owns the whole 160 KB of LDS (a ring of
 // five 64-k pairs, every request a whole 128-byte line), works in 64-k steps (16 MFMAs per wave
 // between barriers instead of 8) and reads its fragments a step ahead.
-template <typename T, bool B_NN, bool SPLIT, bool A_T>
+template <typename T, bool B_NN, int SPLIT, bool A_T>
 __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   constexpr int S = 5;  // ring depth in 64-k pairs
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -1530,8 +1634,15 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing is in flight: the last steps issue no fills)
 
-  if constexpr (SPLIT) store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
-  else store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
+  if constexpr (SPLIT == 1) {
+    store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
+  } else {
+    if constexpr (SPLIT == 2) {  // the parts meet inside this launch: the last one sums and stores
+      if (blockIdx.y + 1 < gridDim.y) return insplit_leave(g, acc, tid, wave, lane);
+      insplit_sum(g, acc, lds, tid, wave, lane);
+    }
+    store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
+  }
 }
 
 // ---------------------------------------------------------------- MFMA kernel, 64x64 tiles
@@ -1555,7 +1666,7 @@ __device__ __forceinline__ int swz_n64(int k, int u) {
 
 // SPLIT: blockIdx.y owns the k range [blockIdx.y * ksplit, + ksplit) (whole 64-k stages) and leaves its raw fp32
 // tile in plane blockIdx.y of the workspace, as the 128x128 kernels do; gemm_splitk_finish_kernel sums the planes.
-template <typename T, bool B_NN, int S, bool SPLIT = false>
+template <typename T, bool B_NN, int S, int SPLIT = 0>
 __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using frag_t = typename Mfma<T>::frag;
@@ -1655,9 +1766,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
   }
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[0][0][e] += acc_odd[e];
-  if constexpr (SPLIT) {
+  if constexpr (SPLIT == 1) {
     store_partial_tile<1, 1>(g, acc, lane, bm + wm * 32, bn + wn * 32);
     return;
+  }
+  if constexpr (SPLIT == 2) {  // the parts meet inside this launch: the last one sums and stores
+    if (blockIdx.y + 1 < gridDim.y) return insplit_leave(g, acc, tid, wave, lane);
+    insplit_sum(g, acc, lds, tid, wave, lane);
   }
   __syncthreads();  // the ring becomes the epilogue's staging area
   store_tile_result<T, 1, 0, 1>(g, acc, lds, wave, lane, bm + wm * 32, bn + wn * 32);
@@ -1927,7 +2042,32 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const T* __restrict__
 // (>= 4 when the output is one or two tiles).
 struct SplitPlan {
   int nsplit, ksplit;
+  int mode;  // how the parts meet: 1 in a summing launch, 2 inside the one launch (insplit_sum; bf16 / f16 only)
 };
+// What the meeting costs, in ns, on top of the longest part's K loop.  A summing launch: 3 us and every plane
+// written and read once at ~4 TB/s.  Inside the launch: the producers' planes go out in ~1.5 us, and the summing
+// workgroup takes them in one after the other, 64 KB (a 128x128 tile: ~1.3 us) or 16 KB (64x64: ~0.9 us) each.
+static double split_meet_ns(int mode, int64_t ns, int64_t M, int64_t N, int tile) {
+  if (ns <= 1) return 0.0;
+  if (mode == 2) return 1500.0 + (tile == 64 ? 900.0 : 1300.0) * (double)(ns - 1);
+  return 3000.0 + (double)ns * (double)M * (double)N * 8.0 / 4000.0;  // 4 TB/s = 4000 B/ns
+}
+// The modes the plan may choose from: both for bf16 / f16 unless the gemm_split knob names one.
+static void split_modes(int elem_size, bool (&allowed)[3]) {
+  const Knobs& kn = knobs();
+  allowed[1] = elem_size == 4 || strcmp(kn.gemm_split, "inlaunch") != 0;
+  allowed[2] = elem_size == 2 && strcmp(kn.gemm_split, "launch2") != 0;
+}
+// Workspace a plan needs: planes of whole rows (a summing launch), or (nsplit - 1) planes of whole tiles and a
+// 64-bit flag each (inside the launch).
+static int64_t split_ws_bytes(const SplitPlan& p, int64_t M, int64_t N, int tile) {
+  if (p.nsplit <= 1) return 0;
+  if (p.mode == 2) {
+    const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
+    return (int64_t)(p.nsplit - 1) * tiles * ((int64_t)tile * tile * 4 + 8);
+  }
+  return (int64_t)p.nsplit * M * ((N + 3) / 4 * 4) * 4;
+}
 // fp32 products that leave most CUs without a 128x128 tile run on 64x64 tiles.
 static int f32_tile(int64_t M, int64_t N) {
   return ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN) < kNumCU * 3 / 4 ? 64 : 128;
@@ -1936,13 +2076,16 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   const int bk = elem_size == 4 ? FBK : BK3;
   const int tile = elem_size == 4 ? f32_tile(M, N) : SBM;
   const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
-  SplitPlan p{1, (int)K};
+  SplitPlan p{1, (int)K, 1};
   if (tiles >= kNumCU || K % bk != 0) return p;
   const double ns_per_k = elem_size == 4 ? (tile == 64 ? 20.0 : 70.0) : 12.8;
   const int min_steps = tiles <= 2 ? 4 : 8;  // one or two tiles: the launch is all latency, shorter splits still pay
   const int64_t max_ns = K / (min_steps * bk) < 64 ? K / (min_steps * bk) : 64;
-  double best = 0;
+  bool allowed[3];
+  split_modes(elem_size, allowed);
+  double best = 1e30;
   int64_t best_ns = 1;
+  int best_mode = 1;
   for (int64_t ns = 1; ns <= max_ns; ++ns) {
     int64_t ks = (K + ns - 1) / ns;
     ks = (ks + bk - 1) / bk * bk;
@@ -1950,11 +2093,18 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
     if (real_ns != ns) continue;  // this count rounds to one already tried
     if (K - (ns - 1) * ks < (int64_t)min_steps * bk) continue;  // the last split would fall under the minimum
     const int64_t per_cu = (tiles * ns + kNumCU - 1) / kNumCU;
-    double t = (double)per_cu * (per_cu >= 2 ? 0.7 : 1.0) * (double)ks * ns_per_k;
-    if (ns > 1) t += 3000.0 + (double)ns * (double)M * (double)N * 8.0 / 4000.0;  // ns; 4 TB/s = 4000 B/ns
-    if (ns == 1 || t < best) {
+    const double t_k = (double)per_cu * (per_cu >= 2 ? 0.7 : 1.0) * (double)ks * ns_per_k;
+    if (ns == 1) {  // the unsplit product: what a split has to beat
+      best = t_k;
+      continue;
+    }
+    // The part count is chosen against the summing launch's cost, which is what the K-loop figures above were
+    // fitted with; the parts then meet whichever way is cheaper for that count.
+    const double t = t_k + split_meet_ns(1, ns, M, N, tile);
+    if (t < best) {
       best = t;
       best_ns = ns;
+      best_mode = allowed[2] && (!allowed[1] || split_meet_ns(2, ns, M, N, tile) < split_meet_ns(1, ns, M, N, tile)) ? 2 : 1;
     }
   }
   if (best_ns <= 1) return p;
@@ -1962,6 +2112,7 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   ks = (ks + bk - 1) / bk * bk;
   p.ksplit = (int)ks;
   p.nsplit = (int)((K + ks - 1) / ks);
+  p.mode = best_mode;
   return p;
 }
 
@@ -1970,25 +2121,34 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
 // least four each; the cost model is the one of plan_splitk with this kernel's figures (2 us to get going,
 // 0.3 us per stage, 1.3 x that with two workgroups on a CU, 3 us and the partial planes for the summing launch).
 static SplitPlan plan_t64_split(int64_t M, int64_t N, int64_t K) {
-  SplitPlan p{1, (int)K};
+  SplitPlan p{1, (int)K, 1};
   const int64_t tiles = ((M + TBM - 1) / TBM) * ((N + TBN - 1) / TBN);
   if (K % 64 != 0 || K < 1024 || tiles > kNumCU / 2) return p;
   const int64_t stages = K / 64;
-  double best = 0;
+  bool allowed[3];
+  split_modes(2, allowed);
+  double best = 1e30;
   int64_t best_ks = stages;
+  int best_mode = 1;
   for (int64_t ns = 1; ns <= stages / 4 && ns <= 64; ++ns) {
     const int64_t ks = (stages + ns - 1) / ns;
     if ((stages + ks - 1) / ks != ns || stages - (ns - 1) * ks < 4) continue;
     const int64_t per_cu = (tiles * ns + kNumCU - 1) / kNumCU;
-    double t = 2000.0 + 300.0 * (double)ks * (per_cu >= 2 ? 1.3 * (double)((per_cu + 1) / 2) : 1.0);
-    if (ns > 1) t += 3000.0 + (double)ns * (double)M * (double)N * 8.0 / 4000.0;
-    if (ns == 1 || t < best) {
+    const double t_k = 2000.0 + 300.0 * (double)ks * (per_cu >= 2 ? 1.3 * (double)((per_cu + 1) / 2) : 1.0);
+    if (ns == 1) {  // the unsplit product: what a split has to beat
+      best = t_k;
+      continue;
+    }
+    const double t = t_k + split_meet_ns(1, ns, M, N, 64);  // (part count against the summing launch, as in plan_splitk)
+    if (t < best) {
       best = t;
       best_ks = ks;
+      best_mode = allowed[2] && (!allowed[1] || split_meet_ns(2, ns, M, N, 64) < split_meet_ns(1, ns, M, N, 64)) ? 2 : 1;
     }
   }
   p.ksplit = (int)(best_ks * 64);
   p.nsplit = (int)((stages + best_ks - 1) / best_ks);
+  p.mode = p.nsplit > 1 ? best_mode : 1;
   return p;
 }
 
@@ -2094,6 +2254,13 @@ static int finish_splitk(const GemmArgs& g, int nsplit, hipStream_t st) {
   return check_launch("mi355_gemm(split-k finish)");
 }
 
+// A flag value of its own for every launch whose workgroups meet through flags in the workspace: odd, and
+// stepped by two - never 0, which is what a flag holds between launches.
+static unsigned long long next_split_epoch() {
+  static std::atomic<unsigned long long> epoch{0x5bd1e9955bd1e995ull};
+  return epoch.fetch_add(2);
+}
+
 template <typename T>
 static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs,
                     const void* c, int64_t c_rs, int64_t c_cs, void* out, int64_t M, int64_t N, int64_t K,
@@ -2143,8 +2310,17 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         if (a_t) return b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, NJ, true> : (const void*)gemm_mfma_w4_kernel<T, true, NJ, true>;
         return b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, NJ, false> : (const void*)gemm_mfma_w4_kernel<T, true, NJ, false>;
       };
+      // The parts of a split K meet inside the launch (SplitPlan::mode 2): planes of whole tiles at the start of the
+      // workspace, one flag per plane behind them.
+      bool meet_inside = false;
+      auto arm_insplit = [&](int64_t tiles, int tile) {
+        meet_inside = true;
+        g.sk_flags = reinterpret_cast<unsigned long long*>(static_cast<unsigned char*>(workspace) + (int64_t)(nsplit - 1) * tiles * tile * tile * 4);
+        g.sk_epoch = next_split_epoch();
+        g.sk_spin_limit = knobs().x16_spin_limit;
+      };
       auto pick_small = [&](auto deep, auto split_c) -> const void* {
-        constexpr bool SP = decltype(split_c)::value;
+        constexpr int SP = decltype(split_c)::value;
         if constexpr (decltype(deep)::value) {
           if (a_t) return b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, SP, true> : (const void*)gemm_mfma_small2_kernel<T, true, SP, true>;
           return b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, SP, false> : (const void*)gemm_mfma_small2_kernel<T, true, SP, false>;
@@ -2182,7 +2358,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool light_b = (int64_t)N * K * (int64_t)sizeof(T) <= 100000000;
       const bool t64_split = ts.nsplit > 1 && M >= 16 && light_b && workspace != nullptr &&
                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
-                             workspace_bytes >= (int64_t)ts.nsplit * M * ((N + 3) / 4 * 4) * 4;
+                             workspace_bytes >= split_ws_bytes(ts, M, N, TBM);
       const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
                                                : (nb128 < kNumCU / 2 || (nb128 == kNumCU / 2 && K <= 2048) ||  // (exactly 128 tiles, [1024,2048]x[2048,2048]: 26.4 -> 21.2 us, K = 512: 10.0 -> 7.0; level at K = 3072, behind from 4096 on)
@@ -2223,14 +2399,13 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                              (forced_tile != nullptr ? strncmp(forced_tile, "x16split", 8) == 0
                                                      : x16_pays && M >= 512 && forced_waves == nullptr);  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
       if (x16_split) {
-        static std::atomic<unsigned long long> epoch{0x5bd1e9955bd1e995ull};  // odd, and stepped by two: odd for ever
         kern = gemm_x16_splitk_kernel(std::is_same<T, bf16_t>::value, !b_nt);
         threads = 256;
         lds_bytes = kX16Lds;
         g.ws = static_cast<float*>(workspace);
         g.sk_splits = xs.splits;
         g.sk_tiles8 = xs.tiles8;
-        g.sk_epoch = epoch.fetch_add(2);  // a value of its own per launch, never 0 (a flag is 0 between launches)
+        g.sk_epoch = next_split_epoch();
         g.sk_spin_limit = kn.x16_spin_limit;
         g.sk_flags = reinterpret_cast<unsigned long long*>(static_cast<unsigned char*>(workspace) + (int64_t)(xs.splits - 1) * nblocks * (BM * BN * 4));
         g.out_rows = N % 64 != 0 || reinterpret_cast<uintptr_t>(out) % 128 != 0;
@@ -2292,12 +2467,16 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
           g.ws = static_cast<float*>(workspace);
           g.ksplit = ts.ksplit;
           g.ws_ld = (int32_t)((N + 3) / 4 * 4);
+          if (ts.mode == 2) arm_insplit(nblocks, TBM);
         }
         const bool deep = nblocks * nsplit <= kNumCU;
         lds_bytes = (deep ? 8 : 4) * kTStage;
-        if (nsplit > 1) {
-          if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8, true> : (const void*)gemm_mfma_t64_kernel<T, true, 8, true>;
-          else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4, true> : (const void*)gemm_mfma_t64_kernel<T, true, 4, true>;
+        if (nsplit > 1 && meet_inside) {
+          if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8, 2> : (const void*)gemm_mfma_t64_kernel<T, true, 8, 2>;
+          else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4, 2> : (const void*)gemm_mfma_t64_kernel<T, true, 4, 2>;
+        } else if (nsplit > 1) {
+          if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8, 1> : (const void*)gemm_mfma_t64_kernel<T, true, 8, 1>;
+          else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4, 1> : (const void*)gemm_mfma_t64_kernel<T, true, 4, 1>;
         } else {
           if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8> : (const void*)gemm_mfma_t64_kernel<T, true, 8>;
           else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4> : (const void*)gemm_mfma_t64_kernel<T, true, 4>;
@@ -2317,18 +2496,22 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         const SplitPlan sp = plan_splitk(M, N, K, sizeof(T));
         const int64_t ws_ld = (N + 3) / 4 * 4;
         const bool split = sp.nsplit > 1 && workspace != nullptr &&
-                           workspace_bytes >= (int64_t)sp.nsplit * M * ws_ld * 4 && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+                           workspace_bytes >= split_ws_bytes(sp, M, N, SBM) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
         if (split) {
           nsplit = sp.nsplit;
           g.ws = static_cast<float*>(workspace);
           g.ksplit = sp.ksplit;
           g.ws_ld = (int32_t)ws_ld;
+          if (sp.mode == 2) arm_insplit(nblocks, SBM);
         }
         // At most one workgroup per CU and whole 64-k pairs per split: the deep-ring kernel.
         const bool pairs = nblocks * nsplit <= kNumCU && K % 64 == 0 && (!split || sp.ksplit % 64 == 0);
         lds_bytes = pairs ? kSmall2Lds : kSmallLds;
-        if (pairs) kern = split ? pick_small(std::true_type{}, std::true_type{}) : pick_small(std::true_type{}, std::false_type{});
-        else kern = split ? pick_small(std::false_type{}, std::true_type{}) : pick_small(std::false_type{}, std::false_type{});
+        using M0 = std::integral_constant<int, 0>;
+        using M1 = std::integral_constant<int, 1>;
+        using M2 = std::integral_constant<int, 2>;
+        if (pairs) kern = !split ? pick_small(std::true_type{}, M0{}) : meet_inside ? pick_small(std::true_type{}, M2{}) : pick_small(std::true_type{}, M1{});
+        else kern = !split ? pick_small(std::false_type{}, M0{}) : meet_inside ? pick_small(std::false_type{}, M2{}) : pick_small(std::false_type{}, M1{});
         threads = 256;
       } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
@@ -2378,7 +2561,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks, (unsigned)nsplit), dim3(threads), params, lds_bytes, st);
       if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma): launch failed: %s", hipGetErrorString(e));
       const int rc = check_launch("mi355_gemm(mfma)");
-      if (rc || nsplit == 1) return rc;
+      if (rc || nsplit == 1 || meet_inside) return rc;
       return finish_splitk<T>(g, nsplit, st);
     }
   }
@@ -2517,8 +2700,8 @@ static int run_gemm_f32out(const void* a, int64_t a_rs, int64_t a_cs, const void
   const bool pairs = nblocks <= kNumCU && K % 64 == 0;  // at most one workgroup per CU: the deep-ring kernel
   const int lds_bytes = pairs ? kSmall2Lds : kSmallLds;
   const void* kern;
-  if (pairs) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, true, false> : (const void*)gemm_mfma_small2_kernel<T, true, true, false>;
-  else kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, true, false> : (const void*)gemm_mfma_small_kernel<T, true, true, false>;
+  if (pairs) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, 1, false> : (const void*)gemm_mfma_small2_kernel<T, true, 1, false>;
+  else kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, 1, false> : (const void*)gemm_mfma_small_kernel<T, true, 1, false>;
   hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   if (e != hipSuccess)
     return set_error(MI355_ERR_LAUNCH, "mi355_gemm_f32out: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
@@ -2544,10 +2727,9 @@ extern "C" int64_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, i
   if (M <= 0 || N <= 0 || K <= 0 || (es != 2 && es != 4)) return 0;
   if (dtype != MI355_BF16 && dtype != MI355_F16 && dtype != MI355_F32) return 0;
   const SplitPlan p = plan_splitk(M, N, K, es);
-  int64_t two_launch = p.nsplit > 1 ? (int64_t)p.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
+  int64_t two_launch = split_ws_bytes(p, M, N, es == 4 ? f32_tile(M, N) : SBM);  // (either way of meeting)
   if (es == 2) {  // the 64x64-tile kernel's own split
-    const SplitPlan t = plan_t64_split(M, N, K);
-    const int64_t t64 = t.nsplit > 1 ? (int64_t)t.nsplit * M * ((N + 3) / 4 * 4) * 4 : 0;
+    const int64_t t64 = split_ws_bytes(plan_t64_split(M, N, K), M, N, TBM);
     two_launch = t64 > two_launch ? t64 : two_launch;
   }
   const int64_t one_launch = es == 2 ? plan_x16_split(M, N, K).ws_bytes : 0;

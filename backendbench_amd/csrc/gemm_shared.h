@@ -174,6 +174,10 @@ __host__ __device__ constexpr int x16_split_summing_units(int units, int splits)
 }
   // 256-wide tile columns, then 192-wide ones (GemmArgs::tail_n)
 
+// gemm.hip: the status word of the in-launch split K of the 128x128- and 64x64-tile kernels, read into *word and
+// cleared when set; a HIP error code, 0 on success.
+int read_insplit_status(unsigned int* word);
+
 // gemm_f64.hip: fp64 products on v_mfma_f64_16x16x4_f64, any strides (c may be null).
 int launch_gemm_f64(const double* a, int64_t a_rs, int64_t a_cs, const double* b, int64_t b_rs, int64_t b_cs, const double* c,
                     int64_t c_rs, int64_t c_cs, double* out, int64_t M, int64_t N, int64_t K, double alpha, double beta,

@@ -964,13 +964,17 @@ const void* gemm_x16_mixed_kernel(bool is_bf16, bool b_nn) {
 }  // namespace mi355
 
 extern "C" int mi355_gemm_status(void) {
-  unsigned int word = 0;
+  unsigned int word = 0, word2 = 0;
   hipError_t e = hipMemcpyFromSymbol(&word, HIP_SYMBOL(mi355::x16_gave_up_word), sizeof(word));
   if (e != hipSuccess) return mi355::set_error(MI355_ERR_LAUNCH, "mi355_gemm_status: reading the status word failed: %s", hipGetErrorString(e));
-  if (word == 0) return MI355_OK;
-  const unsigned int zero = 0;
-  e = hipMemcpyToSymbol(HIP_SYMBOL(mi355::x16_gave_up_word), &zero, sizeof(zero));
-  if (e != hipSuccess) return mi355::set_error(MI355_ERR_LAUNCH, "mi355_gemm_status: clearing the status word failed: %s", hipGetErrorString(e));
+  if (word != 0) {
+    const unsigned int zero = 0;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(mi355::x16_gave_up_word), &zero, sizeof(zero));
+    if (e != hipSuccess) return mi355::set_error(MI355_ERR_LAUNCH, "mi355_gemm_status: clearing the status word failed: %s", hipGetErrorString(e));
+  }
+  const int e2 = mi355::read_insplit_status(&word2);  // the 128x128- and 64x64-tile kernels' word (gemm.hip)
+  if (e2 != 0) return mi355::set_error(MI355_ERR_LAUNCH, "mi355_gemm_status: reading the status word failed: %s", hipGetErrorString((hipError_t)e2));
+  if (word == 0 && word2 == 0) return MI355_OK;
   return mi355::set_error(MI355_ERR_LAUNCH,
                           "mi355_gemm: a split-K launch gave up waiting for a partial product (its output tile holds NaNs)");
 }

@@ -37,6 +37,9 @@ class _GemmKnobs:
     def waves(self, value):
         self._set("gemm_waves", value)
 
+    def split(self, value):
+        self._set("gemm_split", value)
+
     def spin_limit(self, value):
         self._set("x16_spin_limit", value)
 

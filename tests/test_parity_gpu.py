@@ -549,6 +549,66 @@ def test_split_k_on_64x64_tiles(backend, dtype, gemm_knobs):
                 assert ev.bit_equal((0.5 * ref.float() + 2 * full.cpu().float()).to(dtype), out.cpu()), (forced, M, N, K, nt, "full c")
 
 
+@pytest.mark.parametrize("meet", ["inlaunch", "launch2"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_split_k_parts_meet_either_way(backend, dtype, meet, gemm_knobs):
+    """The parts of a K split on the 128x128- and 64x64-tile kernels meet in a summing launch or inside the one
+    launch (the last part polls the others' flags, adds their planes and runs the epilogue): the planner picks
+    per shape, the gemm_split knob forces one.  Shapes for the 64x64 tiles, the two-per-CU and the deep-ring 128x128
+    kernels, part counts from 2 to dozens, ragged tiles and K ranges, both layouts of b, the three epilogues.
+    Small-integer operands: bit-equal to the oracle either way.  Then a HIP graph of in-launch products is replayed
+    with eager work in between: the flags must be back at zero after every run."""
+    from backendbench_amd import _lib
+    announce(f"split-K parts meet {meet}, {dtype}")
+    lib = _lib.load()
+    gemm_knobs.split(meet)
+    g = torch.Generator().manual_seed(47)
+    shapes = [(1536, 2048, 4096), (1024, 2048, 4160), (512, 768, 3072), (197, 768, 3072), (128, 4096, 4096), (64, 64, 4000),
+              (100, 70, 928), (1000, 1752, 2112), (256, 1024, 8192), (16, 4096, 4096), (700, 900, 2048)]
+    split_seen = 0
+    for M, N, K in shapes:
+        split_seen += lib.mi355_gemm_workspace_bytes(M, N, K, _lib.dtype_code(dtype)) > 0
+        for nt in (True, False):
+            if not nt and N % 8:
+                continue
+            a = (torch.randint(-1, 2, (M, K), generator=g) * (torch.randint(0, 4, (M, K), generator=g) == 0)).to(dtype).cuda()
+            b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t() if nt else torch.randint(-1, 2, (K, N), generator=g).to(dtype).cuda()
+            bias = torch.randint(-2, 3, (N,), generator=g).to(dtype).cuda()
+            full = torch.randint(-2, 3, (M, N), generator=g).to(dtype).cuda()
+            ref = aten_cpu.reference(aten.mm.default, [a.float(), b.float()])
+            assert float(ref.abs().max()) <= 192
+            ref = ref.to(dtype)
+            assert ev.bit_equal(ref, backend[aten.mm.default](a, b).cpu()), (meet, M, N, K, nt)
+            out = backend[aten.addmm.default](bias, a, b)
+            assert ev.bit_equal((ref.float() + bias.cpu().float()).to(dtype), out.cpu()), (meet, M, N, K, nt, "bias row")
+            out = backend[aten.addmm.default](full, a, b, beta=2, alpha=0.5)
+            assert ev.bit_equal((0.5 * ref.float() + 2 * full.cpu().float()).to(dtype), out.cpu()), (meet, M, N, K, nt, "full c")
+    assert split_seen >= 9, "these shapes are meant to split K"
+    assert lib.mi355_gemm_status() == 0
+    if meet != "inlaunch":
+        return
+    M, N, K = 1536, 2048, 4096
+    a = torch.randint(-1, 2, (M, K), generator=g).to(dtype).cuda()
+    a2 = torch.randint(-1, 2, (M, K), generator=g).to(dtype).cuda()
+    b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t()
+    want, want2 = backend[aten.mm.default](a, b), backend[aten.mm.default](a2, b)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got = backend[aten.mm.default](a, b)
+        got2 = backend[aten.mm.default](a2, b)
+    for rep in range(4):
+        got.zero_()
+        got2.zero_()
+        junk = torch.full((64 << 20,), float(rep), device="cuda")   # eager work that may land on the freed workspace
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert ev.bit_equal(want, got) and ev.bit_equal(want2, got2), ("replay", rep)
+        del junk
+    assert lib.mi355_gemm_status() == 0
+
+
 def test_f64_addmm_keeps_alpha_and_beta_in_f64(backend):
     """alpha = 0.1 and beta = 0.3 are not fp32 numbers: an f64 addmm must apply them in f64 (1e-12
     against the oracle, where an fp32 round trip of the scalars leaves 1e-8), and a beta too small for

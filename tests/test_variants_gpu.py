@@ -408,6 +408,51 @@ def test_split_k_gives_up_cleanly_and_the_next_launch_is_unharmed(gemm_knobs):
         assert lib.mi355_gemm_status() == 0 and ev.bit_equal(ref, out.cpu())
 
 
+def test_split_k_inside_the_launch_gives_up_and_recovers_on_128x128_tiles(gemm_knobs):
+    """The same bounded wait on the 128x128-tile kernels' in-launch split (four parts here): with a poll limit of
+    0 a summing workgroup whose producers are not done yet writes NaNs and sets the status word; every kernel
+    still runs to its end, tiles that were not given up are exact, and later launches on the same workspace -
+    late flags of the abandoned tiles still in it - are exact again."""
+    print("\n[gpu-case] in-launch split K on 128x128 tiles: give-up path", flush=True)
+    sys.stdout.flush()
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(12)
+    M, K, N = 1024, 8192, 2048
+    dtype = torch.bfloat16
+    code = _lib.dtype_code(dtype)
+    gemm_knobs.split("inlaunch")
+    need = lib.mi355_gemm_workspace_bytes(M, N, K, code)
+    assert need > 0
+    a = (torch.randint(-1, 2, (M, K), generator=g) * (torch.randint(0, 8, (M, K), generator=g) == 0)).to(dtype).cuda()
+    b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t()
+    ref = aten_cpu.reference(aten.mm.default, [a.float(), b.float()]).to(dtype)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    out = torch.empty(M, N, dtype=dtype, device="cuda")
+
+    def launch():
+        _lib.check(lib.mi355_gemm(a.data_ptr(), a.stride(0), a.stride(1), b.data_ptr(), b.stride(0), b.stride(1), None, 0, 0,
+                                  out.data_ptr(), M, N, K, 1.0, 0.0, code, ws.data_ptr(), need, _lib.current_stream_handle()))
+        torch.cuda.synchronize()
+
+    launch()
+    assert lib.mi355_gemm_status() == 0 and ev.bit_equal(ref, out.cpu())
+    gemm_knobs.spin_limit(0)
+    launch()
+    gave_up = bool(torch.isnan(out).any())
+    rc = lib.mi355_gemm_status()
+    assert (rc != 0) == gave_up, "the status word must tell exactly when a tile was given up"
+    if gave_up:
+        assert b"gave up" in lib.mi355_last_error()
+        assert lib.mi355_gemm_status() == 0, "reading the word clears it"
+        clean = ~torch.isnan(out)
+        assert ev.bit_equal(ref[clean.cpu()], out[clean].cpu()), "tiles that were not given up are exact"
+    gemm_knobs.spin_limit(None)
+    for _ in range(3):
+        out.fill_(5)
+        launch()
+        assert lib.mi355_gemm_status() == 0 and ev.bit_equal(ref, out.cpu())
+
+
 def test_set_knob_rejects_unknown_names():
     lib = _lib.load()
     assert lib.mi355_set_knob(b"no_such_knob", b"1") == -1 and b"unknown knob" in lib.mi355_last_error()
