@@ -520,6 +520,9 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
   // couples.  Back-to-back MFMAs on one accumulator block need no wait states; nothing else reads the
   // accumulators before the epilogue.
   auto mfma2 = [&](f32x4& c, const frag_t& b0, const frag_t& a0, const frag_t& b1, const frag_t& a1) __attribute__((always_inline)) {
+    if constexpr ((MI355_X16_ABLATE & 2048) != 0) {  // no MFMAs: the operands are still waited for
+      asm volatile("" : "+a"(c) : "v"(__builtin_bit_cast(u32x4, b0)), "v"(__builtin_bit_cast(u32x4, a0)), "v"(__builtin_bit_cast(u32x4, b1)), "v"(__builtin_bit_cast(u32x4, a1)) : "memory");
+    } else
     if constexpr (std::is_same<T, bf16_t>::value)
       asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tv_mfma_f32_16x16x32_bf16 %0, %3, %4, %0"
                    : "+a"(c)
