@@ -1645,6 +1645,207 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   }
 }
 
+// The deep-ring 128x128 kernel with the fills taken out of the computing waves' instruction streams: eight
+// waves, two per SIMD.  Waves 0 - 3 compute as in gemm_mfma_small2_kernel (fragments of pair p + 1 read during
+// step p, sixteen MFMAs per step) and never touch global memory in the K loop; waves 4 - 7 ("loaders") issue
+// every fill request - wave 4 + w the regions that wave w fills in the four-wave form - wait for them
+// (s_waitcnt vmcnt) and meet the others at the one barrier per step.  Why: a CU takes fills in at about 80 GB/s,
+// which is what a 128x128 tile asks for (32 KB per 64-k step of 0.4 us); at that rate the memory pipeline
+// pushes back, a wave stalls at its next request, and on a SIMD with a single wave the MFMAs behind the
+// request wait with it - fills and MFMAs took turns instead of overlapping (measured on [2048,4096]x
+// [2048,4096]^T, ns per k: 12.5 as built, 6.4 without the fills, 6.3 with the fills alone).  A loader stalls
+// alone.  The loaders end after the last step's barrier; s_barrier counts the waves that are left, so the
+// epilogue's barriers (the in-launch split's exchange) are met by the four computing waves only.
+template <typename T, bool B_NN, int SPLIT, bool A_T>
+__global__ __launch_bounds__(512) void gemm_mfma_small3_kernel(GemmArgs g) {
+  constexpr int S = 5;  // ring depth in 64-k pairs
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  using frag_t = typename Mfma<T>::frag;
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave8 = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const bool loader = wave8 >= 4;
+  const int wave = wave8 & 3;
+  const int wm = wave >> 1, wn = wave & 1;
+  int tm, tn;
+  tile_coords(g, tm, tn);
+  const int bm = tm * SBM, bn = tn * SBN;
+  const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
+  const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
+  const int np = (kend - kbeg) / (2 * BK3);
+  constexpr int kPairPanel = SBM * 64 * 2;  // 16 KB
+  constexpr int kPairSlot = 2 * kPairPanel;
+
+  if (loader) {
+    const T* A = static_cast<const T*>(g.a) + (A_T ? (int64_t)kbeg * g.lda : (int64_t)kbeg);
+    const T* B = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+    // Region q = wave + 4 i (i < 4) of a panel is its bytes [1024 q, 1024 q + 1024); layouts as in the
+    // four-wave form (swz_k64 rows for a K-contiguous operand, swz_n128 k-rows otherwise).
+    const T* a_src[4];
+    const T* b_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int q = wave + 4 * i;
+      const int r = 8 * q + (lane >> 3), slot = lane & 7;
+      const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
+      if constexpr (A_T) {
+        const int k = 4 * q + (lane >> 4), pos = lane & 15;
+        const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+        int gm = bm + u * 8;
+        gm = gm < g.M ? gm : 0;
+        a_src[i] = A + (int64_t)k * g.lda + gm;
+      } else {
+        int gr = bm + r;
+        gr = gr < g.M ? gr : g.M - 1;
+        a_src[i] = A + (int64_t)gr * g.lda + c * 8;
+      }
+      if constexpr (!B_NN) {
+        int gn = bn + r;
+        gn = gn < g.N ? gn : g.N - 1;
+        b_src[i] = B + (int64_t)gn * g.ldb + c * 8;
+      } else {
+        const int k = 4 * q + (lane >> 4), pos = lane & 15;
+        const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
+        int gn = bn + u * 8;
+        gn = gn < g.N ? gn : 0;
+        b_src[i] = B + (int64_t)k * g.ldb + gn;
+      }
+    }
+    auto request_pair = [&](int q, uint32_t slot) __attribute__((always_inline)) {
+      const int64_t k0 = (int64_t)q * 64;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) lds_dma16(slot + (uint32_t)(wave + 4 * i) * 1024u, a_src[i] + (A_T ? k0 * g.lda : k0));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (!B_NN) lds_dma16(slot + kPairPanel + (uint32_t)(wave + 4 * i) * 1024u, b_src[i] + k0);
+        else lds_dma16(slot + kPairPanel + (uint32_t)(wave + 4 * i) * 1024u, b_src[i] + k0 * g.ldb);
+      }
+    };
+    // at most `n` of this wave's requests still in flight (n a multiple of 8: whole pairs)
+    auto wait_fills = [](int n) {
+      if (n >= 24) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+      else if (n == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+      else if (n == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    };
+    uint32_t slot = lds_base;
+    for (int q = 0; q < S && q < np; ++q) request_pair(q, lds_base + (uint32_t)q * kPairSlot);
+    wait_fills(8 * ((np < S ? np : S) - 2 > 0 ? (np < S ? np : S) - 2 : 0));  // pairs 0 and 1 are in
+    __syncthreads();
+    __syncthreads();  // the computing waves hold pair 0: its slot may be refilled
+    // Step p: pair p + 5 goes into the slot pair p left; when the step ends the pairs up to p + 2 are in (the
+    // requests of pairs p + 3 .. p + 5, those that exist, may still fly).
+    for (int p = 0; p < np; ++p) {
+      if (p + S < np) request_pair(p + S, slot);
+      slot = slot + kPairSlot == lds_base + S * kPairSlot ? lds_base : slot + kPairSlot;
+      const int ahead = np - 1 - (p + 2);  // pairs behind p + 2 that have been requested
+      wait_fills(8 * (ahead < 0 ? 0 : ahead > 3 ? 3 : ahead));
+      __syncthreads();
+    }
+    return;
+  }
+
+  const int fr = lane & 31, fg = lane >> 5;
+  const int tr_k = fg * 8 + ((lane & 15) >> 2);
+  const int tr_n = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  frag_t fa[2][4][2], fb[2][4][2];  // [register set][tile of the pair * 2 + 16-k sub-step][block]
+  auto read_pair = [&](int slot_index, frag_t (&xa)[4][2], frag_t (&xb)[4][2]) __attribute__((always_inline)) {
+    const unsigned char* pa = lds + slot_index * kPairSlot;
+    const unsigned char* pb = pa + kPairPanel;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {  // 16-k sub-step u of the pair: chunks 2u, 2u+1 of the 128-byte rows
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if constexpr (A_T) {
+          const int k = u * 16 + tr_k;
+          const int m = wm * 64 + i * 32 + tr_n;
+          const s16x4 lo = lds_read_tr(pa + swz_n128(k, m >> 3) + ((m & 7) << 1));
+          const s16x4 hi = lds_read_tr(pa + swz_n128(k + 4, m >> 3) + ((m & 7) << 1));
+          xa[u][i] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        } else {
+          xa[u][i] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 64 + i * 32 + fr, u * 2 + fg));
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if constexpr (!B_NN) {
+          xb[u][j] = *reinterpret_cast<const frag_t*>(pb + swz_k64(wn * 64 + j * 32 + fr, u * 2 + fg));
+        } else {
+          const int k = u * 16 + tr_k;
+          const int n = wn * 64 + j * 32 + tr_n;
+          const s16x4 lo = lds_read_tr(pb + swz_n128(k, n >> 3) + ((n & 7) << 1));
+          const s16x4 hi = lds_read_tr(pb + swz_n128(k + 4, n >> 3) + ((n & 7) << 1));
+          xb[u][j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      }
+    }
+  };
+  auto mma_pair = [&](frag_t (&xa)[4][2], frag_t (&xb)[4][2]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = Mfma<T>::run(xb[u][j], xa[u][i], acc[i][j]);
+  };
+  // The LDS reads go behind the first eight MFMAs of a step (two each, three with a row-major B), the other
+  // eight MFMAs cover the latency of the last read, and nothing moves across the end of the step.
+#define MI355_MDD                                                                             \
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 2 + (B_NN ? 1 : 0) + (A_T ? 1 : 0), 0);
+#define MI355_X4(X) X X X X
+#define MI355_PAIR_SCHEDULE                                                   \
+  MI355_X4(MI355_MDD) MI355_X4(MI355_MDD)                                     \
+  __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);                         \
+  __builtin_amdgcn_sched_barrier(0);
+
+  __syncthreads();  // pairs 0 and 1 are in
+  read_pair(0, fa[0], fb[0]);
+  __syncthreads();  // every wave has its fragments of pair 0
+  int p = 0, rs = 1;  // rs: the ring slot of pair p + 1
+  auto next_slot = [](int v) { return v + 1 == S ? 0 : v + 1; };
+  for (; p + 2 < np; p += 2) {
+    read_pair(rs, fa[1], fb[1]);
+    mma_pair(fa[0], fb[0]);
+    MI355_PAIR_SCHEDULE
+    __syncthreads();
+    rs = next_slot(rs);
+    read_pair(rs, fa[0], fb[0]);
+    mma_pair(fa[1], fb[1]);
+    MI355_PAIR_SCHEDULE
+    __syncthreads();
+    rs = next_slot(rs);
+  }
+#undef MI355_PAIR_SCHEDULE
+#undef MI355_X4
+#undef MI355_MDD
+  for (; p < np; p += 2) {  // the last one or two steps
+    if (p + 1 < np) read_pair(rs, fa[1], fb[1]);
+    mma_pair(fa[0], fb[0]);
+    __syncthreads();
+    if (p + 1 < np) {
+      mma_pair(fa[1], fb[1]);
+      __syncthreads();
+    }
+  }
+
+  if constexpr (SPLIT == 1) {
+    store_partial_tile<2>(g, acc, lane, bm + wm * 64, bn + wn * 64);
+  } else {
+    if constexpr (SPLIT == 2) {  // the parts meet inside this launch: the last one sums and stores
+      if (blockIdx.y + 1 < gridDim.y) return insplit_leave(g, acc, tid, wave, lane);
+      insplit_sum(g, acc, lds, tid, wave, lane);
+    }
+    store_tile_result<T, 2>(g, acc, lds, wave, lane, bm + wm * 64, bn + wn * 64);
+  }
+}
+
 // ---------------------------------------------------------------- MFMA kernel, 64x64 tiles
 // bf16 / f16 products whose 128x128 tiles would leave most CUs without work (a 197-token ViT
 // layer against a 768-wide weight: 12 tiles; 1024^3: 64) and whose K loop is too short to split:
@@ -2072,6 +2273,22 @@ static int64_t split_ws_bytes(const SplitPlan& p, int64_t M, int64_t N, int tile
 static int f32_tile(int64_t M, int64_t N) {
   return ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN) < kNumCU * 3 / 4 ? 64 : 128;
 }
+// What a 128x128 workgroup of the bf16 / f16 kernels spends per k, in ns, when `wgs` of them run in one launch
+// (measured on [128 tm, 4096] x [128 tn, 4096]^T without a split, whole launches less 3 us of prologue and
+// epilogue): alone on the chip a workgroup is bound by the latency of its fills (128 KB in flight against
+// ~1.8 us), from about 160 on the workgroups slow each other down, and beyond one per CU two share a CU's LDS
+// and fill path.
+static double small_ns_per_k(int64_t wgs) {
+  static const struct { int wgs; double ns; } pts[] = {{64, 7.3}, {128, 7.6}, {160, 7.85}, {192, 8.3}, {224, 9.4},
+                                                       {256, 9.9}, {320, 16.4}, {384, 18.0}, {512, 22.3}};
+  constexpr int n = sizeof(pts) / sizeof(pts[0]);
+  if (wgs <= pts[0].wgs) return pts[0].ns;
+  if (wgs > pts[n - 1].wgs) return pts[n - 1].ns * (double)((wgs + 511) / 512);  // rounds of two per CU
+  for (int i = 1; i < n; ++i)
+    if (wgs <= pts[i].wgs)
+      return pts[i - 1].ns + (pts[i].ns - pts[i - 1].ns) * (double)(wgs - pts[i - 1].wgs) / (double)(pts[i].wgs - pts[i - 1].wgs);
+  return pts[n - 1].ns;
+}
 static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
   const int bk = elem_size == 4 ? FBK : BK3;
   const int tile = elem_size == 4 ? f32_tile(M, N) : SBM;
@@ -2093,18 +2310,22 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
     if (real_ns != ns) continue;  // this count rounds to one already tried
     if (K - (ns - 1) * ks < (int64_t)min_steps * bk) continue;  // the last split would fall under the minimum
     const int64_t per_cu = (tiles * ns + kNumCU - 1) / kNumCU;
-    const double t_k = (double)per_cu * (per_cu >= 2 ? 0.7 : 1.0) * (double)ks * ns_per_k;
+    // (A few rows against a weight that is streamed once - decoding - are bound by that stream, not by the tiles'
+    // K loops: they keep the older figures, under which more, shorter parts win: [8,8192]x[8192,8192]^T 30.9 us
+    // against 37.1.)
+    const double t_k = elem_size == 2 && M > 32 ? (double)ks * small_ns_per_k(tiles * ns)
+                                      : (double)per_cu * (per_cu >= 2 ? 0.7 : 1.0) * (double)ks * ns_per_k;
     if (ns == 1) {  // the unsplit product: what a split has to beat
       best = t_k;
       continue;
     }
-    // The part count is chosen against the summing launch's cost, which is what the K-loop figures above were
-    // fitted with; the parts then meet whichever way is cheaper for that count.
-    const double t = t_k + split_meet_ns(1, ns, M, N, tile);
+    // The parts meet whichever way is cheaper for this count.
+    const int mode = allowed[2] && (!allowed[1] || split_meet_ns(2, ns, M, N, tile) < split_meet_ns(1, ns, M, N, tile)) ? 2 : 1;
+    const double t = t_k + split_meet_ns(elem_size == 2 ? mode : 1, ns, M, N, tile);
     if (t < best) {
       best = t;
       best_ns = ns;
-      best_mode = allowed[2] && (!allowed[1] || split_meet_ns(2, ns, M, N, tile) < split_meet_ns(1, ns, M, N, tile)) ? 2 : 1;
+      best_mode = mode;
     }
   }
   if (best_ns <= 1) return p;
@@ -2319,11 +2540,20 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         g.sk_epoch = next_split_epoch();
         g.sk_spin_limit = knobs().x16_spin_limit;
       };
+      // The deep-ring 128x128 kernel: with loader waves where an operand is transposed by the LDS reads (a row-major
+      // b, an M-contiguous a: three or four DS instructions per MFMA leave the computing waves no slot for
+      // the requests: [2048,4096]x[4096,2048] 43.9 -> 41.7 us, [128,1024]x[1024,128] 12.7 -> 10.6), the four-wave
+      // form otherwise (level or 1 - 3 % ahead there).  gemm_tile = ring4 / ring8 forces one (measurement knobs).
+      const bool four_wave_ring = strcmp(knobs().gemm_tile, "ring4") == 0 || (b_nt && !a_t && strcmp(knobs().gemm_tile, "ring8") != 0);
       auto pick_small = [&](auto deep, auto split_c) -> const void* {
         constexpr int SP = decltype(split_c)::value;
         if constexpr (decltype(deep)::value) {
-          if (a_t) return b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, SP, true> : (const void*)gemm_mfma_small2_kernel<T, true, SP, true>;
-          return b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, SP, false> : (const void*)gemm_mfma_small2_kernel<T, true, SP, false>;
+          if (four_wave_ring) {
+            if (a_t) return b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, SP, true> : (const void*)gemm_mfma_small2_kernel<T, true, SP, true>;
+            return b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, SP, false> : (const void*)gemm_mfma_small2_kernel<T, true, SP, false>;
+          }
+          if (a_t) return b_nt ? (const void*)gemm_mfma_small3_kernel<T, false, SP, true> : (const void*)gemm_mfma_small3_kernel<T, true, SP, true>;
+          return b_nt ? (const void*)gemm_mfma_small3_kernel<T, false, SP, false> : (const void*)gemm_mfma_small3_kernel<T, true, SP, false>;
         } else {
           if (a_t) return b_nt ? (const void*)gemm_mfma_small_kernel<T, false, SP, true> : (const void*)gemm_mfma_small_kernel<T, true, SP, true>;
           return b_nt ? (const void*)gemm_mfma_small_kernel<T, false, SP, false> : (const void*)gemm_mfma_small_kernel<T, true, SP, false>;
@@ -2368,7 +2598,10 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                                                       // vocabulary: 48 us, 128x128 tiles 55) - up to K = 4096 for more than one row of tiles: beyond, the
                                                       // 128x128 kernels with K split over the chip are ahead ([512,8192]x[8192,1536]: 42 us here, 31 there;
                                                       // [768,8192]x[8192,2048]: 62 against 52; at K = 4096 these are level or ahead: 23.4 against 27.5)
-                                                      ((K <= 4096 || M <= 64) && ((nb128 > 32 && nb128 < kNumCU / 2 && M >= 16 && light_b) || nb64 >= 160))));
+                                                      // (from 80 tiles of 128x128 on, two parts of K each on the 128x128 kernels fill the chip and are
+                                                      // ahead at K > 2048: [384,4096]x[4096,4096]^T 34.3 -> 28.4 us, [2048,3072]x[768,3072]^T 26.7 -> 24.8)
+                                                      ((K <= 4096 || M <= 64) && (M <= 64 || nb128 < 80) &&
+                                                       ((nb128 > 32 && nb128 < kNumCU / 2 && M >= 16 && light_b) || nb64 >= 160))));
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
       // with 256x256 tiles when K is a multiple of 128 (from 256 on): measured against the 32x32x16 forms on
       // [4096,K]x[K,16384], it is 11 % faster at K = 256 and 4 - 15 % from K = 768 on (C3: [4096,4096]x
@@ -2512,7 +2745,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         using M2 = std::integral_constant<int, 2>;
         if (pairs) kern = !split ? pick_small(std::true_type{}, M0{}) : meet_inside ? pick_small(std::true_type{}, M2{}) : pick_small(std::true_type{}, M1{});
         else kern = !split ? pick_small(std::false_type{}, M0{}) : meet_inside ? pick_small(std::false_type{}, M2{}) : pick_small(std::false_type{}, M1{});
-        threads = 256;
+        threads = pairs && !four_wave_ring ? 512 : 256;  // the deep-ring kernel: four computing waves and four loaders
       } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
       } else if (K % 64 == 0) {
@@ -2700,13 +2933,13 @@ static int run_gemm_f32out(const void* a, int64_t a_rs, int64_t a_cs, const void
   const bool pairs = nblocks <= kNumCU && K % 64 == 0;  // at most one workgroup per CU: the deep-ring kernel
   const int lds_bytes = pairs ? kSmall2Lds : kSmallLds;
   const void* kern;
-  if (pairs) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, 1, false> : (const void*)gemm_mfma_small2_kernel<T, true, 1, false>;
+  if (pairs) kern = b_nt ? (const void*)gemm_mfma_small2_kernel<T, false, 1, false> : (const void*)gemm_mfma_small3_kernel<T, true, 1, false>;  // (loader waves for a row-major b)
   else kern = b_nt ? (const void*)gemm_mfma_small_kernel<T, false, 1, false> : (const void*)gemm_mfma_small_kernel<T, true, 1, false>;
   hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   if (e != hipSuccess)
     return set_error(MI355_ERR_LAUNCH, "mi355_gemm_f32out: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(e));
   void* params[] = {&g};
-  e = hipLaunchKernel(kern, dim3((unsigned)nblocks, 1), dim3(256), params, lds_bytes, st);
+  e = hipLaunchKernel(kern, dim3((unsigned)nblocks, 1), dim3(pairs && !b_nt ? 512 : 256), params, lds_bytes, st);
   if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm_f32out: launch failed: %s", hipGetErrorString(e));
   int rc = check_launch("mi355_gemm_f32out");
   if (rc) return rc;
