@@ -79,7 +79,9 @@ int mi355_init(void);
 /* Test and measurement knobs; no counterpart in the reference.  The planner's choice of GEMM
  * kernel can be overridden so that a test reaches every kernel form on a shape of its choosing:
  *   "gemm_tile":  "x16" | "x16persist" | "x16split" | "x16split2" .. "x16split4" | "x16mixed" | "256x256" |
- *                 "mixed" | "256x128" | "128x128" | "64x64"  (initial value: the environment's MI355_GEMM_TILE)
+ *                 "mixed" | "256x128" | "128x128" | "64x64" | "ring4" | "ring8"  (initial value: the
+ *                 environment's MI355_GEMM_TILE; ring4 / ring8: the four- / eight-wave form of the 128x128
+ *                 deep-ring kernel on any layout)
  *   "gemm_waves": "4" | "8"                  (initial value: MI355_GEMM_WAVES)
  *   "gemm_split": "launch2" | "inlaunch"     how the parts of a K split over several workgroups of the
  *                 128x128- and 64x64-tile kernels meet: in a summing launch, or inside the one launch
