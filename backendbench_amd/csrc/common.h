@@ -24,6 +24,7 @@ struct Knobs {
   char gemm_waves[8];   // "" / "4" / "8"
   char gemm_split[12];  // "" = the planner decides how a split K meets; "launch2" a summing launch, "inlaunch" inside the one launch
   int x16_spin_limit;   // polls of the in-launch split-K's bounded wait before it gives up
+  int gemm_prefetch;    // workgroups that only warm the last-level cache next to a 128x128-tile launch's tiles: -1 = the planner decides
 };
 const Knobs& knobs();
 constexpr int kX16SpinLimitDefault = 1 << 21;  // about 1 us per poll

@@ -34,6 +34,7 @@ static void knobs_from_env() {
   copy_knob(g_knobs.gemm_tile, sizeof(g_knobs.gemm_tile), getenv("MI355_GEMM_TILE"));
   copy_knob(g_knobs.gemm_waves, sizeof(g_knobs.gemm_waves), getenv("MI355_GEMM_WAVES"));
   g_knobs.x16_spin_limit = kX16SpinLimitDefault;
+  g_knobs.gemm_prefetch = -1;
 }
 
 const Knobs& knobs() {
@@ -105,6 +106,10 @@ extern "C" int mi355_set_knob(const char* name, const char* value) {
     const long v = (value == nullptr || value[0] == 0) ? kX16SpinLimitDefault : strtol(value, nullptr, 10);
     if (v < 0 || v > (1L << 30)) return set_error(MI355_ERR_INVALID, "mi355_set_knob: x16_spin_limit %ld out of range", v);
     g_knobs.x16_spin_limit = (int)v;
+  } else if (strcmp(name, "gemm_prefetch") == 0) {
+    const long v = (value == nullptr || value[0] == 0) ? -1 : strtol(value, nullptr, 10);
+    if (v < -1 || v > kNumCU) return set_error(MI355_ERR_INVALID, "mi355_set_knob: gemm_prefetch %ld out of range", v);
+    g_knobs.gemm_prefetch = (int)v;
   } else {
     return set_error(MI355_ERR_INVALID, "mi355_set_knob: unknown knob '%s'", name);
   }

@@ -1190,6 +1190,7 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
 template <typename T, bool B_NN, int NJ, bool A_T>
 __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  if ((int)blockIdx.x >= g.tiles_m * g.tiles_n) return warm_operands<T, A_T, B_NN>(g, 0, g.K);
   int tm, tn;
   tile_coords(g, tm, tn);
   // the fill requests take their bases in SGPRs: the tile origin is uniform, say so
@@ -1453,6 +1454,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
   const int bm = tm * SBM, bn = tn * SBN;
   const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
   const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
+  if ((int)blockIdx.x >= g.tiles_m * g.tiles_n) return warm_operands<T, A_T, B_NN>(g, kbeg, kend);
   const T* A = static_cast<const T*>(g.a) + (A_T ? (int64_t)kbeg * g.lda : (int64_t)kbeg);
   const T* B = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)kbeg);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -1674,6 +1676,7 @@ __global__ __launch_bounds__(512) void gemm_mfma_small3_kernel(GemmArgs g) {
   const int np = (kend - kbeg) / (2 * BK3);
   constexpr int kPairPanel = SBM * 64 * 2;  // 16 KB
   constexpr int kPairSlot = 2 * kPairPanel;
+  if ((int)blockIdx.x >= g.tiles_m * g.tiles_n) return warm_operands<T, A_T, B_NN>(g, kbeg, kend);
 
   if (loader) {
     const T* A = static_cast<const T*>(g.a) + (A_T ? (int64_t)kbeg * g.lda : (int64_t)kbeg);
@@ -1879,6 +1882,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
   const int bm = tm * TBM, bn = tn * TBN;
   const int kbeg = SPLIT ? (int)blockIdx.y * g.ksplit : 0;
   const int kend = SPLIT ? (kbeg + g.ksplit < g.K ? kbeg + g.ksplit : g.K) : g.K;
+  if ((int)blockIdx.x >= g.tiles_m * g.tiles_n) return warm_operands<T, false, B_NN>(g, kbeg, kend);
   const T* a_base = static_cast<const T*>(g.a) + (int64_t)bm * g.lda + kbeg;
   const T* b_base = static_cast<const T*>(g.b) + (B_NN ? (int64_t)kbeg * g.ldb : (int64_t)bn * g.ldb + kbeg);
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -2526,6 +2530,16 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       int lds_bytes = kGemmLds;
       int threads = 512;
       int nsplit = 1;
+      int warm_blocks = 0;  // workgroups behind the tiles that only warm the last-level cache (warm_operands)
+      // Per part of K, for a launch of one workgroup per CU: up to 32 of the CUs it leaves idle, when a part's K
+      // loop has `min_k` and more (a ring holds the first stages of a K loop itself).  gemm_prefetch = N forces N
+      // (0: none): a measurement knob.
+      auto warm_for = [&](int64_t tiles, int64_t min_k) {
+        const int64_t idle = (kNumCU - tiles * nsplit) / nsplit;
+        const int64_t want = knobs().gemm_prefetch >= 0 ? knobs().gemm_prefetch : K / nsplit >= min_k ? 32 : 0;
+        if (knobs().gemm_prefetch < 0 && idle < 16) return 0;  // too few to stay ahead of the tiles
+        return (int)(idle < 0 ? 0 : idle < want ? idle : want);
+      };
       auto pick_w4 = [&](auto nj) -> const void* {
         constexpr int NJ = decltype(nj)::value;
         if (a_t) return b_nt ? (const void*)gemm_mfma_w4_kernel<T, false, NJ, true> : (const void*)gemm_mfma_w4_kernel<T, true, NJ, true>;
@@ -2570,7 +2584,15 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const char* forced_waves = kn.gemm_waves[0] ? kn.gemm_waves : nullptr;
       const bool mid = !ktail && K % 64 == 0 && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "256x128") == 0
-                                               : K >= 1024 && nblocks < kNumCU * 3 / 4 && tiles_mid > (K >= 2048 ? 228 : 248) && tiles_mid <= kNumCU &&
+                                               : nblocks < kNumCU * 3 / 4 && tiles_mid <= kNumCU &&
+                                                     ((K >= 1024 && tiles_mid > (K >= 2048 ? 228 : 248)) ||
+                                                      // More 128x128 tiles than one round of them, few enough 256x128 tiles to leave CUs for
+                                                      // warm_operands: this kernel runs at fill latency, and with the operands on their way
+                                                      // into the last-level cache it is ahead of the 128x128 kernels with two workgroups on
+                                                      // a CU and of two parts of K on 256x256 tiles ([4096,1536]x[1536,1536]^T 35.1 ->
+                                                      // 29.4 us, [2048,1536]x[1536,2304] 32.9 -> 25.7, [3072,768]x[2048,768]^T 21.6 -> 18.9;
+                                                      // level at K = 512 and from K = 4096 on).
+                                                      (K >= 768 && K <= 3072 && tiles_mid > kNumCU / 2)) &&
                                                      4 * M >= 3 * (int64_t)g.tiles_m * BM);  // rows that are mostly output ([128,4096]x[4096,32000]: 74 us here, 61 on 128x128 tiles)
       // Fewer 128x128 tiles than half the CUs: 64x64 tiles reach four times as many (measured on this
       // chip: [197,768]x[768,768] 11.6 -> 7.5 us, 1024^3 14.6 -> 9.4 us).  A 64x64 workgroup walks K at
@@ -2630,7 +2652,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool x16_split = x16_ok && xs.splits > 1 && workspace != nullptr && workspace_bytes >= xs.ws_bytes &&
                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
                              (forced_tile != nullptr ? strncmp(forced_tile, "x16split", 8) == 0
-                                                     : x16_pays && M >= 512 && forced_waves == nullptr);  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
+                                                     : x16_pays && M >= 512 && forced_waves == nullptr && !mid);  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
       if (x16_split) {
         kern = gemm_x16_splitk_kernel(std::is_same<T, bf16_t>::value, !b_nt);
         threads = 256;
@@ -2690,6 +2712,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         }
         // Output rows off the 128-byte lines: whole tile rows per store instruction (store_tile_rows16).
         g.out_rows = !persist && g.tail_n == 0 && (N % 64 != 0 || reinterpret_cast<uintptr_t>(out) % 128 != 0);
+        if (!persist && g.tail_n == 0) warm_blocks = warm_for(nblocks, 1024);
       } else if (t64) {
         g.tiles_m = (int32_t)((M + TBM - 1) / TBM);
         g.tiles_n = (int32_t)((N + TBN - 1) / TBN);
@@ -2704,6 +2727,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         }
         const bool deep = nblocks * nsplit <= kNumCU;
         lds_bytes = (deep ? 8 : 4) * kTStage;
+        if (deep) warm_blocks = warm_for(nblocks, 1024);
         if (nsplit > 1 && meet_inside) {
           if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8, 2> : (const void*)gemm_mfma_t64_kernel<T, true, 8, 2>;
           else kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 4, 2> : (const void*)gemm_mfma_t64_kernel<T, true, 4, 2>;
@@ -2720,6 +2744,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         kern = pick_w4(std::integral_constant<int, 2>{});
         threads = 256;
         lds_bytes = kGemmLds64;
+        warm_blocks = warm_for(nblocks, 768);
         // (The 16x16x32 kernel on 256x128 tiles was measured for this slot: with half the MFMAs per fill and
         // per LDS read it is level with this form on a transposed b and 10 % behind on a row-major one.)
       } else if (!ktail && nblocks < kNumCU * 3 / 4) {  // 128x128 tiles, two workgroups per CU
@@ -2746,6 +2771,9 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         if (pairs) kern = !split ? pick_small(std::true_type{}, M0{}) : meet_inside ? pick_small(std::true_type{}, M2{}) : pick_small(std::true_type{}, M1{});
         else kern = !split ? pick_small(std::false_type{}, M0{}) : meet_inside ? pick_small(std::false_type{}, M2{}) : pick_small(std::false_type{}, M1{});
         threads = pairs && !four_wave_ring ? 512 : 256;  // the deep-ring kernel: four computing waves and four loaders
+        // CUs without a tile warm the last-level cache for the others (warm_operands): the deep-ring kernels only,
+        // a K loop of 16 stages and more.  gemm_prefetch = N forces that many workgroups per part (a measurement knob).
+        if (pairs) warm_blocks = warm_for(nblocks, 1024);
       } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
       } else if (K % 64 == 0) {
@@ -2791,7 +2819,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       if (nsplit == 1) g.ws = workspace_bytes >= nblocks * 4 * 16 * 8 ? static_cast<float*>(workspace) : nullptr;
 #endif
       void* params[] = {&g};
-      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)nblocks, (unsigned)nsplit), dim3(threads), params, lds_bytes, st);
+      hipError_t e = hipLaunchKernel(kern, dim3((unsigned)(nblocks + warm_blocks), (unsigned)nsplit), dim3(threads), params, lds_bytes, st);
       if (e != hipSuccess) return set_error(MI355_ERR_LAUNCH, "mi355_gemm(mfma): launch failed: %s", hipGetErrorString(e));
       const int rc = check_launch("mi355_gemm(mfma)");
       if (rc || nsplit == 1 || meet_inside) return rc;

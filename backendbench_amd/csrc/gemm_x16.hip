@@ -871,6 +871,7 @@ __device__ __forceinline__ void x16_tile(const GemmArgs& g, unsigned char* lds, 
 template <typename T, bool B_NN>
 __global__ __launch_bounds__(256) void gemm_mfma_x16_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  if ((int)blockIdx.x >= g.tiles_m * g.tiles_n) return warm_operands<T, false, B_NN>(g, 0, g.K);
   int tm, tn;
   tile_coords(g, tm, tn);
   x16_tile<T, B_NN, 4>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * BN));

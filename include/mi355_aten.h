@@ -86,6 +86,9 @@ int mi355_init(void);
  *   "gemm_split": "launch2" | "inlaunch"     how the parts of a K split over several workgroups of the
  *                 128x128- and 64x64-tile kernels meet: in a summing launch, or inside the one launch
  *                 (the planner picks per shape)
+ *   "gemm_prefetch": "0" .. "256"  workgroups per part of K that only read the operands ahead of the tiles, on
+ *                 CUs a launch of one workgroup per CU leaves without a tile (cut down to the CUs left over;
+ *                 unset: up to 32 where 16 and more are left and the K loop is long enough)
  *   "x16_spin_limit": polls of the in-launch split-K's bounded wait for a partial product
  *                 before it gives up (default 2^21, about two seconds); a test sets it to 0
  *                 to walk the give-up path while every kernel still runs to its end.

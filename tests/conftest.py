@@ -43,6 +43,9 @@ class _GemmKnobs:
     def spin_limit(self, value):
         self._set("x16_spin_limit", value)
 
+    def prefetch(self, value):
+        self._set("gemm_prefetch", value)
+
     def restore(self):
         for name in self._touched:
             self._lib.set_knob(name, None)

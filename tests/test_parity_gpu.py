@@ -615,6 +615,40 @@ def test_split_k_parts_meet_either_way(backend, dtype, meet, gemm_knobs):
     assert lib.mi355_gemm_status() == 0
 
 
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+def test_cache_warming_workgroups_change_no_result(backend, layout, gemm_knobs):
+    """A launch that leaves CUs without a tile appends workgroups that only read the operands ahead of the tiles
+    (warm_operands: the deep-ring 128x128 kernels, the 64x64-tile kernel with its deep ring, the 256x128 form, the
+    16x16x32 kernel with one workgroup per tile, with K split inside the launch or not).  With none of them, with
+    the planner's count, with a few and with more than there are idle CUs (the count is cut down) every form must
+    give the same bits, equal to the oracle on small-integer operands; ragged edges and K ranges included."""
+    announce(f"cache-warming workgroups, {layout}")
+    g = torch.Generator().manual_seed(53)
+    # (M, N, K, forced form or None): tiles x parts stay under 256 so that CUs are left over
+    shapes = [(1536, 2048, 4096, None), (1500, 2040, 2112, None), (2048, 768, 3072, None), (1024, 2048, 4096, None),
+              (896, 896, 3584, None), (640, 1280, 4096, "64x64"), (4096, 1536, 1536, None), (3072, 2304, 768, None),
+              (4000, 1480, 1088, "256x128"), (2304, 4096, 2048, "x16"), (1280, 2560, 1024, "x16"), (1024, 1024, 8192, "ring8"),
+              (1024, 1024, 8192, "ring4")]
+    for M, N, K, form in shapes:
+        dtype = torch.bfloat16 if (M + K) % 512 == 0 else torch.float16
+        a = (torch.randint(-1, 2, (M, K), generator=g) * (torch.randint(0, 4, (M, K), generator=g) == 0)).to(dtype).cuda()
+        b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t() if layout == "nt" else torch.randint(-1, 2, (K, N), generator=g).to(dtype).cuda()
+        bias = torch.randint(-2, 3, (N,), generator=g).to(dtype).cuda()
+        ref = aten_cpu.reference(aten.mm.default, [a.float(), b.float()])
+        assert float(ref.abs().max()) <= 250
+        want = (ref + bias.cpu().float()).to(dtype)
+        gemm_knobs.tile(form)
+        for count in (None, "0", "5", "32", "250"):
+            gemm_knobs.prefetch(count)
+            got = backend[aten.addmm.default](bias, a, b)
+            torch.cuda.synchronize()
+            assert ev.bit_equal(want, got.cpu()), (M, N, K, form, layout, count)
+        gemm_knobs.prefetch(None)
+        gemm_knobs.tile(None)
+    from backendbench_amd import _lib
+    assert _lib.load().mi355_gemm_status() == 0
+
+
 def test_f64_addmm_keeps_alpha_and_beta_in_f64(backend):
     """alpha = 0.1 and beta = 0.3 are not fp32 numbers: an f64 addmm must apply them in f64 (1e-12
     against the oracle, where an fp32 round trip of the scalars leaves 1e-8), and a beta too small for
