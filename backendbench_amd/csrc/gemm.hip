@@ -2277,14 +2277,16 @@ static int64_t split_ws_bytes(const SplitPlan& p, int64_t M, int64_t N, int tile
 static int f32_tile(int64_t M, int64_t N) {
   return ((M + SBM - 1) / SBM) * ((N + SBN - 1) / SBN) < kNumCU * 3 / 4 ? 64 : 128;
 }
-// What a 128x128 workgroup of the bf16 / f16 kernels spends per k, in ns, when `wgs` of them run in one launch
-// (measured on [128 tm, 4096] x [128 tn, 4096]^T without a split, whole launches less 3 us of prologue and
-// epilogue): alone on the chip a workgroup is bound by the latency of its fills (128 KB in flight against
-// ~1.8 us), from about 160 on the workgroups slow each other down, and beyond one per CU two share a CU's LDS
-// and fill path.
+// What a 128x128 workgroup of the bf16 / f16 kernels adds per k, in ns, when `wgs` of them run in one launch: the
+// slope between K = 1024 and K = 4096 of [128 tm, K] x [128 tn, K]^T without a split, on inputs that no cache
+// holds.  Up to 128 workgroups the K loop runs at the latency of fills that the warming workgroups have sent ahead
+// (warm_operands; 7.9 ns without them, whatever the count); towards 224 there are fewer CUs left for those and
+// the fills start to queue; beyond one per CU two share a CU's LDS and fill path.
 static double small_ns_per_k(int64_t wgs) {
-  static const struct { int wgs; double ns; } pts[] = {{64, 7.3}, {128, 7.6}, {160, 7.85}, {192, 8.3}, {224, 9.4},
-                                                       {256, 9.9}, {320, 16.4}, {384, 18.0}, {512, 22.3}};
+  // (between a transposed b - 5.5 ns up to 128 workgroups, 6.6 at 192, 8.45 at 256 - and a row-major one - 6.7, 8.0,
+  // 9.5: the plan is made before the layouts are known, mi355_gemm_workspace_bytes has to agree with it)
+  static const struct { int wgs; double ns; } pts[] = {{64, 6.0}, {128, 6.3}, {160, 6.55}, {192, 7.3}, {208, 7.4}, {224, 8.2},
+                                                       {240, 8.6}, {256, 9.0}, {320, 16.4}, {384, 18.0}, {512, 22.3}};
   constexpr int n = sizeof(pts) / sizeof(pts[0]);
   if (wgs <= pts[0].wgs) return pts[0].ns;
   if (wgs > pts[n - 1].wgs) return pts[n - 1].ns * (double)((wgs + 511) / 512);  // rounds of two per CU
@@ -2294,14 +2296,17 @@ static double small_ns_per_k(int64_t wgs) {
   return pts[n - 1].ns;
 }
 static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
-  const int bk = elem_size == 4 ? FBK : BK3;
+  // Parts of whole steps: 64 k where K allows it, so that every part keeps the deep-ring kernel's 64-k pairs
+  // (a part of 3680 k fell back to the 32-k kernel: [1024,11008]x[11008,1024] in three parts 56 us, in four 44).
+  const int bk = elem_size == 4 ? FBK : K % 64 == 0 ? 64 : BK3;
   const int tile = elem_size == 4 ? f32_tile(M, N) : SBM;
   const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
   SplitPlan p{1, (int)K, 1};
   if (tiles >= kNumCU || K % bk != 0) return p;
   const double ns_per_k = elem_size == 4 ? (tile == 64 ? 20.0 : 70.0) : 12.8;
   const int min_steps = tiles <= 2 ? 4 : 8;  // one or two tiles: the launch is all latency, shorter splits still pay
-  const int64_t max_ns = K / (min_steps * bk) < 64 ? K / (min_steps * bk) : 64;
+  const int64_t min_k = (int64_t)min_steps * (elem_size == 4 ? FBK : BK3);  // (steps of the 32-k kernels, as measured)
+  const int64_t max_ns = K / min_k < 64 ? K / min_k : 64;
   bool allowed[3];
   split_modes(elem_size, allowed);
   double best = 1e30;
@@ -2312,7 +2317,7 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
     ks = (ks + bk - 1) / bk * bk;
     const int64_t real_ns = (K + ks - 1) / ks;
     if (real_ns != ns) continue;  // this count rounds to one already tried
-    if (K - (ns - 1) * ks < (int64_t)min_steps * bk) continue;  // the last split would fall under the minimum
+    if (K - (ns - 1) * ks < min_k) continue;  // the last split would fall under the minimum
     const int64_t per_cu = (tiles * ns + kNumCU - 1) / kNumCU;
     // (A few rows against a weight that is streamed once - decoding - are bound by that stream, not by the tiles'
     // K loops: they keep the older figures, under which more, shorter parts win: [8,8192]x[8192,8192]^T 30.9 us

@@ -506,14 +506,17 @@ def test_tile64_gemm_every_k_loop_length(backend, layout, shape, gemm_knobs):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_split_k_with_ragged_k(backend, dtype):
-    """One-tile outputs split along K where K is not a multiple of the split length (K = 672, 544, 416
-    at M = N = 64, plus a 100 x 70 output): every split, the last one included, must cover its own k
-    range exactly.  Small-integer operands: bit-equal to the oracle whatever the order of the partial sums."""
+    """One-tile outputs split along K where K is not a multiple of the split length (K = 4000, 2720, 5216, 3104
+    in parts of whole 32-k steps, plus K = 672 .. 1184 around the length from which a split pays, and a 100 x 70
+    output): every split, the last one included, must cover its own k range exactly.  Small-integer operands:
+    bit-equal to the oracle whatever the order of the partial sums."""
     from backendbench_amd import _lib
     announce(f"split-K with ragged K, {dtype}")
-    assert _lib.load().mi355_gemm_workspace_bytes(64, 64, 672, _lib.dtype_code(dtype)) > 0   # the planner does split these
+    for K in (4000, 2720, 5216):
+        assert _lib.load().mi355_gemm_workspace_bytes(64, 64, K, _lib.dtype_code(dtype)) > 0   # the planner does split these
     g = torch.Generator().manual_seed(9)
-    for M, N, K in [(64, 64, 672), (64, 64, 544), (64, 64, 416), (64, 64, 1184), (100, 70, 928), (64, 64, 4000)]:
+    for M, N, K in [(64, 64, 672), (64, 64, 544), (64, 64, 416), (64, 64, 1184), (100, 70, 928), (64, 64, 4000), (64, 64, 2720),
+                    (64, 64, 5216), (128, 64, 3104), (33, 64, 1696)]:
         for nt in (False, True):
             a = torch.randint(-1, 2, (M, K), generator=g).to(dtype).cuda()
             b = torch.randint(-1, 2, (N, K), generator=g).to(dtype).cuda().t() if nt else torch.randint(-1, 2, (K, N + (-N) % 8), generator=g).to(dtype).cuda()
