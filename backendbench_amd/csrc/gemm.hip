@@ -1872,6 +1872,7 @@ __device__ __forceinline__ int swz_n64(int k, int u) {
 // tile in plane blockIdx.y of the workspace, as the 128x128 kernels do; gemm_splitk_finish_kernel sums the planes.
 template <typename T, bool B_NN, int S, int SPLIT = 0>
 __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
+  static_assert(S == 4 || S == 8, "ring of four or eight stages");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   using frag_t = typename Mfma<T>::frag;
   const int tid = threadIdx.x, lane = tid % kWave;
@@ -1928,7 +1929,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
       case 3: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
       case 4: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
       case 5: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
-      default: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
+      case 6: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
+      default: asm volatile("s_waitcnt vmcnt(28)" ::: "memory"); break;  // seven: the whole ring behind stage 0
     }
   };
 
@@ -1942,14 +1944,13 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
   for (int e = 0; e < 16; ++e) acc[0][0][e] = acc_odd[e] = 0.f;
 
   const int nk = (kend - kbeg) / 64;
-  for (int t = 0; t < S - 1 && t < nk; ++t) request_stage(t);
-  for (int t = 0; t < nk; ++t) {
-    const int last_requested = t + S - 2 < nk - 1 ? t + S - 2 : nk - 1;
-    wait_younger(last_requested - t);
-    __syncthreads();  // stage t has landed for every wave, and every wave is done with stage t-1
+  // Fragments are read one stage ahead: step t computes stage t from one register set while the LDS reads of
+  // stage t + 1 fill the other, so the four MFMAs of a step - all its arithmetic - wait for nothing, and the slot
+  // of stage t, read during step t - 1, takes the request for stage t + S behind the barrier of step t (the ring
+  // is S stages deep in flight).  Two steps per iteration, one per register set.
+  auto read_frags = [&](int t, frag_t (&fa)[4], frag_t (&fb)[4]) __attribute__((always_inline)) {
     const unsigned char* pa = lds + (t % S) * kTStage;
     const unsigned char* pb = pa + kTPanel;
-    frag_t fa[4], fb[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       fa[ks] = *reinterpret_cast<const frag_t*>(pa + swz_k64(wm * 32 + fr, ks * 2 + fg));
@@ -1963,11 +1964,49 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
         fb[ks] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
     }
-    if (t + S - 1 < nk) request_stage(t + S - 1);  // into the slot of stage t-1, behind this stage's LDS reads
+  };
+  auto mma_stage = [&](frag_t (&fa)[4], frag_t (&fb)[4]) __attribute__((always_inline)) {
     acc[0][0] = Mfma<T>::run(fb[0], fa[0], acc[0][0]);
     acc_odd = Mfma<T>::run(fb[1], fa[1], acc_odd);
     acc[0][0] = Mfma<T>::run(fb[2], fa[2], acc[0][0]);
     acc_odd = Mfma<T>::run(fb[3], fa[3], acc_odd);
+  };
+  // One step: stage `t` from `cur`; stage t + 1 (when there is one) lands, is read into `nxt`, and stage t + S is
+  // requested into the slot stage t leaves.  Requests so far reach stage min(t + S - 1, nk - 1).
+  auto step = [&](int t, frag_t (&ca)[4], frag_t (&cb)[4], frag_t (&na)[4], frag_t (&nb)[4]) __attribute__((always_inline)) {
+    const bool more = t + 1 < nk;
+    if (more) wait_younger((t + S - 1 < nk - 1 ? t + S - 1 : nk - 1) - (t + 1));
+    __syncthreads();  // stage t + 1 has landed for every wave, and every wave has read stage t
+    if (more) read_frags(t + 1, na, nb);
+    if (t + S < nk) request_stage(t + S);
+    mma_stage(ca, cb);
+  };
+  for (int t = 0; t < S && t < nk; ++t) request_stage(t);
+  wait_younger((S < nk ? S : nk) - 1);
+  __syncthreads();
+  frag_t fa[2][4], fb[2][4];
+  read_frags(0, fa[0], fb[0]);
+  int t = 0;
+  // Steady state without a branch (with branches around them the accumulators travel between their registers and
+  // the VGPRs in every step): while both steps of an iteration still request a stage, S - 2 stages stay in flight
+  // behind the one that is waited for.
+  for (; t + S + 1 < nk; t += 2) {
+    if constexpr (S == 8) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __syncthreads();
+    read_frags(t + 1, fa[1], fb[1]);
+    request_stage(t + S);
+    mma_stage(fa[0], fb[0]);
+    if constexpr (S == 8) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __syncthreads();
+    read_frags(t + 2, fa[0], fb[0]);
+    request_stage(t + 1 + S);
+    mma_stage(fa[1], fb[1]);
+  }
+  for (; t < nk; t += 2) {  // the last S + 1 steps or fewer: requests and reads run out
+    step(t, fa[0], fb[0], fa[1], fb[1]);
+    if (t + 1 < nk) step(t + 1, fa[1], fb[1], fa[0], fb[0]);
   }
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[0][0][e] += acc_odd[e];
@@ -2347,9 +2386,10 @@ static SplitPlan plan_splitk(int64_t M, int64_t N, int64_t K, int elem_size) {
 }
 
 // Split-K for the 64x64-tile kernel: a handful of tiles with a long K (one image's 197 tokens against a
-// 3072 x 768 weight) leave most CUs idle and walk K at about 0.3 us per 64-k stage.  Splits of whole stages, at
+// 3072 x 768 weight) leave most CUs idle and walk K at about 0.21 us per 64-k stage.  Splits of whole stages, at
 // least four each; the cost model is the one of plan_splitk with this kernel's figures (2 us to get going,
-// 0.3 us per stage, 1.3 x that with two workgroups on a CU, 3 us and the partial planes for the summing launch).
+// 0.21 us per stage - [896,3584]x[896,3584]^T, 196 tiles: 15.7 us for 56 stages - and 1.1 x that per workgroup
+// when several share a CU, 3 us and the partial planes for the summing launch).
 static SplitPlan plan_t64_split(int64_t M, int64_t N, int64_t K) {
   SplitPlan p{1, (int)K, 1};
   const int64_t tiles = ((M + TBM - 1) / TBM) * ((N + TBN - 1) / TBN);
@@ -2364,7 +2404,7 @@ static SplitPlan plan_t64_split(int64_t M, int64_t N, int64_t K) {
     const int64_t ks = (stages + ns - 1) / ns;
     if ((stages + ks - 1) / ks != ns || stages - (ns - 1) * ks < 4) continue;
     const int64_t per_cu = (tiles * ns + kNumCU - 1) / kNumCU;
-    const double t_k = 2000.0 + 300.0 * (double)ks * (per_cu >= 2 ? 1.3 * (double)((per_cu + 1) / 2) : 1.0);
+    const double t_k = 2000.0 + 210.0 * (double)ks * (per_cu >= 2 ? 1.1 * (double)per_cu : 1.0);
     if (ns == 1) {  // the unsplit product: what a split has to beat
       best = t_k;
       continue;
@@ -2618,7 +2658,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                              workspace_bytes >= split_ws_bytes(ts, M, N, TBM);
       const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
-                                               : (nb128 < kNumCU / 2 || (nb128 == kNumCU / 2 && K <= 2048) ||  // (exactly 128 tiles, [1024,2048]x[2048,2048]: 26.4 -> 21.2 us, K = 512: 10.0 -> 7.0; level at K = 3072, behind from 4096 on)
+                                               : (nb128 < kNumCU / 2 || (nb128 == kNumCU / 2 && K < 2048) ||  // (exactly 128 tiles: K = 512 10.0 -> 7.0 us; at K = 2048 the deep-ring 128x128 kernel with its warming workgroups is level on a transposed b, 19 against 21 - 22 us, and ahead on a row-major one)
                                                   ((M <= 64 || N <= 64) && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
                                                      (K <= (M <= 32 ? 1024 : 2048) || t64_split ||
                                                       // enough 64x64 tiles for the chip: no need to split a long K (a few rows against a 32000 x 4096
@@ -2627,8 +2667,11 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                                                       // [768,8192]x[8192,2048]: 62 against 52; at K = 4096 these are level or ahead: 23.4 against 27.5)
                                                       // (from 80 tiles of 128x128 on, two parts of K each on the 128x128 kernels fill the chip and are
                                                       // ahead at K > 2048: [384,4096]x[4096,4096]^T 34.3 -> 28.4 us, [2048,3072]x[768,3072]^T 26.7 -> 24.8)
-                                                      ((K <= 4096 || M <= 64) && (M <= 64 || nb128 < 80) &&
-                                                       ((nb128 > 32 && nb128 < kNumCU / 2 && M >= 16 && light_b) || nb64 >= 160))));
+                                                      // (measured again with the 64x64-tile kernel's fragments read a stage ahead and the 128x128
+                                                      // kernels' warming workgroups: up to 64 tiles of 128x128 at K = 3072 / 4096 this kernel is
+                                                      // 6 - 20 % ahead, at 72 - 96 tiles 4 - 28 % behind; at K = 8192 ahead up to 32 tiles)
+                                                      ((K <= 4096 || M <= 64 || (K <= 8192 && nb128 <= 32)) && (M <= 64 || nb128 <= 64) &&
+                                                       ((nb128 < kNumCU / 2 && M >= 16 && light_b) || nb64 >= 160))));
       // The 16x16x32 form of the four-wave kernel (gemm_x16.hip) takes every product that fills the chip
       // with 256x256 tiles when K is a multiple of 128 (from 256 on): measured against the 32x32x16 forms on
       // [4096,K]x[K,16384], it is 11 % faster at K = 256 and 4 - 15 % from K = 768 on (C3: [4096,4096]x
