@@ -34,7 +34,7 @@ sys.path.insert(0, ROOT)
 # same counter reads for a plain 128 MiB copy): rocprofv3 --pmc runs of `bench.py --only-op <row>`,
 # commands and tables in profiles/C2_row_kernels__softmax_layer_norm.md.  A profiler cannot run inside
 # this script, so the figures are carried here and named as such in the output ("traffic_source").
-MEASURED_TRAFFIC_BYTES = {"C2.layer_norm": 134_670_000, "C2.softmax": 134_290_000}
+MEASURED_TRAFFIC_BYTES = {"C2.layer_norm": 134_670_000, "C2.softmax": 134_280_000}
 
 
 def parse():
