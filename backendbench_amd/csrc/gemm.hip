@@ -151,21 +151,34 @@ __device__ __forceinline__ void insplit_sum(const GemmArgs& g, f32x16 (&acc)[MI]
   __syncthreads();
   const float poison = *gave_up != 0 ? __builtin_nanf("") : -0.f;  // -0: x + -0 == x
   const __amdgpu_buffer_rsrc_t rsrc = insplit_rsrc<NB>(g, first, nprod);
-  for (int p = 0; p < nprod; ++p) {
-    f32x4 part[NB][4];
+  // The planes of several producers are in flight at once (four for a one-block wave tile, two for four blocks:
+  // 64 / 128 registers): a plane comes from another CU's stores through the L2, about a microsecond each when
+  // they are read one after the other.  A batch's last planes may lie past the count: they re-read the last
+  // plane and are not added.  The order of the additions is the order of the parts, as before.
+  constexpr int PB = NB == 1 ? 4 : NB <= 4 ? 2 : 1;
+  for (int p0 = 0; p0 < nprod; p0 += PB) {
+    f32x4 part[PB][NB][4];
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
+    for (int u = 0; u < PB; ++u) {
+      const int p = p0 + u < nprod ? p0 + u : nprod - 1;
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        part[b][q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane * 16, p * (NB * 16384) + ((wave * NB + b) * 4 + q) * 1024, kSc1));
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-      for (int j = 0; j < NJ; ++j)
+      for (int b = 0; b < NB; ++b)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
+          part[u][b][q] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane * 16, p * (NB * 16384) + ((wave * NB + b) * 4 + q) * 1024, kSc1));
+    }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] += part[i * NJ + j][q][e];
+    for (int u = 0; u < PB; ++u) {
+      if (p0 + u >= nprod) break;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] += part[u][i * NJ + j][q][e];
+    }
   }
   acc[0][0][0] += poison;  // NaN marks the tile of a producer that never arrived
   __syncthreads();  // every wave has used what it read of the planes, and has read *gave_up: the epilogue reuses the ring
@@ -2290,10 +2303,10 @@ struct SplitPlan {
 };
 // What the meeting costs, in ns, on top of the longest part's K loop.  A summing launch: 3 us and every plane
 // written and read once at ~4 TB/s.  Inside the launch: the producers' planes go out in ~1.5 us, and the summing
-// workgroup takes them in one after the other, 64 KB (a 128x128 tile: ~1.3 us) or 16 KB (64x64: ~0.9 us) each.
+// workgroup takes them in two (128x128 tiles, 64 KB each: ~1.0 us a plane) or four (64x64, 16 KB: ~0.6 us) at a time.
 static double split_meet_ns(int mode, int64_t ns, int64_t M, int64_t N, int tile) {
   if (ns <= 1) return 0.0;
-  if (mode == 2) return 1500.0 + (tile == 64 ? 900.0 : 1300.0) * (double)(ns - 1);
+  if (mode == 2) return 1500.0 + (tile == 64 ? 600.0 : 1000.0) * (double)(ns - 1);
   return 3000.0 + (double)ns * (double)M * (double)N * 8.0 / 4000.0;  // 4 TB/s = 4000 B/ns
 }
 // The modes the plan may choose from: both for bf16 / f16 unless the gemm_split knob names one.
