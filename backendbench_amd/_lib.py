@@ -97,6 +97,7 @@ SIGNATURES = {
     ),
     "mi355_gemm_status": (c_int, []),
     "mi355_gemm_tile_columns": (c_int, [c_int64, c_int64, c_int64, ctypes.POINTER(c_int32), ctypes.POINTER(c_int32)]),
+    "mi355_gemm_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int, c_char_p, c_int64]),
     "mi355_calib_mfma": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mi355_index_select": (
         c_int,

@@ -2544,6 +2544,16 @@ static unsigned long long next_split_epoch() {
   return epoch.fetch_add(2);
 }
 
+// mi355_gemm_plan: run_gemm stops in front of its launch and leaves what it would have launched here.
+static thread_local char* g_plan_text = nullptr;
+static thread_local int64_t g_plan_cap = 0;
+static int describe_plan(const char* form, int tiles_m, int tiles_n, int64_t grid_x, int grid_y, int threads, int lds_bytes,
+                         int parts, const char* meet, int warm) {
+  snprintf(g_plan_text, (size_t)g_plan_cap, "form=%s tiles=%dx%d grid=%lldx%d threads=%d lds=%d parts=%d meet=%s warm=%d", form, tiles_m,
+           tiles_n, (long long)grid_x, grid_y, threads, lds_bytes, parts, meet, warm);
+  return MI355_OK;
+}
+
 template <typename T>
 static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs,
                     const void* c, int64_t c_rs, int64_t c_cs, void* out, int64_t M, int64_t N, int64_t K,
@@ -2589,6 +2599,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       int threads = 512;
       int nsplit = 1;
       int warm_blocks = 0;  // workgroups behind the tiles that only warm the last-level cache (warm_operands)
+      const char* form = "";  // the kernel form, for mi355_gemm_plan
       // Per part of K, for a launch of one workgroup per CU: up to 32 of the CUs it leaves idle, when a part's K
       // loop has `min_k` and more (a ring holds the first stages of a K loop itself).  gemm_prefetch = N forces N
       // (0: none): a measurement knob.
@@ -2716,6 +2727,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                                                      : x16_pays && M >= 512 && forced_waves == nullptr && !(mid && K <= 4096));  // (a full round of 256x128 tiles: [2048,4096]x[4096,4096] 73.1 us in two parts here, 68.6 there; [2048,11008]x[11008,4096] 155 against 176)  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
       if (x16_split) {
         kern = gemm_x16_splitk_kernel(std::is_same<T, bf16_t>::value, !b_nt);
+        form = "x16_split";
         threads = 256;
         lds_bytes = kX16Lds;
         g.ws = static_cast<float*>(workspace);
@@ -2728,6 +2740,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         nblocks = (int64_t)xs.splits * xs.tiles8;
       } else if (x16) {
         kern = gemm_x16_kernel(std::is_same<T, bf16_t>::value, !b_nt);
+        form = "x16";
         threads = 256;
         lds_bytes = kX16Lds;
         // More tiles than CUs, all of them whole: one workgroup per CU walks its tiles with the fill
@@ -2756,6 +2769,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
 #endif
         if (persist) {
           kern = gemm_x16_persistent_kernel(std::is_same<T, bf16_t>::value, !b_nt);
+          form = "x16_persistent";
           if (nblocks > kNumCU) nblocks = kNumCU;
         }
         // The mixed-width grid (192-wide tiles in the last round) is built for this form too, but it does not
@@ -2769,6 +2783,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
             g.tail_n = mp.narrow;
             nblocks = (int64_t)g.tiles_m * (mp.wide + mp.narrow);
             kern = gemm_x16_mixed_kernel(std::is_same<T, bf16_t>::value, !b_nt);
+            form = "x16_mixed";
           }
         }
         // Output rows off the 128-byte lines: whole tile rows per store instruction (store_tile_rows16).
@@ -2788,6 +2803,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         }
         const bool deep = nblocks * nsplit <= kNumCU;
         lds_bytes = (deep ? 8 : 4) * kTStage;
+        form = deep ? "t64_ring8" : "t64_ring4";
         if (deep) warm_blocks = warm_for(nblocks, 1024);
         if (nsplit > 1 && meet_inside) {
           if (deep) kern = b_nt ? (const void*)gemm_mfma_t64_kernel<T, false, 8, 2> : (const void*)gemm_mfma_t64_kernel<T, true, 8, 2>;
@@ -2803,6 +2819,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         g.tiles_n = (int32_t)((N + 127) / 128);
         nblocks = tiles_mid;
         kern = pick_w4(std::integral_constant<int, 2>{});
+        form = "w4_256x128";
         threads = 256;
         lds_bytes = kGemmLds64;
         warm_blocks = warm_for(nblocks, 768);
@@ -2832,11 +2849,13 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         if (pairs) kern = !split ? pick_small(std::true_type{}, M0{}) : meet_inside ? pick_small(std::true_type{}, M2{}) : pick_small(std::true_type{}, M1{});
         else kern = !split ? pick_small(std::false_type{}, M0{}) : meet_inside ? pick_small(std::false_type{}, M2{}) : pick_small(std::false_type{}, M1{});
         threads = pairs && !four_wave_ring ? 512 : 256;  // the deep-ring kernel: four computing waves and four loaders
+        form = !pairs ? "small_128x128" : four_wave_ring ? "ring4_128x128" : "ring8_128x128";
         // CUs without a tile warm the last-level cache for the others (warm_operands): the deep-ring kernels only,
         // a K loop of 16 stages and more.  gemm_prefetch = N forces that many workgroups per part (a measurement knob).
         if (pairs) warm_blocks = warm_for(nblocks, 1024);
       } else if (ktail) {
         kern = b_nt ? (const void*)gemm_mfma_kernel<T, false, true> : (const void*)gemm_mfma_kernel<T, true, true>;
+        form = "ktail_256x256";
       } else if (K % 64 == 0) {
         // Four waves of 128x128 run the steady state 3-5 % faster and pay ~2 us more per tile
         // (two-pass epilogue), which evens out near K = 2048.  MI355_GEMM_WAVES=4|8 forces one form.
@@ -2845,6 +2864,7 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         lds_bytes = kGemmLds64;
         if (w4) {
           kern = pick_w4(std::integral_constant<int, 4>{});
+          form = "w4_256x256";
           threads = 256;
           // More than one round of tiles with a ragged last round: cut the last columns into 192-wide tiles.
           const bool plain = forced_tile != nullptr && strcmp(forced_tile, "256x256") == 0;
@@ -2855,16 +2875,22 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
               g.tiles_n = mp.wide;
               g.tail_n = mp.narrow;
               nblocks = (int64_t)g.tiles_m * (mp.wide + mp.narrow);
+              form = "w4_mixed";
               if (a_t) kern = b_nt ? (const void*)gemm_mfma_w4_mixed_kernel<T, false, true> : (const void*)gemm_mfma_w4_mixed_kernel<T, true, true>;
               else kern = b_nt ? (const void*)gemm_mfma_w4_mixed_kernel<T, false, false> : (const void*)gemm_mfma_w4_mixed_kernel<T, true, false>;
             }
           }
         } else {
           kern = b_nt ? (const void*)gemm_mfma_dma64_kernel<T, false> : (const void*)gemm_mfma_dma64_kernel<T, true>;
+          form = "dma64_256x256";
         }
       } else {
         kern = b_nt ? (const void*)gemm_mfma_dma_kernel<T, false> : (const void*)gemm_mfma_dma_kernel<T, true>;
+        form = "dma32_256x256";
       }
+      if (g_plan_text != nullptr)
+        return describe_plan(form, g.tiles_m, g.tiles_n + g.tail_n, nblocks + warm_blocks, nsplit, threads, lds_bytes,
+                             x16_split ? xs.splits : nsplit, x16_split || meet_inside ? "inside" : nsplit > 1 ? "launch" : "none", warm_blocks);
       // More than 64 KB of dynamic LDS needs the attribute once per kernel and process.
       static thread_local const void* attr_done[64] = {};
       bool seen = false;
@@ -2929,6 +2955,9 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       else if (deep) kern = MI355_F32_KERNEL(8, 128);
       else kern = MI355_F32_KERNEL(kStages3, 128);
 #undef MI355_F32_KERNEL
+      if (g_plan_text != nullptr)
+        return describe_plan(tile == 64 ? "f32_64x64" : deep ? "f32_128x128_ring8" : "f32_128x128_ring4", g.tiles_m, g.tiles_n, nblocks, nsplit,
+                             256, lds_bytes, nsplit, nsplit > 1 ? "launch" : "none", 0);
       static thread_local const void* attr_done[12] = {};
       bool seen = false;
       for (const void* k : attr_done) seen = seen || k == kern;
@@ -2947,6 +2976,8 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       return finish_splitk<float>(g, nsplit, st);
     }
   }
+  if (g_plan_text != nullptr)
+    return describe_plan(std::is_same<T, double>::value ? "f64_mfma" : "generic", 0, 0, 0, 1, 256, 0, 1, "none", 0);
   if constexpr (std::is_same<T, double>::value) {  // fp64: the MFMA kernel of gemm_f64.hip
     return launch_gemm_f64(static_cast<const double*>(a), a_rs, a_cs, static_cast<const double*>(b), b_rs, b_cs,
                            static_cast<const double*>(c), c_rs, c_cs, static_cast<double*>(out), M, N, K, alpha, beta, st);
@@ -3084,6 +3115,28 @@ extern "C" int mi355_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void*
     case MI355_F64: return run_gemm<double>(a, a_rs, a_cs, b, b_rs, b_cs, c, c_rs, c_cs, out, M, N, K, alpha, beta, workspace, workspace_bytes, st);
     default: return set_error(MI355_ERR_UNSUPPORTED, "mi355_gemm: unsupported dtype %s", dtype_name(dtype));
   }
+}
+
+extern "C" int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int dtype, int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs,
+                               int with_workspace, char* text, int64_t text_bytes) {
+  MI355_REQUIRE(M > 0 && N > 0 && K >= 0 && text != nullptr && text_bytes >= 128, "mi355_gemm_plan: bad argument");
+  // Operand addresses only enter the plan through their alignment: 16-byte aligned stand-ins, never dereferenced.
+  void* const fake = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  void* const ws = with_workspace ? fake : nullptr;
+  const int64_t ws_bytes = with_workspace ? (int64_t(1) << 60) : 0;
+  text[0] = 0;
+  g_plan_text = text;
+  g_plan_cap = text_bytes;
+  int rc;
+  switch (dtype) {
+    case MI355_BF16: rc = run_gemm<bf16_t>(fake, a_rs, a_cs, fake, b_rs, b_cs, nullptr, 0, 0, fake, M, N, K, 1.0, 0.0, ws, ws_bytes, nullptr); break;
+    case MI355_F16: rc = run_gemm<f16_t>(fake, a_rs, a_cs, fake, b_rs, b_cs, nullptr, 0, 0, fake, M, N, K, 1.0, 0.0, ws, ws_bytes, nullptr); break;
+    case MI355_F32: rc = run_gemm<float>(fake, a_rs, a_cs, fake, b_rs, b_cs, nullptr, 0, 0, fake, M, N, K, 1.0, 0.0, ws, ws_bytes, nullptr); break;
+    case MI355_F64: rc = run_gemm<double>(fake, a_rs, a_cs, fake, b_rs, b_cs, nullptr, 0, 0, fake, M, N, K, 1.0, 0.0, ws, ws_bytes, nullptr); break;
+    default: rc = set_error(MI355_ERR_UNSUPPORTED, "mi355_gemm_plan: unsupported dtype %s", dtype_name(dtype));
+  }
+  g_plan_text = nullptr;
+  return rc;
 }
 
 extern "C" int mi355_gemm_f32out(const void* a, int64_t a_rs, int64_t a_cs, const void* b, int64_t b_rs, int64_t b_cs,

@@ -265,6 +265,21 @@ int mi355_gemm_status(void);
  * no counterpart in the reference. */
 int mi355_gemm_tile_columns(int64_t M, int64_t N, int64_t K, int32_t* wide, int32_t* narrow);
 
+/* What mi355_gemm would launch for an [M, K] x [K, N] product of `dtype` with these operand strides
+ * (elements; operands and output taken as 16-byte aligned, no c), with or without a workspace of any
+ * size: one line of text, e.g.
+ *   "form=ring4_128x128 tiles=12x16 grid=224x1 threads=256 lds=163840 parts=1 meet=none warm=32"
+ * form  = the kernel form (x16, x16_persistent, x16_split, x16_mixed, w4_256x256, w4_mixed, w4_256x128,
+ *         ring4_128x128, ring8_128x128, small_128x128, t64_ring8, t64_ring4, dma64_256x256, dma32_256x256,
+ *         ktail_256x256, f32_64x64, f32_128x128_ring8, f32_128x128_ring4, f64_mfma, generic);
+ * tiles = rows x columns of tiles; grid = workgroups per part x parts of K; parts / meet = how many
+ * workgroups share a tile's K range and where they meet ("launch": a summing launch, "inside": in the
+ * one launch); warm = cache-warming workgroups appended per part.  The test knobs apply.  Nothing is
+ * launched and no device is touched: a host-only planning query for tests and documentation, with no
+ * counterpart in the reference.  text_bytes >= 128. */
+int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int dtype, int64_t a_rs, int64_t a_cs, int64_t b_rs,
+                    int64_t b_cs, int with_workspace, char* text, int64_t text_bytes);
+
 /* Measurement only, no counterpart in the reference: the matrix-core instruction stream of the
  * large-tile mm kernel (per wave a 128 x 128 fp32 register tile, 32 v_mfma_f32_32x32x16 per 32-k
  * step) with no memory traffic in the loop.  `blocks` workgroups of four waves run `steps` (a
