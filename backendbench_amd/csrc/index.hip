@@ -235,20 +235,13 @@ __global__ __launch_bounds__(kIxBlock) void gather_rows_lds_kernel(const U* __re
   U* o = out + r * n_idx;
   const bool vec = n_idx % 4 == 0 && per_split % 4 == 0 && (reinterpret_cast<uintptr_t>(ix) & 15) == 0 &&
                    (reinterpret_cast<uintptr_t>(o) % (4 * sizeof(U))) == 0;
-  // The first two batches of indices of every thread are requested before the row is staged, and every
-  // later batch two steps ahead: the index stream (two thirds of the bytes) never waits behind the barrier.
-  constexpr int kAhead = 2;  // batches of indices in flight per thread (one: 23.55 us on [2048,4096] fp32, two: 23.40, four: 24.64)
-  VecN<int64_t, 2> qa[kAhead], qb[kAhead];
+  // The first indices of every thread are requested before the row is staged, and every later batch
+  // one step ahead: the index stream (two thirds of the bytes) never waits behind the barrier.
+  VecN<int64_t, 2> na{}, nb{};
   const int64_t jf = j0 + (int64_t)threadIdx.x * 4;
-  constexpr int64_t kBatch = (int64_t)kIxBlock * 4;
-#pragma unroll
-  for (int d = 0; d < kAhead; ++d) {
-    qa[d] = VecN<int64_t, 2>{};
-    qb[d] = VecN<int64_t, 2>{};
-    if (vec && jf + d * kBatch < j1) {
-      qa[d] = ld_nt<int64_t, 2>(ix + jf + d * kBatch);
-      qb[d] = ld_nt<int64_t, 2>(ix + jf + d * kBatch + 2);
-    }
+  if (vec && jf < j1) {
+    na = ld_nt<int64_t, 2>(ix + jf);
+    nb = ld_nt<int64_t, 2>(ix + jf + 2);
   }
   if (len % UV == 0 && (reinterpret_cast<uintptr_t>(s) & 15) == 0) {
     for (int64_t i = (int64_t)threadIdx.x * UV; i < len; i += (int64_t)kIxBlock * UV)
@@ -258,17 +251,12 @@ __global__ __launch_bounds__(kIxBlock) void gather_rows_lds_kernel(const U* __re
   }
   __syncthreads();
   if (vec) {
-    for (int64_t j = jf; j < j1; j += kBatch) {
-      const VecN<int64_t, 2> a = qa[0], b = qb[0];
-#pragma unroll
-      for (int d = 0; d + 1 < kAhead; ++d) {
-        qa[d] = qa[d + 1];
-        qb[d] = qb[d + 1];
-      }
-      const int64_t jn = j + kAhead * kBatch;
+    for (int64_t j = jf; j < j1; j += (int64_t)kIxBlock * 4) {
+      const VecN<int64_t, 2> a = na, b = nb;
+      const int64_t jn = j + (int64_t)kIxBlock * 4;
       if (jn < j1) {
-        qa[kAhead - 1] = ld_nt<int64_t, 2>(ix + jn);
-        qb[kAhead - 1] = ld_nt<int64_t, 2>(ix + jn + 2);
+        na = ld_nt<int64_t, 2>(ix + jn);
+        nb = ld_nt<int64_t, 2>(ix + jn + 2);
       }
       const int64_t id[4] = {a.v[0], a.v[1], b.v[0], b.v[1]};
       VecN<U, 4> v;
