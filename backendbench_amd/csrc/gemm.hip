@@ -2724,7 +2724,11 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool x16_split = x16_ok && xs.splits > 1 && workspace != nullptr && workspace_bytes >= xs.ws_bytes &&
                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
                              (forced_tile != nullptr ? strncmp(forced_tile, "x16split", 8) == 0
-                                                     : x16_pays && M >= 512 && forced_waves == nullptr && !(mid && K <= 4096));  // (a full round of 256x128 tiles: [2048,4096]x[4096,4096] 73.1 us in two parts here, 68.6 there; [2048,11008]x[11008,4096] 155 against 176)  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
+                                                     // (where the 256x128 form applies it goes first up to K = 3072 with CUs left for its warming
+                                                     // workgroups, and below K = 3072 on 229 - 256 such tiles: there, measured on 21 shapes, the
+                                                     // two forms take 40 - 44 against 47 - 52 us at K = 2048, 56 - 66 against 53 - 57 at 3072 and
+                                                     // 70 - 78 against 65 - 66 at 4096)
+                                                     : x16_pays && M >= 512 && forced_waves == nullptr && !(mid && (K < 3072 || tiles_mid <= 224)));  // (256 rows against 32000 x 4096: 94 us split, 85 unsplit - the planes on top of a weight that is streamed anyway)
       if (x16_split) {
         kern = gemm_x16_splitk_kernel(std::is_same<T, bf16_t>::value, !b_nt);
         form = "x16_split";

@@ -65,9 +65,12 @@ def test_256x128_form_between_one_round_of_128x128_and_one_of_256x128_tiles():
     assert plan(2048, 3136, 2304)["form"] != "w4_256x128"              # K over 3072, 144 tiles
     assert plan(3840, 2048, 2048)["warm"] == 16                        # 240 tiles: 16 CUs left
     assert plan(3584, 3072, 2304, ws=False)["warm"] == 0               # 252 tiles: too few left to stay ahead
-    assert plan(2048, 4096, 4096)["form"] == "w4_256x128"              # a full round, up to K = 4096 ...
+    assert plan(2048, 2048, 3712)["form"] == "w4_256x128"              # 232 tiles: close to a full round, K under 3072 ...
+    assert plan(2048, 3072, 3712)["form"] == "x16_split"               # ... from there two workgroups per 256x256 tile
+    assert plan(2048, 4096, 4096)["form"] == "x16_split"
+    assert plan(2048, 3072, 3712, ws=False)["form"] == "w4_256x128"    # (no workspace, no split)
     p = plan(2048, 11008, 4096)
-    assert p["form"] == "x16_split" and p["parts"] == 2 and p["meet"] == "inside"   # ... two workgroups per 256x256 tile beyond
+    assert p["form"] == "x16_split" and p["parts"] == 2 and p["meet"] == "inside"
     assert plan(2048, 11008, 4096, ws=False)["parts"] == 1
 
 
