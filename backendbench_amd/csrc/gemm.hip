@@ -2680,11 +2680,19 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
       const bool t64_split = ts.nsplit > 1 && M >= 16 && light_b && workspace != nullptr &&
                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
                              workspace_bytes >= split_ws_bytes(ts, M, N, TBM);
+      // More 64x64 tiles than CUs put two workgroups on some CUs, and with a row-major b wider than 1536 columns
+      // (64 columns of a k row are one 128-byte line, 2 N bytes from the next) those then fall behind the 128x128
+      // kernels with K in two parts from K = 2048 on ([512,2048]x[2048,2560] 22.0 -> 17.6 us, [768,2048]x[2048,2560]
+      // 23.2 -> 19.6, [1024,2048]x[2048,1792] 19.9 -> 18.7; at K = 1536 the 64x64 tiles are level or up to 20 % ahead),
+      // with 65 - 256 rows from K = 1536 on ([256,2048]x[2048,5120] 25.7 -> 18.0 us, [256,1536]x[1536,5120] 20.4 ->
+      // 16.8, [128,2048]x[2048,11008] 24.0 -> 20.7).  Narrow products ([3072,2048]x[2048,512]) and a transposed b stay here.
+      const bool t64_crowded_nn = !b_nt && nb64 > kNumCU && N >= 1536 && M > 64;
+      const int64_t t64_k_max = M <= 32 ? 1024 : t64_crowded_nn ? (M <= 256 ? 1024 : 1536) : 2048;
       const bool t64 = !ktail && K % 64 == 0 && !a_t && ld32 &&
                        (forced_tile != nullptr ? strcmp(forced_tile, "64x64") == 0
                                                : (nb128 < kNumCU / 2 || (nb128 == kNumCU / 2 && K < 2048) ||  // (exactly 128 tiles: K = 512 10.0 -> 7.0 us; at K = 2048 the deep-ring 128x128 kernel with its warming workgroups is level on a transposed b, 19 against 21 - 22 us, and ahead on a row-major one)
                                                   ((M <= 64 || N <= 64) && nb64 <= 4 * kNumCU)) && nb64 >= 4 &&
-                                                     (K <= (M <= 32 ? 1024 : 2048) || t64_split ||
+                                                     (K <= t64_k_max || t64_split ||
                                                       // enough 64x64 tiles for the chip: no need to split a long K (a few rows against a 32000 x 4096
                                                       // vocabulary: 48 us, 128x128 tiles 55) - up to K = 4096 for more than one row of tiles: beyond, the
                                                       // 128x128 kernels with K split over the chip are ahead ([512,8192]x[8192,1536]: 42 us here, 31 there;

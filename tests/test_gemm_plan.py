@@ -98,6 +98,16 @@ def test_64x64_tiles_for_few_tiles_and_a_short_k():
     assert p["form"] == "t64_ring8" and p["parts"] > 1 and p["meet"] == "inside"
     assert plan(197, 768, 768)["parts"] == 1
     assert plan(8, 8192, 8192)["form"].endswith("128x128")             # a few rows against 134 MB of weight
+    # more 64x64 tiles than CUs against a wide row-major b: the 128x128 kernels from K = 2048 on (65 - 256 rows: from 1536)
+    assert plan(512, 2048, 2560)["form"] == "t64_ring4"                # (a transposed b stays)
+    p = plan(512, 2048, 2560, nt=False)
+    assert p["form"] == "ring8_128x128" and p["parts"] == 2 and p["meet"] == "inside"
+    assert plan(512, 1536, 2560, nt=False)["form"] == "t64_ring4"
+    assert plan(256, 1536, 5120, nt=False)["form"] == "ring8_128x128"
+    assert plan(256, 1024, 5120, nt=False)["form"] == "t64_ring4"
+    assert plan(192, 2048, 5120, nt=False)["form"] == "t64_ring8"      # 240 tiles: one per CU
+    assert plan(3072, 2048, 512, nt=False)["form"] == "t64_ring4"      # a narrow b
+    assert plan(64, 2048, 11008, nt=False)["form"] == "t64_ring8"      # one row of tiles
 
 
 def test_other_dtypes_and_fallbacks():

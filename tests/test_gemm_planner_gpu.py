@@ -5,7 +5,8 @@
 choosing; this one walks shapes on both sides of every cut-off the planner itself applies -
 256x256-tile counts 64/65, 96, 128/129, 191/192, 228/229, 248/249, 256/257, K = 256, 384, 1024,
 2048, 3072, 4096 (a few tiles), M = 16, 64, 512, a right operand under / over 100 MB, tiles three quarters full or
-less, 128/129, 224/225, 240, 256 tiles of 256x128 with K = 768 and 3072 on both sides - and checks whatever the planner chose against the oracle.
+less, 128/129, 224/225, 240, 256 tiles of 256x128 with K = 768 and 3072 on both sides, more 64x64 tiles than CUs
+against a row-major b of 1536 columns and more with K = 1024, 1536, 2048 on both sides - and checks whatever the planner chose against the oracle.
 
 Operands are small integers (one in four entries of a non-zero), so every sum is an integer far
 inside what bf16 / f16 hold exactly and the order of summation does not matter: bit-equal to the
@@ -120,6 +121,19 @@ def test_planner_boundaries_of_the_256x128_form(backend, grid):
         M = 256 * tm - (56 if ragged else 0)                  # (three quarters of every tile row stay output)
         N = 128 * tn - (40 if ragged else 0)
         _check(backend, M, K, N, layout, dtype, seed=900 * tm + 11 * tn + i, with_bias=(i % 2 == 0))
+
+
+# More 64x64 tiles than CUs: a row-major b of 1536 and more columns moves to the 128x128 kernels from K = 2048 on
+# (65 - 256 rows: from K = 1536 on), a transposed or a narrower one stays on 64x64 tiles.
+@pytest.mark.parametrize("shape", [(512, 2560), (256, 5120), (320, 5120), (264, 4096), (1024, 1792), (1024, 1472), (3072, 512), (64, 11008)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_planner_boundaries_of_crowded_64x64_tiles(backend, shape):
+    M, N = shape
+    print(f"\n[gpu-case] planner boundaries of crowded 64x64 tiles: M = {M}, N = {N}", flush=True)
+    sys.stdout.flush()
+    for i, K in enumerate([1024, 1088, 1536, 1600, 2048]):
+        for layout in ("nn", "nt"):
+            _check(backend, M, K, N, layout, torch.bfloat16 if i % 2 == 0 else torch.float16, seed=13 * M + N + i, with_bias=(i % 2 == 1))
 
 
 @pytest.mark.parametrize("M", [15, 16, 17, 63, 64, 65, 200, 180, 511, 512, 513])
