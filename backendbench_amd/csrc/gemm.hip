@@ -889,8 +889,14 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
   // offset per lane and request (the host checks that they fit: leading dimensions below 4 M elements).
   const T* a_base = A_T ? A : A + (int64_t)bm * g.lda;   // K-contiguous A: offsets are relative to the tile's first row
   const T* b_base = B_NN ? B : B + (int64_t)bn * g.ldb;  // K-contiguous B: relative to the tile's first column
+  // B_PAIR (a K-contiguous B on the 256x128 tile, whose LDS has the room): B is fetched like A, 64 k - one whole
+  // 128-byte line per column - at a time into three pair slots of 128 x 64 (16 KB, swz_k64) instead of four step
+  // slots of 128 x 32.  With 32-k requests every line of B is asked for twice, 64 bytes each time, the second while
+  // the first may still be on its way from HBM.
+  constexpr bool B_PAIR = !B_NN && NJ == 2;
+  constexpr int NB_OFF = B_PAIR ? 4 : NJ;
   uint32_t a_off[8];
-  uint32_t b_off[NJ];
+  uint32_t b_off[NB_OFF];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     if constexpr (A_T) {  // M-contiguous A: the pair slot holds 64 k-rows of 512 B (swz_n), region = two k-rows
@@ -907,8 +913,13 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
     }
   }
 #pragma unroll
-  for (int i = 0; i < NJ; ++i) {
-    if constexpr (B_NN && NJ == 4) {  // 512-byte k-rows (swz_n): region = two k-rows
+  for (int i = 0; i < NB_OFF; ++i) {
+    if constexpr (B_PAIR) {  // 128-byte rows of 64 k (swz_k64): region = eight columns
+      const int r = 8 * (wave + 4 * i) + (lane >> 3), slot = lane & 7;
+      const int c = slot ^ (((r >> 1) & 1) | ((r >> 2) & 6));
+      const int ln = bn + r < g.N ? r : g.N - 1 - bn;
+      b_off[i] = ((uint32_t)ln * (uint32_t)g.ldb + (uint32_t)c * 8u) * 2u;
+    } else if constexpr (B_NN && NJ == 4) {  // 512-byte k-rows (swz_n): region = two k-rows
       const int k = 2 * (wave + 4 * i) + (lane >> 5), pos = lane & 31;
       const int u = (((pos >> 2) ^ (k & 3)) << 2) | (pos & 3);
       int gn = bn + u * 8;
@@ -934,8 +945,12 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
                a_base + (A_T ? (int64_t)t * BK3 * g.lda : (int64_t)t * BK3));
   };
   auto request_b = [&](int i, int t) {
-    lds_dma16s(lds_base + kBRing64 + (uint32_t)(t & 3) * kPanel3 + (uint32_t)(wave + 4 * i) * 1024u, b_off[i],
+    lds_dma16s(lds_base + kBRing64 + (uint32_t)(t & 3) * kPanel3 + (uint32_t)(wave + 4 * i) * 1024u, b_off[i % NB_OFF],
                b_base + (B_NN ? (int64_t)t * BK3 * g.ldb : (int64_t)t * BK3));
+  };
+  // B_PAIR: request i (0..3) of the B pair slot that goes with the A slot at a_slot (steps t, t+1)
+  auto request_b_pair = [&](int i, int t, uint32_t a_slot) {
+    lds_dma16s(lds_base + kBRing64 + a_slot / 2 + (uint32_t)(wave + 4 * i) * 1024u, b_off[i % NB_OFF], b_base + (int64_t)t * BK3);
   };
 
   const int fr = lane & 31, fg = lane >> 5;
@@ -949,10 +964,12 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
   auto io_step = [&](int t, uint32_t a_slot, int half, frag_t (&xa)[2][4], frag_t (&xb)[2][NJA], bool fill_a, int ta,
                      uint32_t fill_slot, int a_first, bool fill_b, int tb) __attribute__((always_inline)) {
     const unsigned char* pa = lds + a_slot;
-    const unsigned char* pb = lds + kBRing64 + (t & 3) * kPanel3;
+    const unsigned char* pb = B_PAIR ? lds + kBRing64 + a_slot / 2 : lds + kBRing64 + (t & 3) * kPanel3;
     auto fill = [&](int q) __attribute__((always_inline)) {
       if (q < 4) {
         if (fill_a) request_a(a_first + q, ta, fill_slot);
+      } else if constexpr (B_PAIR) {  // the B pair follows the A pair: requests 0, 1 with A's 0-3, requests 2, 3 with A's 4-7
+        if (fill_a) request_b_pair(a_first / 2 + q - 4, ta, fill_slot);
       } else if (fill_b) {
         request_b(q - 4, tb);
       }
@@ -982,6 +999,8 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
           const s16x4 lo = lds_read_tr(pb + off_lo + ((n & 7) << 1));
           const s16x4 hi = lds_read_tr(pb + off_hi + ((n & 7) << 1));
           xb[ks][j] = __builtin_bit_cast(frag_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        } else if constexpr (B_PAIR) {
+          xb[ks][j] = *reinterpret_cast<const frag_t*>(pb + swz_k64(wn * (NJA * 32) + j * 32 + fr, half * 4 + ks * 2 + fg));
         } else {
           xb[ks][j] = *reinterpret_cast<const frag_t*>(pb + swz_k32(wn * (NJA * 32) + j * 32 + fr, ks * 2 + fg));
         }
@@ -1056,24 +1075,42 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
   const int nk = g.K / BK3;  // even: K % 64 == 0
 #pragma unroll
   for (int i = 0; i < 8; ++i) request_a(i, 0, 0);
+  if constexpr (B_PAIR) {
 #pragma unroll
-  for (int i = 0; i < NJ; ++i) request_b(i, 0);
+    for (int i = 0; i < 4; ++i) request_b_pair(i, 0, 0);
+    if (nk > 2) {
 #pragma unroll
-  for (int i = 0; i < NJ; ++i) request_b(i, 1);
-  if (nk > 2) {
+      for (int i = 0; i < 8; ++i) request_a(i, 2, kASlot64);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) request_a(i, 2, kASlot64);
+      for (int i = 0; i < 4; ++i) request_b_pair(i, 2, kASlot64);
+      if (nk > 4) {  // what the odd step before step 0 would have asked for: the first half of steps 4, 5
 #pragma unroll
-    for (int i = 0; i < NJ; ++i) request_b(i, 2);
-    if (nk > 4) {
+        for (int i = 0; i < 4; ++i) request_a(i, 4, 2 * kASlot64);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) request_a(i, 4, 2 * kASlot64);
+        for (int i = 0; i < 2; ++i) request_b_pair(i, 4, 2 * kASlot64);
+      }
     }
+  } else {
 #pragma unroll
-    for (int i = 0; i < NJ; ++i) request_b(i, 3);
+    for (int i = 0; i < NJ; ++i) request_b(i, 0);
+#pragma unroll
+    for (int i = 0; i < NJ; ++i) request_b(i, 1);
+    if (nk > 2) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) request_a(i, 2, kASlot64);
+#pragma unroll
+      for (int i = 0; i < NJ; ++i) request_b(i, 2);
+      if (nk > 4) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) request_a(i, 4, 2 * kASlot64);
+      }
+#pragma unroll
+      for (int i = 0; i < NJ; ++i) request_b(i, 3);
+    }
   }
-  // steps 0 and 1 are in when only the 12 + 2 NJ loads behind them still fly
+  // steps 0 and 1 are in when only the 12 + 2 NJ loads behind them still fly (B_PAIR: the 12 of steps 2, 3 and the 6 of 4, 5)
   if (nk > 4 && NJ == 4) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+  else if (nk > 4 && B_PAIR) asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
   else if (nk > 4) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -1153,7 +1190,10 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
 #undef MI355_MD
   // Last steps: the requests thin out.  fills(s) = loads that step s issues; the barrier that
   // ends step s lets exactly those of steps s-1 and s fly, as in the steady state.
-  auto fills = [nk](int s) { return (s & 1) ? NJ * (s + 4 < nk) + 4 * (s + 5 < nk) : (4 + NJ) * (s + 4 < nk); };
+  auto fills = [nk](int s) {
+    if constexpr (B_PAIR) return 6 * ((s & 1) ? s + 5 < nk : s + 4 < nk);
+    else return (s & 1) ? NJ * (s + 4 < nk) + 4 * (s + 5 < nk) : (4 + NJ) * (s + 4 < nk);
+  };
   auto wait_fills = [](int n) {
     switch (n) {
       case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
