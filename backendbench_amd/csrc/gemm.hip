@@ -2883,7 +2883,14 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
         nblocks = (int64_t)g.tiles_m * g.tiles_n;
         const SplitPlan sp = plan_splitk(M, N, K, sizeof(T));
         const int64_t ws_ld = (N + 3) / 4 * 4;
-        const bool split = sp.nsplit > 1 && workspace != nullptr &&
+        // Two parts of K on exactly one round of workgroups (128 tiles x 2) leave no CU for warm_operands and meet
+        // while every CU is busy: with both operands K-contiguous the unsplit launch with its 32 warming workgroups
+        // is ahead up to K = 2048 ([512,2048]x[4096,2048]^T 21.2 -> 19.3 us, [1024,2048]x[2048,2048]^T 20.4 -> 19.0,
+        // [2048,2048]x[1024,2048]^T 21.0 -> 19.0), level at 3072 and behind from 4096 on; a row-major b is 6 % ahead
+        // with the split at K = 2048 already, and so are two rows of tiles against a wide b, which is streamed
+        // more than multiplied ([256,2048]x[8192,2048]^T 23.1 us split, 23.9 unsplit).
+        const bool full_round_nt = b_nt && !a_t && sp.nsplit == 2 && nblocks * 2 >= kNumCU && K <= 2048 && K % 64 == 0 && M >= 512;
+        const bool split = sp.nsplit > 1 && !full_round_nt && workspace != nullptr &&
                            workspace_bytes >= split_ws_bytes(sp, M, N, SBM) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
         if (split) {
           nsplit = sp.nsplit;

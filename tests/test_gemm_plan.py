@@ -83,6 +83,9 @@ def test_128x128_deep_ring_and_its_split():
     assert p["form"] == "ring8_128x128" and p["parts"] >= 3 and p["meet"] == "inside"
     assert plan(1024, 11008, 1024, nt=False, ws=False)["parts"] == 1
     assert plan(1024, 4096, 2048)["parts"] == 2 and plan(1024, 4096, 2048)["warm"] == 0   # 128 tiles x 2 fill the chip
+    p = plan(1024, 2048, 2048)                                         # ... which does not pay up to K = 2048 on a transposed b
+    assert p["parts"] == 1 and p["warm"] == 32
+    assert plan(1024, 2048, 2048, nt=False)["parts"] == 2
     assert plan(2048, 4128, 2048)["form"] == "small_128x128"           # K % 64 != 0: no 64-k pairs
 
 
