@@ -1183,11 +1183,6 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
 #undef MI355_TR_STAMP
 #undef MI355_TR_C0
 #undef MI355_TR_C1
-#undef MI355_W4_SCHEDULE
-#undef MI355_X4
-#undef MI355_MDD
-#undef MI355_MDM
-#undef MI355_MD
   // Last steps: the requests thin out.  fills(s) = loads that step s issues; the barrier that
   // ends step s lets exactly those of steps s-1 and s fly, as in the steady state.
   auto fills = [nk](int s) {
@@ -1207,6 +1202,42 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
       default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
     }
   };
+  if (nk - t == 6) {
+    // The last six steps of any K of 384 and more, written out: which of them still request is known here, so
+    // they keep the steady state's order of MFMAs, reads and requests (in the loop below, whose requests sit
+    // behind run-time conditions, the compiler reads all fragments first and issues the MFMAs in one block:
+    // 1180 clocks a step against 775).  Step t asks for the second half of steps t+4, t+5; step t+1 for b of
+    // step t+5 where b is fetched by the step; nothing after that.
+    constexpr int kPerStep = 4 + NJ;                 // loads a steady-state step issues
+    constexpr int kLateB = B_PAIR ? 0 : NJ;          // loads of step t+1
+    const uint32_t s1 = next_slot(cur), s2 = next_slot(s1);
+    io_step(t + 1, cur, 1, fa[1], fb[1], true, t + 4, s2, 4, true, t + 4);
+    mma_step(fa[0], fb[0]);
+    MI355_W4_SCHEDULE
+    wait_fills(2 * kPerStep);
+    __syncthreads();
+    io_step(t + 2, s1, 0, fa[0], fb[0], false, 0, 0u, 0, !B_PAIR, t + 5);
+    mma_step(fa[1], fb[1]);
+    MI355_W4_SCHEDULE
+    wait_fills(kPerStep + kLateB);
+    __syncthreads();
+    io_step(t + 3, s1, 1, fa[1], fb[1], false, 0, 0u, 0, false, 0);
+    mma_step(fa[0], fb[0]);
+    MI355_W4_SCHEDULE
+    wait_fills(kLateB);
+    __syncthreads();
+    io_step(t + 4, s2, 0, fa[0], fb[0], false, 0, 0u, 0, false, 0);
+    mma_step(fa[1], fb[1]);
+    MI355_W4_SCHEDULE
+    wait_fills(0);
+    __syncthreads();
+    io_step(t + 5, s2, 1, fa[1], fb[1], false, 0, 0u, 0, false, 0);
+    mma_step(fa[0], fb[0]);
+    MI355_W4_SCHEDULE
+    __syncthreads();
+    mma_step(fa[1], fb[1]);
+    t = nk;
+  }
   for (; t < nk; t += 2) {
     const uint32_t nxt = next_slot(cur);
     io_step(t + 1, cur, 1, fa[1], fb[1], t + 4 < nk, t + 4, next_slot(nxt), 4, t + 4 < nk, t + 4);
@@ -1219,6 +1250,11 @@ __device__ __forceinline__ void w4_tile(const GemmArgs& g, unsigned char* lds, c
     __syncthreads();
     cur = nxt;
   }
+#undef MI355_W4_SCHEDULE
+#undef MI355_X4
+#undef MI355_MDD
+#undef MI355_MDM
+#undef MI355_MD
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing is in flight: the last two steps issue no fills)
 #ifdef MI355_GEMM_TRACE
   const uint64_t tr_drained = __builtin_readcyclecounter();
@@ -1658,9 +1694,6 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
     asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
     __syncthreads();
   }
-#undef MI355_PAIR_SCHEDULE
-#undef MI355_X4
-#undef MI355_MDD
   // Last steps: the requests stop at pair np-1; each barrier lets the loads of its last three steps fly.
   auto fills = [np](int q) { return q + 5 < np ? 8 : 0; };
   auto wait_fills = [](int n) {
@@ -1669,6 +1702,35 @@ __global__ __launch_bounds__(256) void gemm_mfma_small2_kernel(GemmArgs g) {
     else if (n == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
+  // The last five or six pairs of a K loop that reached the steady state, written out: which of them still
+  // request (only the first of six) is known at compile time, so they keep the steady state's order of MFMAs and
+  // reads; the loop below decides per step and leaves the order to the compiler.
+  auto last_pairs = [&](auto count) __attribute__((always_inline)) {
+    constexpr int R = decltype(count)::value;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      if (i + 1 < R) {
+        if (i + 5 < R) read_pair(p + i + 1, fa[(i + 1) & 1], fb[(i + 1) & 1], [&](int f) { request(f, p + i + 5); });
+        else read_pair(p + i + 1, fa[(i + 1) & 1], fb[(i + 1) & 1], [](int) {});
+      }
+      mma_pair(fa[i & 1], fb[i & 1]);
+      if (i + 1 < R) {
+        MI355_PAIR_SCHEDULE
+      }
+      wait_fills(8 * ((i - 2 < R - 5) + (i - 1 < R - 5) + (i < R - 5)));  // fills(q - 2) + fills(q - 1) + fills(q), q = p + i
+      __syncthreads();
+    }
+  };
+  if (np - p == 6) {
+    last_pairs(std::integral_constant<int, 6>{});
+    p = np;
+  } else if (np - p == 5) {
+    last_pairs(std::integral_constant<int, 5>{});
+    p = np;
+  }
+#undef MI355_PAIR_SCHEDULE
+#undef MI355_X4
+#undef MI355_MDD
   for (; p < np; p += 2) {
     if (p + 1 < np) {
       const bool fill = p + 5 < np;
@@ -2057,7 +2119,29 @@ __global__ __launch_bounds__(256) void gemm_mfma_t64_kernel(GemmArgs g) {
     request_stage(t + 1 + S);
     mma_stage(fa[1], fb[1]);
   }
-  for (; t < nk; t += 2) {  // the last S + 1 steps or fewer: requests and reads run out
+  // The last S or S + 1 steps of a K loop that reached the steady state, written out: what each of them still
+  // waits for, reads and requests is known at compile time (the loop below decides it per step with a dozen
+  // branches, which cost a 64-k step about as much as its four MFMAs).
+  auto last_steps = [&](auto count) __attribute__((always_inline)) {
+    constexpr int R = decltype(count)::value;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const int left = R - i;  // steps to go, this one included
+      if (left > 1) wait_younger(left > S ? S - 2 : left - 2);
+      __syncthreads();
+      if (left > 1) read_frags(t + i + 1, fa[(i + 1) & 1], fb[(i + 1) & 1]);
+      if (left > S) request_stage(t + i + S);
+      mma_stage(fa[i & 1], fb[i & 1]);
+    }
+  };
+  if (nk - t == S + 1) {
+    last_steps(std::integral_constant<int, S + 1>{});
+    t = nk;
+  } else if (nk - t == S) {
+    last_steps(std::integral_constant<int, S>{});
+    t = nk;
+  }
+  for (; t < nk; t += 2) {  // a K loop shorter than the ring: requests and reads run out
     step(t, fa[0], fb[0], fa[1], fb[1]);
     if (t + 1 < nk) step(t + 1, fa[1], fb[1], fa[0], fb[0]);
   }
