@@ -1487,7 +1487,6 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
     asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     __syncthreads();
   }
-#undef MI355_SMALL_SCHEDULE
   // Last steps: the requests stop at tile nk-1; each barrier lets the loads of its last two steps fly.
   auto fills = [nk](int q) { return q + 4 < nk ? 4 : 0; };
   auto wait_fills = [](int n) {
@@ -1495,6 +1494,33 @@ __global__ __launch_bounds__(256) void gemm_mfma_small_kernel(GemmArgs g) {
     else if (n == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
+  // The last four or five steps of a K loop that reached the steady state, written out: which of them still
+  // request (only the first of five) is known at compile time, so they keep the steady state's order of MFMAs
+  // and reads; the loop below decides per step.
+  auto last_tiles = [&](auto count) __attribute__((always_inline)) {
+    constexpr int R = decltype(count)::value;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      if (i + 1 < R) {
+        if (i + 4 < R) read_tile(it + i + 1, fa[(i + 1) & 1], fb[(i + 1) & 1], [&](int f) { request1(f, it + i + 4); });
+        else read_tile(it + i + 1, fa[(i + 1) & 1], fb[(i + 1) & 1], [](int) {});
+      }
+      mma_tile(fa[i & 1], fb[i & 1]);
+      if (i + 1 < R) {
+        MI355_SMALL_SCHEDULE
+      }
+      wait_fills(4 * ((i - 1 < R - 4) + (i < R - 4)));  // fills(q - 1) + fills(q), q = it + i
+      __syncthreads();
+    }
+  };
+  if (nk - it == 5) {
+    last_tiles(std::integral_constant<int, 5>{});
+    it = nk;
+  } else if (nk - it == 4) {
+    last_tiles(std::integral_constant<int, 4>{});
+    it = nk;
+  }
+#undef MI355_SMALL_SCHEDULE
   for (; it < nk; it += 2) {
     if (it + 1 < nk) {
       const bool fill = it + 4 < nk;
@@ -2784,8 +2810,12 @@ static int run_gemm(const void* a, int64_t a_rs, int64_t a_cs, const void* b, in
                                                       // into the last-level cache it is ahead of the 128x128 kernels with two workgroups on
                                                       // a CU and of two parts of K on 256x256 tiles ([4096,1536]x[1536,1536]^T 35.1 ->
                                                       // 29.4 us, [2048,1536]x[1536,2304] 32.9 -> 25.7, [3072,768]x[2048,768]^T 21.6 -> 18.9;
-                                                      // level at K = 512 and from K = 4096 on).
-                                                      (K >= 768 && K <= 3072 && tiles_mid > kNumCU / 2)) &&
+                                                      // level from K = 4096 on.  Below K = 768 no warming workgroups are added,
+                                                      // and with the last six steps of its K loop written out this form is 17 - 30 %
+                                                      // ahead of two 128x128 workgroups per CU there too, on either layout of b:
+                                                      // [2048,512]x[512,3072] 20.1 -> 15.4 us, [4096,256]x[1536,256]^T 14.3 -> 11.4,
+                                                      // [1024,640]x[640,6144] 24.4 -> 17.5; 85 shapes, K = 256 .. 704).
+                                                      (K >= 256 && K <= 3072 && tiles_mid > kNumCU / 2)) &&
                                                      4 * M >= 3 * (int64_t)g.tiles_m * BM);  // rows that are mostly output ([128,4096]x[4096,32000]: 74 us here, 61 on 128x128 tiles)
       // Fewer 128x128 tiles than half the CUs: 64x64 tiles reach four times as many (measured on this
       // chip: [197,768]x[768,768] 11.6 -> 7.5 us, 1024^3 14.6 -> 9.4 us).  A 64x64 workgroup walks K at

@@ -60,7 +60,10 @@ def test_256x128_form_between_one_round_of_128x128_and_one_of_256x128_tiles():
     assert plan(2048, 768, 2304, nt=False)["form"] == "w4_256x128"
     assert plan(2048, 768, 2048)["form"] != "w4_256x128"               # 128 tiles of 256x128: one round of 128x128 tiles
     assert plan(2048, 768, 2176)["form"] == "w4_256x128"               # 136
-    assert plan(2048, 704, 2304)["form"] != "w4_256x128"               # K under 768
+    p = plan(2048, 704, 2304)
+    assert p["form"] == "w4_256x128" and p["warm"] == 0               # K under 768: no warming workgroups
+    assert plan(2048, 256, 2304, nt=False)["form"] == "w4_256x128"
+    assert plan(2048, 192, 2304)["form"] != "w4_256x128"              # K under 256
     assert plan(2048, 3072, 2304)["form"] == "w4_256x128"
     assert plan(2048, 3136, 2304)["form"] != "w4_256x128"              # K over 3072, 144 tiles
     assert plan(3840, 2048, 2048)["warm"] == 16                        # 240 tiles: 16 CUs left

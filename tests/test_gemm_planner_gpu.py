@@ -5,7 +5,7 @@
 choosing; this one walks shapes on both sides of every cut-off the planner itself applies -
 256x256-tile counts 64/65, 96, 128/129, 191/192, 228/229, 248/249, 256/257, K = 256, 384, 1024,
 2048, 3072, 4096 (a few tiles), M = 16, 64, 512, a right operand under / over 100 MB, tiles three quarters full or
-less, 128/129, 224/225, 240, 256 tiles of 256x128 with K = 768 and 3072 on both sides, more 64x64 tiles than CUs
+less, 128/129, 224/225, 240, 256 tiles of 256x128 with K = 256 and 3072 on both sides, more 64x64 tiles than CUs
 against a row-major b of 1536 columns and more with K = 1024, 1536, 2048 on both sides - and checks whatever the planner chose against the oracle.
 
 Operands are small integers (one in four entries of a non-zero), so every sum is an integer far
@@ -103,7 +103,7 @@ def test_planner_boundaries_in_k_for_a_few_tiles(backend, grid):
         _check(backend, 256 * tm - (24 if i % 3 == 2 else 0), K, 256 * tn, layout, dtype, seed=31 * tm + 7 * tn + i, with_bias=(i % 2 == 0))
 
 
-# The 256x128 form takes 129 - 256 tiles of 256x128 (under 192 tiles of 256x256) for K = 768 .. 3072, and above
+# The 256x128 form takes 129 - 256 tiles of 256x128 (under 192 tiles of 256x256) for K = 256 .. 3072, and above
 # 228 / 248 such tiles from K = 1024 on; with 16 and more CUs left over it adds cache-warming workgroups.
 # (rows of 256, columns of 128): 128 / 136 / 224 / 232 / 240 / 245 / 256 tiles of 256x128
 _MID_GRIDS = [(8, 16), (8, 17), (8, 28), (8, 29), (15, 16), (7, 35), (16, 16), (4, 33)]
@@ -114,7 +114,7 @@ def test_planner_boundaries_of_the_256x128_form(backend, grid):
     tm, tn = grid
     print(f"\n[gpu-case] planner boundaries of the 256x128 form: {tm} x {tn} tiles", flush=True)
     sys.stdout.flush()
-    for i, K in enumerate([704, 768, 1024, 2048, 3072, 3136]):
+    for i, K in enumerate([192, 256, 704, 1024, 2048, 3072, 3136]):
         layout = "nt" if (i + tm + tn) % 2 else "nn"
         dtype = torch.bfloat16 if i % 2 == 0 else torch.float16
         ragged = i % 3 == 1
