@@ -1281,7 +1281,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_w4_kernel(GemmArgs g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   if ((int)blockIdx.x >= g.tiles_m * g.tiles_n) return warm_operands<T, A_T, B_NN>(g, 0, g.K);
   int tm, tn;
-  tile_coords(g, tm, tn);
+  tile_coords<NJ == 2 ? 4 : 8>(g, tm, tn);
   // the fill requests take their bases in SGPRs: the tile origin is uniform, say so
   w4_tile<T, B_NN, NJ, A_T>(g, lds, __builtin_amdgcn_readfirstlane(tm * BM), __builtin_amdgcn_readfirstlane(tn * (NJ * 64)));
 }

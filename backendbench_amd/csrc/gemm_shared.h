@@ -50,8 +50,10 @@ struct GemmArgs {
 };
 
 // Tile id for this block: blocks land on XCD (blockIdx % 8); give each XCD a contiguous
-// band of tile ids, then walk the band in groups of 8 tile-rows so A and B panels repeat
-// in that XCD's L2.
+// band of tile ids, then walk the band in groups of GROUP tile-rows so A and B panels repeat
+// in that XCD's L2 (32 tiles of an XCD: 8 rows x 4 columns of square tiles; 256x128 tiles take 4 rows x 8
+// columns, 1024 + 1024 operand rows per XCD instead of 2048 + 512).
+template <int GROUP = 8>
 __device__ __forceinline__ void tile_coords(const int tiles_m, const int tiles_n, int pid, int& tm, int& tn) {
   const int nblocks = tiles_m * tiles_n;
   const int per_xcd = (nblocks + kNumXCD - 1) / kNumXCD;
@@ -59,7 +61,6 @@ __device__ __forceinline__ void tile_coords(const int tiles_m, const int tiles_n
   const int xcd = pid % kNumXCD, local = pid / kNumXCD;
   if (full == 0) pid = xcd * per_xcd + local;
   else pid = (xcd < full ? xcd * per_xcd : full * per_xcd + (xcd - full) * (per_xcd - 1)) + local;
-  constexpr int GROUP = 8;
   const int in_group = GROUP * tiles_n;
   const int group = pid / in_group;
   const int first_m = group * GROUP;
@@ -67,8 +68,9 @@ __device__ __forceinline__ void tile_coords(const int tiles_m, const int tiles_n
   tm = first_m + (pid % in_group) % rows;
   tn = (pid % in_group) / rows;
 }
+template <int GROUP = 8>
 __device__ __forceinline__ void tile_coords(const GemmArgs& g, int& tm, int& tn) {
-  tile_coords(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
+  tile_coords<GROUP>(g.tiles_m, g.tiles_n, blockIdx.x, tm, tn);
 }
 
 // Epilogue of the MFMA kernels for output rows that start at any 2-byte offset (N % 8 != 0: a 50257-wide
